@@ -1,0 +1,129 @@
+"""CPU oracle for the storage-access path.  TEST INFRASTRUCTURE ONLY.
+
+Only tests/, the smoke check and the benchmark's CPU-baseline leg may import
+this package; the shipped library never does.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = None
+
+u64 = ctypes.c_uint64
+u32 = ctypes.c_uint32
+_p64 = np.ctypeslib.ndpointer(dtype=np.uint64, flags="C_CONTIGUOUS")
+_p32 = np.ctypeslib.ndpointer(dtype=np.uint32, flags="C_CONTIGUOUS")
+
+
+def build(force=False):
+    """Compile the C oracle in place (gcc, seconds)."""
+    so = os.path.join(_HERE, "libbam_oracle.so")
+    if force and os.path.exists(so):
+        os.remove(so)
+    subprocess.run(["make", "-s", "-C", _HERE], check=True)
+    return so
+
+
+def lib():
+    global _LIB
+    if _LIB is not None:
+        return _LIB
+    so = os.path.join(_HERE, "libbam_oracle.so")
+    if not os.path.exists(so):
+        build()
+    L = ctypes.CDLL(so)
+    sig = {
+        "bo_splitmix64": (u64, [u64, u64]),
+        "bo_fill_store": (None, [u64, u64, u64, _p64]),
+        "bo_store_sum": (u64, [u64, u64, u64, u64]),
+        "bo_gather_indices": (None, [u64, u64, u64, u64, _p64]),
+        "bo_gather_sum": (u64, [u64, u64, u64, u64, u64]),
+        "bo_block_lbas": (None, [u64, u64, u64, u64, u32, u32, _p64]),
+        "bo_block_checksum": (u64, [u64, u64, u32, u32]),
+        "bo_rmat_edges": (None, [u64, u32, u64, u64, _p64, _p64]),
+        "bo_uniform_edges": (None, [u64, u64, u64, u64, _p64, _p64]),
+        "bo_build_csr": (u64, [u64, u64, _p64, _p64, _p64, _p64]),
+        "bo_bfs_sources": (None, [u64, u64, _p64, u32, _p64]),
+        "bo_bfs_levels": (u32, [u64, _p64, _p64, u64, _p32]),
+        "bo_bfs_levels_sweep": (u32, [u64, _p64, _p64, u64, _p32]),
+        "bo_cc_labels": (u64, [u64, _p64, _p64, _p64]),
+        "bo_cc_labels_sweep": (u64, [u64, _p64, _p64, _p64, ctypes.POINTER(u32)]),
+        "bo_bfs_edges_scanned": (u64, [u64, _p64, _p32]),
+        "bo_cmd_rw": (None, [_p32, ctypes.c_uint16, ctypes.c_uint8, u32, u64, u64, u64, ctypes.c_uint16]),
+    }
+    for name, (res, args) in sig.items():
+        f = getattr(L, name)
+        f.restype = res
+        f.argtypes = args
+    _LIB = L
+    return L
+
+
+# ---- convenience wrappers -------------------------------------------------
+
+def store(seed, first, n):
+    out = np.empty(n, dtype=np.uint64)
+    lib().bo_fill_store(seed, first, n, out)
+    return out
+
+
+def gather_indices(seed, first_k, n, n_elems):
+    out = np.empty(n, dtype=np.uint64)
+    lib().bo_gather_indices(seed, first_k, n, n_elems, out)
+    return out
+
+
+def block_lbas(seed, first_k, n, ns_bytes, req_bytes, lba_bytes):
+    out = np.empty(n, dtype=np.uint64)
+    lib().bo_block_lbas(seed, first_k, n, ns_bytes, req_bytes, lba_bytes, out)
+    return out
+
+
+def rmat_csr(seed, scale, edge_factor=16):
+    n_v, n_p = 1 << scale, edge_factor << scale
+    u = np.empty(n_p, dtype=np.uint64)
+    v = np.empty(n_p, dtype=np.uint64)
+    lib().bo_rmat_edges(seed, scale, 0, n_p, u, v)
+    return _csr(n_v, u, v)
+
+
+def uniform_csr(seed, n_vertices, n_pairs):
+    u = np.empty(n_pairs, dtype=np.uint64)
+    v = np.empty(n_pairs, dtype=np.uint64)
+    lib().bo_uniform_edges(seed, n_vertices, 0, n_pairs, u, v)
+    return _csr(n_vertices, u, v)
+
+
+def _csr(n_v, u, v):
+    off = np.empty(n_v + 1, dtype=np.uint64)
+    nb = np.empty(max(2 * len(u), 1), dtype=np.uint64)
+    e = lib().bo_build_csr(n_v, len(u), u, v, off, nb)
+    return off, nb[:e].copy()
+
+
+def bfs_sources(seed, offsets, n_src=8):
+    out = np.empty(n_src, dtype=np.uint64)
+    lib().bo_bfs_sources(seed, len(offsets) - 1, offsets, n_src, out)
+    return out
+
+
+def bfs_levels(offsets, neigh, src, sweep=False):
+    lv = np.empty(len(offsets) - 1, dtype=np.uint32)
+    nb = neigh if len(neigh) else np.zeros(1, dtype=np.uint64)
+    f = lib().bo_bfs_levels_sweep if sweep else lib().bo_bfs_levels
+    iters = f(len(offsets) - 1, offsets, nb, int(src), lv)
+    return lv, iters
+
+
+def cc_labels(offsets, neigh, sweep=False):
+    lb = np.empty(len(offsets) - 1, dtype=np.uint64)
+    nb = neigh if len(neigh) else np.zeros(1, dtype=np.uint64)
+    if sweep:
+        it = u32(0)
+        comps = lib().bo_cc_labels_sweep(len(offsets) - 1, offsets, nb, lb, ctypes.byref(it))
+        return lb, comps, it.value
+    comps = lib().bo_cc_labels(len(offsets) - 1, offsets, nb, lb)
+    return lb, comps

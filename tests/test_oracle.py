@@ -1,0 +1,153 @@
+"""Pins the CPU oracle: golden vectors, library routines, an independent numpy restatement."""
+import json
+import os
+
+import numpy as np
+import pytest
+import scipy.sparse as sp
+import scipy.sparse.csgraph as csg
+
+import oracle
+from oracle import oracle_np as onp
+
+G = os.path.join(os.path.dirname(__file__), "golden")
+
+
+def _j(name):
+    with open(os.path.join(G, name)) as f:
+        return json.load(f)
+
+
+def test_splitmix64_published_vectors():
+    g = _j("splitmix64.json")
+    L = oracle.lib()
+    assert [L.bo_splitmix64(1234567, i) for i in range(5)] == [int(x) for x in g["seed_1234567"]]
+    assert [L.bo_splitmix64(0, i) for i in range(3)] == [int(x, 16) for x in g["seed_0"]]
+    # the sequential generator form: state += golden; out = mix(state)
+    state, out = 1234567, []
+    for _ in range(5):
+        state = (state + 0x9E3779B97F4A7C15) & (2**64 - 1)
+        z = state
+        z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & (2**64 - 1)
+        z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & (2**64 - 1)
+        out.append(z ^ (z >> 31))
+    assert out == [int(x) for x in g["seed_1234567"]]
+
+
+def test_store_sums_closed_form():
+    g = _j("splitmix64.json")
+    L = oracle.lib()
+    for seed in (0, 42):
+        assert L.bo_store_sum(seed, 0, 1, 4096) == int(g["sum_first_4096"][str(seed)], 16)
+        assert L.bo_store_sum(seed, 0, 8, 1 << 21) == int(g["cfg1_stride8_sum_2p21"][str(seed)], 16)
+        ref = int(np.sum(onp.splitmix64(seed, np.arange(0, 1 << 24, 8, dtype=np.uint64)), dtype=np.uint64))
+        assert ref == int(g["cfg1_stride8_sum_2p21"][str(seed)], 16)
+
+
+def test_store_and_gather_match_numpy():
+    s = oracle.store(42, 1000, 5000)
+    assert np.array_equal(s, onp.splitmix64(42, np.arange(1000, 6000, dtype=np.uint64)))
+    idx = oracle.gather_indices(42, 7, 4096, 1 << 20)
+    ref = onp.splitmix64(42 ^ 0x5eed, np.arange(7, 7 + 4096, dtype=np.uint64)) % np.uint64(1 << 20)
+    assert np.array_equal(idx, ref)
+    tot = int(np.sum(onp.splitmix64(42, ref), dtype=np.uint64))
+    assert oracle.lib().bo_gather_sum(42, 42, 7, 4096, 1 << 20) == tot
+
+
+def test_block_lbas_and_checksum():
+    lb = oracle.block_lbas(42, 0, 1000, 64 << 30, 4096, 512)
+    ref = (onp.splitmix64(42, np.arange(1000, dtype=np.uint64)) % np.uint64((64 << 30) // 4096)) * np.uint64(8)
+    assert np.array_equal(lb, ref)
+    assert int(lb.max()) * 512 + 4096 <= 64 << 30
+    for lba in (0, 8, int(lb[3])):
+        w0 = lba * 64
+        ref = int(np.sum(onp.splitmix64(7, np.arange(w0, w0 + 512, dtype=np.uint64)), dtype=np.uint64))
+        assert oracle.lib().bo_block_checksum(7, lba, 512, 4096) == ref
+
+
+def test_sqe_image_matches_nvme_spec_layout():
+    d = np.zeros(16, dtype=np.uint32)
+    oracle.lib().bo_cmd_rw(d, 0xBEEF, 0x02, 1, 0x1122334455667000, 0xAABBCCDD00112000, 0x0123456789ABCDEF, 8)
+    b = d.tobytes()
+    assert len(b) == 64
+    assert b[0] == 0x02 and b[1] == 0x00          # opcode, FUSE/PSDT = 0
+    assert b[2:4] == bytes([0xEF, 0xBE])          # CID, little endian
+    assert b[4:8] == (1).to_bytes(4, "little")    # NSID
+    assert b[8:24] == bytes(16)                   # CDW2-3, MPTR
+    assert b[24:32] == (0x1122334455667000).to_bytes(8, "little")   # PRP1
+    assert b[32:40] == (0xAABBCCDD00112000).to_bytes(8, "little")   # PRP2
+    assert b[40:48] == (0x0123456789ABCDEF).to_bytes(8, "little")   # SLBA
+    assert b[48:50] == (7).to_bytes(2, "little")  # NLB is zero based
+    assert b[50:64] == bytes(14)
+
+
+def test_reference_sample_graph():
+    g = _j("sample_graph.json")
+    off = np.array(g["offsets"], dtype=np.uint64)
+    nb = np.array(g["edges"], dtype=np.uint64)
+    for src, exp in g["bfs"].items():
+        for sweep in (False, True):
+            lv, it = oracle.bfs_levels(off, nb, int(src), sweep=sweep)
+            assert lv.tolist() == exp["levels"], (src, sweep)
+            assert it == exp["iterations"], (src, sweep)
+    lb, comps = oracle.cc_labels(off, nb)
+    assert lb.tolist() == g["cc"]["labels"] and comps == g["cc"]["components"]
+    lb2, comps2, _ = oracle.cc_labels(off, nb, sweep=True)
+    assert lb2.tolist() == g["cc"]["labels"] and comps2 == 2
+
+
+@pytest.mark.parametrize("scale", [6, 10, 13])
+def test_rmat_generator_and_csr_match_numpy(scale):
+    n = 16 << scale
+    u = np.empty(n, dtype=np.uint64)
+    v = np.empty(n, dtype=np.uint64)
+    oracle.lib().bo_rmat_edges(42, scale, 0, n, u, v)
+    u2, v2 = onp.rmat_edges(42, scale, 0, n)
+    assert np.array_equal(u, u2) and np.array_equal(v, v2)
+    assert int(u.max()) < (1 << scale) and int(v.max()) < (1 << scale)
+    # quadrant (0,0) must dominate: about a^scale-ish skew, at least more low ids than high
+    assert (u < (1 << (scale - 1))).mean() > 0.7
+    off, nb = oracle.rmat_csr(42, scale)
+    off2, nb2 = onp.build_csr(1 << scale, u2, v2)
+    assert np.array_equal(off, off2) and np.array_equal(nb, nb2)
+    # symmetric, no self loops, sorted unique rows
+    A = sp.csr_matrix((np.ones(len(nb), dtype=np.int8), nb.astype(np.int64), off.astype(np.int64)), shape=(1 << scale,) * 2)
+    assert (A != A.T).nnz == 0 and A.diagonal().sum() == 0
+    for r in range(0, 1 << scale, 97):
+        row = nb[int(off[r]):int(off[r + 1])]
+        assert np.all(row[1:] > row[:-1])
+
+
+def _scipy_graph(off, nb):
+    n = len(off) - 1
+    return sp.csr_matrix((np.ones(len(nb), dtype=np.int8), nb.astype(np.int64), off.astype(np.int64)), shape=(n, n))
+
+
+@pytest.mark.parametrize("seed,scale", [(42, 8), (0, 11), (7, 13)])
+def test_bfs_against_scipy(seed, scale):
+    off, nb = oracle.rmat_csr(seed, scale)
+    A = _scipy_graph(off, nb)
+    for src in oracle.bfs_sources(seed, off, 4):
+        d = csg.shortest_path(A, method="D", unweighted=True, indices=int(src))
+        exp = np.where(np.isinf(d), 0xFFFFFFFF, d).astype(np.uint32)
+        lv, it = oracle.bfs_levels(off, nb, src)
+        lv2, it2 = oracle.bfs_levels(off, nb, src, sweep=True)
+        assert np.array_equal(lv, exp) and np.array_equal(lv2, exp)
+        assert it == it2 == int(exp[exp != 0xFFFFFFFF].max()) + 1
+        assert off[int(src) + 1] > off[int(src)]
+
+
+@pytest.mark.parametrize("n_v,n_p", [(64, 40), (1000, 700), (5000, 9000)])
+def test_cc_against_scipy(n_v, n_p):
+    off, nb = oracle.uniform_csr(42, n_v, n_p)
+    u, v = onp.uniform_edges(42, n_v, 0, n_p)
+    off2, nb2 = onp.build_csr(n_v, u, v)
+    assert np.array_equal(off, off2) and np.array_equal(nb, nb2)
+    ncomp, lab = csg.connected_components(_scipy_graph(off, nb), directed=False)
+    lb, comps = oracle.cc_labels(off, nb)
+    lb2, comps2, iters = oracle.cc_labels(off, nb, sweep=True)
+    assert comps == comps2 == ncomp and np.array_equal(lb, lb2) and iters >= 1
+    # label = smallest vertex id of the component
+    mins = np.full(ncomp, n_v, dtype=np.int64)
+    np.minimum.at(mins, lab, np.arange(n_v))
+    assert np.array_equal(lb.astype(np.int64), mins[lab])
