@@ -1,0 +1,770 @@
+// C-ABI of the GPU-side storage-access path: handle management over the C++
+// host objects (ctrl.h, page_cache.h) and the gfx950 kernels that drive them.
+// Kernel shapes follow the reference's benchmark kernels (cited per kernel);
+// lane arithmetic is for 64-wide waves.
+#include "bam_amd.h"
+
+#include <hip/hip_runtime.h>
+#include <cerrno>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <thread>
+#include <vector>
+
+#include "ctrl.h"
+#include "event.h"
+#include "nvmt.h"
+#include "page_cache.h"
+
+// ---------------------------------------------------------------------------
+// error plumbing
+// ---------------------------------------------------------------------------
+static thread_local std::string g_err;
+
+#define BAM_API_BEGIN try {
+#define BAM_API_END                                                        \
+    return 0;                                                              \
+    } catch (const std::exception& e) { g_err = e.what(); return EIO; }    \
+      catch (...) { g_err = "unknown error"; return EIO; }
+
+static int fail(int code, const char* msg) { g_err = msg; return code; }
+
+struct bam_target {
+    nvmt_t* t = nullptr;
+    void* bar = nullptr;
+    void* backing = nullptr;
+    size_t backing_bytes = 0;
+    nvmt_config_t cfg{};
+};
+struct bam_ctrl { Controller* c; };
+struct bam_page_cache { page_cache_t* pc; Controller* ctrl; };
+struct bam_range { range_t<uint64_t>* r; };
+struct bam_array { array_t<uint64_t>* a; };
+
+// ---------------------------------------------------------------------------
+// device helpers
+// ---------------------------------------------------------------------------
+namespace {
+
+__device__ __forceinline__ uint64_t mix64(uint64_t z)
+{
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+__device__ __forceinline__ uint64_t splitmix64(uint64_t seed, uint64_t i) { return mix64(seed + (i + 1) * 0x9E3779B97F4A7C15ull); }
+
+/* sum over the 64 lanes of a wave (all lanes active); result valid in every lane */
+__device__ __forceinline__ uint64_t wave_sum(uint64_t v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += bam::shfl(v, bam::lane() ^ o);
+    return v;
+}
+
+/* add this block's values into *sum with one atomic per wave */
+__device__ __forceinline__ void block_accumulate(unsigned long long* sum, uint64_t v)
+{
+    v = wave_sum(v);
+    if (bam::lane() == 0 && v) atomicAdd(sum, (unsigned long long)v);
+}
+
+// ---- array benchmark (benchmarks/array/main.cu:43-65), with a checksum ----
+__global__ void k_array_read(array_d_t<uint64_t>* dr, uint64_t n_reqs, const uint64_t* assignment, uint64_t stride, uint64_t reqs_per_thread, unsigned long long* sum)
+{
+    const uint64_t tid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    uint64_t v = 0;
+    if (tid < n_reqs) {
+        const uint64_t idx = assignment ? assignment[tid] : tid * stride;
+        for (uint64_t i = 0; i < reqs_per_thread; i++) v += (*dr)[idx];
+    }
+    block_accumulate(sum, v);
+}
+
+__global__ void k_array_write(array_d_t<uint64_t>* dr, uint64_t n_reqs, const uint64_t* assignment, uint64_t stride, const uint64_t* values)
+{
+    const uint64_t tid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (tid < n_reqs) (*dr)(assignment ? assignment[tid] : tid * stride, values[tid]);
+}
+
+// ---- cache / pattern benchmark (benchmarks/cache/main.cu:44-114): a wave streams whole pages ----
+template <int MODE>
+__global__ __launch_bounds__(256) void k_cache_stream(array_d_t<uint64_t>* dr, uint64_t n_waves, uint64_t n_pages_per_wave, const uint64_t* assignment, unsigned long long* sum)
+{
+    const uint64_t tid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const uint64_t wave = tid / BAM_WAVE_SIZE, lane = tid % BAM_WAVE_SIZE;
+    uint64_t v = 0;
+    if (wave < n_waves) {
+        range_d_t<uint64_t>* r0 = dr->d_ranges;
+        const uint64_t epp = r0->n_elems_per_page;
+        const uint64_t start_page = assignment ? assignment[wave] : wave * n_pages_per_wave;
+        if (MODE == 2) {
+            /* one acquire per page, then 16 bytes per lane per load */
+            for (uint64_t p = 0; p < n_pages_per_wave; p++) {
+                data_page_t* pg; size_t s, e; int64_t r;
+                const uint4* base = (const uint4*)dr->acquire_page((start_page + p) * epp, pg, s, e, r);
+                const uint32_t n16 = (uint32_t)(r0->cache.page_size / 16);
+                uint64_t a0 = 0, a1 = 0;
+                for (uint32_t i = (uint32_t)lane; i < n16; i += 4 * BAM_WAVE_SIZE) {
+                    uint4 x0 = base[i], x1 = {0, 0, 0, 0}, x2 = {0, 0, 0, 0}, x3 = {0, 0, 0, 0};
+                    if (i + BAM_WAVE_SIZE < n16) x1 = base[i + BAM_WAVE_SIZE];
+                    if (i + 2 * BAM_WAVE_SIZE < n16) x2 = base[i + 2 * BAM_WAVE_SIZE];
+                    if (i + 3 * BAM_WAVE_SIZE < n16) x3 = base[i + 3 * BAM_WAVE_SIZE];
+                    a0 += (((uint64_t)x0.y << 32) | x0.x) + (((uint64_t)x1.y << 32) | x1.x) + (((uint64_t)x2.y << 32) | x2.x) + (((uint64_t)x3.y << 32) | x3.x);
+                    a1 += (((uint64_t)x0.w << 32) | x0.z) + (((uint64_t)x1.w << 32) | x1.z) + (((uint64_t)x2.w << 32) | x2.z) + (((uint64_t)x3.w << 32) | x3.z);
+                }
+                v += a0 + a1;
+                dr->release_page(pg, r, s);
+            }
+        } else {
+            bam_ptr<uint64_t> ptr(dr);
+            for (uint64_t p = 0; p < n_pages_per_wave; p++) {
+                const uint64_t start_idx = (start_page + p) * epp + lane;
+                for (uint64_t j = 0; j < epp; j += BAM_WAVE_SIZE) {
+                    if (MODE == 0) v += (*dr)[start_idx + j];
+                    else v += ptr[start_idx + j];
+                }
+            }
+        }
+    }
+    block_accumulate(sum, v);
+}
+
+// ---- raw block benchmark (benchmarks/block/main.cu:99-200) ----
+__global__ void k_block_io(Controller** ctrls, page_cache_d_t* pc, uint32_t req_size, uint64_t n_reqs, const uint64_t* lbas, int write, int queue_policy)
+{
+    const uint64_t tid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const uint64_t act = bam::active_mask();
+    const uint32_t leader = bam::first_lane(act);
+    uint32_t ctrl = 0, queue = 0;
+    if (bam::lane() == leader) {
+        ctrl = pc->n_ctrls == 1 ? 0 : (uint32_t)(pc->ctrl_counter->fetch_add(1, simt::memory_order_relaxed) % pc->n_ctrls);
+        queue = queue_policy == 0 ? get_smid() % ctrls[ctrl]->n_qps
+                                  : (uint32_t)(ctrls[ctrl]->queue_counter.fetch_add(1, simt::memory_order_relaxed) % ctrls[ctrl]->n_qps);
+    }
+    ctrl = bam::bcast(ctrl, leader);
+    queue = bam::bcast(queue, leader);
+    if (tid < n_reqs) {
+        QueuePair* qp = ctrls[ctrl]->d_qps + queue;
+        const uint64_t start_block = lbas ? lbas[tid] : (tid * req_size) >> qp->block_size_log;
+        const uint64_t n_blocks = req_size >> qp->block_size_log;
+        if (write) write_data(pc, qp, start_block, n_blocks, tid);
+        else read_data(pc, qp, start_block, n_blocks, tid);
+    }
+}
+
+__global__ void k_block_checksum(page_cache_d_t* pc, uint64_t n_slots, uint32_t req_bytes, uint64_t* out)
+{
+    /* one wave per slot */
+    const uint64_t wave = ((uint64_t)blockIdx.x * blockDim.x + threadIdx.x) / BAM_WAVE_SIZE;
+    uint64_t v = 0;
+    if (wave < n_slots) {
+        const uint64_t* p = (const uint64_t*)(pc->base_addr + wave * pc->page_size);
+        for (uint32_t i = bam::lane(); i < req_bytes / 8; i += BAM_WAVE_SIZE) v += p[i];
+    }
+    v = wave_sum(v);
+    if (wave < n_slots && bam::lane() == 0) out[wave] = v;
+}
+
+// ---- BFS: wave per `coarse` vertices, edges through bam_ptr (benchmarks/bfs/main.cu:658-689) ----
+#define MYINFINITY 0xFFFFFFFFu
+__global__ __launch_bounds__(128) void k_bfs_coalesce_coarse_ptr_pc(array_d_t<uint64_t>* da, uint32_t* label, const uint32_t level, const uint64_t vertex_count,
+                                                                   const uint64_t* vertexList, uint64_t* changed, uint64_t coarse)
+{
+    const uint64_t tid = (uint64_t)blockDim.x * blockIdx.x + threadIdx.x;
+    const uint64_t waveIdx = tid / BAM_WAVE_SIZE, laneIdx = tid % BAM_WAVE_SIZE;
+    bam_ptr<uint64_t> ptr(da);
+    bool any = false;
+    for (uint64_t j = 0; j < coarse; j++) {
+        const uint64_t v = waveIdx * coarse + j;
+        if (v < vertex_count && label[v] == level) {
+            const uint64_t start = vertexList[v];
+            const uint64_t shift_start = start & 0xFFFFFFFFFFFFFFF0ull;      /* 128-byte aligned first access */
+            const uint64_t end = vertexList[v + 1];
+            for (uint64_t i = shift_start + laneIdx; i < end; i += BAM_WAVE_SIZE) {
+                if (i >= start) {
+                    const uint64_t next = ptr[i];
+                    if (label[next] == MYINFINITY) {
+                        label[next] = level + 1;
+                        any = true;
+                    }
+                }
+            }
+        }
+    }
+    if (any) *changed = 1;
+}
+
+// ---- CC: min-label propagation (benchmarks/cc/main.cu:123-144, 595-617) ----
+__device__ __forceinline__ void cc_compute(uint64_t cid, unsigned long long* comp, uint64_t next, bool* next_visit, bool* changed)
+{
+    const unsigned long long comp_src = comp[cid], comp_next = comp[next];
+    if (comp_next == comp_src) return;
+    uint64_t next_target;
+    unsigned long long comp_target;
+    if (comp_src < comp_next) { next_target = next; comp_target = comp_src; }
+    else { next_target = cid; comp_target = comp_next; }
+    atomicMin(&comp[next_target], comp_target);
+    next_visit[next_target] = true;
+    *changed = true;
+}
+
+__global__ __launch_bounds__(128) void k_cc_coalesce_coarse_ptr_pc(array_d_t<uint64_t>* da, bool* curr_visit, bool* next_visit, uint64_t vertex_count,
+                                                                  const uint64_t* vertexList, unsigned long long* comp, bool* changed, uint64_t coarse)
+{
+    const uint64_t tid = (uint64_t)blockDim.x * blockIdx.x + threadIdx.x;
+    const uint64_t waveIdx = tid / BAM_WAVE_SIZE, laneIdx = tid % BAM_WAVE_SIZE;
+    bam_ptr<uint64_t> ptr(da);
+    for (uint64_t j = 0; j < coarse; j++) {
+        const uint64_t v = waveIdx * coarse + j;
+        if (v < vertex_count && curr_visit[v] == true) {
+            const uint64_t start = vertexList[v];
+            const uint64_t shift_start = start & 0xFFFFFFFFFFFFFFF0ull;
+            const uint64_t end = vertexList[v + 1];
+            for (uint64_t i = shift_start + laneIdx; i < end; i += BAM_WAVE_SIZE)
+                if (i >= start) cc_compute(v, comp, ptr[i], next_visit, changed);
+        }
+    }
+}
+
+__global__ void k_iota(unsigned long long* p, uint64_t n)
+{
+    const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = i;
+}
+
+// ---- synthetic inputs ----
+__global__ void k_gen_words(uint64_t seed, uint64_t first, uint64_t n, uint64_t* out)
+{
+    const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = splitmix64(seed, first + i);
+}
+__global__ void k_gen_mod(uint64_t seed, uint64_t first, uint64_t n, uint64_t modulus, uint64_t scale, uint64_t* out)
+{
+    const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = (splitmix64(seed, first + i) % modulus) * scale;
+}
+/* RMAT a=.57 b=.19 c=.19 d=.05 as 32-bit thresholds floor(p * 2^32); one quadrant draw per level from splitmix64(seed, edge * scale + level) */
+__global__ void k_gen_rmat(uint64_t seed, uint32_t scale, uint64_t first, uint64_t n, uint64_t* u, uint64_t* v)
+{
+    const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const uint32_t T1 = 2448131358u, T2 = T1 + 816043786u, T3 = T2 + 816043786u;
+    const uint64_t e = first + i;
+    uint64_t uu = 0, vv = 0;
+    for (uint32_t l = 0; l < scale; l++) {
+        const uint32_t x = (uint32_t)(splitmix64(seed, e * scale + l) >> 32);
+        const uint32_t q = x < T1 ? 0 : x < T2 ? 1 : x < T3 ? 2 : 3;
+        uu = (uu << 1) | (q >> 1);
+        vv = (vv << 1) | (q & 1);
+    }
+    u[i] = uu; v[i] = vv;
+}
+__global__ void k_gen_uniform(uint64_t seed, uint64_t n_vertices, uint64_t first, uint64_t n, uint64_t* u, uint64_t* v)
+{
+    const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const uint64_t p = first + i;
+    u[i] = splitmix64(seed, 2 * p) % n_vertices;
+    v[i] = splitmix64(seed, 2 * p + 1) % n_vertices;
+}
+
+// ---- measurement helpers ----
+__global__ void k_copy16(const uint4* __restrict__ src, uint4* __restrict__ dst, uint64_t n16)
+{
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (uint64_t)gridDim.x * blockDim.x) dst[i] = src[i];
+}
+/* every wave pulls whole chunks of host-pinned memory into device memory, 16 bytes per lane per load */
+__global__ void k_host_pull(const uint4* __restrict__ host, uint4* __restrict__ dev, uint64_t n_chunks, uint32_t chunk16, uint64_t host_chunks)
+{
+    const uint64_t wave = ((uint64_t)blockIdx.x * blockDim.x + threadIdx.x) / BAM_WAVE_SIZE;
+    const uint64_t n_waves = (uint64_t)gridDim.x * blockDim.x / BAM_WAVE_SIZE;
+    for (uint64_t c = wave; c < n_chunks; c += n_waves) {
+        const uint4* s = host + (c % host_chunks) * chunk16;
+        uint4* d = dev + (c % host_chunks) * chunk16;
+        for (uint32_t i = bam::lane(); i < chunk16; i += BAM_WAVE_SIZE) d[i] = s[i];
+    }
+}
+
+inline uint32_t blocks_for(uint64_t n, uint32_t bs) { return (uint32_t)((n + bs - 1) / bs); }
+
+void fill_backing(uint64_t seed, uint64_t* p, uint64_t n_words)
+{
+    unsigned nt = std::thread::hardware_concurrency();
+    if (nt < 1) nt = 1;
+    if (nt > 16) nt = 16;
+    std::vector<std::thread> th;
+    const uint64_t per = (n_words + nt - 1) / nt;
+    for (unsigned t = 0; t < nt; t++) {
+        const uint64_t a = t * per, b = a + per < n_words ? a + per : n_words;
+        if (a < b) th.emplace_back([=]() { nvmt_fill_words(seed, a, b - a, p + a); });
+    }
+    for (auto& x : th) x.join();
+}
+
+} // namespace
+
+// ---------------------------------------------------------------------------
+// C entry points
+// ---------------------------------------------------------------------------
+extern "C" {
+
+const char* bam_last_error(void) { return g_err.c_str(); }
+
+int bam_device_count(int* count)
+{
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (count) *count = e == hipSuccess ? n : 0;
+    return e == hipSuccess ? 0 : fail(ENODEV, hipGetErrorString(e));
+}
+
+int bam_target_create(bam_target_t** out, const char* path, uint64_t ns_bytes, uint32_t lba_bytes, int backing, uint64_t seed,
+                      uint32_t n_io_threads, uint32_t max_queue_entries, uint32_t max_io_queues, uint32_t completion_order,
+                      uint32_t fail_every, uint32_t drop_every)
+{
+    if (!out || !path) return fail(EINVAL, "bam_target_create: null argument");
+    *out = nullptr;
+    BAM_API_BEGIN
+    bam_target* bt = new bam_target();
+    nvmt_config_t& c = bt->cfg;
+    c.ns_bytes = ns_bytes; c.lba_bytes = lba_bytes; c.seed = seed; c.n_io_threads = n_io_threads;
+    c.max_queue_entries = max_queue_entries; c.max_io_queues = max_io_queues; c.dstrd = 4;     /* one doorbell per 64-byte line */
+    c.order = completion_order; c.fail_every = fail_every; c.drop_every = drop_every;
+    if (backing) {
+        if (posix_memalign(&bt->backing, 4096, ns_bytes)) { delete bt; return fail(ENOMEM, "bam_target_create: backing store allocation failed"); }
+        bt->backing_bytes = ns_bytes;
+        fill_backing(seed, (uint64_t*)bt->backing, ns_bytes / 8);
+        c.backing = bt->backing;
+    }
+    const size_t bar_size = nvmt_bar_size(&c);
+    hip_err_chk(hipHostMalloc(&bt->bar, bar_size, hipHostMallocMapped));
+    memset(bt->bar, 0, bar_size);
+    bt->t = nvmt_create(&c, bt->bar);
+    if (!bt->t) { (void)hipHostFree(bt->bar); free(bt->backing); delete bt; return fail(EINVAL, "bam_target_create: invalid target configuration"); }
+    int err = nvmt_publish(path, bt->t);
+    if (err) { nvmt_destroy(bt->t); (void)hipHostFree(bt->bar); free(bt->backing); delete bt; return fail(err, "bam_target_create: path already published"); }
+    *out = bt;
+    BAM_API_END
+}
+
+void bam_target_destroy(bam_target_t* t)
+{
+    if (!t) return;
+    nvmt_destroy(t->t);
+    (void)hipHostFree(t->bar);
+    free(t->backing);
+    delete t;
+}
+
+int bam_target_stats(bam_target_t* t, uint64_t* out, int reset)
+{
+    if (!t || !out) return fail(EINVAL, "bam_target_stats: null argument");
+    nvmt_stats_t s;
+    nvmt_stats(t->t, &s);
+    const uint64_t v[10] = {s.admin_cmds, s.io_cmds, s.read_cmds, s.write_cmds, s.bytes_read, s.bytes_written, s.error_cpls, s.sq_doorbells, s.cq_full_stalls, s.dropped};
+    memcpy(out, v, sizeof(v));
+    if (reset) nvmt_reset_stats(t->t);
+    return 0;
+}
+
+void* bam_target_backing(bam_target_t* t) { return t ? t->backing : nullptr; }
+
+int bam_ctrl_create(bam_ctrl_t** out, const char* path, uint32_t ns_id, uint32_t device, uint64_t queue_depth, uint64_t n_queues,
+                    uint32_t stage_bytes, uint32_t spin_limit)
+{
+    if (!out || !path) return fail(EINVAL, "bam_ctrl_create: null argument");
+    *out = nullptr;
+    BAM_API_BEGIN
+    Controller* c = new Controller(path, ns_id, device, queue_depth, n_queues, stage_bytes, spin_limit);
+    *out = new bam_ctrl{c};
+    BAM_API_END
+}
+
+void bam_ctrl_destroy(bam_ctrl_t* c)
+{
+    if (!c) return;
+    delete c->c;
+    delete c;
+}
+
+int bam_ctrl_info(bam_ctrl_t* c, uint64_t* out, int reset)
+{
+    if (!c || !out) return fail(EINVAL, "bam_ctrl_info: null argument");
+    BAM_API_BEGIN
+    out[0] = c->c->n_qps;
+    out[1] = c->c->n_qps ? c->c->h_qps[0]->sq.qs : 0;
+    out[2] = c->c->blk_size;
+    out[3] = c->c->ns.size;
+    if (reset) out[4] = c->c->reset_stats();
+    else hip_err_chk(hipMemcpy(&out[4], c->c->d_ctrl_ptr, sizeof(uint64_t), hipMemcpyDeviceToHost));
+    out[5] = c->c->completion_errors();
+    BAM_API_END
+}
+
+int bam_ctrl_aborted(bam_ctrl_t* c, int clear)
+{
+    if (!c) return 0;
+    int a = c->c->aborted();
+    if (clear) c->c->clear_abort();
+    return a;
+}
+
+int bam_page_cache_create(bam_page_cache_t** out, uint64_t page_size, uint64_t n_pages, uint32_t device, bam_ctrl_t* ctrl, uint64_t max_range)
+{
+    if (!out || !ctrl) return fail(EINVAL, "bam_page_cache_create: null argument");
+    *out = nullptr;
+    BAM_API_BEGIN
+    std::vector<Controller*> ctrls{ctrl->c};
+    page_cache_t* pc = new page_cache_t(page_size, n_pages, device, *ctrl->c, max_range, ctrls);
+    *out = new bam_page_cache{pc, ctrl->c};
+    BAM_API_END
+}
+
+void bam_page_cache_destroy(bam_page_cache_t* pc)
+{
+    if (!pc) return;
+    delete pc->pc;
+    delete pc;
+}
+
+int bam_page_cache_info(bam_page_cache_t* pc, uint64_t* out)
+{
+    if (!pc || !out) return fail(EINVAL, "bam_page_cache_info: null argument");
+    out[0] = pc->pc->pdt.n_pages;
+    out[1] = pc->pc->pdt.page_size;
+    out[2] = pc->pc->pdt.wave_batch;
+    out[3] = pc->pc->pdt.prp1 == nullptr;
+    return 0;
+}
+
+int bam_page_cache_flush(bam_page_cache_t* pc)
+{
+    if (!pc) return fail(EINVAL, "bam_page_cache_flush: null argument");
+    BAM_API_BEGIN
+    pc->pc->flush_cache();
+    hip_err_chk(hipDeviceSynchronize());
+    BAM_API_END
+}
+
+int bam_range_create(bam_range_t** out, uint64_t index_start, uint64_t count, uint64_t page_start, uint64_t page_count,
+                     uint64_t page_start_offset, uint64_t page_size, bam_page_cache_t* pc, uint32_t device, int dist)
+{
+    if (!out || !pc) return fail(EINVAL, "bam_range_create: null argument");
+    *out = nullptr;
+    if (dist != REPLICATE && dist != STRIPE) return fail(EINVAL, "bam_range_create: unknown distribution");
+    if (page_size != pc->pc->pdt.page_size) return fail(EINVAL, "bam_range_create: page size differs from the cache's");
+    if (page_start_offset >= page_size || count <= index_start || page_count == 0) return fail(EINVAL, "bam_range_create: empty or misaligned range");
+    if (((count - index_start) * sizeof(uint64_t) + page_start_offset + page_size - 1) / page_size > page_count)
+        return fail(EINVAL, "bam_range_create: page_count does not cover the elements");
+    BAM_API_BEGIN
+    *out = new bam_range{new range_t<uint64_t>(index_start, count, page_start, page_count, page_start_offset, page_size, pc->pc, device, (data_dist_t)dist)};
+    BAM_API_END
+}
+
+void bam_range_destroy(bam_range_t* r)
+{
+    if (!r) return;
+    delete r->r;
+    delete r;
+}
+
+int bam_array_create(bam_array_t** out, uint64_t n_elems, uint64_t disk_start_offset, bam_range_t** ranges, uint32_t n_ranges, uint32_t device)
+{
+    if (!out || !ranges || !n_ranges) return fail(EINVAL, "bam_array_create: null argument");
+    *out = nullptr;
+    BAM_API_BEGIN
+    std::vector<range_t<uint64_t>*> rs;
+    for (uint32_t i = 0; i < n_ranges; i++) rs.push_back(ranges[i]->r);
+    *out = new bam_array{new array_t<uint64_t>(n_elems, disk_start_offset, rs, device)};
+    BAM_API_END
+}
+
+void bam_array_destroy(bam_array_t* a)
+{
+    if (!a) return;
+    delete a->a;
+    delete a;
+}
+
+int bam_array_stats(bam_array_t* a, uint64_t* out, int reset)
+{
+    if (!a || !out) return fail(EINVAL, "bam_array_stats: null argument");
+    BAM_API_BEGIN
+    hip_err_chk(hipDeviceSynchronize());
+    if (!reset) {
+        /* read without clearing: read-and-reset, then put the totals back into shard 0 */
+        std::vector<bam_array_counters> per;
+        a->a->reset_stats(&per);
+        for (size_t i = 0; i < per.size(); i++) {
+            bam_stat_shard_t s0 = {per[i].access_cnt, per[i].miss_cnt, per[i].hit_cnt, per[i].read_io_cnt, {0, 0, 0, 0}};
+            hip_err_chk(hipMemcpy(a->a->h_ranges[i].stats, &s0, sizeof(s0), hipMemcpyHostToDevice));
+        }
+        out[0] = out[1] = out[2] = out[3] = 0;
+        for (auto& p : per) { out[0] += p.read_io_cnt; out[1] += p.access_cnt; out[2] += p.miss_cnt; out[3] += p.hit_cnt; }
+    } else {
+        bam_array_counters t = a->a->reset_stats();
+        out[0] = t.read_io_cnt; out[1] = t.access_cnt; out[2] = t.miss_cnt; out[3] = t.hit_cnt;
+    }
+    BAM_API_END
+}
+
+int bam_array_read(bam_array_t* a, uint64_t n_reqs, const uint64_t* d_assignment, uint64_t stride, uint64_t reqs_per_thread,
+                   uint32_t block_size, uint64_t* d_sum, void* stream)
+{
+    if (!a || !d_sum) return fail(EINVAL, "bam_array_read: null argument");
+    if (!block_size || block_size % BAM_WAVE_SIZE || block_size > 1024) return fail(EINVAL, "bam_array_read: block size must be a multiple of 64, at most 1024");
+    if (!n_reqs) return 0;
+    BAM_API_BEGIN
+    hipLaunchKernelGGL(k_array_read, dim3(blocks_for(n_reqs, block_size)), dim3(block_size), 0, (hipStream_t)stream,
+                       a->a->d_array_ptr, n_reqs, d_assignment, stride, reqs_per_thread, (unsigned long long*)d_sum);
+    hip_err_chk(hipGetLastError());
+    BAM_API_END
+}
+
+int bam_array_write(bam_array_t* a, uint64_t n_reqs, const uint64_t* d_assignment, uint64_t stride, const uint64_t* d_values,
+                    uint32_t block_size, void* stream)
+{
+    if (!a || !d_values) return fail(EINVAL, "bam_array_write: null argument");
+    if (!block_size || block_size % BAM_WAVE_SIZE || block_size > 1024) return fail(EINVAL, "bam_array_write: block size must be a multiple of 64, at most 1024");
+    if (!n_reqs) return 0;
+    BAM_API_BEGIN
+    hipLaunchKernelGGL(k_array_write, dim3(blocks_for(n_reqs, block_size)), dim3(block_size), 0, (hipStream_t)stream,
+                       a->a->d_array_ptr, n_reqs, d_assignment, stride, d_values);
+    hip_err_chk(hipGetLastError());
+    BAM_API_END
+}
+
+int bam_cache_stream(bam_array_t* a, uint64_t n_waves, uint64_t n_pages_per_wave, const uint64_t* d_assignment, int mode,
+                     uint64_t* d_sum, void* stream)
+{
+    if (!a || !d_sum) return fail(EINVAL, "bam_cache_stream: null argument");
+    if (mode < 0 || mode > 2) return fail(EINVAL, "bam_cache_stream: mode must be 0, 1 or 2");
+    if (!n_waves || !n_pages_per_wave) return 0;
+    BAM_API_BEGIN
+    const uint32_t bs = 256;
+    const dim3 grid(blocks_for(n_waves * BAM_WAVE_SIZE, bs)), block(bs);
+    array_d_t<uint64_t>* d = a->a->d_array_ptr;
+    unsigned long long* s = (unsigned long long*)d_sum;
+    if (mode == 0) hipLaunchKernelGGL(k_cache_stream<0>, grid, block, 0, (hipStream_t)stream, d, n_waves, n_pages_per_wave, d_assignment, s);
+    else if (mode == 1) hipLaunchKernelGGL(k_cache_stream<1>, grid, block, 0, (hipStream_t)stream, d, n_waves, n_pages_per_wave, d_assignment, s);
+    else hipLaunchKernelGGL(k_cache_stream<2>, grid, block, 0, (hipStream_t)stream, d, n_waves, n_pages_per_wave, d_assignment, s);
+    hip_err_chk(hipGetLastError());
+    BAM_API_END
+}
+
+int bam_block_io(bam_ctrl_t* c, bam_page_cache_t* pc, uint64_t n_reqs, uint32_t req_bytes, const uint64_t* d_lbas, int write,
+                 int queue_policy, uint32_t block_size, void* stream)
+{
+    if (!c || !pc) return fail(EINVAL, "bam_block_io: null argument");
+    if (!block_size || block_size % BAM_WAVE_SIZE || block_size > 1024) return fail(EINVAL, "bam_block_io: block size must be a multiple of 64, at most 1024");
+    if (n_reqs > pc->pc->pdt.n_pages) return fail(EINVAL, "bam_block_io: needs one cache page per request");
+    if (!req_bytes || req_bytes % c->c->blk_size || req_bytes > pc->pc->pdt.page_size) return fail(EINVAL, "bam_block_io: request size must be a multiple of the block size and fit a page");
+    if (!n_reqs) return 0;
+    BAM_API_BEGIN
+    hipLaunchKernelGGL(k_block_io, dim3(blocks_for(n_reqs, block_size)), dim3(block_size), 0, (hipStream_t)stream,
+                       pc->pc->pdt.d_ctrls, pc->pc->d_pc_ptr, req_bytes, n_reqs, d_lbas, write, queue_policy);
+    hip_err_chk(hipGetLastError());
+    BAM_API_END
+}
+
+int bam_block_checksum(bam_page_cache_t* pc, uint64_t n_slots, uint32_t req_bytes, uint64_t* d_out, void* stream)
+{
+    if (!pc || !d_out) return fail(EINVAL, "bam_block_checksum: null argument");
+    if (n_slots > pc->pc->pdt.n_pages || req_bytes > pc->pc->pdt.page_size || req_bytes % 8) return fail(EINVAL, "bam_block_checksum: out of range");
+    if (!n_slots) return 0;
+    BAM_API_BEGIN
+    hipLaunchKernelGGL(k_block_checksum, dim3(blocks_for(n_slots * BAM_WAVE_SIZE, 256)), dim3(256), 0, (hipStream_t)stream,
+                       pc->pc->d_pc_ptr, n_slots, req_bytes, d_out);
+    hip_err_chk(hipGetLastError());
+    BAM_API_END
+}
+
+int bam_bfs(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t src, uint32_t* d_labels,
+            uint32_t coarse, uint32_t* iterations, void* stream)
+{
+    if (!edges || !d_offsets || !d_labels) return fail(EINVAL, "bam_bfs: null argument");
+    if (src >= n_vertices || !coarse) return fail(EINVAL, "bam_bfs: source out of range or coarse = 0");
+    BAM_API_BEGIN
+    hipStream_t st = (hipStream_t)stream;
+    BufferPtr changed_buf = createBuffer(sizeof(uint64_t), edges->a->adt.n_ranges ? 0 : 0);
+    uint64_t* changed_d = (uint64_t*)changed_buf.get();
+    const uint32_t zero = 0;
+    hip_err_chk(hipMemsetAsync(d_labels, 0xFF, n_vertices * sizeof(uint32_t), st));
+    hip_err_chk(hipMemcpyAsync(d_labels + src, &zero, sizeof(uint32_t), hipMemcpyHostToDevice, st));
+    const uint32_t threads = 128;
+    const uint64_t n_waves = (n_vertices + coarse - 1) / coarse;
+    const uint32_t blocks = blocks_for(n_waves * BAM_WAVE_SIZE, threads);
+    uint32_t level = 0, iter = 0;
+    uint64_t changed_h;
+    do {
+        changed_h = 0;
+        hip_err_chk(hipMemcpyAsync(changed_d, &changed_h, sizeof(uint64_t), hipMemcpyHostToDevice, st));
+        hipLaunchKernelGGL(k_bfs_coalesce_coarse_ptr_pc, dim3(blocks), dim3(threads), 0, st,
+                           edges->a->d_array_ptr, d_labels, level, n_vertices, d_offsets, changed_d, (uint64_t)coarse);
+        hip_err_chk(hipGetLastError());
+        iter++; level++;
+        hip_err_chk(hipMemcpyAsync(&changed_h, changed_d, sizeof(uint64_t), hipMemcpyDeviceToHost, st));
+        hip_err_chk(hipStreamSynchronize(st));
+    } while (changed_h);
+    if (iterations) *iterations = iter;
+    BAM_API_END
+}
+
+int bam_cc(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t* d_labels,
+           uint32_t coarse, uint32_t* iterations, void* stream)
+{
+    if (!edges || !d_offsets || !d_labels) return fail(EINVAL, "bam_cc: null argument");
+    if (!coarse || !n_vertices) return fail(EINVAL, "bam_cc: empty graph or coarse = 0");
+    BAM_API_BEGIN
+    hipStream_t st = (hipStream_t)stream;
+    BufferPtr visit_a = createBuffer(n_vertices, 0), visit_b = createBuffer(n_vertices, 0), changed_buf = createBuffer(sizeof(uint64_t), 0);
+    bool* curr = (bool*)visit_a.get();
+    bool* next = (bool*)visit_b.get();
+    bool* changed_d = (bool*)changed_buf.get();
+    hipLaunchKernelGGL(k_iota, dim3(blocks_for(n_vertices, 256)), dim3(256), 0, st, (unsigned long long*)d_labels, n_vertices);
+    hip_err_chk(hipMemsetAsync(curr, 0x01, n_vertices, st));
+    hip_err_chk(hipMemsetAsync(next, 0x00, n_vertices, st));
+    const uint32_t threads = 128;
+    const uint64_t n_waves = (n_vertices + coarse - 1) / coarse;
+    const uint32_t blocks = blocks_for(n_waves * BAM_WAVE_SIZE, threads);
+    uint32_t iter = 0;
+    bool changed_h;
+    do {
+        changed_h = false;
+        hip_err_chk(hipMemcpyAsync(changed_d, &changed_h, sizeof(bool), hipMemcpyHostToDevice, st));
+        hipLaunchKernelGGL(k_cc_coalesce_coarse_ptr_pc, dim3(blocks), dim3(threads), 0, st,
+                           edges->a->d_array_ptr, curr, next, n_vertices, d_offsets, (unsigned long long*)d_labels, changed_d, (uint64_t)coarse);
+        hip_err_chk(hipGetLastError());
+        hip_err_chk(hipMemsetAsync(curr, 0x00, n_vertices, st));
+        bool* t = curr; curr = next; next = t;
+        iter++;
+        hip_err_chk(hipMemcpyAsync(&changed_h, changed_d, sizeof(bool), hipMemcpyDeviceToHost, st));
+        hip_err_chk(hipStreamSynchronize(st));
+    } while (changed_h);
+    if (iterations) *iterations = iter;
+    BAM_API_END
+}
+
+int bam_gen_words(uint64_t seed, uint64_t first, uint64_t n, uint64_t* d_out, void* stream)
+{
+    if (!d_out) return fail(EINVAL, "bam_gen_words: null argument");
+    if (!n) return 0;
+    BAM_API_BEGIN
+    hipLaunchKernelGGL(k_gen_words, dim3(blocks_for(n, 256)), dim3(256), 0, (hipStream_t)stream, seed, first, n, d_out);
+    hip_err_chk(hipGetLastError());
+    BAM_API_END
+}
+
+int bam_gen_mod(uint64_t seed, uint64_t first, uint64_t n, uint64_t modulus, uint64_t scale, uint64_t* d_out, void* stream)
+{
+    if (!d_out || !modulus) return fail(EINVAL, "bam_gen_mod: null argument or zero modulus");
+    if (!n) return 0;
+    BAM_API_BEGIN
+    hipLaunchKernelGGL(k_gen_mod, dim3(blocks_for(n, 256)), dim3(256), 0, (hipStream_t)stream, seed, first, n, modulus, scale, d_out);
+    hip_err_chk(hipGetLastError());
+    BAM_API_END
+}
+
+int bam_gen_rmat(uint64_t seed, uint32_t scale, uint64_t first_edge, uint64_t n, uint64_t* d_u, uint64_t* d_v, void* stream)
+{
+    if (!d_u || !d_v || !scale || scale > 40) return fail(EINVAL, "bam_gen_rmat: bad argument");
+    if (!n) return 0;
+    BAM_API_BEGIN
+    hipLaunchKernelGGL(k_gen_rmat, dim3(blocks_for(n, 256)), dim3(256), 0, (hipStream_t)stream, seed, scale, first_edge, n, d_u, d_v);
+    hip_err_chk(hipGetLastError());
+    BAM_API_END
+}
+
+int bam_gen_uniform(uint64_t seed, uint64_t n_vertices, uint64_t first_pair, uint64_t n, uint64_t* d_u, uint64_t* d_v, void* stream)
+{
+    if (!d_u || !d_v || !n_vertices) return fail(EINVAL, "bam_gen_uniform: bad argument");
+    if (!n) return 0;
+    BAM_API_BEGIN
+    hipLaunchKernelGGL(k_gen_uniform, dim3(blocks_for(n, 256)), dim3(256), 0, (hipStream_t)stream, seed, n_vertices, first_pair, n, d_u, d_v);
+    hip_err_chk(hipGetLastError());
+    BAM_API_END
+}
+
+int bam_copy_kernel(const void* d_src, void* d_dst, uint64_t n_bytes, float* ms, void* stream)
+{
+    if (!d_src || !d_dst || n_bytes % 16) return fail(EINVAL, "bam_copy_kernel: bad argument");
+    BAM_API_BEGIN
+    hipStream_t st = (hipStream_t)stream;
+    Event a(st);
+    hipLaunchKernelGGL(k_copy16, dim3(256 * 16), dim3(256), 0, st, (const uint4*)d_src, (uint4*)d_dst, n_bytes / 16);
+    hip_err_chk(hipGetLastError());
+    Event b(st);
+    if (ms) *ms = (float)((b - a) / 1e3);
+    BAM_API_END
+}
+
+int bam_host_read_ceiling(uint64_t n_bytes, uint32_t chunk_bytes, float* ms)
+{
+    if (!n_bytes || !chunk_bytes || chunk_bytes % 1024) return fail(EINVAL, "bam_host_read_ceiling: chunk must be a multiple of 1024 bytes");
+    BAM_API_BEGIN
+    const uint64_t window = n_bytes < (256ull << 20) ? n_bytes : (256ull << 20);
+    const uint64_t host_chunks = window / chunk_bytes;
+    if (!host_chunks) return fail(EINVAL, "bam_host_read_ceiling: less than one chunk");
+    BufferPtr host = createHostBuffer(window), dev = createBuffer(window, 0);
+    const uint64_t n_chunks = n_bytes / chunk_bytes;
+    for (int rep = 0; rep < 2; rep++) {           /* first pass warms mappings */
+        Event a(0);
+        hipLaunchKernelGGL(k_host_pull, dim3(256 * 8), dim3(256), 0, 0, (const uint4*)host.get(), (uint4*)dev.get(), n_chunks, chunk_bytes / 16, host_chunks);
+        hip_err_chk(hipGetLastError());
+        Event b(0);
+        if (ms) *ms = (float)((b - a) / 1e3);
+    }
+    BAM_API_END
+}
+
+int bam_event_create(void** ev)
+{
+    if (!ev) return fail(EINVAL, "bam_event_create: null argument");
+    BAM_API_BEGIN
+    hipEvent_t e;
+    hip_err_chk(hipEventCreate(&e));
+    *ev = (void*)e;
+    BAM_API_END
+}
+
+int bam_event_record(void* ev, void* stream)
+{
+    BAM_API_BEGIN
+    hip_err_chk(hipEventRecord((hipEvent_t)ev, (hipStream_t)stream));
+    BAM_API_END
+}
+
+int bam_event_elapsed_ms(void* start, void* stop, float* ms)
+{
+    if (!ms) return fail(EINVAL, "bam_event_elapsed_ms: null argument");
+    BAM_API_BEGIN
+    hip_err_chk(hipEventSynchronize((hipEvent_t)stop));
+    hip_err_chk(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+    BAM_API_END
+}
+
+void bam_event_destroy(void* ev)
+{
+    if (ev) (void)hipEventDestroy((hipEvent_t)ev);
+}
+
+double bam_target_ceiling_iops(uint64_t ns_bytes, uint32_t lba_bytes, int backing, uint32_t n_io_threads, uint32_t n_clients,
+                               uint32_t depth, uint64_t n_cmds, uint32_t req_bytes)
+{
+    nvmt_config_t c{};
+    c.ns_bytes = ns_bytes; c.lba_bytes = lba_bytes; c.seed = 42; c.n_io_threads = n_io_threads;
+    c.max_queue_entries = 1024; c.max_io_queues = 128; c.dstrd = 4;
+    void* mem = nullptr;
+    if (backing) {
+        if (posix_memalign(&mem, 4096, ns_bytes)) return -1.0;
+        fill_backing(42, (uint64_t*)mem, ns_bytes / 8);
+        c.backing = mem;
+    }
+    double r = nvmt_selftest_iops(&c, n_clients, depth, n_cmds, req_bytes);
+    free(mem);
+    return r;
+}
+
+} // extern "C"

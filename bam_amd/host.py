@@ -1,0 +1,240 @@
+"""Host-side mirror of the reference's host objects over the C-ABI.
+
+Controller / PageCache / Range / Array correspond to Controller
+(include/ctrl.h:39-78), page_cache_t (include/page_cache.h:631-887),
+range_t<uint64_t> (:964-1030) and array_t<uint64_t> (:1718-1774) of the
+reference, with the same constructor arguments in the same order.  Device
+buffers are torch tensors on the handle's device; 64-bit unsigned data travels
+as int64 tensors (same bits).
+"""
+import ctypes
+
+import torch
+
+from . import _lib
+
+c_u64, c_u32, c_vp = ctypes.c_uint64, ctypes.c_uint32, ctypes.c_void_p
+MASK64 = (1 << 64) - 1
+
+
+class BamError(RuntimeError):
+    pass
+
+
+# a target must outlive the controllers attached to it: controllers tear their queues down through it
+_TARGETS = {}
+
+
+def _chk(status, what):
+    if status != 0:
+        msg = _lib.load().bam_last_error()
+        raise BamError(f"{what}: {msg.decode() if msg else 'error'} (status {status})")
+
+
+def _ptr(t):
+    if t is None:
+        return None
+    if not t.is_cuda or not t.is_contiguous():
+        raise BamError("expected a contiguous tensor in device memory")
+    return c_vp(t.data_ptr())
+
+
+def _stream():
+    return c_vp(torch.cuda.current_stream().cuda_stream)
+
+
+class Target:
+    """Software NVMe target published under `path` (stands where /dev/libnvmN does in the reference)."""
+
+    def __init__(self, path, ns_bytes, lba_bytes=512, backing=False, seed=42, n_io_threads=4,
+                 max_queue_entries=1024, max_io_queues=128, completion_order=0, fail_every=0, drop_every=0):
+        self.L = _lib.load()
+        self.h = c_vp()
+        self.path = path
+        _chk(self.L.bam_target_create(ctypes.byref(self.h), path.encode(), ns_bytes, lba_bytes, int(backing), seed,
+                                      n_io_threads, max_queue_entries, max_io_queues, completion_order, fail_every, drop_every),
+             "bam_target_create")
+        _TARGETS[path] = self
+
+    def stats(self, reset=False):
+        out = (c_u64 * 10)()
+        _chk(self.L.bam_target_stats(self.h, out, int(reset)), "bam_target_stats")
+        keys = ("admin_cmds", "io_cmds", "read_cmds", "write_cmds", "bytes_read", "bytes_written", "error_cpls",
+                "sq_doorbells", "cq_full_stalls", "dropped")
+        return dict(zip(keys, list(out)))
+
+    def close(self):
+        if self.h:
+            _TARGETS.pop(self.path, None)
+            self.L.bam_target_destroy(self.h)
+            self.h = c_vp()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class Controller:
+    def __init__(self, path, ns_id=1, device=0, queue_depth=1024, n_queues=128, stage_bytes=4096, spin_limit=1 << 24):
+        self.L = _lib.load()
+        self.h = c_vp()
+        self.device = device
+        self._target = _TARGETS.get(path)
+        _chk(self.L.bam_ctrl_create(ctypes.byref(self.h), path.encode(), ns_id, device, queue_depth, n_queues, stage_bytes, spin_limit),
+             "bam_ctrl_create")
+
+    def info(self, reset=False):
+        out = (c_u64 * 6)()
+        _chk(self.L.bam_ctrl_info(self.h, out, int(reset)), "bam_ctrl_info")
+        keys = ("n_qps", "queue_depth", "blk_size", "ns_blocks", "ssd_accesses", "error_completions")
+        return dict(zip(keys, list(out)))
+
+    def aborted(self, clear=False):
+        return bool(self.L.bam_ctrl_aborted(self.h, int(clear)))
+
+    def close(self):
+        if self.h:
+            self.L.bam_ctrl_destroy(self.h)
+            self.h = c_vp()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class PageCache:
+    def __init__(self, page_size, n_pages, device, ctrl, max_range=64):
+        self.L = _lib.load()
+        self.h = c_vp()
+        self.ctrl = ctrl
+        self.device = device
+        _chk(self.L.bam_page_cache_create(ctypes.byref(self.h), page_size, n_pages, device, ctrl.h, max_range), "bam_page_cache_create")
+
+    def info(self):
+        out = (c_u64 * 4)()
+        _chk(self.L.bam_page_cache_info(self.h, out), "bam_page_cache_info")
+        return dict(zip(("n_pages", "page_size", "wave_batch", "staged"), list(out)))
+
+    def flush(self):
+        _chk(self.L.bam_page_cache_flush(self.h), "bam_page_cache_flush")
+
+    def block_io(self, n_reqs, req_bytes, lbas=None, write=False, queue_policy=1, block_size=64):
+        """One thread per NVMe command into cache slot tid (benchmarks/block/main.cu:99-200)."""
+        _chk(self.L.bam_block_io(self.ctrl.h, self.h, n_reqs, req_bytes, _ptr(lbas), int(write), queue_policy, block_size, _stream()),
+             "bam_block_io")
+
+    def block_checksums(self, n_slots, req_bytes):
+        out = torch.empty(n_slots, dtype=torch.int64, device=f"cuda:{self.device}")
+        _chk(self.L.bam_block_checksum(self.h, n_slots, req_bytes, _ptr(out), _stream()), "bam_block_checksum")
+        return out
+
+    def close(self):
+        if self.h:
+            self.L.bam_page_cache_destroy(self.h)
+            self.h = c_vp()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class Range:
+    REPLICATE, STRIPE = 0, 1
+
+    def __init__(self, index_start, count, page_start, page_count, page_start_offset, page_size, cache, device, dist=0):
+        self.L = _lib.load()
+        self.h = c_vp()
+        self.cache = cache
+        _chk(self.L.bam_range_create(ctypes.byref(self.h), index_start, count, page_start, page_count, page_start_offset,
+                                     page_size, cache.h, device, dist), "bam_range_create")
+
+    def close(self):
+        if self.h:
+            self.L.bam_range_destroy(self.h)
+            self.h = c_vp()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class Array:
+    def __init__(self, n_elems, disk_start_offset, ranges, device):
+        self.L = _lib.load()
+        self.h = c_vp()
+        self.ranges = list(ranges)
+        self.device = device
+        arr = (c_vp * len(ranges))(*[r.h for r in ranges])
+        _chk(self.L.bam_array_create(ctypes.byref(self.h), n_elems, disk_start_offset, arr, len(ranges), device), "bam_array_create")
+
+    def _sum_buf(self):
+        return torch.zeros(1, dtype=torch.int64, device=f"cuda:{self.device}")
+
+    def read_async(self, n_reqs, d_sum, assignment=None, stride=1, reqs_per_thread=1, block_size=64):
+        _chk(self.L.bam_array_read(self.h, n_reqs, _ptr(assignment), stride, reqs_per_thread, block_size, _ptr(d_sum), _stream()),
+             "bam_array_read")
+
+    def read(self, n_reqs, assignment=None, stride=1, reqs_per_thread=1, block_size=64):
+        """Sum (mod 2^64) of the elements read: thread t reads assignment[t] (or t * stride)."""
+        s = self._sum_buf()
+        self.read_async(n_reqs, s, assignment, stride, reqs_per_thread, block_size)
+        return int(s.item()) & MASK64
+
+    def write(self, n_reqs, values, assignment=None, stride=1, block_size=64):
+        _chk(self.L.bam_array_write(self.h, n_reqs, _ptr(assignment), stride, _ptr(values), block_size, _stream()), "bam_array_write")
+
+    def stream_async(self, n_waves, n_pages_per_wave, d_sum, assignment=None, mode=2):
+        _chk(self.L.bam_cache_stream(self.h, n_waves, n_pages_per_wave, _ptr(assignment), mode, _ptr(d_sum), _stream()), "bam_cache_stream")
+
+    def stream(self, n_waves, n_pages_per_wave, assignment=None, mode=2):
+        s = self._sum_buf()
+        self.stream_async(n_waves, n_pages_per_wave, s, assignment, mode)
+        return int(s.item()) & MASK64
+
+    def bfs(self, offsets, src, coarse=1):
+        """Levels (uint32 as int32 bits... returned as int64-safe uint32 tensor) and launch count."""
+        n_v = offsets.numel() - 1
+        labels = torch.empty(n_v, dtype=torch.int32, device=offsets.device)
+        it = c_u32(0)
+        _chk(self.L.bam_bfs(self.h, _ptr(offsets), n_v, int(src), _ptr(labels), coarse, ctypes.byref(it), _stream()), "bam_bfs")
+        return labels, it.value
+
+    def cc(self, offsets, coarse=1):
+        n_v = offsets.numel() - 1
+        labels = torch.empty(n_v, dtype=torch.int64, device=offsets.device)
+        it = c_u32(0)
+        _chk(self.L.bam_cc(self.h, _ptr(offsets), n_v, _ptr(labels), coarse, ctypes.byref(it), _stream()), "bam_cc")
+        return labels, it.value
+
+    def stats(self, reset=True):
+        out = (c_u64 * 4)()
+        _chk(self.L.bam_array_stats(self.h, out, int(reset)), "bam_array_stats")
+        return dict(zip(("read_io_cnt", "access_cnt", "miss_cnt", "hit_cnt"), list(out)))
+
+    def close(self):
+        if self.h:
+            self.L.bam_array_destroy(self.h)
+            self.h = c_vp()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def make_array(ctrl, n_elems, page_size, cache_pages, device=0, disk_offset_bytes=0, max_range=64):
+    """page cache + one range + array over n_elems u64 stored from byte disk_offset_bytes (page aligned)."""
+    pc = PageCache(page_size, cache_pages, device, ctrl, max_range)
+    n_pages = (n_elems * 8 + page_size - 1) // page_size
+    r = Range(0, n_elems, disk_offset_bytes // page_size, n_pages, 0, page_size, pc, device)
+    a = Array(n_elems, disk_offset_bytes, [r], device)
+    return pc, r, a

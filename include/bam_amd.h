@@ -1,0 +1,130 @@
+/*
+ * C-ABI of the GPU-side storage-access path (libbam_amd.so).
+ *
+ * Plain pointers and sizes only.  Handles are opaque; they wrap the C++ host
+ * objects of ctrl.h / page_cache.h, which mirror the reference's.  Every entry
+ * point returns 0 on success or a non-zero errno-style code; bam_last_error()
+ * gives the message of the last failure on the calling thread.  Device
+ * pointers (d_*) must be valid on the device the handle was created for.
+ * Kernels are launched on the given stream (0 = the null stream) and the
+ * calls that return results through host pointers synchronise that stream.
+ */
+#ifndef __BAM_AMD_H__
+#define __BAM_AMD_H__
+#include <stddef.h>
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct bam_target bam_target_t;       /* software NVMe target + its register window and backing store */
+typedef struct bam_ctrl bam_ctrl_t;           /* Controller */
+typedef struct bam_page_cache bam_page_cache_t;
+typedef struct bam_range bam_range_t;         /* range_t<uint64_t> */
+typedef struct bam_array bam_array_t;         /* array_t<uint64_t> */
+
+const char* bam_last_error(void);
+/* 1 when the library was built with the gfx950 device path and a HIP device is present */
+int bam_device_count(int* count);
+
+/* ---- backing store ----
+ * Stands where the reference opens /dev/libnvmN (benchmarks/array/main.cu:39-40,
+ * include/ctrl.h:148-163): creates a software NVMe target and publishes it under
+ * `path`.  backing = 0: procedural namespace (word w = splitmix64(seed, w));
+ * backing = 1: memory-backed namespace in host-pinned memory, initialised to
+ * the same words so that both read identically until written. */
+int bam_target_create(bam_target_t** out, const char* path, uint64_t ns_bytes, uint32_t lba_bytes, int backing, uint64_t seed,
+                      uint32_t n_io_threads, uint32_t max_queue_entries, uint32_t max_io_queues, uint32_t completion_order,
+                      uint32_t fail_every, uint32_t drop_every);
+void bam_target_destroy(bam_target_t* t);
+/* out[10]: admin_cmds, io_cmds, read_cmds, write_cmds, bytes_read, bytes_written, error_cpls, sq_doorbells, cq_full_stalls, dropped */
+int bam_target_stats(bam_target_t* t, uint64_t* out, int reset);
+/* host pointer to the memory-backed namespace (NULL for procedural) */
+void* bam_target_backing(bam_target_t* t);
+
+/* ---- Controller (include/ctrl.h:148-199 of the reference) ----
+ * stage_bytes: size of the per-command staging page (0 = PRPs address device memory directly, needs CPU-visible VRAM);
+ * spin_limit: bound of every device-side wait loop, in back-off steps (0 = unbounded). */
+int bam_ctrl_create(bam_ctrl_t** out, const char* path, uint32_t ns_id, uint32_t device, uint64_t queue_depth, uint64_t n_queues,
+                    uint32_t stage_bytes, uint32_t spin_limit);
+void bam_ctrl_destroy(bam_ctrl_t* c);
+/* out[6]: n_qps, queue depth, block size, namespace blocks, #SSDAccesses since last reset, error completions */
+int bam_ctrl_info(bam_ctrl_t* c, uint64_t* out, int reset);
+/* 1 if a device-side wait gave up (lost completion / spin limit); clear = reset the flag */
+int bam_ctrl_aborted(bam_ctrl_t* c, int clear);
+
+/* ---- page_cache_t / range_t<uint64_t> / array_t<uint64_t> (include/page_cache.h:697-875, 984-1030, 1754-1772) ---- */
+int bam_page_cache_create(bam_page_cache_t** out, uint64_t page_size, uint64_t n_pages, uint32_t device, bam_ctrl_t* ctrl, uint64_t max_range);
+void bam_page_cache_destroy(bam_page_cache_t* pc);
+/* out[4]: n_pages, page_size, wave_batch, staged(0/1) */
+int bam_page_cache_info(bam_page_cache_t* pc, uint64_t* out);
+int bam_page_cache_flush(bam_page_cache_t* pc);
+int bam_range_create(bam_range_t** out, uint64_t index_start, uint64_t count, uint64_t page_start, uint64_t page_count,
+                     uint64_t page_start_offset, uint64_t page_size, bam_page_cache_t* pc, uint32_t device, int dist);
+void bam_range_destroy(bam_range_t* r);
+int bam_array_create(bam_array_t** out, uint64_t n_elems, uint64_t disk_start_offset, bam_range_t** ranges, uint32_t n_ranges, uint32_t device);
+void bam_array_destroy(bam_array_t* a);
+/* array_t::print_reset_stats (include/page_cache.h:1731-1752) as numbers; out[4]: read_io_cnt, access_cnt, miss_cnt, hit_cnt */
+int bam_array_stats(bam_array_t* a, uint64_t* out, int reset);
+
+/* ---- array benchmark kernels (benchmarks/array/main.cu:43-65) ----
+ * One thread per request: thread t reads element d_assignment[t] (or t * stride when d_assignment is NULL)
+ * reqs_per_thread times through array_d_t::operator[] and the launch adds every value read into *d_sum
+ * (mod 2^64).  The reference discards the values; the checksum is what makes the result checkable. */
+int bam_array_read(bam_array_t* a, uint64_t n_reqs, const uint64_t* d_assignment, uint64_t stride, uint64_t reqs_per_thread,
+                   uint32_t block_size, uint64_t* d_sum, void* stream);
+/* same request pattern through array_d_t::operator() (seq_write): element <- d_values[t] */
+int bam_array_write(bam_array_t* a, uint64_t n_reqs, const uint64_t* d_assignment, uint64_t stride, const uint64_t* d_values,
+                    uint32_t block_size, void* stream);
+
+/* ---- cache / pattern benchmark kernels (benchmarks/cache/main.cu:44-114, benchmarks/pattern/main.cu:105-170) ----
+ * One wave per run of n_pages_per_wave whole pages starting at page d_assignment[w] (or w * n_pages_per_wave),
+ * every element read once and summed into *d_sum.  mode 0: array_d_t::operator[] per element,
+ * mode 1: bam_ptr per element (the reference's kernel, 64-wide), mode 2: one acquire per page and
+ * 16-byte loads (what the hit-path roofline is measured on). */
+int bam_cache_stream(bam_array_t* a, uint64_t n_waves, uint64_t n_pages_per_wave, const uint64_t* d_assignment, int mode,
+                     uint64_t* d_sum, void* stream);
+
+/* ---- raw block benchmark kernels (benchmarks/block/main.cu:99-200) ----
+ * One thread per command: thread t transfers req_bytes between LBA d_lbas[t] (or t * req_bytes / lba_size when
+ * NULL) and cache slot t with read_data / write_data; no cache lookup.  Needs n_pages >= n_reqs.
+ * queue_policy 0: queue = compute unit % n_qps (sequential kernel), 1: round-robin counter (random kernel). */
+int bam_block_io(bam_ctrl_t* c, bam_page_cache_t* pc, uint64_t n_reqs, uint32_t req_bytes, const uint64_t* d_lbas, int write,
+                 int queue_policy, uint32_t block_size, void* stream);
+/* sum of the 64-bit words of the first req_bytes of slots 0..n-1, one sum per slot */
+int bam_block_checksum(bam_page_cache_t* pc, uint64_t n_slots, uint32_t req_bytes, uint64_t* d_out, void* stream);
+
+/* ---- BFS (benchmarks/bfs/main.cu:658-689 kernel_coalesce_coarse_ptr_pc, host loop :1557-1566, 1577-1736) ----
+ * Level-synchronous BFS from src: d_offsets[V+1] in device memory, neighbour ids read through the array,
+ * d_labels[V] receives the level of every vertex (0xFFFFFFFF = unreachable).  *iterations = kernel launches. */
+int bam_bfs(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t src, uint32_t* d_labels,
+            uint32_t coarse, uint32_t* iterations, void* stream);
+/* ---- CC (benchmarks/cc/main.cu:123-144 cc_compute, :595-617 kernel, host loop :1410-1425, 1515-1521) ----
+ * Min-label propagation; d_labels[V] receives the smallest vertex id of each vertex's component. */
+int bam_cc(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t* d_labels,
+           uint32_t coarse, uint32_t* iterations, void* stream);
+
+/* ---- synthetic inputs on the device (no counterpart in the reference, which reads dataset files) ---- */
+int bam_gen_words(uint64_t seed, uint64_t first, uint64_t n, uint64_t* d_out, void* stream);                 /* out[k] = splitmix64(seed, first + k) */
+int bam_gen_mod(uint64_t seed, uint64_t first, uint64_t n, uint64_t modulus, uint64_t scale, uint64_t* d_out, void* stream); /* (splitmix64(seed, first+k) % modulus) * scale */
+int bam_gen_rmat(uint64_t seed, uint32_t scale, uint64_t first_edge, uint64_t n, uint64_t* d_u, uint64_t* d_v, void* stream);
+int bam_gen_uniform(uint64_t seed, uint64_t n_vertices, uint64_t first_pair, uint64_t n, uint64_t* d_u, uint64_t* d_v, void* stream);
+
+/* ---- measurement helpers ----
+ * plain device copy of n bytes (calibration of traffic counters), and a bulk read of host-pinned memory by the
+ * GPU (the interconnect ceiling of staged transfers); both return elapsed milliseconds measured with HIP events. */
+int bam_copy_kernel(const void* d_src, void* d_dst, uint64_t n_bytes, float* ms, void* stream);
+int bam_host_read_ceiling(uint64_t n_bytes, uint32_t chunk_bytes, float* ms);
+/* time a callback-free region: record/elapsed on the stream the kernels above were launched on */
+int bam_event_create(void** ev);
+int bam_event_record(void* ev, void* stream);
+int bam_event_elapsed_ms(void* start, void* stop, float* ms);
+void bam_event_destroy(void* ev);
+/* protocol ceiling of the target with plain host clients (nvmt_selftest_iops) */
+double bam_target_ceiling_iops(uint64_t ns_bytes, uint32_t lba_bytes, int backing, uint32_t n_io_threads, uint32_t n_clients,
+                               uint32_t depth, uint64_t n_cmds, uint32_t req_bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* __BAM_AMD_H__ */

@@ -1,0 +1,122 @@
+/*
+ * gfx950 wavefront-64 primitives used by the device path.
+ *
+ * Stands where the reference uses CUDA warp intrinsics and inline PTX:
+ * lane_id / warp_id / get_smid (include/nvm_util.h:276-295), __activemask,
+ * __match_any_sync, __shfl_sync, __any_sync, __syncwarp and __nanosleep call
+ * sites throughout include/page_cache.h and include/nvm_parallel_queue.h.
+ * Masks are 64 bits wide; gfx950 has no match-any instruction, so grouping
+ * lanes by key is a readfirstlane/ballot loop (one trip per distinct key).
+ *
+ * Memory operations on shared words go through __hip_atomic_* with an explicit
+ * scope: agent for state shared between waves, system for anything the NVMe
+ * controller (a device, or host threads of the software target) reads or writes.
+ */
+#ifndef __BAM_WAVE_H__
+#define __BAM_WAVE_H__
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define BAM_WAVE_SIZE 64
+
+namespace bam {
+
+__device__ __forceinline__ uint32_t lane() { return __lane_id(); }
+__device__ __forceinline__ uint64_t ballot(bool p) { return __builtin_amdgcn_ballot_w64(p); }
+__device__ __forceinline__ uint64_t active_mask() { return __builtin_amdgcn_ballot_w64(true); }
+__device__ __forceinline__ uint32_t popc(uint64_t m) { return (uint32_t)__builtin_popcountll(m); }
+__device__ __forceinline__ uint32_t first_lane(uint64_t m) { return (uint32_t)__builtin_ctzll(m); }
+__device__ __forceinline__ uint64_t lanes_below(uint32_t l) { return (1ull << l) - 1ull; }
+/* position of this lane among the set lanes of m */
+__device__ __forceinline__ uint32_t rank_in(uint64_t m) { return popc(m & lanes_below(lane())); }
+
+/* value held by lane `src` (wave-uniform src) */
+__device__ __forceinline__ uint32_t bcast(uint32_t v, uint32_t src) { return (uint32_t)__builtin_amdgcn_readlane((int)v, (int)src); }
+__device__ __forceinline__ uint64_t bcast(uint64_t v, uint32_t src)
+{
+    return ((uint64_t)bcast((uint32_t)(v >> 32), src) << 32) | bcast((uint32_t)v, src);
+}
+/* value held by the first active lane */
+__device__ __forceinline__ uint32_t first(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); }
+__device__ __forceinline__ uint64_t first(uint64_t v)
+{
+    return ((uint64_t)first((uint32_t)(v >> 32)) << 32) | first((uint32_t)v);
+}
+/* value held by lane `src`, src differing per lane (ds_bpermute) */
+__device__ __forceinline__ uint32_t shfl(uint32_t v, uint32_t src) { return (uint32_t)__builtin_amdgcn_ds_bpermute((int)(src << 2), (int)v); }
+__device__ __forceinline__ uint64_t shfl(uint64_t v, uint32_t src)
+{
+    return ((uint64_t)shfl((uint32_t)(v >> 32), src) << 32) | shfl((uint32_t)v, src);
+}
+
+/*
+ * Group the active lanes by a 64-bit key: returns the mask of active lanes
+ * holding the same key as the caller.  One loop trip per distinct key.
+ */
+__device__ __forceinline__ uint64_t match_any(uint64_t key)
+{
+    uint64_t mine = 0;
+    bool done = false;
+    while (!done) {
+        uint64_t k = first(key);            /* key of the first lane still looping */
+        bool eq = key == k;
+        uint64_t grp = ballot(eq);
+        if (eq) { mine = grp; done = true; }
+    }
+    return mine;
+}
+__device__ __forceinline__ uint64_t match_any(uint64_t key_a, uint64_t key_b)
+{
+    uint64_t mine = 0;
+    bool done = false;
+    while (!done) {
+        uint64_t a = first(key_a), b = first(key_b);
+        bool eq = key_a == a && key_b == b;
+        uint64_t grp = ballot(eq);
+        if (eq) { mine = grp; done = true; }
+    }
+    return mine;
+}
+
+/* compute-unit identity across the whole device: XCC, shader engine and CU bits */
+__device__ __forceinline__ uint32_t cu_id() { return __smid(); }
+
+/* back-off: n * 64 clocks, doubling up to 32 */
+__device__ __forceinline__ void backoff(uint32_t& n)
+{
+    switch (n) {
+    case 1: __builtin_amdgcn_s_sleep(1); break;
+    case 2: __builtin_amdgcn_s_sleep(2); break;
+    case 4: __builtin_amdgcn_s_sleep(4); break;
+    case 8: __builtin_amdgcn_s_sleep(8); break;
+    case 16: __builtin_amdgcn_s_sleep(16); break;
+    default: __builtin_amdgcn_s_sleep(32); break;
+    }
+    if (n < 32) n <<= 1;
+}
+
+/* ---- scoped atomics on plain words ---- */
+#define BAM_AGENT  __HIP_MEMORY_SCOPE_AGENT
+#define BAM_SYSTEM __HIP_MEMORY_SCOPE_SYSTEM
+
+template <typename T> __device__ __forceinline__ T ld_relaxed(const T* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, BAM_AGENT); }
+template <typename T> __device__ __forceinline__ T ld_acquire(const T* p) { return __hip_atomic_load(p, __ATOMIC_ACQUIRE, BAM_AGENT); }
+template <typename T> __device__ __forceinline__ T ld_relaxed_sys(const volatile T* p) { return __hip_atomic_load((const T*)p, __ATOMIC_RELAXED, BAM_SYSTEM); }
+template <typename T> __device__ __forceinline__ T ld_acquire_sys(const volatile T* p) { return __hip_atomic_load((const T*)p, __ATOMIC_ACQUIRE, BAM_SYSTEM); }
+template <typename T> __device__ __forceinline__ void st_relaxed(T* p, T v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, BAM_AGENT); }
+template <typename T> __device__ __forceinline__ void st_release(T* p, T v) { __hip_atomic_store(p, v, __ATOMIC_RELEASE, BAM_AGENT); }
+template <typename T> __device__ __forceinline__ void st_relaxed_sys(volatile T* p, T v) { __hip_atomic_store((T*)p, v, __ATOMIC_RELAXED, BAM_SYSTEM); }
+template <typename T> __device__ __forceinline__ void st_release_sys(volatile T* p, T v) { __hip_atomic_store((T*)p, v, __ATOMIC_RELEASE, BAM_SYSTEM); }
+
+__device__ __forceinline__ void fence_release_sys() { __builtin_amdgcn_fence(__ATOMIC_RELEASE, ""); }
+__device__ __forceinline__ void fence_acquire_sys() { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, ""); }
+__device__ __forceinline__ void fence_acq_rel_agent() { __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "agent"); }
+
+} // namespace bam
+
+/* names the reference's kernels use */
+__device__ __forceinline__ uint32_t lane_id() { return bam::lane(); }
+__device__ __forceinline__ uint32_t get_smid() { return bam::cu_id(); }
+__device__ __forceinline__ uint32_t warp_id() { return (threadIdx.x + threadIdx.y * blockDim.x) / BAM_WAVE_SIZE; }
+
+#endif /* __BAM_WAVE_H__ */

@@ -1,0 +1,299 @@
+/*
+ * Concurrent NVMe submission/completion protocol for gfx950 wavefronts.
+ *
+ * Same job and same entry points as include/nvm_parallel_queue.h of the
+ * reference (get_cid :35-52, put_cid :54-57, move_tail :59-80, move_head_cq
+ * :82-123, sq_enqueue :167-330, cq_poll :378-422, cq_dequeue :424-535), and
+ * the same wire behaviour towards the controller: ticketed SQ slots, one tail
+ * doorbell per contiguous run of written entries, SQ slots recycled from the
+ * SQHD field of completions, one CQ-head doorbell per run of consumed entries.
+ *
+ * The execution model is different.  A gfx950 wave runs its 64 lanes in lock
+ * step, so a lane must never spin on something a masked-off sibling produces.
+ * Every operation here is therefore done by the whole group of active lanes
+ * that target the same queue:
+ *   - one in_ticket fetch_add(n) per group reserves n consecutive SQ slots;
+ *   - lanes write their own 64-byte entries and set tail_mark; the group's
+ *     leader try-locks tail_lock and the group sweeps up to 64 marks per load;
+ *   - completions are not searched for per thread.  Whichever group holds
+ *     head_lock drains the CQ 64 entries per load and flags each completed
+ *     command in the cid table (cid[c] = LOCKED|DONE); waiters poll their own
+ *     word.  The drainer frees SQ slots from SQHD and rings the CQ doorbell
+ *     once per sweep.
+ * All waits are bounded (bam_guard_t).
+ */
+#ifndef __NVM_PARALLEL_QUEUE_H_
+#define __NVM_PARALLEL_QUEUE_H_
+
+#include "bam_wave.h"
+#include "nvm_types.h"
+#include "nvm_util.h"
+
+#define LOCKED   1
+#define UNLOCKED 0
+#define BAM_CID_DONE 2u
+
+namespace bam {
+
+struct spin_t { uint32_t n = 0, slp = 1; };
+
+/* one back-off step of a wait loop on queue q; true = give up (abort raised or spin limit hit) */
+__device__ __forceinline__ bool spin_giveup(const nvm_queue_t* q, spin_t& s)
+{
+    backoff(s.slp);
+    s.n++;
+    bam_guard_t* g = q->guard;
+    if (!g) return false;
+    if ((s.n & 127u) == 0 && ld_relaxed_sys(&g->abort)) return true;
+    uint32_t lim = q->spin_limit;
+    if (lim && s.n > lim) { st_relaxed_sys(&g->abort, 1u); return true; }
+    return false;
+}
+
+/* lanes of `act` with rank below `run` where run = length of the leading all-true prefix of `ok` in rank order */
+__device__ __forceinline__ uint32_t leading_run(uint64_t act, uint64_t ok)
+{
+    uint64_t miss = act & ~ok;
+    return miss ? popc(act & lanes_below(first_lane(miss))) : popc(act);
+}
+
+/* ---- command ids ---- */
+/*
+ * One allocation attempt for every active lane: true and an id in `id` for the
+ * lanes that got one.  A lane must never wait for an id while siblings hold
+ * theirs (two waves sharing a queue would starve each other), so callers let
+ * the lucky lanes run their command to completion and retry for the rest.
+ */
+__device__ __forceinline__ bool try_get_cid_group(nvm_queue_t* sq, uint32_t& id)
+{
+    const uint64_t act = active_mask();
+    const uint32_t ld = first_lane(act);
+    uint32_t base = 0;
+    if (lane() == ld) base = __hip_atomic_fetch_add(&sq->cid_ticket, popc(act), __ATOMIC_RELAXED, BAM_AGENT);
+    base = bcast(base, ld);
+    const uint32_t probe = (base + rank_in(act)) & sq->cid_mask;
+    const uint32_t old = __hip_atomic_fetch_or(&sq->cid[probe].val, (uint32_t)LOCKED, __ATOMIC_ACQUIRE, BAM_AGENT);
+    id = probe;
+    return old == 0;
+}
+
+/* blocking form for callers that hold nothing else: every active lane ends up with an id */
+__device__ __forceinline__ uint32_t get_cid_group(nvm_queue_t* sq)
+{
+    uint32_t id = 0;
+    bool got = false;
+    spin_t sp;
+    for (;;) {
+        if (!got) got = try_get_cid_group(sq, id);
+        if (!ballot(!got)) break;
+        if (spin_giveup(sq, sp)) break;
+    }
+    return got ? id : 0;
+}
+
+__device__ __forceinline__ void cq_drain_group(nvm_queue_t* cq, nvm_queue_t* sq, uint64_t act);
+
+/* drain the completion queue if nobody else is doing so; true if this group did */
+__device__ __forceinline__ bool try_drain_group(nvm_queue_t* cq, nvm_queue_t* sq)
+{
+    const uint64_t act = active_mask();
+    const uint32_t leader = first_lane(act);
+    uint32_t got = 0;
+    if (lane() == leader)
+        got = ld_relaxed(&cq->head_lock) == UNLOCKED &&
+              __hip_atomic_exchange(&cq->head_lock, (uint32_t)LOCKED, __ATOMIC_ACQUIRE, BAM_AGENT) == UNLOCKED;
+    got = bcast(got, leader);
+    if (got) {
+        cq_drain_group(cq, sq, act);
+        if (lane() == leader) st_release(&cq->head_lock, (uint32_t)UNLOCKED);
+    }
+    return got != 0;
+}
+
+/*
+ * Submit one command per active lane to `sq` (wave-uniform).  Returns the
+ * slot the lane's entry went to.  On return every entry is covered by a
+ * doorbell write.
+ */
+__device__ __forceinline__ uint32_t sq_enqueue_group(nvm_queue_t* sq, const nvm_cmd_t* cmd)
+{
+    const uint64_t act = active_mask();
+    const uint32_t n = popc(act), rank = rank_in(act), leader = first_lane(act);
+    const uint32_t mask = sq->qs_minus_1;
+    uint32_t t0 = 0;
+    if (lane() == leader) t0 = __hip_atomic_fetch_add(&sq->in_ticket, n, __ATOMIC_RELAXED, BAM_AGENT);
+    t0 = bcast(t0, leader);
+    const uint32_t ticket = t0 + rank, pos = ticket & mask;
+    const uint32_t want = (ticket >> sq->qs_log2) * 2u;      /* slot is free for my lap when tickets[pos] == want */
+    bool written = false;
+    spin_t sp;
+    for (;;) {
+        if (!written && ld_acquire(&sq->tickets[pos].val) == want) {
+            uint4* dst = (uint4*)(((nvm_cmd_t*)sq->vaddr) + pos);
+            const uint4* src = (const uint4*)cmd->dword;
+            dst[0] = src[0]; dst[1] = src[1]; dst[2] = src[2]; dst[3] = src[3];
+            /* the entry must be visible to the controller before the mark can be swept into a doorbell */
+            st_release_sys(&sq->tail_mark[pos].val, 1u);
+            written = true;
+        }
+        const uint32_t tl = ld_acquire(&sq->tail);
+        const bool covered = written && (int32_t)(tl - ticket) > 0;
+        if (!ballot(!covered)) break;
+        bool progressed = false;
+        if (ballot(written && !covered)) {
+            /* try to become the tail mover for this queue */
+            uint32_t got = 0;
+            if (lane() == leader)
+                got = ld_relaxed(&sq->tail_lock) == UNLOCKED &&
+                      __hip_atomic_exchange(&sq->tail_lock, (uint32_t)LOCKED, __ATOMIC_ACQUIRE, BAM_AGENT) == UNLOCKED;
+            got = bcast(got, leader);
+            if (got) {
+                const uint32_t cur = ld_relaxed(&sq->tail);
+                /* never let tail + 1 == head (mod qs): at most qs - 1 entries outstanding */
+                const uint32_t room = ld_acquire(&sq->head) + sq->qs - 1u - cur;
+                uint32_t total = 0;
+                for (;;) {
+                    const uint32_t k = total + rank;
+                    const bool m = k < room && ld_acquire(&sq->tail_mark[(cur + k) & mask].val) == 1u;
+                    const uint32_t run = leading_run(act, ballot(m));
+                    if (rank < run) st_relaxed(&sq->tail_mark[(cur + k) & mask].val, 0u);
+                    total += run;
+                    if (run < n) break;
+                }
+                if (lane() == leader) {
+                    if (total) {
+                        fence_release_sys();
+                        st_relaxed_sys(sq->db, (cur + total) & mask);     /* one doorbell for the whole run */
+                        st_release(&sq->tail, cur + total);
+                    }
+                    st_release(&sq->tail_lock, (uint32_t)UNLOCKED);
+                }
+                progressed = total != 0;
+            }
+        }
+        if (!progressed) {
+            /* a full SQ only empties when completions are consumed: do that here too, or a
+             * group larger than the queue would wait on itself */
+            try_drain_group((nvm_queue_t*)sq->pair, sq);
+            if (spin_giveup(sq, sp)) break;
+        }
+    }
+    return pos;
+}
+
+/*
+ * Drain the completion queue: caller's group holds cq->head_lock.  Flags every
+ * completed command in sq->cid[], frees the SQ slots the controller has
+ * consumed (SQHD of the newest completion) and rings the CQ head doorbell once.
+ */
+__device__ __forceinline__ void cq_drain_group(nvm_queue_t* cq, nvm_queue_t* sq, uint64_t act)
+{
+    const uint32_t n = popc(act), rank = rank_in(act), leader = first_lane(act);
+    const uint32_t mask = cq->qs_minus_1;
+    const uint32_t h = ld_relaxed(&cq->head);
+    nvm_cpl_t* ring = (nvm_cpl_t*)cq->vaddr;
+    uint32_t moved = 0, sqhd = 0;
+    for (;;) {
+        const uint32_t idx = h + moved + rank, loc = idx & mask;
+        const uint32_t phase = (~(idx >> cq->qs_log2)) & 1u;          /* first lap carries phase 1 */
+        const uint32_t dw3 = ld_acquire_sys(&ring[loc].dword[3]);
+        const bool valid = ((dw3 >> 16) & 1u) == phase && moved + rank < mask;
+        const uint32_t run = leading_run(act, ballot(valid));
+        if (rank < run) {
+            if (dw3 >> 17) __hip_atomic_fetch_add(&cq->n_errors, 1u, __ATOMIC_RELAXED, BAM_AGENT);
+            st_release(&sq->cid[dw3 & sq->cid_mask].val, (uint32_t)LOCKED | BAM_CID_DONE);
+        }
+        if (run) {
+            uint32_t v = 0;
+            if (rank == run - 1) v = ld_relaxed_sys(&ring[loc].dword[2]) & 0xffffu;
+            /* lane holding the newest entry of the run */
+            uint64_t holder = ballot(rank == run - 1);
+            sqhd = bcast(v, first_lane(holder));
+        }
+        moved += run;
+        if (run < n) break;
+    }
+    if (moved) {
+        const uint32_t smask = sq->qs_minus_1;
+        const uint32_t sh = ld_relaxed(&sq->head);
+        const uint32_t freed = (sqhd - sh) & smask;
+        for (uint32_t i = rank; i < freed; i += n)
+            __hip_atomic_fetch_add(&sq->tickets[(sh + i) & smask].val, 2u, __ATOMIC_RELEASE, BAM_AGENT);
+        if (lane() == leader) {
+            if (freed) st_release(&sq->head, sh + freed);
+            st_relaxed_sys(cq->db, (h + moved) & mask);                /* one doorbell for the whole run */
+            st_release(&cq->head, h + moved);
+        }
+    }
+}
+
+/* Wait until the command `cid` of every active lane has completed on (sq, cq) (wave-uniform). */
+__device__ __forceinline__ void cq_wait_group(nvm_queue_t* cq, nvm_queue_t* sq, uint32_t cid)
+{
+    spin_t sp;
+    for (;;) {
+        const bool done = (ld_acquire(&sq->cid[cid].val) & BAM_CID_DONE) != 0;
+        if (!ballot(!done)) break;
+        try_drain_group(cq, sq);
+        if (spin_giveup(cq, sp)) break;
+    }
+    /* what the controller wrote before posting the completion is visible from here on */
+    fence_acquire_sys();
+}
+
+} // namespace bam
+
+/* ---- per-thread entry points with the reference's names ---- */
+
+inline __device__ uint16_t get_cid(nvm_queue_t* sq)
+{
+    uint32_t id = 0;
+    for (bool done = false; !done;) {
+        nvm_queue_t* cur = (nvm_queue_t*)bam::first((uint64_t)sq);
+        if (cur == sq) { id = bam::get_cid_group(cur); done = true; }
+    }
+    return (uint16_t)id;
+}
+
+inline __device__ void put_cid(nvm_queue_t* sq, uint16_t id)
+{
+    bam::st_release(&sq->cid[id].val, (uint32_t)UNLOCKED);
+}
+
+/* returns the SQ slot used */
+inline __device__ uint16_t sq_enqueue(nvm_queue_t* sq, nvm_cmd_t* cmd)
+{
+    uint32_t pos = 0;
+    for (bool done = false; !done;) {
+        nvm_queue_t* cur = (nvm_queue_t*)bam::first((uint64_t)sq);
+        if (cur == sq) { pos = bam::sq_enqueue_group(cur, cmd); done = true; }
+    }
+    return (uint16_t)pos;
+}
+
+/*
+ * Wait for the completion of command `search_cid` submitted on the SQ paired
+ * with `cq` (cq->pair).  The reference scans the ring and hands back the entry's position
+ * for cq_dequeue; here the drainer has already consumed the entry, so the
+ * out-parameters (which the reference dereferences even when NULL,
+ * nvm_parallel_queue.h:406-407) are optional and receive the current head.
+ */
+inline __device__ uint32_t cq_poll(nvm_queue_t* cq, uint16_t search_cid, uint32_t* loc_ = nullptr, uint32_t* cq_head = nullptr)
+{
+    for (bool done = false; !done;) {
+        nvm_queue_t* cur = (nvm_queue_t*)bam::first((uint64_t)cq);
+        if (cur == cq) { bam::cq_wait_group(cur, (nvm_queue_t*)cur->pair, search_cid); done = true; }
+    }
+    uint32_t h = bam::ld_relaxed(&cq->head);
+    if (loc_) *loc_ = h;
+    if (cq_head) *cq_head = h;
+    return h & cq->qs_minus_1;
+}
+
+/* Completions are consumed by the drainer inside cq_poll; nothing is left to do per entry. */
+inline __device__ void cq_dequeue(nvm_queue_t* cq, uint16_t pos, nvm_queue_t* sq, uint32_t loc_ = 0, uint32_t cur_head_ = 0)
+{
+    (void)cq; (void)pos; (void)sq; (void)loc_; (void)cur_head_;
+}
+
+#endif /* __NVM_PARALLEL_QUEUE_H_ */

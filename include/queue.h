@@ -1,0 +1,118 @@
+/*
+ * I/O queue pair as the device sees it, plus the host code that creates it.
+ * Replaces include/queue.h of the reference (QueuePair :27-49, queue sizing
+ * :95-107, init_gpu_specific_struct :58-85, admin creation :181-203).
+ *
+ * Differences that follow from the wave-cooperative engine: per-slot state is
+ * dense 32-bit words, the command-id table has as many entries as the queue
+ * (ids index a staging window, see below) instead of 65536, and the pos_locks
+ * and head_mark arrays are gone.
+ *
+ * Staged transfers.  When the controller cannot address device memory (the
+ * software target on a machine without CPU-visible VRAM) every queue pair owns
+ * a window of controller-visible staging pages, one per command id; commands
+ * carry the staging page as PRP1 and the submitting lanes move the payload
+ * between staging and device memory themselves.
+ */
+#ifndef __BAM_QUEUE_H__
+#define __BAM_QUEUE_H__
+#include <algorithm>
+#include <cstdint>
+#include <stdexcept>
+#include <string>
+#include "buffer.h"
+#include "nvm_admin.h"
+#include "nvm_aq.h"
+#include "nvm_error.h"
+#include "nvm_types.h"
+#include "util.h"
+
+struct QueuePair
+{
+    uint32_t            pageSize;
+    uint32_t            block_size;
+    uint32_t            block_size_log;
+    uint32_t            block_size_minus_1;
+    uint32_t            nvmNamespace;
+    nvm_queue_t         sq;
+    nvm_queue_t         cq;
+    uint16_t            qp_id;
+    uint8_t*            stage;          /* staging window (NULL: PRPs address device memory directly) */
+    uint64_t            stage_ioaddr;
+    uint32_t            stage_stride;   /* bytes per command id */
+
+    /* host-side owners; a raw pointer keeps the struct trivially copyable to the device */
+    struct Owners {
+        DmaPtr sq_mem, cq_mem, stage_mem;
+        BufferPtr sq_tickets, sq_tail_mark, sq_cid;
+    };
+    Owners*             own;
+    nvm_aq_ref          aq;
+
+    QueuePair(const nvm_ctrl_t* ctrl, const uint32_t hipDevice, const struct nvm_ns_info ns, const struct nvm_ctrl_info info,
+              nvm_aq_ref& aq_ref, const uint16_t qp_id, const uint64_t queueDepth,
+              bam_guard_t* guard = nullptr, uint32_t stage_bytes = 4096, bam_dma_place ring_place = BAM_DMA_HOST)
+    {
+        own = new Owners();
+        aq = aq_ref;
+        /* depth: what was asked for, capped by MQES + 1 and rounded down to a power of two */
+        uint64_t depth = std::min<uint64_t>(queueDepth, (uint64_t)info.max_entries + 1);
+        uint32_t qs = 2;
+        while ((uint64_t)qs * 2 <= depth) qs *= 2;
+
+        own->sq_mem = createDma(ctrl, NVM_PAGE_ALIGN(qs * sizeof(nvm_cmd_t), 1UL << 16), hipDevice, ring_place);
+        own->cq_mem = createDma(ctrl, NVM_PAGE_ALIGN(qs * sizeof(nvm_cpl_t), 1UL << 16), hipDevice, ring_place);
+
+        pageSize = info.page_size;
+        block_size = ns.lba_data_size;
+        block_size_minus_1 = ns.lba_data_size - 1;
+        block_size_log = (uint32_t)__builtin_ctzl(ns.lba_data_size);
+        nvmNamespace = ns.ns_id;
+        this->qp_id = qp_id;
+
+        int status = nvm_admin_cq_create(aq_ref, &cq, qp_id, own->cq_mem.get(), 0, qs);
+        if (!nvm_ok(status)) { delete own; throw std::runtime_error(std::string("Failed to create completion queue: ") + nvm_strerror(status)); }
+        status = nvm_admin_sq_create(aq_ref, &sq, &cq, qp_id, own->sq_mem.get(), 0, qs);
+        if (!nvm_ok(status)) { nvm_admin_cq_delete(aq_ref, &cq); delete own; throw std::runtime_error(std::string("Failed to create submission queue: ") + nvm_strerror(status)); }
+
+        /* device-side protocol state */
+        const uint32_t n_cids = qs;
+        own->sq_tickets = createBuffer(qs * sizeof(padded_struct), hipDevice);
+        own->sq_tail_mark = createBuffer(qs * sizeof(padded_struct), hipDevice);
+        own->sq_cid = createBuffer(n_cids * sizeof(padded_struct), hipDevice);
+        sq.tickets = (padded_struct*)own->sq_tickets.get();
+        sq.tail_mark = (padded_struct*)own->sq_tail_mark.get();
+        sq.cid = (padded_struct*)own->sq_cid.get();
+        sq.cid_mask = n_cids - 1;
+        cq.cid = sq.cid;
+        cq.cid_mask = sq.cid_mask;
+        sq.guard = cq.guard = guard;
+        sq.spin_limit = cq.spin_limit = guard ? guard->spin_limit : 0;
+
+        stage = nullptr; stage_ioaddr = 0; stage_stride = 0;
+        if (stage_bytes) {
+            own->stage_mem = createDma(ctrl, (size_t)n_cids * stage_bytes);
+            stage = (uint8_t*)own->stage_mem->vaddr;
+            stage_ioaddr = own->stage_mem->ioaddrs[0];
+            stage_stride = stage_bytes;
+        }
+    }
+
+    /* the device copy lives at d_self: let each queue find its partner there */
+    void bind_device(QueuePair* d_self)
+    {
+        sq.pair = &d_self->cq;
+        cq.pair = &d_self->sq;
+    }
+
+    QueuePair(const QueuePair&) = delete;
+    QueuePair& operator=(const QueuePair&) = delete;
+
+    ~QueuePair()
+    {
+        if (sq.db) nvm_admin_sq_delete(aq, &sq, &cq);
+        if (cq.db) nvm_admin_cq_delete(aq, &cq);
+        delete own;
+    }
+};
+#endif
