@@ -100,22 +100,26 @@ __global__ __launch_bounds__(256) void k_cache_stream(array_d_t<uint64_t>* dr, u
         const uint64_t epp = r0->n_elems_per_page;
         const uint64_t start_page = assignment ? assignment[wave] : wave * n_pages_per_wave;
         if (MODE == 2) {
-            /* one acquire per page, then 16 bytes per lane per load */
+            /* descriptor read once; per page one acquire, eight loads in flight per lane, one release */
+            bam::range_view<uint64_t> view;
+            view.load(r0);
+            const uint32_t n8 = view.page_size / 8;
             for (uint64_t p = 0; p < n_pages_per_wave; p++) {
-                data_page_t* pg; size_t s, e; int64_t r;
-                const uint4* base = (const uint4*)dr->acquire_page((start_page + p) * epp, pg, s, e, r);
-                const uint32_t n16 = (uint32_t)(r0->cache.page_size / 16);
+                const uint64_t page = view.page_of((start_page + p) * epp);
                 uint64_t a0 = 0, a1 = 0;
-                for (uint32_t i = (uint32_t)lane; i < n16; i += 4 * BAM_WAVE_SIZE) {
-                    uint4 x0 = base[i], x1 = {0, 0, 0, 0}, x2 = {0, 0, 0, 0}, x3 = {0, 0, 0, 0};
-                    if (i + BAM_WAVE_SIZE < n16) x1 = base[i + BAM_WAVE_SIZE];
-                    if (i + 2 * BAM_WAVE_SIZE < n16) x2 = base[i + 2 * BAM_WAVE_SIZE];
-                    if (i + 3 * BAM_WAVE_SIZE < n16) x3 = base[i + 3 * BAM_WAVE_SIZE];
-                    a0 += (((uint64_t)x0.y << 32) | x0.x) + (((uint64_t)x1.y << 32) | x1.x) + (((uint64_t)x2.y << 32) | x2.x) + (((uint64_t)x3.y << 32) | x3.x);
-                    a1 += (((uint64_t)x0.w << 32) | x0.z) + (((uint64_t)x1.w << 32) | x1.z) + (((uint64_t)x2.w << 32) | x2.z) + (((uint64_t)x3.w << 32) | x3.z);
-                }
+                auto sum_page = [&](uint32_t slot) {
+                    const uint64_t* base = (const uint64_t*)view.slot_addr(slot);
+                    for (uint32_t i = (uint32_t)lane; i < n8; i += 8 * BAM_WAVE_SIZE) {
+                        uint64_t x[8];
+#pragma unroll
+                        for (int k = 0; k < 8; k++) x[k] = i + k * BAM_WAVE_SIZE < n8 ? bam::ld_payload(base + i + k * BAM_WAVE_SIZE) : 0;
+                        a0 += x[0] + x[2] + x[4] + x[6];
+                        a1 += x[1] + x[3] + x[5] + x[7];
+                    }
+                    return true;
+                };
+                view.acquire(page, false, sum_page, sum_page);
                 v += a0 + a1;
-                dr->release_page(pg, r, s);
             }
         } else {
             bam_ptr<uint64_t> ptr(dr);

@@ -6,6 +6,9 @@
 #include "nvm_cmd.h"
 #include "nvm_types.h"
 
+#if defined(__x86_64__)
+#include <immintrin.h>
+#endif
 #include <atomic>
 #include <cerrno>
 #include <chrono>
@@ -60,17 +63,23 @@ struct Sq {
     volatile uint32_t* tail_db = nullptr;
 };
 
+// Counters are kept per service thread (relaxed atomics on a private cache line: uncontended) and summed on read.
+struct alignas(128) Stats {
+    std::atomic<uint64_t> admin_cmds{0}, io_cmds{0}, read_cmds{0}, write_cmds{0}, bytes_read{0},
+        bytes_written{0}, error_cpls{0}, sq_doorbells{0}, cq_full_stalls{0}, dropped{0};
+    void bump(std::atomic<uint64_t>& c, uint64_t v = 1) { c.store(c.load(std::memory_order_relaxed) + v, std::memory_order_relaxed); }
+    void clear() { for (auto* c : {&admin_cmds, &io_cmds, &read_cmds, &write_cmds, &bytes_read, &bytes_written, &error_cpls, &sq_doorbells, &cq_full_stalls, &dropped}) c->store(0, std::memory_order_relaxed); }
+};
+
 struct IoThread {
+    Stats stats;
     std::thread th;
     std::mutex mu;                 // guards `sqs` (held by the service loop for one pass)
     std::vector<uint16_t> sqs;     // SQ ids served by this thread
     uint64_t rng = 0x9E3779B97F4A7C15ull;
 };
 
-struct Stats {
-    std::atomic<uint64_t> admin_cmds{0}, io_cmds{0}, read_cmds{0}, write_cmds{0}, bytes_read{0},
-        bytes_written{0}, error_cpls{0}, sq_doorbells{0}, cq_full_stalls{0}, dropped{0};
-};
+
 
 } // namespace
 
@@ -126,13 +135,67 @@ bool for_each_prp(const nvmt* t, const nvm_cmd_t& c, uint64_t bytes, F&& fn)
     return true;
 }
 
-void gen_words(uint64_t seed, uint64_t w0, uint64_t n, uint64_t* out)
+// words w0.. of a procedural namespace.  The loop has independent iterations and 64-bit multiplies, so it
+// vectorises; it is built three times and the widest variant the CPU supports is picked once.
+#define BAM_GEN_WORDS_BODY                                              \
+    const uint64_t s0 = seed + (w0 + 1) * 0x9E3779B97F4A7C15ull;        \
+    for (uint64_t k = 0; k < n; k++) {                                  \
+        uint64_t z = s0 + k * 0x9E3779B97F4A7C15ull;                    \
+        z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;                    \
+        z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;                    \
+        out[k] = z ^ (z >> 31);                                         \
+    }
+#if defined(__x86_64__)
+__attribute__((target("avx512f,avx512dq,avx512vl"), optimize("O3")))
+void gen_words_avx512(uint64_t seed, uint64_t w0, uint64_t n, uint64_t* __restrict__ out) { BAM_GEN_WORDS_BODY }
+__attribute__((target("avx2"), optimize("O3")))
+void gen_words_avx2(uint64_t seed, uint64_t w0, uint64_t n, uint64_t* __restrict__ out) { BAM_GEN_WORDS_BODY }
+#endif
+void gen_words_base(uint64_t seed, uint64_t w0, uint64_t n, uint64_t* __restrict__ out) { BAM_GEN_WORDS_BODY }
+
+// Copy to a DMA destination with streaming stores: the destination is read next by the device over the
+// interconnect, never by this core, so it should neither be read for ownership nor stay in this core's cache.
+#if defined(__x86_64__)
+__attribute__((target("avx2")))
+void copy_out_avx2(void* dst, const void* src, size_t n)
 {
-    uint64_t s = seed + (w0 + 1) * 0x9E3779B97F4A7C15ull;
-    for (uint64_t k = 0; k < n; k++, s += 0x9E3779B97F4A7C15ull) out[k] = mix64(s);
+    if (((uintptr_t)dst | (uintptr_t)src | n) & 31) { memcpy(dst, src, n); return; }
+    const __m256i* s = (const __m256i*)src;
+    __m256i* d = (__m256i*)dst;
+    for (size_t i = 0; i < n / 32; i++) _mm256_stream_si256(d + i, _mm256_load_si256(s + i));
+}
+#endif
+void copy_out_base(void* dst, const void* src, size_t n) { memcpy(dst, src, n); }
+typedef void (*copy_out_fn)(void*, const void*, size_t);
+copy_out_fn pick_copy_out()
+{
+#if defined(__x86_64__)
+    __builtin_cpu_init();
+    if (__builtin_cpu_supports("avx2") && !getenv("NVMT_NO_STREAMING_STORES")) return copy_out_avx2;
+#endif
+    return copy_out_base;
+}
+const copy_out_fn copy_out = pick_copy_out();
+inline void copy_out_fence()
+{
+#if defined(__x86_64__)
+    _mm_sfence();
+#endif
 }
 
-uint16_t do_rw(nvmt* t, const nvm_cmd_t& c, bool write)
+typedef void (*gen_words_fn)(uint64_t, uint64_t, uint64_t, uint64_t*);
+gen_words_fn pick_gen_words()
+{
+#if defined(__x86_64__)
+    __builtin_cpu_init();
+    if (__builtin_cpu_supports("avx512dq") && __builtin_cpu_supports("avx512vl")) return gen_words_avx512;
+    if (__builtin_cpu_supports("avx2")) return gen_words_avx2;
+#endif
+    return gen_words_base;
+}
+const gen_words_fn gen_words = pick_gen_words();
+
+uint16_t do_rw(nvmt* t, Stats& st_, const nvm_cmd_t& c, bool write)
 {
     const uint32_t lba = t->cfg.lba_bytes;
     uint64_t slba = ((uint64_t)c.dword[11] << 32) | c.dword[10];
@@ -142,37 +205,38 @@ uint16_t do_rw(nvmt* t, const nvm_cmd_t& c, bool write)
     if (c.dword[1] != 1) return ST_INVALID_FIELD;
     if (write && !t->cfg.backing) return ST_WRITE_RO;
     uint64_t done = 0;
-    alignas(64) uint64_t tmp[512];
+    alignas(64) uint64_t tmp[512];      /* sizeof(tmp) is the generation chunk */
     bool ok = for_each_prp(t, c, bytes, [&](uint64_t addr, uint64_t len) {
         uint8_t* p = (uint8_t*)addr;
         if (write) {
             memcpy((uint8_t*)t->cfg.backing + off + done, p, len);
         } else if (t->cfg.backing) {
-            memcpy(p, (const uint8_t*)t->cfg.backing + off + done, len);
+            copy_out(p, (const uint8_t*)t->cfg.backing + off + done, len);
         } else {
             // procedural content, generated in cache then copied out (pieces are multiples of 8 bytes)
             for (uint64_t k = 0; k < len; k += sizeof(tmp)) {
                 uint64_t n = len - k < sizeof(tmp) ? len - k : sizeof(tmp);
                 gen_words(t->cfg.seed, (off + done + k) / 8, n / 8, tmp);
-                memcpy(p + k, tmp, n);
+                copy_out(p + k, tmp, n);
             }
         }
         done += len;
     });
     if (!ok) return ST_INVALID_FIELD;
-    if (write) { t->stats.write_cmds++; t->stats.bytes_written += bytes; }
-    else       { t->stats.read_cmds++;  t->stats.bytes_read += bytes; }
+    if (!write) copy_out_fence();       /* streaming stores are weakly ordered: drain them before the completion is posted */
+    if (write) { st_.bump(st_.write_cmds); st_.bump(st_.bytes_written, bytes); }
+    else       { st_.bump(st_.read_cmds);  st_.bump(st_.bytes_read, bytes); }
     return ST_OK;
 }
 
 // Post one completion; waits while the CQ is full (head doorbell not advanced).
-bool post_cpl(nvmt* t, Cq& cq, uint16_t sqid, uint16_t sqhd, uint16_t cid, uint16_t status, uint32_t dw0)
+bool post_cpl(nvmt* t, Stats& st_, Cq& cq, uint16_t sqid, uint16_t sqhd, uint16_t cid, uint16_t status, uint32_t dw0)
 {
     // tail is an index in [0, qs); admin queues need not be powers of two
     const uint32_t next = cq.tail + 1 == cq.qs ? 0 : cq.tail + 1;
     bool stalled = false;
     while (next == ld<uint32_t>(cq.head_db) % cq.qs) {
-        if (!stalled) { t->stats.cq_full_stalls++; stalled = true; }
+        if (!stalled) { st_.bump(st_.cq_full_stalls); stalled = true; }
         if (t->stop.load(std::memory_order_relaxed)) return false;
         cpu_relax();
     }
@@ -184,7 +248,7 @@ bool post_cpl(nvmt* t, Cq& cq, uint16_t sqid, uint16_t sqhd, uint16_t cid, uint1
     st<uint32_t>(&e->dword[3], (uint32_t)cid | (cq.phase << 16) | ((uint32_t)status << 17));
     cq.tail = next;
     if (next == 0) cq.phase ^= 1;
-    if (status) t->stats.error_cpls++;
+    if (status) st_.bump(st_.error_cpls);
     return true;
 }
 
@@ -193,7 +257,8 @@ void serve_sq(nvmt* t, IoThread* me, Sq& sq)
     Cq& cq = t->cqs[sq.cqid];
     const uint32_t mask = sq.qs - 1;
     uint32_t tail = ld<uint32_t>(sq.tail_db) & mask;
-    if (tail != sq.last_tail) { t->stats.sq_doorbells++; sq.last_tail = tail; }
+    Stats& st_ = me->stats;
+    if (tail != sq.last_tail) { st_.bump(st_.sq_doorbells); sq.last_tail = tail; }
     while (((tail - sq.head) & mask) != 0) {
         nvm_cmd_t batch[64];
         uint32_t n = (tail - sq.head) & mask;
@@ -212,18 +277,19 @@ void serve_sq(nvmt* t, IoThread* me, Sq& sq)
             const nvm_cmd_t& c = batch[order[k]];
             uint8_t op = c.dword[0] & 0xff;
             uint16_t cid = c.dword[0] >> 16, status;
-            uint64_t seq = ++t->cmd_seq;
-            t->stats.io_cmds++;
-            if (t->cfg.drop_every && seq % t->cfg.drop_every == 0) { t->stats.dropped++; continue; }
+            const bool inject = t->cfg.drop_every || t->cfg.fail_every;
+            const uint64_t seq = inject ? ++t->cmd_seq : 0;       // a shared counter only when fault injection needs one
+            st_.bump(st_.io_cmds);
+            if (t->cfg.drop_every && seq % t->cfg.drop_every == 0) { st_.bump(st_.dropped); continue; }
             if (t->cfg.fail_every && seq % t->cfg.fail_every == 0) status = ST_DATA_XFER_ERROR;
-            else if (op == NVM_IO_READ) status = do_rw(t, c, false);
-            else if (op == NVM_IO_WRITE) status = do_rw(t, c, true);
+            else if (op == NVM_IO_READ) status = do_rw(t, st_, c, false);
+            else if (op == NVM_IO_WRITE) status = do_rw(t, st_, c, true);
             else if (op == NVM_IO_FLUSH) status = ST_OK;
             else status = ST_INVALID_OPCODE;
             if (status && t->trace_errors.load(std::memory_order_relaxed) > 0 && t->trace_errors.fetch_sub(1) > 0)
                 fprintf(stderr, "[nvmt] sq %u status %#x: dw0 %08x nsid %u prp1 %08x%08x prp2 %08x%08x slba %08x%08x dw12 %08x (sq head %u)\n",
                         sq.id, status, c.dword[0], c.dword[1], c.dword[7], c.dword[6], c.dword[9], c.dword[8], c.dword[11], c.dword[10], c.dword[12], sq.head);
-            if (!post_cpl(t, cq, sq.id, (uint16_t)sq.head, cid, status, 0)) return;
+            if (!post_cpl(t, st_, cq, sq.id, (uint16_t)sq.head, cid, status, 0)) return;
         }
     }
 }
@@ -294,7 +360,7 @@ void admin_cmd(nvmt* t, const nvm_cmd_t& c)
     uint64_t prp1 = ((uint64_t)c.dword[7] << 32) | c.dword[6];
     uint16_t qid = c.dword[10] & 0xffff;
     uint32_t qs = (c.dword[10] >> 16) + 1;
-    t->stats.admin_cmds++;
+    t->stats.bump(t->stats.admin_cmds);
     switch (op) {
     case NVM_ADMIN_IDENTIFY: identify(t, c, status); break;
     case NVM_ADMIN_SET_FEATURES:
@@ -353,7 +419,7 @@ void admin_cmd(nvmt* t, const nvm_cmd_t& c)
     case NVM_ADMIN_ABORT: break;
     default: status = ST_INVALID_OPCODE;
     }
-    post_cpl(t, t->acq, 0, (uint16_t)t->asq.head, cid, status, dw0);
+    post_cpl(t, t->stats, t->acq, 0, (uint16_t)t->asq.head, cid, status, dw0);
 }
 
 void teardown_io(nvmt* t)
@@ -486,17 +552,20 @@ volatile void* nvmt_bar(nvmt_t* t) { return t->bar; }
 
 void nvmt_stats(nvmt_t* t, nvmt_stats_t* o)
 {
-    o->admin_cmds = t->stats.admin_cmds; o->io_cmds = t->stats.io_cmds; o->read_cmds = t->stats.read_cmds;
-    o->write_cmds = t->stats.write_cmds; o->bytes_read = t->stats.bytes_read; o->bytes_written = t->stats.bytes_written;
-    o->error_cpls = t->stats.error_cpls; o->sq_doorbells = t->stats.sq_doorbells;
-    o->cq_full_stalls = t->stats.cq_full_stalls; o->dropped = t->stats.dropped;
+    memset(o, 0, sizeof(*o));
+    auto add = [&](const Stats& s) {
+        o->admin_cmds += s.admin_cmds; o->io_cmds += s.io_cmds; o->read_cmds += s.read_cmds; o->write_cmds += s.write_cmds;
+        o->bytes_read += s.bytes_read; o->bytes_written += s.bytes_written; o->error_cpls += s.error_cpls;
+        o->sq_doorbells += s.sq_doorbells; o->cq_full_stalls += s.cq_full_stalls; o->dropped += s.dropped;
+    };
+    add(t->stats);
+    for (IoThread* th : t->io) add(th->stats);
 }
 
 void nvmt_reset_stats(nvmt_t* t)
 {
-    t->stats.admin_cmds = 0; t->stats.io_cmds = 0; t->stats.read_cmds = 0; t->stats.write_cmds = 0;
-    t->stats.bytes_read = 0; t->stats.bytes_written = 0; t->stats.error_cpls = 0; t->stats.sq_doorbells = 0;
-    t->stats.cq_full_stalls = 0; t->stats.dropped = 0;
+    t->stats.clear();
+    for (IoThread* th : t->io) th->stats.clear();
 }
 
 void nvmt_fill_words(uint64_t seed, uint64_t first_word, uint64_t n, uint64_t* out) { gen_words(seed, first_word, n, out); }

@@ -77,7 +77,7 @@ class Target:
 
 
 class Controller:
-    def __init__(self, path, ns_id=1, device=0, queue_depth=1024, n_queues=128, stage_bytes=4096, spin_limit=1 << 24):
+    def __init__(self, path, ns_id=1, device=0, queue_depth=1024, n_queues=128, stage_bytes=4096, spin_limit=10_000_000):
         self.L = _lib.load()
         self.h = c_vp()
         self.device = device

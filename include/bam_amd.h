@@ -44,7 +44,7 @@ void* bam_target_backing(bam_target_t* t);
 
 /* ---- Controller (include/ctrl.h:148-199 of the reference) ----
  * stage_bytes: size of the per-command staging page (0 = PRPs address device memory directly, needs CPU-visible VRAM);
- * spin_limit: bound of every device-side wait loop, in back-off steps (0 = unbounded). */
+ * spin_limit: bound of every device-side wait loop, in microseconds (0 = unbounded). */
 int bam_ctrl_create(bam_ctrl_t** out, const char* path, uint32_t ns_id, uint32_t device, uint64_t queue_depth, uint64_t n_queues,
                     uint32_t stage_bytes, uint32_t spin_limit);
 void bam_ctrl_destroy(bam_ctrl_t* c);

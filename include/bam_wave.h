@@ -108,6 +108,28 @@ template <typename T> __device__ __forceinline__ void st_release(T* p, T v) { __
 template <typename T> __device__ __forceinline__ void st_relaxed_sys(volatile T* p, T v) { __hip_atomic_store((T*)p, v, __ATOMIC_RELAXED, BAM_SYSTEM); }
 template <typename T> __device__ __forceinline__ void st_release_sys(volatile T* p, T v) { __hip_atomic_store((T*)p, v, __ATOMIC_RELEASE, BAM_SYSTEM); }
 
+/*
+ * Load of page-cache payload.  A cache slot is refilled by other compute units
+ * over the life of a kernel, so payload must never be served from this compute
+ * unit's vector L1: an agent-scope load goes to L2, which the hardware keeps
+ * coherent for device memory.  This is what lets the hit path take its page
+ * reference with a relaxed atomic instead of an acquire (an acquire at agent
+ * scope invalidates caches on every page visit).
+ */
+template <typename T> __device__ __forceinline__ T ld_payload(const T* p)
+{
+    if constexpr (sizeof(T) == 8) { uint64_t v = __hip_atomic_load((const uint64_t*)p, __ATOMIC_RELAXED, BAM_AGENT); return *(T*)&v; }
+    else if constexpr (sizeof(T) == 4) { uint32_t v = __hip_atomic_load((const uint32_t*)p, __ATOMIC_RELAXED, BAM_AGENT); return *(T*)&v; }
+    else if constexpr (sizeof(T) == 2) { uint16_t v = __hip_atomic_load((const uint16_t*)p, __ATOMIC_RELAXED, BAM_AGENT); return *(T*)&v; }
+    else if constexpr (sizeof(T) == 1) { uint8_t v = __hip_atomic_load((const uint8_t*)p, __ATOMIC_RELAXED, BAM_AGENT); return *(T*)&v; }
+    else if constexpr (sizeof(T) == 16) {
+        uint64_t v[2];
+        v[0] = __hip_atomic_load((const uint64_t*)p, __ATOMIC_RELAXED, BAM_AGENT);
+        v[1] = __hip_atomic_load((const uint64_t*)p + 1, __ATOMIC_RELAXED, BAM_AGENT);
+        return *(T*)v;
+    } else { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent"); return *p; }
+}
+
 __device__ __forceinline__ void fence_release_sys() { __builtin_amdgcn_fence(__ATOMIC_RELEASE, ""); }
 __device__ __forceinline__ void fence_acquire_sys() { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, ""); }
 __device__ __forceinline__ void fence_acq_rel_agent() { __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "agent"); }

@@ -56,7 +56,7 @@ struct Controller
     Owners*                 own;
 
     Controller(const char* path, uint32_t nvmNamespace, uint32_t hipDevice, uint64_t queueDepth, uint64_t numQueues,
-               uint32_t stage_bytes = 4096, uint32_t spin_limit = 1u << 24)
+               uint32_t stage_bytes = 4096, uint32_t spin_limit = 10000000)
         : ctrl(nullptr), aq_ref(nullptr), deviceId(hipDevice)
     {
         nvmt_t* target = nvmt_lookup(path);
@@ -66,7 +66,7 @@ struct Controller
 
     /* register window supplied directly (a target the caller owns, or a mapped BAR0) */
     Controller(volatile void* mm_ptr, size_t mm_size, uint32_t nvmNamespace, uint32_t hipDevice, uint64_t queueDepth, uint64_t numQueues,
-               uint32_t stage_bytes = 4096, uint32_t spin_limit = 1u << 24)
+               uint32_t stage_bytes = 4096, uint32_t spin_limit = 10000000)
         : ctrl(nullptr), aq_ref(nullptr), deviceId(hipDevice)
     {
         bringup(mm_ptr, mm_size, nvmNamespace, queueDepth, numQueues, stage_bytes, spin_limit);

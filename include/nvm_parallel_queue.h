@@ -35,20 +35,26 @@
 
 namespace bam {
 
-struct spin_t { uint32_t n = 0, slp = 1; };
+struct spin_t { uint32_t n = 0, slp = 1; uint64_t t0 = 0; };
 
-/* one back-off step of a wait loop on queue q; true = give up (abort raised or spin limit hit) */
-__device__ __forceinline__ bool spin_giveup(const nvm_queue_t* q, spin_t& s)
+/*
+ * One back-off step of a wait loop; true = give up.  Every 64 steps the loop
+ * looks at the shared abort flag and at the wall clock (100 MHz constant
+ * counter): a wait that has lasted longer than `limit_us` microseconds raises
+ * the abort flag itself.  limit_us = 0 waits for ever.
+ */
+__device__ __forceinline__ bool spin_giveup(bam_guard_t* g, uint32_t limit_us, spin_t& s)
 {
     backoff(s.slp);
-    s.n++;
-    bam_guard_t* g = q->guard;
-    if (!g) return false;
-    if ((s.n & 127u) == 0 && ld_relaxed_sys(&g->abort)) return true;
-    uint32_t lim = q->spin_limit;
-    if (lim && s.n > lim) { st_relaxed_sys(&g->abort, 1u); return true; }
+    if ((++s.n & 63u) != 0 || !g) return false;
+    if (ld_relaxed_sys(&g->abort)) return true;
+    if (!limit_us) return false;
+    const uint64_t now = wall_clock64();
+    if (!s.t0) { s.t0 = now; return false; }
+    if (now - s.t0 > (uint64_t)limit_us * 100u) { st_relaxed_sys(&g->abort, 1u); return true; }
     return false;
 }
+__device__ __forceinline__ bool spin_giveup(const nvm_queue_t* q, spin_t& s) { return spin_giveup(q->guard, q->spin_limit, s); }
 
 /* lanes of `act` with rank below `run` where run = length of the leading all-true prefix of `ok` in rank order */
 __device__ __forceinline__ uint32_t leading_run(uint64_t act, uint64_t ok)
@@ -59,36 +65,40 @@ __device__ __forceinline__ uint32_t leading_run(uint64_t act, uint64_t ok)
 
 /* ---- command ids ---- */
 /*
- * One allocation attempt for every active lane: true and an id in `id` for the
- * lanes that got one.  A lane must never wait for an id while siblings hold
- * theirs (two waves sharing a queue would starve each other), so callers let
- * the lucky lanes run their command to completion and retry for the rest.
+ * Command ids are handed out to a group of lanes as one block of 64 (ids
+ * 64*b .. 64*b+63): one atomic per wave instead of one per command, and a
+ * wave never sits on a few ids while it waits for more, which would leave two
+ * waves that share a queue each holding part of what the other needs.
+ * Returns the lane's id (block base + rank of the lane in the group); the
+ * caller holds nothing else it would have to give up while this waits.
  */
-__device__ __forceinline__ bool try_get_cid_group(nvm_queue_t* sq, uint32_t& id)
-{
-    const uint64_t act = active_mask();
-    const uint32_t ld = first_lane(act);
-    uint32_t base = 0;
-    if (lane() == ld) base = __hip_atomic_fetch_add(&sq->cid_ticket, popc(act), __ATOMIC_RELAXED, BAM_AGENT);
-    base = bcast(base, ld);
-    const uint32_t probe = (base + rank_in(act)) & sq->cid_mask;
-    const uint32_t old = __hip_atomic_fetch_or(&sq->cid[probe].val, (uint32_t)LOCKED, __ATOMIC_ACQUIRE, BAM_AGENT);
-    id = probe;
-    return old == 0;
-}
-
-/* blocking form for callers that hold nothing else: every active lane ends up with an id */
 __device__ __forceinline__ uint32_t get_cid_group(nvm_queue_t* sq)
 {
-    uint32_t id = 0;
-    bool got = false;
-    spin_t sp;
-    for (;;) {
-        if (!got) got = try_get_cid_group(sq, id);
-        if (!ballot(!got)) break;
-        if (spin_giveup(sq, sp)) break;
+    const uint64_t act = active_mask();
+    const uint32_t leader = first_lane(act);
+    const uint32_t n_blocks = (sq->cid_mask + 1u) >> 6;
+    uint32_t base = 0;
+    if (lane() == leader) {
+        spin_t sp;
+        for (;;) {
+            const uint32_t b = __hip_atomic_fetch_add(&sq->cid_ticket, 1u, __ATOMIC_RELAXED, BAM_AGENT) % n_blocks;
+            if (ld_relaxed(&sq->pos_locks[b].val) == UNLOCKED &&
+                __hip_atomic_exchange(&sq->pos_locks[b].val, (uint32_t)LOCKED, __ATOMIC_ACQUIRE, BAM_AGENT) == UNLOCKED) { base = b << 6; break; }
+            if (spin_giveup(sq, sp)) break;
+        }
     }
-    return got ? id : 0;
+    base = bcast(base, leader);
+    const uint32_t id = base + rank_in(act);
+    st_relaxed(&sq->cid[id].val, (uint32_t)LOCKED);
+    return id;
+}
+
+/* give the group's block of command ids back (every lane of the group that called get_cid_group) */
+__device__ __forceinline__ void put_cid_group(nvm_queue_t* sq, uint32_t id)
+{
+    const uint64_t act = active_mask();
+    st_relaxed(&sq->cid[id].val, (uint32_t)UNLOCKED);
+    if (lane() == first_lane(act)) st_release(&sq->pos_locks[id >> 6].val, (uint32_t)UNLOCKED);
 }
 
 __device__ __forceinline__ void cq_drain_group(nvm_queue_t* cq, nvm_queue_t* sq, uint64_t act);
@@ -255,9 +265,13 @@ inline __device__ uint16_t get_cid(nvm_queue_t* sq)
     return (uint16_t)id;
 }
 
+/* to be called by the same lanes that called get_cid together */
 inline __device__ void put_cid(nvm_queue_t* sq, uint16_t id)
 {
-    bam::st_release(&sq->cid[id].val, (uint32_t)UNLOCKED);
+    for (bool done = false; !done;) {
+        nvm_queue_t* cur = (nvm_queue_t*)bam::first((uint64_t)sq);
+        if (cur == sq) { bam::put_cid_group(cur, id); done = true; }
+    }
 }
 
 /* returns the SQ slot used */

@@ -49,10 +49,10 @@ typedef struct
 } nvm_dma_t;
 
 /*
- * Bounded waits of the device path.  Every spin loop gives up after
- * spin_limit trips (0 = never) or as soon as `abort` is non-zero, and sets
- * `abort` when it does, so that a lost completion ends the kernel instead of
- * hanging the GPU.  Lives in host-pinned memory; the host reads it after the
+ * Bounded waits of the device path.  Every spin loop gives up once it has
+ * waited spin_limit microseconds (0 = never) or as soon as `abort` is
+ * non-zero, and sets `abort` when it does, so that a lost completion ends the
+ * kernel instead of hanging the GPU.  Lives in host-pinned memory; the host reads it after the
  * kernel to tell whether results are valid.
  */
 typedef struct bam_guard
@@ -82,8 +82,8 @@ typedef struct
     padded_struct*          tickets;        /* SQ [qs]: 2*lap = free for lap, odd = submitted */
     padded_struct*          head_mark;      /* unused by the wave-cooperative engine (kept for layout parity) */
     padded_struct*          tail_mark;      /* SQ [qs]: 1 = written, waiting for the tail sweep */
-    padded_struct*          cid;            /* SQ [n_cids]: 0 free, 1 in flight, 3 in flight + completed */
-    padded_struct*          pos_locks;      /* unused by the wave-cooperative engine */
+    padded_struct*          cid;            /* SQ [n_cids]: per command id, 0 idle, 1 in flight, 3 in flight + completed */
+    padded_struct*          pos_locks;      /* SQ [n_cids / 64]: command ids are handed out to a wave in blocks of 64; 1 = block taken */
     uint32_t                cid_mask;       /* n_cids - 1 */
     struct bam_guard*       guard;          /* device path: bounded-wait control (may be NULL) */
     uint32_t                spin_limit;     /* device path: copy of guard->spin_limit */

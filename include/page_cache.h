@@ -66,7 +66,7 @@ enum data_dist_t { REPLICATE = 0, STRIPE = 1 };
 #define V_NB  0x02U
 #define V_B   0x03U
 
-#define BAM_STAT_SHARDS 64
+#define BAM_STAT_SHARDS 256
 
 struct page_cache_t;
 struct page_cache_d_t;
@@ -75,8 +75,9 @@ template <typename T> struct array_d_t;
 template <typename T> struct range_d_t;
 
 /* one per backing page */
-typedef struct { uint32_t state; uint32_t offset; } data_page_t;
+typedef struct __attribute__((aligned(8))) { uint32_t state; uint32_t offset; } data_page_t;   /* read as one 64-bit word on the hit path */
 typedef data_page_t* pages_t;
+__forceinline__ __device__ void bam_release_refs(data_page_t* dp, const uint32_t count, const bool wrote);
 
 /* one per cache slot */
 typedef struct { uint32_t page_take_lock; uint32_t pad; uint64_t page_translation; } cache_page_t;
@@ -118,21 +119,13 @@ struct page_cache_d_t {
     uint64_t n_ctrls;
     bool prps;
     uint64_t n_blocks_per_page;
-    uint32_t wave_batch;             /* distinct pages one wave may hold referenced while it loads (1..64) */
+    uint32_t wave_batch;             /* distinct pages one wave loads side by side (64: a whole wave) */
     bam_guard_t* guard;
     uint32_t spin_limit;
 
     __forceinline__ __device__ cache_page_t* get_cache_page(const uint32_t page) const { return &cache_pages[page]; }
     __forceinline__ __device__ uint32_t find_slot(uint64_t address, uint64_t range_id, const uint32_t queue_);
-    __forceinline__ __device__ bool spin_giveup(bam::spin_t& s) const
-    {
-        bam::backoff(s.slp);
-        s.n++;
-        if (!guard) return false;
-        if ((s.n & 127u) == 0 && bam::ld_relaxed_sys(&guard->abort)) return true;
-        if (spin_limit && s.n > spin_limit) { bam::st_relaxed_sys(&guard->abort, 1u); return true; }
-        return false;
-    }
+    __forceinline__ __device__ bool spin_giveup(bam::spin_t& s) const { return bam::spin_giveup(guard, spin_limit, s); }
 };
 
 __device__ void read_data(page_cache_d_t* pc, QueuePair* qp, const uint64_t starting_lba, const uint64_t n_blocks, const unsigned long long pc_entry);
@@ -156,66 +149,62 @@ uint64_t get_backing_ctrl_(const size_t page_offset, const uint64_t n_ctrls, con
 namespace bam {
 
 /*
+ * Move each active lane's payload (dst/src/bytes differ per lane) with the
+ * whole group: one lane's payload at a time, 16 bytes per lane per access.
+ * All loads of a 4 KiB page are issued before its stores so that one page
+ * costs one trip over the interconnect, not four.
+ */
+__device__ __forceinline__ void copy_pages(uint8_t* dst, const uint8_t* src, uint32_t bytes, uint64_t act, uint32_t n, uint32_t rank)
+{
+    for (uint64_t m = act; m; m &= m - 1) {
+        const uint32_t j = first_lane(m);
+        const uint4* s = (const uint4*)bcast((uint64_t)src, j);
+        uint4* d = (uint4*)bcast((uint64_t)dst, j);
+        const uint32_t nb = bcast(bytes, j) / 16;
+        uint32_t i = rank;
+        for (; i + 3 * n < nb; i += 4 * n) {
+            const uint4 x0 = s[i], x1 = s[i + n], x2 = s[i + 2 * n], x3 = s[i + 3 * n];
+            d[i] = x0; d[i + n] = x1; d[i + 2 * n] = x2; d[i + 3 * n] = x3;
+        }
+        for (; i < nb; i += n) d[i] = s[i];
+    }
+}
+
+/*
  * One command per active lane on queue pair `qp` (wave-uniform): allocate ids,
  * build and submit the entries as one batch, wait for all completions, move
  * staged payload, recycle ids.  `pc_entry` is the cache slot the data belongs to.
  */
 __device__ __forceinline__ void io_group(page_cache_d_t* pc, QueuePair* qp, uint64_t lba, uint32_t n_blocks, uint64_t pc_entry, uint8_t opcode)
 {
+    const uint64_t act = active_mask();
+    const uint32_t n = popc(act), rank = rank_in(act);
     const uint32_t bytes = n_blocks << qp->block_size_log;
     uint8_t* slot_addr = pc->base_addr + pc_entry * pc->page_size;
-    bool pending = true;
-    spin_t sp;
-    for (;;) {
-        /* lanes that get a command id run their command to completion; the others try again afterwards */
-        uint32_t cid = 0;
-        const bool ready = pending && try_get_cid_group(&qp->sq, cid);
-        if (ready) {
-            const uint64_t act = active_mask();
-            const uint32_t n = popc(act), rank = rank_in(act);
-            uint64_t prp1, prp2 = 0;
-            uint8_t* stage = nullptr;
-            if (qp->stage) {
-                stage = qp->stage + (size_t)cid * qp->stage_stride;
-                prp1 = qp->stage_ioaddr + (uint64_t)cid * qp->stage_stride;
-                if (opcode == NVM_IO_WRITE) {
-                    /* payload to staging, one lane's page at a time, 16 bytes per lane per trip */
-                    for (uint64_t m = act; m; m &= m - 1) {
-                        const uint32_t j = first_lane(m);
-                        uint4* d = (uint4*)bcast((uint64_t)stage, j);
-                        const uint4* s = (const uint4*)bcast((uint64_t)slot_addr, j);
-                        const uint32_t nb = bcast(bytes, j) / 16;
-                        for (uint32_t i = rank; i < nb; i += n) d[i] = s[i];
-                    }
-                    fence_release_sys();
-                }
-            } else {
-                prp1 = pc->prp1[pc_entry];
-                if (pc->prps) prp2 = pc->prp2[pc_entry];
-            }
-            nvm_cmd_t cmd;
-#pragma unroll
-            for (int i = 0; i < 16; i++) cmd.dword[i] = 0;
-            nvm_cmd_header(&cmd, (uint16_t)cid, opcode, qp->nvmNamespace);
-            nvm_cmd_data_ptr(&cmd, prp1, prp2);
-            nvm_cmd_rw_blks(&cmd, lba, (uint16_t)n_blocks);
-            sq_enqueue_group(&qp->sq, &cmd);
-            cq_wait_group(&qp->cq, &qp->sq, cid);
-            if (stage && opcode == NVM_IO_READ) {
-                for (uint64_t m = act; m; m &= m - 1) {
-                    const uint32_t j = first_lane(m);
-                    const uint4* s = (const uint4*)bcast((uint64_t)stage, j);
-                    uint4* d = (uint4*)bcast((uint64_t)slot_addr, j);
-                    const uint32_t nb = bcast(bytes, j) / 16;
-                    for (uint32_t i = rank; i < nb; i += n) d[i] = s[i];
-                }
-            }
-            st_release(&qp->sq.cid[cid].val, (uint32_t)UNLOCKED);
-            pending = false;
+    const uint32_t cid = get_cid_group(&qp->sq);
+    uint64_t prp1, prp2 = 0;
+    uint8_t* stage = nullptr;
+    if (qp->stage) {
+        stage = qp->stage + (size_t)cid * qp->stage_stride;
+        prp1 = qp->stage_ioaddr + (uint64_t)cid * qp->stage_stride;
+        if (opcode == NVM_IO_WRITE) {
+            copy_pages(stage, slot_addr, bytes, act, n, rank);
+            fence_release_sys();
         }
-        if (!ballot(pending)) break;
-        if (!ballot(ready) && spin_giveup(&qp->sq, sp)) break;
+    } else {
+        prp1 = pc->prp1[pc_entry];
+        if (pc->prps) prp2 = pc->prp2[pc_entry];
     }
+    nvm_cmd_t cmd;
+#pragma unroll
+    for (int i = 0; i < 16; i++) cmd.dword[i] = 0;
+    nvm_cmd_header(&cmd, (uint16_t)cid, opcode, qp->nvmNamespace);
+    nvm_cmd_data_ptr(&cmd, prp1, prp2);
+    nvm_cmd_rw_blks(&cmd, lba, (uint16_t)n_blocks);
+    sq_enqueue_group(&qp->sq, &cmd);
+    cq_wait_group(&qp->cq, &qp->sq, cid);
+    if (stage && opcode == NVM_IO_READ) copy_pages(slot_addr, stage, bytes, act, n, rank);
+    put_cid_group(&qp->sq, cid);
 }
 
 } // namespace bam
@@ -243,26 +232,31 @@ inline __device__ void write_data(page_cache_d_t* pc, QueuePair* qp, const uint6
 /* eviction                                                           */
 /* ------------------------------------------------------------------ */
 
+#define BAM_NO_SLOT 0xffffffffu
+#define BAM_FIND_SLOT_TRIES 64
+
 /*
  * Find a cache slot for page `address` of range `range_id`: a global
  * round-robin hand (page_ticket); a slot is taken if it is free, or if its
  * current page has no references and is not busy, in which case that page is
  * invalidated (and written back first when dirty).  Called by all lanes of a
  * wave that need a slot; they advance side by side and take one ticket grab
- * per trip for the whole group.
+ * per trip for the whole group.  A lane gives up after BAM_FIND_SLOT_TRIES
+ * slots and returns BAM_NO_SLOT: its caller then lets the lanes that did get
+ * a slot finish their loads before trying again, so that waves never wait for
+ * slots while sitting on slots other waves wait for.
  */
 __forceinline__ __device__
 uint32_t page_cache_d_t::find_slot(uint64_t address, uint64_t range_id, const uint32_t queue_)
 {
     using namespace bam;
     const uint64_t global_address = (address << n_ranges_bits) | range_id;
-    uint32_t page = 0;
-    bool found = false;
-    spin_t sp;
-    for (;;) {
-        const uint64_t need = ballot(!found);
+    uint32_t page = BAM_NO_SLOT;
+    bool looking = true;
+    for (uint32_t tries = 0;; tries++) {
+        const uint64_t need = ballot(looking);
         if (!need) break;
-        if (!found) {
+        if (looking) {
             const uint32_t ld = first_lane(need);
             uint32_t base = 0;
             if (lane() == ld) base = __hip_atomic_fetch_add(page_ticket, popc(need), __ATOMIC_RELAXED, BAM_AGENT);
@@ -274,7 +268,7 @@ uint32_t page_cache_d_t::find_slot(uint64_t address, uint64_t range_id, const ui
                 if (__hip_atomic_compare_exchange_strong(&cp->page_take_lock, &v, (uint32_t)LOCKED, __ATOMIC_ACQUIRE, __ATOMIC_RELAXED, BAM_AGENT)) {
                     cp->page_translation = global_address;
                     st_release(&cp->page_take_lock, (uint32_t)UNLOCKED);
-                    page = p; found = true;
+                    page = p; looking = false;
                 }
             } else if (v == UNLOCKED) {
                 if (__hip_atomic_compare_exchange_strong(&cp->page_take_lock, &v, (uint32_t)LOCKED, __ATOMIC_ACQUIRE, __ATOMIC_RELAXED, BAM_AGENT)) {
@@ -299,7 +293,7 @@ uint32_t page_cache_d_t::find_slot(uint64_t address, uint64_t range_id, const ui
                                 /* -> INVALID; references taken meanwhile stay counted and their owners reload */
                                 __hip_atomic_fetch_and(&victim->state, CNT_MASK, __ATOMIC_RELEASE, BAM_AGENT);
                                 cp->page_translation = global_address;
-                                page = p; found = true;
+                                page = p; looking = false;
                             } else {
                                 __hip_atomic_fetch_and(&victim->state, DISABLE_BUSY_MASK, __ATOMIC_RELEASE, BAM_AGENT);
                             }
@@ -308,8 +302,8 @@ uint32_t page_cache_d_t::find_slot(uint64_t address, uint64_t range_id, const ui
                     st_release(&cp->page_take_lock, (uint32_t)UNLOCKED);
                 }
             }
+            if (looking && tries + 1 >= BAM_FIND_SLOT_TRIES) looking = false;
         }
-        if (ballot(!found) && (++sp.n & 1023u) == 0 && spin_giveup(sp)) break;
     }
     return page;
 }
@@ -344,93 +338,274 @@ struct range_d_t {
     __forceinline__ __device__ uint64_t get_page(const size_t i) const { return ((i - index_start) * sizeof(T) + page_start_offset) >> cache.page_size_log; }
     __forceinline__ __device__ uint64_t get_subindex(const size_t i) const { return ((i - index_start) * sizeof(T) + page_start_offset) & cache.page_size_minus_1; }
     __forceinline__ __device__ uint64_t get_global_address(const size_t page) const { return (page << cache.n_ranges_bits) | range_id; }
-    __forceinline__ __device__ void release_page(const size_t pg) const { __hip_atomic_fetch_add(&pages[pg].state, (uint32_t)-1, __ATOMIC_RELEASE, BAM_AGENT); }
-    __forceinline__ __device__ void release_page(const size_t pg, const uint32_t count) const { __hip_atomic_fetch_add(&pages[pg].state, 0u - count, __ATOMIC_RELEASE, BAM_AGENT); }
+    __forceinline__ __device__ void release_page(const size_t pg, const uint32_t count, const bool wrote) const { bam_release_refs(&pages[pg], count, wrote); }
+    __forceinline__ __device__ void release_page(const size_t pg) const { release_page(pg, 1, true); }
+    __forceinline__ __device__ void release_page(const size_t pg, const uint32_t count) const { release_page(pg, count, true); }
     __forceinline__ __device__ cache_page_t* get_cache_page(const size_t pg) const { return cache.get_cache_page(pages[pg].offset); }
     __forceinline__ __device__ uint64_t get_cache_page_addr(const uint32_t page_trans) const { return (uint64_t)(cache.base_addr + (uint64_t)page_trans * cache.page_size); }
     __forceinline__ __device__ void mark_page_dirty(const size_t index) { __hip_atomic_fetch_or(&pages[index].state, DIRTY, __ATOMIC_RELAXED, BAM_AGENT); }
     __forceinline__ __device__ uint64_t acquire_page(const size_t pg, const uint32_t count, const bool write, const uint32_t ctrl, const uint32_t queue);
-    __forceinline__ __device__ bam_stat_shard_t* shard() const { return stats + (bam::cu_id() & (BAM_STAT_SHARDS - 1)); }
+    /* spread by workgroup so that no counter word is shared by more than a few waves at a time */
+    __forceinline__ __device__ bam_stat_shard_t* shard() const { return stats + (((blockIdx.x + blockIdx.y * gridDim.x) * 0x9E3779B1u) >> 24) % BAM_STAT_SHARDS; }
+    __forceinline__ __device__ bool slow_step(const size_t pg, const bool write, const uint32_t queue, uint64_t& sv, uint32_t& slot, bool& was_hit, bool& progressed);
 };
 
+/*
+ * Drop `count` references of a page.  A reader only has to have its loads of
+ * the page returned before the count drops (a wave-level wait); only a writer
+ * must also make its stores visible to the other compute units before an
+ * evictor may write the page back, which costs an L2 write-back.
+ */
+__forceinline__ __device__ void bam_release_refs(data_page_t* dp, const uint32_t count, const bool wrote)
+{
+    if (bam::ballot(wrote)) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    else __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __hip_atomic_fetch_add(&dp->state, 0u - count, __ATOMIC_RELAXED, BAM_AGENT);
+}
+
+/*
+ * Take `count` references on a page with one 64-bit fetch-add on
+ * {state, offset}.  True on a hit (VALID, not BUSY): `slot` is the cache slot,
+ * learnt from the same round trip.  On false the references are taken all the
+ * same and `sv` holds the word as it was; acquire_page_slow carries on from it.
+ * Relaxed on purpose: payload is read past the vector L1 (bam::ld_payload), so
+ * no cache invalidation is needed on a page visit.
+ */
+__forceinline__ __device__ bool bam_try_hit(data_page_t* dp, const uint32_t count, const bool write, uint64_t& sv, uint32_t& slot)
+{
+    sv = __hip_atomic_fetch_add((uint64_t*)dp, (uint64_t)count, __ATOMIC_RELAXED, BAM_AGENT);
+    const uint32_t s = (uint32_t)sv;
+    if ((s >> (CNT_SHIFT + 1)) != V_NB) return false;
+    if (write && (s & DIRTY) == 0) __hip_atomic_fetch_or(&dp->state, DIRTY, __ATOMIC_RELAXED, BAM_AGENT);
+    slot = (uint32_t)(sv >> 32);
+    return true;
+}
+
 namespace bam {
-/* add to a counter; when every active lane names the same word the address is made
- * wave-uniform so that the compiler folds the wave's adds into one atomic */
+/*
+ * Add v (0..127) of every active lane to a counter with one atomic per distinct
+ * counter word: the lane values are summed with seven ballots (bit-sliced
+ * population count), which works for any set of active lanes.
+ */
 __device__ __forceinline__ void stat_add(unsigned long long* ctr, uint32_t v)
 {
-    const uint64_t a0 = first((uint64_t)ctr);
-    if (!ballot((uint64_t)ctr != a0)) __hip_atomic_fetch_add((unsigned long long*)a0, (unsigned long long)v, __ATOMIC_RELAXED, BAM_AGENT);
-    else __hip_atomic_fetch_add(ctr, (unsigned long long)v, __ATOMIC_RELAXED, BAM_AGENT);
+    for (bool done = false; !done;) {
+        const uint64_t a0 = first((uint64_t)ctr);
+        if ((uint64_t)ctr == a0) {
+            uint32_t total = 0;
+#pragma unroll
+            for (uint32_t b = 0; b < 7; b++) total += popc(ballot((v >> b) & 1u)) << b;
+            if (lane() == first_lane(active_mask()) && total)
+                __hip_atomic_fetch_add((unsigned long long*)a0, (unsigned long long)total, __ATOMIC_RELAXED, BAM_AGENT);
+            done = true;
+        }
+    }
 }
 } // namespace bam
 
 /*
- * The page state machine.  Takes `count` references on page `pg` and returns
- * the cache slot that holds it, loading it first if needed.  Callable by any
- * subset of a wave's lanes, each for a different page: the lanes step through
- * the states together, and those that have to load a page do their victim
- * search and their NVMe reads as one batch.
+ * One pass of the page state machine past the hit test: the caller holds its
+ * references (bam_try_hit) and `sv` is the state word it last saw.  True once
+ * the page is valid, with its cache slot in `slot`.  Callable by any subset of
+ * a wave's lanes, each for a different page: the lanes look at their pages
+ * together, and those that have to load one do their victim search and their
+ * NVMe reads as one batch.  `progressed` tells whether this pass loaded a page.
  *
- *   VALID, not BUSY : hit
+ *   VALID, not BUSY     : hit (somebody else loaded it while we waited)
  *   not VALID, not BUSY : whoever sets BUSY first loads the page, then flips BUSY->VALID
- *   BUSY : somebody else is loading or evicting; wait and look again
+ *   BUSY                : somebody else is loading or evicting; look again later
+ *
+ * Callers use a resolved page and drop its references before they make the
+ * next pass for the lanes still waiting: a lane that sat on a resident page
+ * while its siblings look for slots could pin the last evictable slot.
  */
 template <typename T>
 __forceinline__ __device__
-uint64_t range_d_t<T>::acquire_page(const size_t pg, const uint32_t count, const bool write, const uint32_t ctrl_, const uint32_t queue)
+bool range_d_t<T>::slow_step(const size_t pg, const bool write, const uint32_t queue, uint64_t& sv, uint32_t& slot, bool& was_hit, bool& progressed)
 {
     using namespace bam;
-    (void)ctrl_;
     data_page_t* dp = &pages[pg];
-    bam_stat_shard_t* sh = shard();
-    stat_add(&sh->access_cnt, count);
-    uint32_t s = __hip_atomic_fetch_add(&dp->state, count, __ATOMIC_ACQUIRE, BAM_AGENT);
-    uint32_t slot = 0;
-    bool resolved = false;
-    spin_t sp;
-    for (;;) {
-        bool load_me = false;
-        if (!resolved) {
-            const uint32_t st = s >> (CNT_SHIFT + 1);
-            if (st == V_NB) {
-                if (write && (s & DIRTY) == 0) __hip_atomic_fetch_or(&dp->state, DIRTY, __ATOMIC_RELAXED, BAM_AGENT);
-                slot = ld_relaxed(&dp->offset);
-                stat_add(&sh->hit_cnt, count);
-                resolved = true;
-            } else if (st == NV_NB) {
-                const uint32_t o = __hip_atomic_fetch_or(&dp->state, BUSY, __ATOMIC_ACQUIRE, BAM_AGENT);
-                if ((o & BUSY) == 0) {
-                    if ((o >> (CNT_SHIFT + 1)) == NV_NB) load_me = true;
-                    else __hip_atomic_fetch_and(&dp->state, DISABLE_BUSY_MASK, __ATOMIC_RELEASE, BAM_AGENT);  /* became valid meanwhile */
-                }
-            }
+    bool load_me = false, resolved = false;
+    const uint32_t s = (uint32_t)sv, st = s >> (CNT_SHIFT + 1);
+    progressed = false;
+    if (st == V_NB) {
+        if (write && (s & DIRTY) == 0) __hip_atomic_fetch_or(&dp->state, DIRTY, __ATOMIC_RELAXED, BAM_AGENT);
+        slot = (uint32_t)(sv >> 32);
+        was_hit = true;
+        resolved = true;
+    } else if (st == NV_NB) {
+        const uint32_t o = __hip_atomic_fetch_or(&dp->state, BUSY, __ATOMIC_ACQUIRE, BAM_AGENT);
+        if ((o & BUSY) == 0) {
+            if ((o >> (CNT_SHIFT + 1)) == NV_NB) load_me = true;
+            else __hip_atomic_fetch_and(&dp->state, DISABLE_BUSY_MASK, __ATOMIC_RELEASE, BAM_AGENT);  /* became valid meanwhile */
         }
-        const uint64_t loaders = ballot(load_me);
-        if (load_me) {
-            slot = cache.find_slot(pg, range_id, queue);
+    }
+    if (load_me) {
+        const uint32_t found = cache.find_slot(pg, range_id, queue);
+        if (found == BAM_NO_SLOT) {
+            /* no evictable slot right now: hand the page back; a later pass tries again */
+            __hip_atomic_fetch_and(&dp->state, DISABLE_BUSY_MASK, __ATOMIC_RELEASE, BAM_AGENT);
+        } else {
             uint64_t c = get_backing_ctrl(pg);
             if (c == ALL_CTRLS) c = cache.n_ctrls == 1 ? 0 : cache.ctrl_counter->fetch_add(1, simt::memory_order_relaxed) % cache.n_ctrls;
             Controller* ctl = cache.d_ctrls[c];
             stat_add((unsigned long long*)&ctl->access_counter, 1);
-            stat_add(&sh->read_io_cnt, 1);
-            read_data(&cache, ctl->d_qps + (queue % ctl->n_qps), get_backing_page(pg) * cache.n_blocks_per_page, cache.n_blocks_per_page, slot);
-            st_relaxed(&dp->offset, slot);
-            stat_add(&sh->miss_cnt, count);
+            stat_add(&shard()->read_io_cnt, 1);
+            read_data(&cache, ctl->d_qps + (queue % ctl->n_qps), get_backing_page(pg) * cache.n_blocks_per_page, cache.n_blocks_per_page, found);
+            st_relaxed(&dp->offset, found);
             if (write) __hip_atomic_fetch_or(&dp->state, DIRTY, __ATOMIC_RELAXED, BAM_AGENT);
             /* BUSY -> 0 and VALID -> 1 in one step; publishes the payload and the offset */
             __hip_atomic_fetch_xor(&dp->state, DISABLE_BUSY_ENABLE_VALID, __ATOMIC_RELEASE, BAM_AGENT);
+            slot = found;
+            was_hit = false;
             resolved = true;
+            progressed = true;
         }
-        if (!ballot(!resolved)) break;
-        if (!loaders && cache.spin_giveup(sp)) break;
-        if (!resolved) s = ld_acquire(&dp->state);
     }
+    if (!resolved) sv = __hip_atomic_load((uint64_t*)dp, __ATOMIC_RELAXED, BAM_AGENT);
+    return resolved;
+}
+
+/* the reference's entry point: references + slot, and the access is accounted in the range's counters */
+template <typename T>
+__forceinline__ __device__
+uint64_t range_d_t<T>::acquire_page(const size_t pg, const uint32_t count, const bool write, const uint32_t ctrl_, const uint32_t queue)
+{
+    (void)ctrl_;
+    uint64_t sv;
+    uint32_t slot = 0;
+    bool hit = bam_try_hit(&pages[pg], count, write, sv, slot);
+    if (!hit) {
+        /* every lane keeps its references until all are in: callers of this entry point hold pages anyway */
+        bool resolved = false;
+        bam::spin_t sp;
+        for (;;) {
+            bool progressed = false;
+            if (!resolved) resolved = slow_step(pg, write, queue, sv, slot, hit, progressed);
+            if (!bam::ballot(!resolved)) break;
+            if (!bam::ballot(progressed) && cache.spin_giveup(sp)) { if (!resolved) slot = 0; break; }
+        }
+    }
+    bam_stat_shard_t* sh = shard();
+    bam::stat_add(&sh->access_cnt, count);
+    bam::stat_add(&sh->hit_cnt, hit ? count : 0);
+    bam::stat_add(&sh->miss_cnt, hit ? 0 : count);
     return slot;
 }
 
 /* ------------------------------------------------------------------ */
 /* arrays                                                             */
 /* ------------------------------------------------------------------ */
+
+namespace bam {
+/*
+ * What the device path needs to know about a range, read once and kept in
+ * registers: a kernel that walks an array re-derives page numbers and
+ * addresses from these instead of re-reading the descriptors from memory
+ * around every atomic.
+ */
+template <typename T>
+struct range_view {
+    range_d_t<T>* r = nullptr;       /* full descriptor, for the miss path */
+    data_page_t* pages;
+    uint8_t* base_addr;
+    bam_stat_shard_t* shard;
+    uint64_t index_start, index_end, pso;
+    uint32_t page_size_log, page_size;
+
+    __forceinline__ __device__ void load(range_d_t<T>* r_)
+    {
+        r = r_;
+        pages = r_->pages;
+        base_addr = r_->cache.base_addr;
+        shard = r_->shard();
+        index_start = r_->index_start;
+        index_end = r_->count;
+        pso = r_->page_start_offset;
+        page_size_log = (uint32_t)r_->cache.page_size_log;
+        page_size = (uint32_t)r_->cache.page_size;
+    }
+    __forceinline__ __device__ bool holds(const size_t i) const { return r && i >= index_start && i < index_end; }
+    __forceinline__ __device__ uint64_t byte_of(const size_t i) const { return (i - index_start) * sizeof(T) + pso; }
+    __forceinline__ __device__ uint64_t page_of(const size_t i) const { return byte_of(i) >> page_size_log; }
+    __forceinline__ __device__ uint8_t* slot_addr(const uint32_t slot) const { return base_addr + ((uint64_t)slot << page_size_log); }
+    /* element window [start, end) covered by `page`, clipped to the range */
+    __forceinline__ __device__ void window(const uint64_t page, size_t& start, size_t& end) const
+    {
+        const uint64_t first_byte = page << page_size_log;
+        start = index_start + (first_byte <= pso ? 0 : (first_byte - pso + sizeof(T) - 1) / sizeof(T));
+        end = index_start + (first_byte + page_size - pso) / sizeof(T);
+        if (end > index_end) end = index_end;
+    }
+    /* one access per active lane: hit or miss as its group's master found the page */
+    __forceinline__ __device__ void account(const bool hit) const
+    {
+        stat_add(&shard->access_cnt, 1);
+        stat_add(&shard->hit_cnt, hit ? 1 : 0);
+        stat_add(&shard->miss_cnt, hit ? 0 : 1);
+    }
+
+    /*
+     * Wave-level request coalescing + acquire.  Lanes that want the same page
+     * form a group; the lowest lane of each group (its master) takes the
+     * group's references with one atomic.  Groups whose page is resident are
+     * served first: `on_hit(slot)` runs for their lanes and, if it returns
+     * true, their references are dropped right away.  Only then do the
+     * masters of the remaining groups go through the miss path together, so a
+     * wave that waits for I/O holds no reference on anything but the pages it
+     * is loading.  `on_miss(slot)` runs for those lanes once their page is in.
+     */
+    template <typename FH, typename FM>
+    __forceinline__ __device__ void acquire(const uint64_t page, const bool write, FH&& on_hit, FM&& on_miss) const
+    {
+        const uint32_t me = lane();
+        const uint64_t eq_mask = match_any(page, (uint64_t)r);
+        const uint32_t master = first_lane(eq_mask), count = popc(eq_mask);
+        const bool dirty = (ballot(write) & eq_mask) != 0;
+        data_page_t* dp = pages + page;
+        uint64_t sv = 0, pack = 0;
+        uint32_t slot = 0;
+        if (master == me) { const bool h = bam_try_hit(dp, count, dirty, sv, slot); pack = (uint64_t)slot | ((uint64_t)h << 63); }
+        pack = shfl(pack, master);
+        if (pack >> 63) {
+            account(true);
+            const bool drop = on_hit((uint32_t)pack);
+            __builtin_amdgcn_wave_barrier();
+            if (drop && master == me) bam_release_refs(dp, count, dirty);
+        } else {
+            /* miss path: pass after pass; groups whose page came in are served and release before the next pass */
+            const uint32_t queue = get_smid();
+            bool done = false;
+            spin_t sp;
+            for (;;) {
+                bool progressed = false;
+                if (!done) {
+                    bool hit = false, resolved = false;
+                    if (master == me) { resolved = r->slow_step(page, dirty, queue, sv, slot, hit, progressed); pack = (uint64_t)slot | ((uint64_t)hit << 63) | ((uint64_t)resolved << 62); }
+                    pack = shfl(pack, master);
+                    if ((pack >> 62) & 1) {
+                        account((pack >> 63) != 0);
+                        const bool drop = on_miss((uint32_t)pack);
+                        __builtin_amdgcn_wave_barrier();
+                        if (drop && master == me) bam_release_refs(dp, count, dirty);
+                        done = true;
+                    }
+                }
+                if (!ballot(!done)) break;
+                if (!ballot(progressed) && r->cache.spin_giveup(sp)) break;
+            }
+        }
+    }
+
+    /* drop the reference each active lane holds on `page` (one atomic per group of lanes on the same page) */
+    __forceinline__ __device__ void release(const uint64_t page, const bool wrote) const
+    {
+        const uint64_t eq_mask = match_any(page, (uint64_t)r);
+        const bool any_wrote = (ballot(wrote) & eq_mask) != 0;
+        if (first_lane(eq_mask) == lane()) bam_release_refs(pages + page, popc(eq_mask), any_wrote);
+    }
+};
+} // namespace bam
 
 template <typename T>
 struct array_d_t {
@@ -447,64 +622,50 @@ struct array_d_t {
         return -1;
     }
 
+    /* the view of the range holding element i; false if no range does */
+    __forceinline__ __device__ bool view_of(const size_t i, bam::range_view<T>& v) const
+    {
+        const int64_t r = find_range(i);
+        if (r == -1) return false;
+        v.load(d_ranges + r);
+        return true;
+    }
+
     /*
-     * Wave-level request coalescing: lanes that want the same page of the same
-     * array form a group; the lowest lane of each group ("master") takes the
-     * group's references in one go.  eq_mask/master/count describe the caller's
-     * group, base_master is the cache slot.
+     * The reference's coalescing entry point (include/page_cache.h:1330-1366):
+     * eq_mask/master/count describe the caller's group of same-page lanes,
+     * base_master is the cache slot; the group's references stay taken.
      */
     __forceinline__ __device__ void coalesce_page(const uint32_t lane, const uint64_t mask, const int64_t r, const uint64_t page, const uint64_t gaddr, const bool write,
                                                   uint64_t& eq_mask, int& master, uint32_t& count, uint64_t& base_master) const
     {
-        (void)mask;
-        range_d_t<T>* r_ = d_ranges + r;
-        const uint32_t queue = get_smid();        /* reduced modulo the controller's queue count at the point of use */
-        eq_mask = bam::match_any(gaddr, (uint64_t)this);
+        (void)mask; (void)lane; (void)gaddr;
+        bam::range_view<T> v;
+        v.load(d_ranges + r);
+        eq_mask = bam::match_any(page, (uint64_t)v.r);
         master = (int)bam::first_lane(eq_mask);
         count = bam::popc(eq_mask);
-        const bool dirty = (bam::ballot(write) & eq_mask) != 0;
-        uint64_t base = 0;
-        if (master == (int)lane) base = r_->acquire_page(page, count, dirty, 0, queue);
-        base_master = bam::shfl(base, (uint32_t)master);
+        uint32_t slot = 0;
+        auto keep = [&](uint32_t s_) { slot = s_; return false; };
+        v.acquire(page, write, keep, keep);
+        base_master = slot;
     }
 
-    /*
-     * Run `fn(address of element i in the cache)` with the page referenced, for
-     * every active lane, holding at most cache.wave_batch distinct pages of
-     * this wave referenced at any time.
-     */
+    /* run fn(address of element i in the cache) with the page referenced, for every active lane */
     template <typename F>
     __forceinline__ __device__ void with_element(const size_t i, const bool write, F&& fn) const
     {
-        const int64_t r = find_range(i);
-        if (r == -1) return;
-        range_d_t<T>* r_ = d_ranges + r;
-        const uint32_t lane = lane_id();
-        const uint64_t page = r_->get_page(i), subindex = r_->get_subindex(i), gaddr = r_->get_global_address(page);
-        const uint64_t eq_mask = bam::match_any(gaddr, (uint64_t)this);
-        const uint32_t master = bam::first_lane(eq_mask), count = bam::popc(eq_mask);
-        const bool dirty = (bam::ballot(write) & eq_mask) != 0;
-        const uint64_t masters = bam::ballot(master == lane);
-        const uint32_t n_masters = bam::popc(masters), my_group = bam::popc(masters & bam::lanes_below(master));
-        const uint32_t batch = bam::first(r_->cache.wave_batch);
-        const uint32_t queue = get_smid();
-        for (uint32_t g0 = 0; g0 < n_masters; g0 += batch) {
-            if (my_group >= g0 && my_group < g0 + batch) {
-                uint64_t base = 0;
-                if (master == lane) base = r_->acquire_page(page, count, dirty, 0, queue);
-                base = bam::shfl(base, master);
-                fn((T*)(r_->get_cache_page_addr((uint32_t)base) + subindex));
-                /* every lane of the group has used the page before the master drops the references */
-                __builtin_amdgcn_wave_barrier();
-                if (master == lane) r_->release_page(page, count);
-            }
-        }
+        bam::range_view<T> v;
+        if (!view_of(i, v)) return;
+        const uint64_t byte = v.byte_of(i);
+        auto use = [&](uint32_t slot) { fn((T*)(v.slot_addr(slot) + (byte & (v.page_size - 1)))); return true; };
+        v.acquire(byte >> v.page_size_log, write, use, use);
     }
 
     __forceinline__ __device__ T seq_read(const size_t i) const
     {
         T ret = T();
-        with_element(i, false, [&](T* p) { ret = *p; });
+        with_element(i, false, [&](T* p) { ret = bam::ld_payload(p); });
         return ret;
     }
 
@@ -525,38 +686,32 @@ struct array_d_t {
 
     /*
      * Reference the page holding element i and keep it referenced: returns the
-     * address of the page in the cache, the element window [start, end) it
-     * covers, the page descriptor and the range index.  Pair with release_page.
+     * address of the first element of the window [start, end) the page covers,
+     * the page descriptor and the range index.  Pair with release_page.
      */
     __forceinline__ __device__ void* acquire_page(const size_t i, data_page_t*& page_, size_t& start, size_t& end, int64_t& r) const
     {
-        const uint32_t lane = lane_id();
         r = find_range(i);
         page_ = nullptr;
         if (r == -1) return nullptr;
-        range_d_t<T>* r_ = d_ranges + r;
-        uint64_t eq_mask, base_master;
-        int master;
-        uint32_t count;
-        const uint64_t page = r_->get_page(i);
-        coalesce_page(lane, bam::active_mask(), r, page, r_->get_global_address(page), false, eq_mask, master, count, base_master);
-        page_ = &r_->pages[page];
-        /* first element of the page; a page may start before the range when page_start_offset != 0 */
-        const uint64_t first_byte = (page << r_->cache.page_size_log);
-        const uint64_t first_elem = first_byte <= r_->page_start_offset ? 0 : (first_byte - r_->page_start_offset) / sizeof(T);
-        start = r_->index_start + first_elem;
-        end = r_->index_start + ((first_byte + r_->cache.page_size - r_->page_start_offset) / sizeof(T));
-        return (void*)(r_->get_cache_page_addr((uint32_t)base_master) + r_->get_subindex(start));
+        bam::range_view<T> v;
+        v.load(d_ranges + r);
+        const uint64_t page = v.page_of(i);
+        uint32_t slot = 0;
+        auto keep = [&](uint32_t s_) { slot = s_; return false; };
+        v.acquire(page, false, keep, keep);
+        page_ = v.pages + page;
+        v.window(page, start, end);
+        return (void*)(v.slot_addr(slot) + (v.byte_of(start) & (v.page_size - 1)));
     }
 
-    __forceinline__ __device__ void release_page(data_page_t* page_, const int64_t r, const size_t i) const
+    __forceinline__ __device__ void release_page(data_page_t* page_, const int64_t r, const size_t i, const bool wrote = true) const
     {
         (void)page_;
         if (r == -1) return;
-        range_d_t<T>* r_ = d_ranges + r;
-        const uint64_t page = r_->get_page(i);
-        const uint64_t eq_mask = bam::match_any(r_->get_global_address(page), (uint64_t)this);
-        if (bam::first_lane(eq_mask) == lane_id()) r_->release_page(page, bam::popc(eq_mask));
+        bam::range_view<T> v;
+        v.load(d_ranges + r);
+        v.release(v.page_of(i), wrote);
     }
 };
 
@@ -585,7 +740,9 @@ struct bam_ref {
  * release.  Same contract as the reference's bam_ptr (include/page_cache.h:414-485).
  * A thread holds one page referenced for as long as the window stays on it, so
  * the cache must have more pages than the threads of the resident waves can
- * hold at once (the reference has the same requirement).
+ * hold at once (the reference has the same requirement).  The range
+ * descriptor is read once and kept in registers for as long as the accesses
+ * stay inside that range.
  */
 template <typename T>
 struct bam_ptr {
@@ -596,6 +753,9 @@ struct bam_ptr {
     int64_t range_id = -1;
     T* addr = nullptr;
     bool dirty = false;
+#if defined(__HIP_DEVICE_COMPILE__)
+    bam::range_view<T> view;
+#endif
 
     __forceinline__ __host__ __device__ bam_ptr(array_d_t<T>* a) { init(a); }
     __forceinline__ __host__ __device__ ~bam_ptr() { fini(); }
@@ -605,7 +765,7 @@ struct bam_ptr {
     {
 #if defined(__HIP_DEVICE_COMPILE__)
         if (page) {
-            array->release_page(page, range_id, start);
+            view.release((uint64_t)(page - view.pages), dirty);
             page = nullptr;
         }
 #endif
@@ -615,8 +775,21 @@ struct bam_ptr {
     {
 #if defined(__HIP_DEVICE_COMPILE__)
         fini();
-        addr = (T*)array->acquire_page(i, page, start, end, range_id);
+        start = end = 0;
+        addr = nullptr;
         dirty = false;
+        if (!view.holds(i)) {
+            range_id = array->find_range(i);
+            if (range_id == -1) { view.r = nullptr; return nullptr; }
+            view.load(array->d_ranges + range_id);
+        }
+        const uint64_t pg = view.page_of(i);
+        uint32_t slot = 0;
+        auto keep = [&](uint32_t s_) { slot = s_; return false; };
+        view.acquire(pg, false, keep, keep);
+        page = view.pages + pg;
+        view.window(pg, start, end);
+        addr = (T*)(view.slot_addr(slot) + (view.byte_of(start) & (view.page_size - 1)));
 #endif
         return addr;
     }
@@ -624,7 +797,11 @@ struct bam_ptr {
     __forceinline__ __host__ __device__ T read(const size_t i)
     {
         if (i < start || i >= end) update_page(i);
+#if defined(__HIP_DEVICE_COMPILE__)
+        return bam::ld_payload(addr + (i - start));
+#else
         return addr[i - start];
+#endif
     }
 
     __forceinline__ __host__ __device__ void mark_dirty()
@@ -781,13 +958,7 @@ struct page_cache_t {
         page_ticket_buf = createBuffer(sizeof(uint32_t), hipDevice);
         pdt.page_ticket = (uint32_t*)page_ticket_buf.get();
 
-        /* how many pages a wave may pin while loading: leave at least half of the cache evictable */
-        hipDeviceProp_t prop;
-        hip_err_chk(hipGetDeviceProperties(&prop, hipDevice));
-        const uint64_t max_waves = (uint64_t)prop.multiProcessorCount * prop.maxThreadsPerMultiProcessor / BAM_WAVE_SIZE;
-        uint64_t batch = np / (2 * (max_waves ? max_waves : 1));
-        pdt.wave_batch = (uint32_t)(batch < 1 ? 1 : batch > BAM_WAVE_SIZE ? BAM_WAVE_SIZE : batch);
-        if (const char* e = getenv("BAM_WAVE_BATCH")) { int v = atoi(e); if (v >= 1 && v <= BAM_WAVE_SIZE) pdt.wave_batch = (uint32_t)v; }
+        pdt.wave_batch = BAM_WAVE_SIZE;
 
         const bool staged = ctrl.n_qps && ctrl.h_qps[0]->stage != nullptr;
         const uint64_t cache_size = ps * np;

@@ -5,8 +5,8 @@
  *
  * Differences that follow from the wave-cooperative engine: per-slot state is
  * dense 32-bit words, the command-id table has as many entries as the queue
- * (ids index a staging window, see below) instead of 65536, and the pos_locks
- * and head_mark arrays are gone.
+ * (ids index a staging window, see below) instead of 65536 and is handed out
+ * to waves in blocks of 64 ids, and the head_mark array is gone.
  *
  * Staged transfers.  When the controller cannot address device memory (the
  * software target on a machine without CPU-visible VRAM) every queue pair owns
@@ -44,7 +44,7 @@ struct QueuePair
     /* host-side owners; a raw pointer keeps the struct trivially copyable to the device */
     struct Owners {
         DmaPtr sq_mem, cq_mem, stage_mem;
-        BufferPtr sq_tickets, sq_tail_mark, sq_cid;
+        BufferPtr sq_tickets, sq_tail_mark, sq_cid, sq_cid_blocks;
     };
     Owners*             own;
     nvm_aq_ref          aq;
@@ -76,7 +76,7 @@ struct QueuePair
         if (!nvm_ok(status)) { nvm_admin_cq_delete(aq_ref, &cq); delete own; throw std::runtime_error(std::string("Failed to create submission queue: ") + nvm_strerror(status)); }
 
         /* device-side protocol state */
-        const uint32_t n_cids = qs;
+        const uint32_t n_cids = qs < 64 ? 64 : qs;      /* handed out in blocks of 64, one block per wave */
         own->sq_tickets = createBuffer(qs * sizeof(padded_struct), hipDevice);
         own->sq_tail_mark = createBuffer(qs * sizeof(padded_struct), hipDevice);
         own->sq_cid = createBuffer(n_cids * sizeof(padded_struct), hipDevice);
@@ -84,6 +84,8 @@ struct QueuePair
         sq.tail_mark = (padded_struct*)own->sq_tail_mark.get();
         sq.cid = (padded_struct*)own->sq_cid.get();
         sq.cid_mask = n_cids - 1;
+        own->sq_cid_blocks = createBuffer((n_cids / 64) * sizeof(padded_struct), hipDevice);
+        sq.pos_locks = (padded_struct*)own->sq_cid_blocks.get();
         cq.cid = sq.cid;
         cq.cid_mask = sq.cid_mask;
         sq.guard = cq.guard = guard;
