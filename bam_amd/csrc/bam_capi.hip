@@ -367,7 +367,7 @@ int bam_target_stats(bam_target_t* t, uint64_t* out, int reset)
     if (!t || !out) return fail(EINVAL, "bam_target_stats: null argument");
     nvmt_stats_t s;
     nvmt_stats(t->t, &s);
-    const uint64_t v[10] = {s.admin_cmds, s.io_cmds, s.read_cmds, s.write_cmds, s.bytes_read, s.bytes_written, s.error_cpls, s.sq_doorbells, s.cq_full_stalls, s.dropped};
+    const uint64_t v[12] = {s.admin_cmds, s.io_cmds, s.read_cmds, s.write_cmds, s.bytes_read, s.bytes_written, s.error_cpls, s.sq_doorbells, s.cq_full_stalls, s.dropped, s.sqe_retries, s.stale_doorbells};
     memcpy(out, v, sizeof(v));
     if (reset) nvmt_reset_stats(t->t);
     return 0;

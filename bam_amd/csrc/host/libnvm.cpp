@@ -466,6 +466,18 @@ int nvm_admin_sq_create(nvm_aq_ref ref, nvm_queue_t* sq, const nvm_queue_t* cq, 
     return create_queue(ref, sq, false, id, cq->no, dma, page_offset, qs, need_prp);
 }
 
+int nvm_admin_sq_set_sealed(nvm_aq_ref ref, nvm_queue_t* sq)
+{
+    if (!ref || !sq || sq->no == 0) return EINVAL;
+    nvm_cmd_t cmd; nvm_cpl_t cpl;
+    admin_cmd(&cmd, 0, 0);
+    cmd.dword[0] = NVM_ADMIN_VS_SEAL_SQ;        /* full 8-bit opcode: nvm_cmd_header keeps only the low seven bits */
+    cmd.dword[10] = sq->no;
+    int err = nvm_raw_rpc(ref, &cmd, &cpl);
+    if (!err) sq->sealed = 1;
+    return err;
+}
+
 int nvm_admin_cq_delete(nvm_aq_ref ref, nvm_queue_t* cq) { return delete_queue(ref, cq, true); }
 int nvm_admin_sq_delete(nvm_aq_ref ref, nvm_queue_t* sq, const nvm_queue_t* cq) { (void)cq; return delete_queue(ref, sq, false); }
 } // extern "C"

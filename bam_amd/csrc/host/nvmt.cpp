@@ -51,6 +51,7 @@ template <typename T> inline void st(volatile void* p, T v) { __atomic_store_n((
 struct Cq {
     bool valid = false;
     uint32_t qs = 0, tail = 0, phase = 1;
+    uint32_t head_seen = 0;        // newest plausible value of the head doorbell
     nvm_cpl_t* mem = nullptr;
     volatile uint32_t* head_db = nullptr;
 };
@@ -59,6 +60,9 @@ struct Sq {
     bool valid = false;
     uint16_t id = 0, cqid = 0;
     uint32_t qs = 0, head = 0, last_tail = 0;
+    bool sealed = false;           // entries carry sequence number + checksum (nvm_cmd_seal)
+    uint32_t fetched = 0;          // commands fetched so far = sequence number expected next
+    bool retry_counted = false;
     nvm_cmd_t* mem = nullptr;
     volatile uint32_t* tail_db = nullptr;
 };
@@ -66,9 +70,9 @@ struct Sq {
 // Counters are kept per service thread (relaxed atomics on a private cache line: uncontended) and summed on read.
 struct alignas(128) Stats {
     std::atomic<uint64_t> admin_cmds{0}, io_cmds{0}, read_cmds{0}, write_cmds{0}, bytes_read{0},
-        bytes_written{0}, error_cpls{0}, sq_doorbells{0}, cq_full_stalls{0}, dropped{0};
+        bytes_written{0}, error_cpls{0}, sq_doorbells{0}, cq_full_stalls{0}, dropped{0}, sqe_retries{0}, stale_doorbells{0};
     void bump(std::atomic<uint64_t>& c, uint64_t v = 1) { c.store(c.load(std::memory_order_relaxed) + v, std::memory_order_relaxed); }
-    void clear() { for (auto* c : {&admin_cmds, &io_cmds, &read_cmds, &write_cmds, &bytes_read, &bytes_written, &error_cpls, &sq_doorbells, &cq_full_stalls, &dropped}) c->store(0, std::memory_order_relaxed); }
+    void clear() { for (auto* c : {&admin_cmds, &io_cmds, &read_cmds, &write_cmds, &bytes_read, &bytes_written, &error_cpls, &sq_doorbells, &cq_full_stalls, &dropped, &sqe_retries, &stale_doorbells}) c->store(0, std::memory_order_relaxed); }
 };
 
 struct IoThread {
@@ -235,7 +239,14 @@ bool post_cpl(nvmt* t, Stats& st_, Cq& cq, uint16_t sqid, uint16_t sqhd, uint16_
     // tail is an index in [0, qs); admin queues need not be powers of two
     const uint32_t next = cq.tail + 1 == cq.qs ? 0 : cq.tail + 1;
     bool stalled = false;
-    while (next == ld<uint32_t>(cq.head_db) % cq.qs) {
+    for (;;) {
+        // the consumer can only have acknowledged entries that were posted: a doorbell value outside
+        // [head_seen, tail] is an old one that arrived late, and is ignored
+        const uint32_t hd = ld<uint32_t>(cq.head_db) % cq.qs;
+        const uint32_t adv = (hd + cq.qs - cq.head_seen) % cq.qs, outstanding = (cq.tail + cq.qs - cq.head_seen) % cq.qs;
+        if (adv <= outstanding) cq.head_seen = hd;
+        else st_.bump(st_.stale_doorbells);
+        if (next != cq.head_seen) break;
         if (!stalled) { st_.bump(st_.cq_full_stalls); stalled = true; }
         if (t->stop.load(std::memory_order_relaxed)) return false;
         cpu_relax();
@@ -263,7 +274,23 @@ void serve_sq(nvmt* t, IoThread* me, Sq& sq)
         nvm_cmd_t batch[64];
         uint32_t n = (tail - sq.head) & mask;
         if (n > 64) n = 64;
-        for (uint32_t i = 0; i < n; i++) batch[i] = sq.mem[(sq.head + i) & mask];
+        if (sq.sealed) {
+            // take entries only while sequence number and checksum match: one that is stale, torn or still in
+            // flight (entry and doorbell are not ordered on the way here) is looked at again on a later pass
+            uint32_t got = 0;
+            for (; got < n; got++) {
+                batch[got] = sq.mem[(sq.head + got) & mask];
+                std::atomic_thread_fence(std::memory_order_acquire);
+                if (!nvm_cmd_seal_ok(&batch[got], sq.fetched + got)) break;
+            }
+            if (got < n && !sq.retry_counted) { st_.bump(st_.sqe_retries); sq.retry_counted = true; }
+            if (!got) return;
+            sq.retry_counted = false;
+            n = got;
+            sq.fetched += n;
+        } else {
+            for (uint32_t i = 0; i < n; i++) batch[i] = sq.mem[(sq.head + i) & mask];
+        }
         sq.head = (sq.head + n) & mask;
         uint32_t order[64];
         for (uint32_t i = 0; i < n; i++) order[i] = t->cfg.order == NVMT_ORDER_REVERSE ? n - 1 - i : i;
@@ -379,7 +406,7 @@ void admin_cmd(nvmt* t, const nvm_cmd_t& c)
         if (!prp1 || !(c.dword[11] & 1)) { status = ST_INVALID_FIELD; break; }
         {
             Cq& q = t->cqs[qid];
-            q.qs = qs; q.tail = 0; q.phase = 1; q.mem = (nvm_cpl_t*)prp1; q.head_db = t->cq_db(qid);
+            q.qs = qs; q.tail = 0; q.phase = 1; q.head_seen = 0; q.mem = (nvm_cpl_t*)prp1; q.head_db = t->cq_db(qid);
             st<uint32_t>(q.head_db, 0);
             q.valid = true;
         }
@@ -391,7 +418,7 @@ void admin_cmd(nvmt* t, const nvm_cmd_t& c)
         if (qs < 2 || qs > t->cfg.max_queue_entries || (qs & (qs - 1))) { status = ST_QSIZE_INVALID; break; }
         if (!prp1 || !(c.dword[11] & 1)) { status = ST_INVALID_FIELD; break; }
         Sq& q = t->sqs[qid];
-        q.id = qid; q.cqid = cqid; q.qs = qs; q.head = 0; q.last_tail = 0; q.mem = (nvm_cmd_t*)prp1; q.tail_db = t->sq_db(qid);
+        q.id = qid; q.cqid = cqid; q.qs = qs; q.head = 0; q.last_tail = 0; q.sealed = false; q.fetched = 0; q.retry_counted = false; q.mem = (nvm_cmd_t*)prp1; q.tail_db = t->sq_db(qid);
         st<uint32_t>(q.tail_db, 0);
         q.valid = true;
         assign_sq(t, qid, true);
@@ -417,6 +444,14 @@ void admin_cmd(nvmt* t, const nvm_cmd_t& c)
         break;
     }
     case NVM_ADMIN_ABORT: break;
+    case NVM_ADMIN_VS_SEAL_SQ:
+        if (qid == 0 || qid > t->cfg.max_io_queues || !t->sqs[qid].valid) { status = ST_QID_INVALID; break; }
+        {
+            IoThread* th = t->io[t->sqs[qid].cqid % t->io.size()];
+            std::lock_guard<std::mutex> g(th->mu);
+            t->sqs[qid].sealed = true;
+        }
+        break;
     default: status = ST_INVALID_OPCODE;
     }
     post_cpl(t, t->stats, t->acq, 0, (uint16_t)t->asq.head, cid, status, dw0);
@@ -557,6 +592,7 @@ void nvmt_stats(nvmt_t* t, nvmt_stats_t* o)
         o->admin_cmds += s.admin_cmds; o->io_cmds += s.io_cmds; o->read_cmds += s.read_cmds; o->write_cmds += s.write_cmds;
         o->bytes_read += s.bytes_read; o->bytes_written += s.bytes_written; o->error_cpls += s.error_cpls;
         o->sq_doorbells += s.sq_doorbells; o->cq_full_stalls += s.cq_full_stalls; o->dropped += s.dropped;
+        o->sqe_retries += s.sqe_retries; o->stale_doorbells += s.stale_doorbells;
     };
     add(t->stats);
     for (IoThread* th : t->io) add(th->stats);

@@ -57,10 +57,10 @@ class Target:
         _TARGETS[path] = self
 
     def stats(self, reset=False):
-        out = (c_u64 * 10)()
+        out = (c_u64 * 12)()
         _chk(self.L.bam_target_stats(self.h, out, int(reset)), "bam_target_stats")
         keys = ("admin_cmds", "io_cmds", "read_cmds", "write_cmds", "bytes_read", "bytes_written", "error_cpls",
-                "sq_doorbells", "cq_full_stalls", "dropped")
+                "sq_doorbells", "cq_full_stalls", "dropped", "sqe_retries", "stale_doorbells")
         return dict(zip(keys, list(out)))
 
     def close(self):

@@ -37,7 +37,8 @@ int bam_target_create(bam_target_t** out, const char* path, uint64_t ns_bytes, u
                       uint32_t n_io_threads, uint32_t max_queue_entries, uint32_t max_io_queues, uint32_t completion_order,
                       uint32_t fail_every, uint32_t drop_every);
 void bam_target_destroy(bam_target_t* t);
-/* out[10]: admin_cmds, io_cmds, read_cmds, write_cmds, bytes_read, bytes_written, error_cpls, sq_doorbells, cq_full_stalls, dropped */
+/* out[12]: admin_cmds, io_cmds, read_cmds, write_cmds, bytes_read, bytes_written, error_cpls, sq_doorbells, cq_full_stalls, dropped,
+ *          sqe_retries, stale_doorbells */
 int bam_target_stats(bam_target_t* t, uint64_t* out, int reset);
 /* host pointer to the memory-backed namespace (NULL for procedural) */
 void* bam_target_backing(bam_target_t* t);

@@ -81,6 +81,22 @@ __device__ __forceinline__ uint64_t match_any(uint64_t key_a, uint64_t key_b)
 /* compute-unit identity across the whole device: XCC, shader engine and CU bits */
 __device__ __forceinline__ uint32_t cu_id() { return __smid(); }
 
+/*
+ * A number that differs between the waves resident on the device at one time
+ * and is spread evenly: hash of the hardware wave slot (XCC, SE, CU, SIMD,
+ * wave).  Used to pick an I/O queue per wave: the CU number alone (what the
+ * reference uses, smid % n_qps) has gaps and repeats across the eight XCDs,
+ * which would leave most queues idle and a few overrun.
+ */
+__device__ __forceinline__ uint32_t wave_slot_hash()
+{
+    const uint32_t hw = __builtin_amdgcn_s_getreg((31 << 11) | (0 << 6) | 4);          /* HW_ID, all 32 bits */
+    const uint32_t xcc = __builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20);          /* XCC_ID[3:0] */
+    uint32_t h = (hw & 0xffffu) | (xcc << 16);
+    h *= 0x9E3779B1u;
+    return h ^ (h >> 15);
+}
+
 /* back-off: n * 64 clocks, doubling up to 32 */
 __device__ __forceinline__ void backoff(uint32_t& n)
 {

@@ -25,6 +25,8 @@ int nvm_admin_cq_create(nvm_aq_ref ref, nvm_queue_t* cq, uint16_t id, const nvm_
 int nvm_admin_cq_delete(nvm_aq_ref ref, nvm_queue_t* cq);
 int nvm_admin_sq_create(nvm_aq_ref ref, nvm_queue_t* sq, const nvm_queue_t* cq, uint16_t id, const nvm_dma_t* dma, size_t page_offset, size_t qs, bool need_prp NVM_DEFAULT(false));
 int nvm_admin_sq_delete(nvm_aq_ref ref, nvm_queue_t* sq, const nvm_queue_t* cq);
+/* extension: from now on the controller only takes entries of `sq` that pass nvm_cmd_seal_ok (software target only) */
+int nvm_admin_sq_set_sealed(nvm_aq_ref ref, nvm_queue_t* sq);
 int nvm_admin_get_log_page(nvm_aq_ref ref, uint32_t ns_id, void* ptr, uint64_t ioaddr, uint8_t log_id, uint64_t log_offset);
 #ifdef __cplusplus
 }

@@ -31,7 +31,8 @@ enum nvm_admin_command_set
     NVM_ADMIN_IDENTIFY      = 0x06,
     NVM_ADMIN_ABORT         = 0x08,
     NVM_ADMIN_SET_FEATURES  = 0x09,
-    NVM_ADMIN_GET_FEATURES  = 0x0A
+    NVM_ADMIN_GET_FEATURES  = 0x0A,
+    NVM_ADMIN_VS_SEAL_SQ    = 0xC1      /* vendor specific: CDW10[15:0] = SQ id whose entries are sealed from now on */
 };
 
 /* DW0 (opcode, FUSE = PSDT = 0, CID) and DW1 (NSID) */
@@ -60,6 +61,44 @@ void nvm_cmd_rw_blks(nvm_cmd_t* cmd, uint64_t start_lba, uint16_t n_blks)
     cmd->dword[10] = (uint32_t)start_lba;
     cmd->dword[11] = (uint32_t)(start_lba >> 32);
     cmd->dword[12] = (cmd->dword[12] & 0xffff0000u) | ((uint32_t)(n_blks - 1) & 0xffffu);
+}
+
+/*
+ * Sealed submission entries (extension; no counterpart in the reference).
+ *
+ * A queue whose entries are written by one agent and fetched by another over
+ * an interconnect that may reorder posted writes (a GPU filling a ring in host
+ * memory for the software target) cannot rely on "entry first, doorbell
+ * second" arriving in that order.  On a sealed SQ the writer stores the
+ * entry's absolute sequence number (its slot ticket) in CDW2 and a checksum of
+ * the other fifteen dwords, keyed by that number, in CDW3 (both reserved in
+ * NVM read/write/flush commands); the fetching side takes an entry only when
+ * both match, so an entry that is stale, torn or not yet complete is simply
+ * looked at again later.
+ */
+__host__ __device__ static inline
+uint32_t nvm_cmd_seal_value(const nvm_cmd_t* cmd, uint32_t ticket)
+{
+    uint32_t h = ticket * 0x9E3779B1u + 0x7F4A7C15u;
+    for (int i = 0; i < 16; i++) {
+        if (i == 3) continue;
+        h = (h ^ cmd->dword[i]) * 0x85EBCA6Bu;
+        h ^= h >> 13;
+    }
+    return h | 1u;
+}
+
+__host__ __device__ static inline
+void nvm_cmd_seal(nvm_cmd_t* cmd, uint32_t ticket)
+{
+    cmd->dword[2] = ticket;
+    cmd->dword[3] = nvm_cmd_seal_value(cmd, ticket);
+}
+
+__host__ __device__ static inline
+int nvm_cmd_seal_ok(const nvm_cmd_t* cmd, uint32_t ticket)
+{
+    return cmd->dword[2] == ticket && cmd->dword[3] == nvm_cmd_seal_value(cmd, ticket);
 }
 
 /*

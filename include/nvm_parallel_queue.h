@@ -26,6 +26,7 @@
 #define __NVM_PARALLEL_QUEUE_H_
 
 #include "bam_wave.h"
+#include "nvm_cmd.h"
 #include "nvm_types.h"
 #include "nvm_util.h"
 
@@ -69,23 +70,26 @@ __device__ __forceinline__ uint32_t leading_run(uint64_t act, uint64_t ok)
  * 64*b .. 64*b+63): one atomic per wave instead of one per command, and a
  * wave never sits on a few ids while it waits for more, which would leave two
  * waves that share a queue each holding part of what the other needs.
- * Returns the lane's id (block base + rank of the lane in the group); the
- * caller holds nothing else it would have to give up while this waits.
+ * Blocks are ticket locks: the n-th wave to ask gets block n mod n_blocks and
+ * waits for that block's turn counter to reach n div n_blocks, so waves are
+ * served in arrival order and none starves.  Returns the lane's id (block
+ * base + rank of the lane in the group); the caller holds nothing else it
+ * would have to give up while this waits.
  */
 __device__ __forceinline__ uint32_t get_cid_group(nvm_queue_t* sq)
 {
     const uint64_t act = active_mask();
     const uint32_t leader = first_lane(act);
-    const uint32_t n_blocks = (sq->cid_mask + 1u) >> 6;
+    const uint32_t n_blocks = (sq->cid_mask + 1u) >> 6;          /* power of two */
     uint32_t base = 0;
     if (lane() == leader) {
+        const uint32_t t = __hip_atomic_fetch_add(&sq->cid_ticket, 1u, __ATOMIC_RELAXED, BAM_AGENT);
+        const uint32_t b = t & (n_blocks - 1), shift = (uint32_t)__builtin_ctz(n_blocks);
+        const uint32_t turn_mask = 0xffffffffu >> shift;
         spin_t sp;
-        for (;;) {
-            const uint32_t b = __hip_atomic_fetch_add(&sq->cid_ticket, 1u, __ATOMIC_RELAXED, BAM_AGENT) % n_blocks;
-            if (ld_relaxed(&sq->pos_locks[b].val) == UNLOCKED &&
-                __hip_atomic_exchange(&sq->pos_locks[b].val, (uint32_t)LOCKED, __ATOMIC_ACQUIRE, BAM_AGENT) == UNLOCKED) { base = b << 6; break; }
+        while (((ld_acquire(&sq->pos_locks[b].val) - (t >> shift)) & turn_mask) != 0)
             if (spin_giveup(sq, sp)) break;
-        }
+        base = b << 6;
     }
     base = bcast(base, leader);
     const uint32_t id = base + rank_in(act);
@@ -98,7 +102,7 @@ __device__ __forceinline__ void put_cid_group(nvm_queue_t* sq, uint32_t id)
 {
     const uint64_t act = active_mask();
     st_relaxed(&sq->cid[id].val, (uint32_t)UNLOCKED);
-    if (lane() == first_lane(act)) st_release(&sq->pos_locks[id >> 6].val, (uint32_t)UNLOCKED);
+    if (lane() == first_lane(act)) __hip_atomic_fetch_add(&sq->pos_locks[id >> 6].val, 1u, __ATOMIC_RELEASE, BAM_AGENT);   /* next turn */
 }
 
 __device__ __forceinline__ void cq_drain_group(nvm_queue_t* cq, nvm_queue_t* sq, uint64_t act);
@@ -125,7 +129,7 @@ __device__ __forceinline__ bool try_drain_group(nvm_queue_t* cq, nvm_queue_t* sq
  * slot the lane's entry went to.  On return every entry is covered by a
  * doorbell write.
  */
-__device__ __forceinline__ uint32_t sq_enqueue_group(nvm_queue_t* sq, const nvm_cmd_t* cmd)
+__device__ __forceinline__ uint32_t sq_enqueue_group(nvm_queue_t* sq, nvm_cmd_t* cmd)
 {
     const uint64_t act = active_mask();
     const uint32_t n = popc(act), rank = rank_in(act), leader = first_lane(act);
@@ -135,6 +139,7 @@ __device__ __forceinline__ uint32_t sq_enqueue_group(nvm_queue_t* sq, const nvm_
     t0 = bcast(t0, leader);
     const uint32_t ticket = t0 + rank, pos = ticket & mask;
     const uint32_t want = (ticket >> sq->qs_log2) * 2u;      /* slot is free for my lap when tickets[pos] == want */
+    if (sq->sealed) nvm_cmd_seal(cmd, ticket);
     bool written = false;
     spin_t sp;
     for (;;) {

@@ -83,8 +83,9 @@ typedef struct
     padded_struct*          head_mark;      /* unused by the wave-cooperative engine (kept for layout parity) */
     padded_struct*          tail_mark;      /* SQ [qs]: 1 = written, waiting for the tail sweep */
     padded_struct*          cid;            /* SQ [n_cids]: per command id, 0 idle, 1 in flight, 3 in flight + completed */
-    padded_struct*          pos_locks;      /* SQ [n_cids / 64]: command ids are handed out to a wave in blocks of 64; 1 = block taken */
+    padded_struct*          pos_locks;      /* SQ [n_cids / 64]: command ids are handed out to a wave in blocks of 64; turn counter of each block */
     uint32_t                cid_mask;       /* n_cids - 1 */
+    uint32_t                sealed;         /* SQ: entries carry a sequence number and checksum (nvm_cmd_seal) */
     struct bam_guard*       guard;          /* device path: bounded-wait control (may be NULL) */
     uint32_t                spin_limit;     /* device path: copy of guard->spin_limit */
     void*                   pair;           /* device path: the CQ of an SQ / the SQ of a CQ (device address) */

@@ -56,6 +56,8 @@ typedef struct
     uint64_t sq_doorbells;      /* distinct tail values observed */
     uint64_t cq_full_stalls;    /* times a completion had to wait for CQ space */
     uint64_t dropped;           /* commands swallowed by drop_every */
+    uint64_t sqe_retries;       /* sealed SQ: entries found stale or incomplete when first looked at */
+    uint64_t stale_doorbells;   /* doorbell values that pointed behind what had already been seen */
 } nvmt_stats_t;
 
 /* bytes of register window needed for this configuration (>= 0x2000) */

@@ -187,6 +187,7 @@ __device__ __forceinline__ void io_group(page_cache_d_t* pc, QueuePair* qp, uint
     if (qp->stage) {
         stage = qp->stage + (size_t)cid * qp->stage_stride;
         prp1 = qp->stage_ioaddr + (uint64_t)cid * qp->stage_stride;
+        if (bytes > qp->pageSize) prp2 = prp1 + qp->pageSize;         /* staging pages are contiguous: second controller page */
         if (opcode == NVM_IO_WRITE) {
             copy_pages(stage, slot_addr, bytes, act, n, rank);
             fence_release_sys();
@@ -574,7 +575,7 @@ struct range_view {
             if (drop && master == me) bam_release_refs(dp, count, dirty);
         } else {
             /* miss path: pass after pass; groups whose page came in are served and release before the next pass */
-            const uint32_t queue = get_smid();
+            const uint32_t queue = wave_slot_hash();
             bool done = false;
             spin_t sp;
             for (;;) {

@@ -75,6 +75,11 @@ struct QueuePair
         status = nvm_admin_sq_create(aq_ref, &sq, &cq, qp_id, own->sq_mem.get(), 0, qs);
         if (!nvm_ok(status)) { nvm_admin_cq_delete(aq_ref, &cq); delete own; throw std::runtime_error(std::string("Failed to create submission queue: ") + nvm_strerror(status)); }
 
+        /* the ring is filled by the GPU across the interconnect and fetched by the controller from the other side:
+         * have entries sealed so that one that has not fully arrived is never taken (see nvm_cmd_seal) */
+        status = nvm_admin_sq_set_sealed(aq_ref, &sq);
+        if (!nvm_ok(status)) { nvm_admin_sq_delete(aq_ref, &sq, &cq); nvm_admin_cq_delete(aq_ref, &cq); delete own; throw std::runtime_error(std::string("Failed to seal submission queue: ") + nvm_strerror(status)); }
+
         /* device-side protocol state */
         const uint32_t n_cids = qs < 64 ? 64 : qs;      /* handed out in blocks of 64, one block per wave */
         own->sq_tickets = createBuffer(qs * sizeof(padded_struct), hipDevice);
@@ -92,6 +97,8 @@ struct QueuePair
         sq.spin_limit = cq.spin_limit = guard ? guard->spin_limit : 0;
 
         stage = nullptr; stage_ioaddr = 0; stage_stride = 0;
+        if (stage_bytes > 2 * ctrl->page_size || (stage_bytes & (stage_bytes - 1)))
+            throw std::runtime_error("QueuePair: the staging page must be a power of two of at most two controller pages (PRP1 + PRP2)");
         if (stage_bytes) {
             own->stage_mem = createDma(ctrl, (size_t)n_cids * stage_bytes);
             stage = (uint8_t*)own->stage_mem->vaddr;

@@ -127,3 +127,91 @@ def cc_labels(offsets, neigh, sweep=False):
         return lb, comps, it.value
     comps = lib().bo_cc_labels(len(offsets) - 1, offsets, nb, lb)
     return lb, comps
+
+
+# ---- CPU restatement of the page-cache + queue protocol (cpu_path.c) -------
+_CPU = None
+
+
+def cpu_lib():
+    global _CPU
+    if _CPU is not None:
+        return _CPU
+    so = os.path.join(_HERE, "libbam_cpu_path.so")
+    if not os.path.exists(so):
+        build()
+    L = ctypes.CDLL(so)
+    vp = ctypes.c_void_p
+    L.bo_cpu_path_create.restype = vp
+    L.bo_cpu_path_create.argtypes = [u64, u32, u64, vp, u32, u32, u32, u64, u64, u64, u64]
+    L.bo_cpu_path_destroy.argtypes = [vp]
+    L.bo_cpu_path_stats.argtypes = [vp, ctypes.POINTER(u64), ctypes.c_int]
+    L.bo_cpu_path_check.restype = ctypes.c_int
+    L.bo_cpu_path_check.argtypes = [vp]
+    L.bo_cpu_array_sum.restype = u64
+    L.bo_cpu_array_sum.argtypes = [vp, u32, u64, vp, u64]
+    L.bo_cpu_block_reads.restype = u64
+    L.bo_cpu_block_reads.argtypes = [vp, u32, u64, _p64, u32, vp]
+    L.bo_cpu_bfs.restype = u32
+    L.bo_cpu_bfs.argtypes = [vp, u32, _p64, u64, u64, _p32]
+    L.bo_cpu_cc.restype = u32
+    L.bo_cpu_cc.argtypes = [vp, u32, _p64, u64, _p64]
+    _CPU = L
+    return L
+
+
+class CpuPath:
+    """The reference's path restated on CPU threads, over the software NVMe target.
+
+    backing: None for a procedural namespace (word w = splitmix64(seed, w)), or a
+    C-contiguous numpy array that is the namespace content (kept alive here).
+    """
+
+    def __init__(self, ns_bytes, n_elems, page_size=4096, cache_pages=1024, lba_bytes=512, seed=42, backing=None,
+                 n_io_threads=2, n_queues=4, queue_depth=64, disk_offset_bytes=0):
+        self.L = cpu_lib()
+        self._backing = backing
+        bp = backing.ctypes.data if backing is not None else None
+        self.h = self.L.bo_cpu_path_create(ns_bytes, lba_bytes, seed, bp, n_io_threads, n_queues, queue_depth,
+                                           page_size, cache_pages, n_elems, disk_offset_bytes)
+        if not self.h:
+            raise RuntimeError("bo_cpu_path_create failed")
+
+    def array_sum(self, n_reqs, idx=None, stride=1, n_threads=4):
+        p = idx.ctypes.data if idx is not None else None
+        return self.L.bo_cpu_array_sum(self.h, n_threads, n_reqs, p, stride)
+
+    def block_reads(self, lbas, req_bytes, n_threads=4):
+        cs = np.empty(len(lbas), dtype=np.uint64)
+        self.L.bo_cpu_block_reads(self.h, n_threads, len(lbas), lbas, req_bytes, cs.ctypes.data)
+        return cs
+
+    def bfs(self, offsets, src, n_threads=4):
+        lv = np.empty(len(offsets), dtype=np.uint32)      # one spare slot: the current level is parked there
+        it = self.L.bo_cpu_bfs(self.h, n_threads, offsets, len(offsets) - 1, int(src), lv)
+        return lv[:-1].copy(), it
+
+    def cc(self, offsets, n_threads=4):
+        lb = np.empty(len(offsets) - 1, dtype=np.uint64)
+        it = self.L.bo_cpu_cc(self.h, n_threads, offsets, len(offsets) - 1, lb)
+        return lb, it
+
+    def stats(self, reset=True):
+        out = (u64 * 4)()
+        self.L.bo_cpu_path_stats(self.h, out, int(reset))
+        return dict(zip(("read_io_cnt", "access_cnt", "miss_cnt", "hit_cnt"), list(out)))
+
+    def check(self):
+        """0 when the quiescent-state invariants hold."""
+        return self.L.bo_cpu_path_check(self.h)
+
+    def close(self):
+        if self.h:
+            self.L.bo_cpu_path_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

@@ -1,0 +1,339 @@
+"""GPU parity: the gfx950 path, called through the C-ABI, against the CPU oracle.  Bit-exact everywhere (integer work)."""
+import ctypes
+import json
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+
+pytestmark = pytest.mark.gpu
+
+G = os.path.join(os.path.dirname(__file__), "golden")
+SEED = 42
+LIMIT_US = 20_000_000      # bound of every device-side wait in these tests
+
+
+@pytest.fixture(scope="module")
+def bam():
+    import torch
+    import bam_amd
+    if not torch.cuda.is_available():
+        pytest.fail("gpu tests need a GPU")
+    bam_amd.load()          # raises when the HIP library is missing: there is no fallback
+    return bam_amd
+
+
+_n = [0]
+
+
+def _path():
+    _n[0] += 1
+    return "/dev/libnvm-t%d" % _n[0]
+
+
+class Rig:
+    """target + controller (+ array) with teardown in the right order"""
+
+    def __init__(self, bam, ns_bytes, lba=512, backing=False, seed=SEED, n_queues=8, depth=256, io_threads=4, order=0,
+                 fail_every=0, drop_every=0, stage_bytes=4096, limit=LIMIT_US):
+        self.bam = bam
+        self.path = _path()
+        self.t = bam.Target(self.path, ns_bytes, lba, backing=backing, seed=seed, n_io_threads=io_threads,
+                            completion_order=order, fail_every=fail_every, drop_every=drop_every)
+        self.c = bam.Controller(self.path, 1, 0, queue_depth=depth, n_queues=n_queues, stage_bytes=stage_bytes, spin_limit=limit)
+        self.objs = []
+
+    def array(self, n_elems, page_size, cache_pages, disk_offset=0):
+        from bam_amd.host import make_array
+        pc, r, a = make_array(self.c, n_elems, page_size, cache_pages, 0, disk_offset)
+        self.objs.append((a, r, pc))
+        return a
+
+    def backing(self, n_words):
+        p = self.t.L.bam_target_backing(self.t.h)
+        return np.ctypeslib.as_array(ctypes.cast(p, ctypes.POINTER(ctypes.c_uint64)), shape=(n_words,))
+
+    def close(self):
+        for a, r, pc in self.objs:
+            a.close(); r.close(); pc.close()
+        self.c.close(); self.t.close()
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+
+def _dev(x):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(x).view(np.int64)).cuda()
+
+
+def _u64(t):
+    return t.cpu().numpy().view(np.uint64)
+
+
+# ---------------------------------------------------------------- generators
+
+def test_device_generators_match_oracle(bam):
+    from bam_amd import gen
+    assert np.array_equal(_u64(gen.words(SEED, 1000, 5000)), oracle.store(SEED, 1000, 5000))
+    assert np.array_equal(_u64(gen.gather_indices(SEED, 4096, 1 << 20, first=7)), oracle.gather_indices(SEED, 7, 4096, 1 << 20))
+    assert np.array_equal(_u64(gen.block_lbas(SEED, 1000, 64 << 30, 4096, 512)), oracle.block_lbas(SEED, 0, 1000, 64 << 30, 4096, 512))
+    for scale in (6, 12):
+        u, v = gen.rmat_pairs(SEED, scale, 0, 16 << scale)
+        ru = np.empty(16 << scale, dtype=np.uint64); rv = np.empty(16 << scale, dtype=np.uint64)
+        oracle.lib().bo_rmat_edges(SEED, scale, 0, 16 << scale, ru, rv)
+        assert np.array_equal(_u64(u), ru) and np.array_equal(_u64(v), rv)
+        off, nb = gen.rmat_csr(SEED, scale)
+        roff, rnb = oracle.rmat_csr(SEED, scale)
+        assert np.array_equal(_u64(off), roff) and np.array_equal(_u64(nb), rnb)
+    off, nb = gen.uniform_csr(SEED, 5000, 9000)
+    roff, rnb = oracle.uniform_csr(SEED, 5000, 9000)
+    assert np.array_equal(_u64(off), roff) and np.array_equal(_u64(nb), rnb)
+
+
+# ---------------------------------------------------------------- array
+
+def test_config1_reduction_on_gpu(bam):
+    """2^24 u64, 128 MiB store, 4 KiB pages, 64 MiB cache, stride-8 reads: the reference's plumbing case"""
+    with open(os.path.join(G, "splitmix64.json")) as f:
+        g = json.load(f)
+    for seed in (0, 42):
+        with Rig(bam, 128 << 20, seed=seed, n_queues=32, depth=1024) as r:
+            a = r.array(1 << 24, 4096, 16384)
+            s = a.read(1 << 21, stride=8, block_size=64)
+            st = a.stats()
+            assert s == int(g["cfg1_stride8_sum_2p21"][str(seed)], 16)
+            assert st["access_cnt"] == 1 << 21 and st["hit_cnt"] + st["miss_cnt"] == 1 << 21
+            assert 32768 <= st["read_io_cnt"] < 32768 + 8192
+            assert not r.c.aborted() and r.c.info()["error_completions"] == 0
+            assert r.t.stats()["read_cmds"] == st["read_io_cnt"]
+
+
+def test_counter_invariants_without_eviction(bam):
+    """read I/Os = distinct pages first touched; accesses = lane accesses; second pass all hits (reference logs)"""
+    n = 1 << 20
+    with Rig(bam, 16 << 20) as r:
+        a = r.array(n, 4096, 4096)
+        assert a.read(n, block_size=64) == oracle.lib().bo_store_sum(SEED, 0, 1, n)
+        st = a.stats()
+        assert st["read_io_cnt"] == n // 512 and st["access_cnt"] == n and st["hit_cnt"] + st["miss_cnt"] == n
+        assert a.read(n, block_size=256) == oracle.lib().bo_store_sum(SEED, 0, 1, n)
+        st = a.stats()
+        assert st == {"read_io_cnt": 0, "access_cnt": n, "miss_cnt": 0, "hit_cnt": n}
+        assert r.c.info(reset=True)["ssd_accesses"] == n // 512
+
+
+@pytest.mark.parametrize("cache_pages,n_queues,depth,block", [(64, 4, 64, 64), (1024, 2, 16, 256), (4096, 16, 1024, 128)])
+def test_random_gather_with_eviction(bam, cache_pages, n_queues, depth, block):
+    from bam_amd import gen
+    n_elems, n = 1 << 22, 1 << 18          # 8192 pages of data
+    with Rig(bam, 64 << 20, n_queues=n_queues, depth=depth) as r:
+        a = r.array(n_elems, 4096, cache_pages)
+        idx = gen.gather_indices(SEED, n, n_elems)
+        for _ in range(2):
+            assert a.read(n, idx, block_size=block) == oracle.lib().bo_gather_sum(SEED, SEED, 0, n, n_elems)
+            st = a.stats()
+            assert st["access_cnt"] == n and st["hit_cnt"] + st["miss_cnt"] == n and st["read_io_cnt"] > 0
+        assert a.read(n // 2, idx, reqs_per_thread=2, block_size=block) == (2 * oracle.lib().bo_gather_sum(SEED, SEED, 0, n // 2, n_elems)) % 2**64
+        assert not r.c.aborted()
+
+
+def test_ragged_and_empty_and_last_element(bam):
+    n_elems = (1 << 16) + 37                 # last page partly used
+    with Rig(bam, 1 << 20) as r:
+        a = r.array(n_elems, 4096, 32)
+        assert a.read(0) == 0
+        assert a.read(1) == oracle.lib().bo_splitmix64(SEED, 0)
+        assert a.read(77) == oracle.lib().bo_store_sum(SEED, 0, 1, 77)          # one and a bit waves
+        idx = np.array([n_elems - 1, 0, n_elems - 1, 511, 512, n_elems - 37], dtype=np.uint64)
+        assert a.read(len(idx), _dev(idx)) == int(np.sum(oracle.store(SEED, 0, n_elems)[idx.astype(np.int64)], dtype=np.uint64))
+        st = a.stats()
+        assert st["access_cnt"] == 0 + 1 + 77 + 6
+
+
+def test_memory_backed_store_disk_offset_and_small_pages(bam):
+    data = (np.arange(1 << 18, dtype=np.uint64) * np.uint64(0x9E3779B97F4A7C15)) ^ np.uint64(0xABCDEF)
+    with Rig(bam, data.nbytes, backing=True) as r:
+        r.backing(len(data))[:] = data
+        off_elems = 4096
+        a = r.array(len(data) - off_elems, 512, 256, disk_offset=off_elems * 8)     # 512-byte lines as in the reference's Optane runs
+        idx = oracle.gather_indices(7, 0, 1 << 16, len(data) - off_elems)
+        assert a.read(len(idx), _dev(idx), block_size=64) == int(np.sum(data[idx.astype(np.int64) + off_elems], dtype=np.uint64))
+        st = a.stats()
+        assert st["access_cnt"] == len(idx) and st["read_io_cnt"] > 256
+        assert r.t.stats()["bytes_read"] == st["read_io_cnt"] * 512
+
+
+def test_large_pages_through_bigger_staging(bam):
+    with Rig(bam, 32 << 20, stage_bytes=8192) as r:
+        a = r.array(1 << 20, 8192, 64)
+        assert a.read(1 << 18, stride=3) == oracle.lib().bo_store_sum(SEED, 0, 3, 1 << 18)
+        assert r.t.stats()["bytes_read"] == a.stats()["read_io_cnt"] * 8192
+
+
+# ---------------------------------------------------------------- cache / pattern streaming
+
+@pytest.mark.parametrize("mode", [0, 1, 2])
+def test_page_streaming_modes(bam, mode):
+    n_pages = 4096
+    with Rig(bam, 64 << 20) as r:
+        a = r.array(n_pages * 512, 4096, n_pages)
+        ref = oracle.lib().bo_store_sum(SEED, 0, 1, n_pages * 512)
+        assert a.stream(n_pages // 2, 2, mode=mode) == ref          # cold: every page read once
+        st = a.stats()
+        # per-element operator[]: the wave's first access to a page misses, its seven others hit; bam_ptr and the
+        # page-wise kernel take each page once per wave
+        assert st["read_io_cnt"] == n_pages and st["hit_cnt"] == (n_pages * 448 if mode == 0 else 0)
+        assert st["access_cnt"] == (n_pages * 512 if mode == 0 else n_pages * 64)
+        assert a.stream(n_pages // 2, 2, mode=mode) == ref          # hot: no I/O at all
+        st = a.stats()
+        assert st["read_io_cnt"] == 0 and st["miss_cnt"] == 0
+        # permuted page assignment, smaller cache than data
+    with Rig(bam, 64 << 20) as r:
+        a = r.array(n_pages * 512, 4096, 512)
+        perm = np.random.default_rng(3).permutation(n_pages).astype(np.uint64)
+        assert a.stream(n_pages, 1, _dev(perm), mode=mode) == ref
+        assert not r.c.aborted()
+
+
+# ---------------------------------------------------------------- raw block
+
+@pytest.mark.parametrize("req,lba,order", [(4096, 512, 0), (512, 512, 2), (4096, 4096, 1)])
+def test_block_reads_payload_checksums(bam, req, lba, order):
+    from bam_amd import gen
+    n, ns = 1 << 16, 64 << 30
+    with Rig(bam, ns, lba=lba, n_queues=16, depth=256, order=order) as r:
+        pc = bam.PageCache(4096, n, 0, r.c)
+        lbas = gen.block_lbas(SEED, n, ns, req, lba)
+        for policy in (0, 1):
+            pc.block_io(n, req, lbas, queue_policy=policy)
+            cs = _u64(pc.block_checksums(n, req))
+            ref = np.array([oracle.lib().bo_block_checksum(SEED, int(x), lba, req) for x in _u64(lbas)], dtype=np.uint64)
+            assert np.array_equal(cs, ref)
+        pc.block_io(1000, req, None)            # sequential LBAs, ragged last wave
+        cs = _u64(pc.block_checksums(1000, req))
+        ref = np.array([oracle.lib().bo_block_checksum(SEED, k * req // lba, lba, req) for k in range(1000)], dtype=np.uint64)
+        assert np.array_equal(cs, ref)
+        ts = r.t.stats()
+        assert ts["read_cmds"] == 2 * n + 1000 and ts["error_cpls"] == 0 and ts["sq_doorbells"] < ts["read_cmds"]
+        assert not r.c.aborted()
+        pc.close()
+
+
+def test_block_write_then_read_back(bam):
+    n = 4096
+    with Rig(bam, 64 << 20, backing=True) as r:
+        pc = bam.PageCache(4096, n, 0, r.c)
+        pc.block_io(n, 4096, None)                                   # slots <- LBAs 0..
+        before = _u64(pc.block_checksums(n, 4096)).copy()
+        shifted = _dev(np.arange(n, dtype=np.uint64) * np.uint64(8) + np.uint64(8 * n))
+        pc.block_io(n, 4096, shifted, write=True)                    # same payload to LBAs further on
+        store = r.backing((64 << 20) // 8)
+        assert np.array_equal(store[n * 512: 2 * n * 512], oracle.store(SEED, 0, n * 512))
+        pc.block_io(n, 4096, shifted)
+        assert np.array_equal(_u64(pc.block_checksums(n, 4096)), before)
+        assert r.t.stats()["write_cmds"] == n
+        pc.close()
+
+
+# ---------------------------------------------------------------- write path through the cache
+
+def test_array_write_eviction_write_back_and_flush(bam):
+    n_elems = 1 << 16
+    with Rig(bam, n_elems * 8, backing=True) as r:
+        a = r.array(n_elems, 4096, 16)                               # 128 pages of data, 16 cached: dirty pages get evicted
+        vals = np.arange(n_elems, dtype=np.uint64) * np.uint64(3) + np.uint64(1)
+        a.write(n_elems, _dev(vals), block_size=64)
+        r.objs[0][2].flush()
+        assert np.array_equal(r.backing(n_elems), vals)
+        assert a.read(n_elems) == int(np.sum(vals, dtype=np.uint64))
+        assert r.t.stats()["write_cmds"] >= 128 and not r.c.aborted()
+
+
+# ---------------------------------------------------------------- graphs
+
+def _graph_rig(bam, nb, cache_pages, **kw):
+    pad = (-len(nb)) % 512
+    r = Rig(bam, (len(nb) + pad) * 8, backing=True, **kw)
+    r.backing(len(nb) + pad)[:len(nb)] = nb
+    return r, r.array(max(len(nb), 1), 4096, cache_pages)
+
+
+def test_reference_sample_graph(bam):
+    with open(os.path.join(G, "sample_graph.json")) as f:
+        g = json.load(f)
+    off = np.array(g["offsets"], dtype=np.uint64)
+    nb = np.array(g["edges"], dtype=np.uint64)
+    r, a = _graph_rig(bam, nb, 64)
+    with r:
+        for src, exp in g["bfs"].items():
+            lv, it = a.bfs(_dev(off), int(src))
+            assert lv.cpu().numpy().view(np.uint32).tolist() == exp["levels"] and it == exp["iterations"]
+        lb, it = a.cc(_dev(off))
+        assert _u64(lb).tolist() == g["cc"]["labels"]
+
+
+@pytest.mark.parametrize("scale,cache_pages,coarse", [(10, 4096, 1), (14, 512, 128), (16, 8192, 8)])
+def test_bfs_levels_rmat(bam, scale, cache_pages, coarse):
+    off, nb = oracle.rmat_csr(SEED, scale)
+    r, a = _graph_rig(bam, nb, cache_pages, n_queues=16, depth=256)
+    with r:
+        doff = _dev(off)
+        for src in oracle.bfs_sources(SEED, off, 4):
+            lv, it = a.bfs(doff, int(src), coarse=coarse)
+            ref, rit = oracle.bfs_levels(off, nb, int(src))
+            assert np.array_equal(lv.cpu().numpy().view(np.uint32), ref) and it == rit
+        assert not r.c.aborted()
+
+
+@pytest.mark.parametrize("n_v,n_p,cache_pages,coarse", [(1 << 12, 3000, 256, 1), (1 << 16, 1 << 18, 512, 512), (1 << 14, 1 << 17, 4096, 4)])
+def test_cc_labels_uniform(bam, n_v, n_p, cache_pages, coarse):
+    off, nb = oracle.uniform_csr(SEED, n_v, n_p)
+    r, a = _graph_rig(bam, nb, cache_pages, n_queues=16, depth=256)
+    with r:
+        lb, it = a.cc(_dev(off), coarse=coarse)
+        ref, comps = oracle.cc_labels(off, nb)
+        assert np.array_equal(_u64(lb), ref)
+        assert len(np.unique(_u64(lb))) == comps and it >= 1
+        assert not r.c.aborted()
+
+
+# ---------------------------------------------------------------- failure handling
+
+def test_lost_completion_ends_the_kernel_with_the_abort_flag(bam):
+    """the target swallows one command in 500; the waits are bounded, so the launch returns and says so"""
+    with Rig(bam, 16 << 20, drop_every=500, limit=300_000) as r:
+        a = r.array(1 << 20, 4096, 4096)
+        a.read(1 << 18, block_size=64)
+        assert r.c.aborted() and r.t.stats()["dropped"] >= 1
+        assert r.c.aborted(clear=True) and not r.c.aborted()
+
+
+def test_error_completions_are_counted(bam):
+    with Rig(bam, 16 << 20, fail_every=100) as r:
+        a = r.array(1 << 20, 4096, 4096)
+        a.read(1 << 18, block_size=64)
+        assert not r.c.aborted()
+        assert r.c.info()["error_completions"] == r.t.stats()["error_cpls"] > 0
+
+
+# ---------------------------------------------------------------- full size (config 2)
+
+def test_config2_full_size_gather(bam):
+    """2^28 u64 behind a 1 GiB cache, 2^26 uniform reads, one thread per read: checksum against the closed form"""
+    from bam_amd import gen
+    n_elems, n = 1 << 28, 1 << 26
+    with Rig(bam, n_elems * 8, n_queues=128, depth=1024, io_threads=12) as r:
+        a = r.array(n_elems, 4096, 1 << 18)
+        idx = gen.gather_indices(SEED, n, n_elems)
+        assert a.read(n, idx, block_size=256) == oracle.lib().bo_gather_sum(SEED, SEED, 0, n, n_elems)
+        st = a.stats()
+        assert st["access_cnt"] == n and st["hit_cnt"] + st["miss_cnt"] == n
+        # a page can be fetched at most once per distinct wave-level miss: between #distinct pages and #misses
+        assert (1 << 18) < st["read_io_cnt"] <= st["miss_cnt"]
+        assert not r.c.aborted() and r.c.info()["error_completions"] == 0
