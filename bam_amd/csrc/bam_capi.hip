@@ -40,7 +40,8 @@ struct bam_target {
 struct bam_ctrl { Controller* c; };
 struct bam_page_cache { page_cache_t* pc; Controller* ctrl; };
 struct bam_range { range_t<uint64_t>* r; };
-struct bam_array { array_t<uint64_t>* a; };
+#define BAM_SUM_PARTIALS 4096
+struct bam_array { array_t<uint64_t>* a; BufferPtr partials; };      /* partials: [BAM_SUM_PARTIALS] checksum shards, zero between launches */
 
 // ---------------------------------------------------------------------------
 // device helpers
@@ -63,9 +64,22 @@ __device__ __forceinline__ uint64_t wave_sum(uint64_t v)
     return v;
 }
 
-/* add this block's values into *sum with one atomic per wave */
-__device__ __forceinline__ void block_accumulate(unsigned long long* sum, uint64_t v)
+/*
+ * Add the wave's values into the launch's checksum.  A single word would take one atomic per wave of the
+ * whole grid, all serialised on one address (about 12 ns each: a million waves cost more than the reads they
+ * sum), so the sum is kept in BAM_SUM_PARTIALS shards picked by workgroup and folded by k_fold_partials.
+ */
+__device__ __forceinline__ void block_accumulate(unsigned long long* partials, uint64_t v)
 {
+    v = wave_sum(v);
+    if (bam::lane() == 0 && v) atomicAdd(&partials[(blockIdx.x * 0x9E3779B1u) >> 20], (unsigned long long)v);
+}
+
+/* one block of 1024 threads: *sum += all shards; shards are left zero for the next launch */
+__global__ void k_fold_partials(unsigned long long* partials, unsigned long long* sum)
+{
+    uint64_t v = 0;
+    for (uint32_t i = threadIdx.x; i < BAM_SUM_PARTIALS; i += blockDim.x) { v += partials[i]; partials[i] = 0; }
     v = wave_sum(v);
     if (bam::lane() == 0 && v) atomicAdd(sum, (unsigned long long)v);
 }
@@ -100,27 +114,37 @@ __global__ __launch_bounds__(256) void k_cache_stream(array_d_t<uint64_t>* dr, u
         const uint64_t epp = r0->n_elems_per_page;
         const uint64_t start_page = assignment ? assignment[wave] : wave * n_pages_per_wave;
         if (MODE == 2) {
-            /* descriptor read once; per page one acquire, eight loads in flight per lane, one release */
+            /*
+             * Descriptor read once.  Pages are taken sixteen at a time: lane l of the wave asks for page l of the
+             * batch, so the sixteen reference counts go out as one vector atomic; then the whole wave streams the
+             * sixteen pages, eight loads in flight per lane, and the sixteen references are dropped together.
+             */
             bam::range_view<uint64_t> view;
             view.load(r0);
             const uint32_t n8 = view.page_size / 8;
-            for (uint64_t p = 0; p < n_pages_per_wave; p++) {
-                const uint64_t page = view.page_of((start_page + p) * epp);
-                uint64_t a0 = 0, a1 = 0;
-                auto sum_page = [&](uint32_t slot) {
-                    const uint64_t* base = (const uint64_t*)view.slot_addr(slot);
+            uint64_t a0 = 0, a1 = 0;
+            for (uint64_t p0 = 0; p0 < n_pages_per_wave; p0 += 16) {
+                const uint32_t nb = (uint32_t)(n_pages_per_wave - p0 < 16 ? n_pages_per_wave - p0 : 16);
+                uint32_t slot = 0;
+                const uint64_t page = view.page_of((start_page + p0 + (lane < nb ? lane : 0)) * epp);
+                if (lane < nb) {
+                    auto keep = [&](uint32_t s_) { slot = s_; return false; };
+                    view.acquire(page, false, keep, keep);
+                }
+                for (uint32_t k = 0; k < nb; k++) {
+                    const uint64_t* base = (const uint64_t*)view.slot_addr(bam::bcast(slot, k));
                     for (uint32_t i = (uint32_t)lane; i < n8; i += 8 * BAM_WAVE_SIZE) {
                         uint64_t x[8];
 #pragma unroll
-                        for (int k = 0; k < 8; k++) x[k] = i + k * BAM_WAVE_SIZE < n8 ? bam::ld_payload(base + i + k * BAM_WAVE_SIZE) : 0;
+                        for (int j = 0; j < 8; j++) x[j] = i + j * BAM_WAVE_SIZE < n8 ? bam::ld_payload(base + i + j * BAM_WAVE_SIZE) : 0;
                         a0 += x[0] + x[2] + x[4] + x[6];
                         a1 += x[1] + x[3] + x[5] + x[7];
                     }
-                    return true;
-                };
-                view.acquire(page, false, sum_page, sum_page);
-                v += a0 + a1;
+                }
+                if (lane < nb) view.release(page, false);
             }
+            v += a0 + a1;
+            view.flush_stats();
         } else {
             bam_ptr<uint64_t> ptr(dr);
             for (uint64_t p = 0; p < n_pages_per_wave; p++) {
@@ -481,7 +505,7 @@ int bam_array_create(bam_array_t** out, uint64_t n_elems, uint64_t disk_start_of
     BAM_API_BEGIN
     std::vector<range_t<uint64_t>*> rs;
     for (uint32_t i = 0; i < n_ranges; i++) rs.push_back(ranges[i]->r);
-    *out = new bam_array{new array_t<uint64_t>(n_elems, disk_start_offset, rs, device)};
+    *out = new bam_array{new array_t<uint64_t>(n_elems, disk_start_offset, rs, device), createBuffer(BAM_SUM_PARTIALS * sizeof(uint64_t), device)};
     BAM_API_END
 }
 
@@ -502,7 +526,7 @@ int bam_array_stats(bam_array_t* a, uint64_t* out, int reset)
         std::vector<bam_array_counters> per;
         a->a->reset_stats(&per);
         for (size_t i = 0; i < per.size(); i++) {
-            bam_stat_shard_t s0 = {per[i].access_cnt, per[i].miss_cnt, per[i].hit_cnt, per[i].read_io_cnt, {0, 0, 0, 0}};
+            bam_stat_shard_t s0 = {per[i].access_cnt, 0, per[i].hit_cnt, per[i].read_io_cnt, {0, 0, 0, 0}};
             hip_err_chk(hipMemcpy(a->a->h_ranges[i].stats, &s0, sizeof(s0), hipMemcpyHostToDevice));
         }
         out[0] = out[1] = out[2] = out[3] = 0;
@@ -522,7 +546,8 @@ int bam_array_read(bam_array_t* a, uint64_t n_reqs, const uint64_t* d_assignment
     if (!n_reqs) return 0;
     BAM_API_BEGIN
     hipLaunchKernelGGL(k_array_read, dim3(blocks_for(n_reqs, block_size)), dim3(block_size), 0, (hipStream_t)stream,
-                       a->a->d_array_ptr, n_reqs, d_assignment, stride, reqs_per_thread, (unsigned long long*)d_sum);
+                       a->a->d_array_ptr, n_reqs, d_assignment, stride, reqs_per_thread, (unsigned long long*)a->partials.get());
+    hipLaunchKernelGGL(k_fold_partials, dim3(1), dim3(1024), 0, (hipStream_t)stream, (unsigned long long*)a->partials.get(), (unsigned long long*)d_sum);
     hip_err_chk(hipGetLastError());
     BAM_API_END
 }
@@ -550,10 +575,11 @@ int bam_cache_stream(bam_array_t* a, uint64_t n_waves, uint64_t n_pages_per_wave
     const uint32_t bs = 256;
     const dim3 grid(blocks_for(n_waves * BAM_WAVE_SIZE, bs)), block(bs);
     array_d_t<uint64_t>* d = a->a->d_array_ptr;
-    unsigned long long* s = (unsigned long long*)d_sum;
+    unsigned long long* s = (unsigned long long*)a->partials.get();
     if (mode == 0) hipLaunchKernelGGL(k_cache_stream<0>, grid, block, 0, (hipStream_t)stream, d, n_waves, n_pages_per_wave, d_assignment, s);
     else if (mode == 1) hipLaunchKernelGGL(k_cache_stream<1>, grid, block, 0, (hipStream_t)stream, d, n_waves, n_pages_per_wave, d_assignment, s);
     else hipLaunchKernelGGL(k_cache_stream<2>, grid, block, 0, (hipStream_t)stream, d, n_waves, n_pages_per_wave, d_assignment, s);
+    hipLaunchKernelGGL(k_fold_partials, dim3(1), dim3(1024), 0, (hipStream_t)stream, s, (unsigned long long*)d_sum);
     hip_err_chk(hipGetLastError());
     BAM_API_END
 }

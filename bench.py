@@ -1,0 +1,292 @@
+#!/usr/bin/env python3
+"""Benchmark of the GPU-side storage-access path on one MI355X.
+
+A step is one launch of the random-gather array benchmark: 2^26 element reads,
+one thread per read, at uniform-random indices into a 2^28-element u64 array
+(2 GiB store) behind a 1 GiB page cache with 4 KiB pages, the store being the
+software NVMe target.  The index tensors are generated and resident in HBM
+before the timed region.  `value` is 4 KiB read I/Os per second over the timed
+steps.  On the same JSON line:
+
+  roofline      the hit-path page-streaming kernel over the resident 1 GiB
+                cache (HBM bound), timed with HIP events on its stream
+  cpu_baseline  the CPU restatement of the reference path (oracle/cpu_path.c)
+                on a bounded sample of the same workload, on the host cores
+  store         what the backing store can do: the target's service ceiling
+                with plain host clients and the interconnect ceiling for the
+                staged payload, both measured in this run
+  block         raw block benchmark (2^22 reads, 128 queue pairs x 1024)
+  bfs           RMAT BFS through bam_ptr (with --bfs-scale)
+
+Everything is checked against the closed-form oracle while it is measured.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+SEED = 42
+N_ELEMS = 1 << 28
+CACHE_PAGES = 1 << 18
+PAGE = 4096
+N_READS = 1 << 26
+HBM_PEAK_GBS = 8000.0
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=3)
+    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--io-threads", type=int, default=12, help="service threads of the software NVMe target")
+    ap.add_argument("--queues", type=int, default=128)
+    ap.add_argument("--depth", type=int, default=1024)
+    ap.add_argument("--block", type=int, default=256, help="threads per block of the gather kernel")
+    ap.add_argument("--cpu-reads", type=int, default=1 << 22, help="size of the CPU-baseline sample (element reads)")
+    ap.add_argument("--cpu-threads", type=int, default=8)
+    ap.add_argument("--bfs-scale", type=int, default=24, help="RMAT scale of the BFS leg (0 = skip)")
+    ap.add_argument("--bfs-sources", type=int, default=8)
+    ap.add_argument("--skip-cpu", action="store_true")
+    ap.add_argument("--skip-block", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this path runs on one GPU; --gpus %d is not supported (a GPU box here has one GPU, "
+                 "and the path has no collective step to scale)" % args.gpus)
+
+    import numpy as np
+    import torch
+    import bam_amd
+    from bam_amd import gen, _lib
+    from bam_amd.host import make_array
+    import oracle
+
+    L = _lib.load()                     # raises if the HIP library is missing: nothing here falls back to the CPU
+    O = oracle.lib()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def event():
+        e = ctypes.c_void_p()
+        assert L.bam_event_create(ctypes.byref(e)) == 0
+        return e
+
+    def elapsed_ms(a, b):
+        ms = ctypes.c_float(0)
+        assert L.bam_event_elapsed_ms(a, b, ctypes.byref(ms)) == 0
+        return ms.value
+
+    # ------------------------------------------------------------------ set-up
+    t0 = time.time()
+    target = bam_amd.Target("/dev/libnvm0", N_ELEMS * 8, 512, backing=False, seed=SEED, n_io_threads=args.io_threads)
+    ctrl = bam_amd.Controller("/dev/libnvm0", 1, 0, queue_depth=args.depth, n_queues=args.queues, spin_limit=60_000_000)
+    pc, rng, arr = make_array(ctrl, N_ELEMS, PAGE, CACHE_PAGES)
+    n_steps = args.warmup + args.steps
+    idx = [gen.gather_indices(SEED, N_READS, N_ELEMS, first=s * N_READS) for s in range(n_steps)]
+    sums = [torch.zeros(1, dtype=torch.int64, device=dev) for _ in range(n_steps)]
+    torch.cuda.synchronize()
+    log("[bench] set-up %.1fs: %s %s" % (time.time() - t0, ctrl.info(), pc.info()))
+
+    # ------------------------------------------------------------------ hit path (roofline): stream the resident cache
+    arr.stream(CACHE_PAGES // 4, 4, mode=2)             # cold pass fills the cache with pages 0 .. CACHE_PAGES-1
+    arr.stats()
+    ref_stream = O.bo_store_sum(SEED, 0, 1, 1 << 24)
+    assert arr.stream((1 << 24) // 512 // 4, 4, mode=2) == ref_stream, "hit-path checksum mismatch"
+    hit_reps = 20
+    s_hit = torch.zeros(1, dtype=torch.int64, device=dev)
+    for mode, name in ((2, "page_wise"), (1, "bam_ptr")):
+        arr.stream_async(CACHE_PAGES // 4, 4, s_hit, mode=mode)
+    torch.cuda.synchronize()
+    hit = {}
+    for mode, name in ((2, "page_wise"), (1, "bam_ptr")):
+        a, b = event(), event()
+        L.bam_event_record(a, stream)
+        for _ in range(hit_reps):
+            arr.stream_async(CACHE_PAGES // 4, 4, s_hit, mode=mode)
+        L.bam_event_record(b, stream)
+        ms = elapsed_ms(a, b) / hit_reps
+        hit[name] = {"ms_per_launch": ms, "GBps": CACHE_PAGES * PAGE / ms / 1e6}
+    st = arr.stats()
+    assert st["read_io_cnt"] == 0 and st["miss_cnt"] == 0, "hit-path pass did I/O"
+    roofline = {"bound": "hbm", "kernel": "k_cache_stream<2> (page-wise streaming of the resident cache)",
+                "achieved": hit["page_wise"]["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": hit["page_wise"]["GBps"] / HBM_PEAK_GBS, "traffic": None,
+                "bytes_per_launch": CACHE_PAGES * PAGE, "ms_per_launch": hit["page_wise"]["ms_per_launch"],
+                "bam_ptr_kernel_GBps": hit["bam_ptr"]["GBps"]}
+    log("[bench] hit path: %s" % hit)
+
+    # 100 %-hit element gather (indices restricted to the resident half)
+    idx_hit = gen.gather_indices(SEED, N_READS, CACHE_PAGES * 512)
+    arr.read_async(N_READS, s_hit.zero_(), idx_hit, block_size=args.block)
+    torch.cuda.synchronize()
+    a, b = event(), event()
+    L.bam_event_record(a, stream)
+    arr.read_async(N_READS, s_hit.zero_(), idx_hit, block_size=args.block)
+    L.bam_event_record(b, stream)
+    ms = elapsed_ms(a, b)
+    assert int(s_hit.item()) & (2**64 - 1) == O.bo_gather_sum(SEED, SEED, 0, N_READS, CACHE_PAGES * 512), "hit gather checksum mismatch"
+    gather_hit = {"reads_per_s": N_READS / ms * 1e3, "GBps_of_u64": N_READS * 8 / ms / 1e6, "ms": ms}
+    arr.stats()
+    del idx_hit
+    log("[bench] hit gather: %s" % gather_hit)
+
+    # ------------------------------------------------------------------ timed steps (configuration 2)
+    for s in range(args.warmup):
+        arr.read_async(N_READS, sums[s], idx[s], block_size=args.block)
+    torch.cuda.synchronize()
+    arr.stats(); target.stats(reset=True)
+    a, b = event(), event()
+    t_wall = time.time()
+    L.bam_event_record(a, stream)
+    for s in range(args.warmup, n_steps):
+        arr.read_async(N_READS, sums[s], idx[s], block_size=args.block)
+    L.bam_event_record(b, stream)
+    torch.cuda.synchronize()
+    t_wall = time.time() - t_wall
+    ms_total = elapsed_ms(a, b)
+    st = arr.stats()
+    ts = target.stats()
+    ok = not ctrl.aborted() and ctrl.info()["error_completions"] == 0
+    for s in range(n_steps):
+        want = O.bo_gather_sum(SEED, SEED, s * N_READS, N_READS, N_ELEMS)
+        ok = ok and (int(sums[s].item()) & (2**64 - 1)) == want
+    assert ok, "configuration-2 checksum mismatch or aborted wait"
+    assert st["access_cnt"] == args.steps * N_READS and st["read_io_cnt"] == ts["read_cmds"]
+    iops = st["read_io_cnt"] / ms_total * 1e3
+    ms_per_step = ms_total / max(args.steps, 1)
+    cfg2_hit_rate = st["hit_cnt"] / max(st["access_cnt"], 1)
+    log("[bench] cfg2: %.1f ms/step, %.2f M IOPS, %.1f M reads/s, hit rate %.3f, doorbells %d, sqe_retries %d (wall %.2fs)" %
+        (ms_per_step, iops / 1e6, args.steps * N_READS / ms_total / 1e3, st["hit_cnt"] / st["access_cnt"], ts["sq_doorbells"], ts["sqe_retries"], t_wall))
+    del idx, sums
+
+    # ------------------------------------------------------------------ what the store can do
+    ms_c = ctypes.c_float(0)
+    assert L.bam_host_read_ceiling(8 << 30, 4096, ctypes.byref(ms_c)) == 0
+    link_gbps = (8 << 30) / ms_c.value / 1e6
+    n_clients = max(2, min(8, (os.cpu_count() or 8) // 2))
+    target_iops = L.bam_target_ceiling_iops(64 << 30, 512, 0, args.io_threads, n_clients, 256, 400000, 4096)
+    ceiling = min(target_iops, link_gbps * 1e9 / PAGE)
+    store = {"target_service_iops": target_iops, "target_clients": n_clients, "interconnect_pull_GBps": link_gbps,
+             "interconnect_iops_4k": link_gbps * 1e9 / PAGE, "ceiling_iops_4k": ceiling, "cfg2_frac_of_ceiling": iops / ceiling}
+    log("[bench] store: %s" % store)
+
+    # ------------------------------------------------------------------ raw block benchmark (configuration 3)
+    block = None
+    if not args.skip_block:
+        arr.close(); rng.close(); pc.close(); ctrl.close(); target.close()
+        target = bam_amd.Target("/dev/libnvm0", 64 << 30, 512, backing=False, seed=SEED, n_io_threads=args.io_threads)
+        ctrl = bam_amd.Controller("/dev/libnvm0", 1, 0, queue_depth=1024, n_queues=128, spin_limit=60_000_000)
+        n_blk = 1 << 22
+        pcb = bam_amd.PageCache(PAGE, n_blk, 0, ctrl)
+        block = {}
+        for req in (4096, 512):
+            lbas = gen.block_lbas(SEED, n_blk, 64 << 30, req, 512)
+            pcb.block_io(n_blk, req, lbas, block_size=64)           # warm-up launch
+            torch.cuda.synchronize()
+            a, b = event(), event()
+            L.bam_event_record(a, stream)
+            pcb.block_io(n_blk, req, lbas, block_size=64)
+            L.bam_event_record(b, stream)
+            ms = elapsed_ms(a, b)
+            cs = pcb.block_checksums(n_blk, req).cpu().numpy().view(np.uint64)
+            sample = np.random.default_rng(1).integers(0, n_blk, 4096)
+            lb = lbas.cpu().numpy().view(np.uint64)
+            good = all(int(cs[k]) == O.bo_block_checksum(SEED, int(lb[k]), 512, req) for k in sample)
+            assert good and not ctrl.aborted(), "raw block payload checksum mismatch"
+            block["read_%dB" % req] = {"iops": n_blk / ms * 1e3, "GBps": n_blk * req / ms / 1e6, "ms": ms}
+        block["frac_of_ceiling_4k"] = block["read_4096B"]["iops"] / ceiling
+        log("[bench] block: %s" % block)
+        pcb.close()
+
+    # ------------------------------------------------------------------ BFS on RMAT (configuration 4)
+    bfs = None
+    if args.bfs_scale:
+        t0 = time.time()
+        ctrl.close(); target.close()
+        off, nb = gen.rmat_csr(SEED, args.bfs_scale)
+        n_e = nb.numel()
+        ns_bytes = (n_e * 8 + PAGE - 1) // PAGE * PAGE
+        target = bam_amd.Target("/dev/libnvm0", ns_bytes, 512, backing=True, seed=SEED, n_io_threads=args.io_threads)
+        dst = (ctypes.c_char * (n_e * 8)).from_address(target.L.bam_target_backing(target.h))
+        nb_h = nb.cpu().numpy()
+        ctypes.memmove(dst, nb_h.ctypes.data, n_e * 8)
+        ctrl = bam_amd.Controller("/dev/libnvm0", 1, 0, queue_depth=1024, n_queues=128, spin_limit=60_000_000)
+        cache_pages = max(1 << 14, (n_e * 8 // PAGE) // 4)              # 25 % of the edge array
+        pcg, rg, ag = make_array(ctrl, n_e, PAGE, cache_pages)
+        off_h = off.cpu().numpy().view(np.uint64)
+        srcs = oracle.bfs_sources(SEED, off_h, args.bfs_sources)
+        del nb
+        log("[bench] bfs graph: V=2^%d E=%d cache_pages=%d (%.1fs to build)" % (args.bfs_scale, n_e, cache_pages, time.time() - t0))
+        tot_ms, tot_edges, levels_ok, iters = 0.0, 0, True, []
+        nb_u = nb_h.view(np.uint64)
+        for k, src in enumerate(srcs):
+            a, b = event(), event()
+            L.bam_event_record(a, stream)
+            lv, it = ag.bfs(off, int(src), coarse=4)
+            L.bam_event_record(b, stream)
+            ms = elapsed_ms(a, b)
+            lv_h = lv.cpu().numpy().view(np.uint32)
+            if k == 0:                                                  # full-size parity against the serial oracle (timed: the CPU figure)
+                t1 = time.time()
+                ref, rit = oracle.bfs_levels(off_h, nb_u, int(src))
+                cpu_bfs_s = time.time() - t1
+                cpu_bfs_edges = O.bo_bfs_edges_scanned(len(off_h) - 1, off_h, ref)
+                levels_ok = levels_ok and np.array_equal(lv_h, ref) and it == rit
+            tot_edges += O.bo_bfs_edges_scanned(len(off_h) - 1, off_h, lv_h)
+            tot_ms += ms
+            iters.append(it)
+        assert levels_ok and not ctrl.aborted(), "BFS levels differ from the oracle"
+        st = ag.stats()
+        bfs = {"scale": args.bfs_scale, "edges": n_e, "sources": len(srcs), "GTEPS": tot_edges / tot_ms / 1e6,
+               "ms_per_source": tot_ms / len(srcs), "iterations": iters, "read_ios": st["read_io_cnt"],
+               "hit_rate": st["hit_cnt"] / max(st["access_cnt"], 1)}
+        # CPU figure: the oracle's uncached in-RAM serial BFS on one core, same graph, first source
+        bfs["cpu_serial_GTEPS"] = cpu_bfs_edges / cpu_bfs_s / 1e9
+        log("[bench] bfs: %s" % bfs)
+        ag.close(); rg.close(); pcg.close()
+
+    ctrl.close(); target.close()
+
+    # ------------------------------------------------------------------ CPU baseline (the reference path restated on host cores)
+    cpu = None
+    if not args.skip_cpu:
+        n_s = args.cpu_reads
+        cp = oracle.CpuPath(N_ELEMS * 8, N_ELEMS, PAGE, CACHE_PAGES, seed=SEED, n_io_threads=4, n_queues=args.cpu_threads, queue_depth=1024)
+        idx_h = oracle.gather_indices(SEED, 0, n_s, N_ELEMS)
+        t1 = time.time()
+        s = cp.array_sum(n_s, idx_h, n_threads=args.cpu_threads)
+        dt = time.time() - t1
+        cst = cp.stats()
+        assert s == O.bo_gather_sum(SEED, SEED, 0, n_s, N_ELEMS) and cp.check() == 0, "CPU baseline checksum mismatch"
+        cp.close()
+        cpu = {"value": cst["read_io_cnt"] / dt, "unit": "IOPS", "cores": args.cpu_threads + 4, "kind": "port",
+               "sample": "first %d of the 2^26 reads of one step, cold cache, %d lane threads + 4 target threads; %.1f s" % (n_s, args.cpu_threads, dt),
+               "reads_per_s": n_s / dt}
+        log("[bench] cpu baseline: %s" % cpu)
+
+    out = {
+        "metric": "4KiB read IOPS (random gather through the page cache); cache-hit GB/s and BFS GTEPS alongside",
+        "value": iops, "unit": "IOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "u64", "data": "synthetic",
+        "config": {"workload": "random gather array bench: 2^28 u64 (2 GiB store), 4 KiB pages, 1 GiB page cache, 2^26 uniform-random reads per launch, one thread per read",
+                   "store": "software NVMe target, procedural namespace, %d service threads, %d queue pairs x %d" % (args.io_threads, args.queues, args.depth),
+                   "seed": SEED, "block_size": args.block},
+        "reads_per_s": args.steps * N_READS / ms_total * 1e3,
+        "hit_rate": cfg2_hit_rate,
+        "roofline": roofline, "cpu_baseline": cpu, "store": store, "hit_gather": gather_hit, "block": block, "bfs": bfs,
+    }
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -66,7 +66,7 @@ enum data_dist_t { REPLICATE = 0, STRIPE = 1 };
 #define V_NB  0x02U
 #define V_B   0x03U
 
-#define BAM_STAT_SHARDS 256
+#define BAM_STAT_SHARDS 4096
 
 struct page_cache_t;
 struct page_cache_d_t;
@@ -347,7 +347,7 @@ struct range_d_t {
     __forceinline__ __device__ void mark_page_dirty(const size_t index) { __hip_atomic_fetch_or(&pages[index].state, DIRTY, __ATOMIC_RELAXED, BAM_AGENT); }
     __forceinline__ __device__ uint64_t acquire_page(const size_t pg, const uint32_t count, const bool write, const uint32_t ctrl, const uint32_t queue);
     /* spread by workgroup so that no counter word is shared by more than a few waves at a time */
-    __forceinline__ __device__ bam_stat_shard_t* shard() const { return stats + (((blockIdx.x + blockIdx.y * gridDim.x) * 0x9E3779B1u) >> 24) % BAM_STAT_SHARDS; }
+    __forceinline__ __device__ bam_stat_shard_t* shard() const { return stats + (((blockIdx.x + blockIdx.y * gridDim.x) * 0x9E3779B1u) >> 20) % BAM_STAT_SHARDS; }
     __forceinline__ __device__ bool slow_step(const size_t pg, const bool write, const uint32_t queue, uint64_t& sv, uint32_t& slot, bool& was_hit, bool& progressed);
 };
 
@@ -384,20 +384,21 @@ __forceinline__ __device__ bool bam_try_hit(data_page_t* dp, const uint32_t coun
 
 namespace bam {
 /*
- * Add v (0..127) of every active lane to a counter with one atomic per distinct
- * counter word: the lane values are summed with seven ballots (bit-sliced
- * population count), which works for any set of active lanes.
+ * Add v (below 2^BITS) of every active lane to a counter with one atomic per
+ * distinct counter word: the lane values are summed with BITS ballots
+ * (bit-sliced population count), which works for any set of active lanes.
  */
+template <int BITS = 7>
 __device__ __forceinline__ void stat_add(unsigned long long* ctr, uint32_t v)
 {
     for (bool done = false; !done;) {
         const uint64_t a0 = first((uint64_t)ctr);
         if ((uint64_t)ctr == a0) {
-            uint32_t total = 0;
+            unsigned long long total = 0;
 #pragma unroll
-            for (uint32_t b = 0; b < 7; b++) total += popc(ballot((v >> b) & 1u)) << b;
+            for (uint32_t b = 0; b < BITS; b++) total += (unsigned long long)popc(ballot((v >> b) & 1u)) << b;
             if (lane() == first_lane(active_mask()) && total)
-                __hip_atomic_fetch_add((unsigned long long*)a0, (unsigned long long)total, __ATOMIC_RELAXED, BAM_AGENT);
+                __hip_atomic_fetch_add((unsigned long long*)a0, total, __ATOMIC_RELAXED, BAM_AGENT);
             done = true;
         }
     }
@@ -490,7 +491,6 @@ uint64_t range_d_t<T>::acquire_page(const size_t pg, const uint32_t count, const
     bam_stat_shard_t* sh = shard();
     bam::stat_add(&sh->access_cnt, count);
     bam::stat_add(&sh->hit_cnt, hit ? count : 0);
-    bam::stat_add(&sh->miss_cnt, hit ? 0 : count);
     return slot;
 }
 
@@ -513,9 +513,11 @@ struct range_view {
     bam_stat_shard_t* shard;
     uint64_t index_start, index_end, pso;
     uint32_t page_size_log, page_size;
+    uint32_t n_access = 0, n_hit = 0;   /* this lane's accesses since the last flush_stats() */
 
     __forceinline__ __device__ void load(range_d_t<T>* r_)
     {
+        flush_stats();
         r = r_;
         pages = r_->pages;
         base_addr = r_->cache.base_addr;
@@ -538,12 +540,22 @@ struct range_view {
         end = index_start + (first_byte + page_size - pso) / sizeof(T);
         if (end > index_end) end = index_end;
     }
-    /* one access per active lane: hit or miss as its group's master found the page */
-    __forceinline__ __device__ void account(const bool hit) const
+    /*
+     * One access per active lane, hit or miss as its group's master found the
+     * page.  Counted in registers; flush_stats() adds the lanes' totals to the
+     * range's counters with one atomic per counter per wave.  Misses are not
+     * counted separately: every access is either one or the other.
+     */
+    __forceinline__ __device__ void account(const bool hit) { n_access++; n_hit += hit ? 1u : 0u; }
+
+    /* WIDE: the lanes may hold more than one access each (a view that lived through many acquires) */
+    template <bool WIDE = true>
+    __forceinline__ __device__ void flush_stats()
     {
-        stat_add(&shard->access_cnt, 1);
-        stat_add(&shard->hit_cnt, hit ? 1 : 0);
-        stat_add(&shard->miss_cnt, hit ? 0 : 1);
+        if (!r) return;
+        stat_add<WIDE ? 32 : 1>(&shard->access_cnt, n_access);
+        stat_add<WIDE ? 32 : 1>(&shard->hit_cnt, n_hit);
+        n_access = n_hit = 0;
     }
 
     /*
@@ -557,7 +569,7 @@ struct range_view {
      * is loading.  `on_miss(slot)` runs for those lanes once their page is in.
      */
     template <typename FH, typename FM>
-    __forceinline__ __device__ void acquire(const uint64_t page, const bool write, FH&& on_hit, FM&& on_miss) const
+    __forceinline__ __device__ void acquire(const uint64_t page, const bool write, FH&& on_hit, FM&& on_miss)
     {
         const uint32_t me = lane();
         const uint64_t eq_mask = match_any(page, (uint64_t)r);
@@ -649,6 +661,7 @@ struct array_d_t {
         uint32_t slot = 0;
         auto keep = [&](uint32_t s_) { slot = s_; return false; };
         v.acquire(page, write, keep, keep);
+        v.template flush_stats<false>();
         base_master = slot;
     }
 
@@ -661,6 +674,7 @@ struct array_d_t {
         const uint64_t byte = v.byte_of(i);
         auto use = [&](uint32_t slot) { fn((T*)(v.slot_addr(slot) + (byte & (v.page_size - 1)))); return true; };
         v.acquire(byte >> v.page_size_log, write, use, use);
+        v.template flush_stats<false>();
     }
 
     __forceinline__ __device__ T seq_read(const size_t i) const
@@ -701,6 +715,7 @@ struct array_d_t {
         uint32_t slot = 0;
         auto keep = [&](uint32_t s_) { slot = s_; return false; };
         v.acquire(page, false, keep, keep);
+        v.template flush_stats<false>();
         page_ = v.pages + page;
         v.window(page, start, end);
         return (void*)(v.slot_addr(slot) + (v.byte_of(start) & (v.page_size - 1)));
@@ -759,7 +774,13 @@ struct bam_ptr {
 #endif
 
     __forceinline__ __host__ __device__ bam_ptr(array_d_t<T>* a) { init(a); }
-    __forceinline__ __host__ __device__ ~bam_ptr() { fini(); }
+    __forceinline__ __host__ __device__ ~bam_ptr()
+    {
+        fini();
+#if defined(__HIP_DEVICE_COMPILE__)
+        view.flush_stats();
+#endif
+    }
     __forceinline__ __host__ __device__ void init(array_d_t<T>* a) { array = a; }
 
     __forceinline__ __host__ __device__ void fini(void)
@@ -1076,7 +1097,8 @@ struct array_t {
             hip_err_chk(hipMemcpy(sh.data(), h_ranges[i].stats, sh.size() * sizeof(bam_stat_shard_t), hipMemcpyDeviceToHost));
             hip_err_chk(hipMemset(h_ranges[i].stats, 0, sh.size() * sizeof(bam_stat_shard_t)));
             bam_array_counters r = {0, 0, 0, 0};
-            for (auto& s : sh) { r.read_io_cnt += s.read_io_cnt; r.access_cnt += s.access_cnt; r.miss_cnt += s.miss_cnt; r.hit_cnt += s.hit_cnt; }
+            for (auto& s : sh) { r.read_io_cnt += s.read_io_cnt; r.access_cnt += s.access_cnt; r.hit_cnt += s.hit_cnt; }
+            r.miss_cnt = r.access_cnt - r.hit_cnt;      /* every access is a hit or a miss; only hits are counted on the device */
             if (per_range) per_range->push_back(r);
             tot.read_io_cnt += r.read_io_cnt; tot.access_cnt += r.access_cnt; tot.miss_cnt += r.miss_cnt; tot.hit_cnt += r.hit_cnt;
         }
