@@ -467,6 +467,16 @@ int bam_page_cache_info(bam_page_cache_t* pc, uint64_t* out)
     return 0;
 }
 
+int bam_page_cache_profile(bam_page_cache_t* pc, uint64_t* out16, int reset)
+{
+    if (!pc || !out16) return fail(EINVAL, "bam_page_cache_profile: null argument");
+    BAM_API_BEGIN
+    hip_err_chk(hipDeviceSynchronize());
+    hip_err_chk(hipMemcpy(out16, pc->pc->pdt.prof, 16 * sizeof(uint64_t), hipMemcpyDeviceToHost));
+    if (reset) hip_err_chk(hipMemset(pc->pc->pdt.prof, 0, 16 * sizeof(uint64_t)));
+    BAM_API_END
+}
+
 int bam_page_cache_flush(bam_page_cache_t* pc)
 {
     if (!pc) return fail(EINVAL, "bam_page_cache_flush: null argument");

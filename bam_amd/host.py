@@ -122,6 +122,13 @@ class PageCache:
     def flush(self):
         _chk(self.L.bam_page_cache_flush(self.h), "bam_page_cache_flush")
 
+    def profile(self, reset=True):
+        """Miss-path phase timers (only a library built with -DBAM_PROFILE fills them)."""
+        out = (c_u64 * 16)()
+        _chk(self.L.bam_page_cache_profile(self.h, out, int(reset)), "bam_page_cache_profile")
+        keys = ("batches", "commands", "t_cid", "t_submit", "t_wait", "t_copy", "t_find_slot", "find_slot_calls", "find_slot_lanes")
+        return dict(zip(keys, list(out)))
+
     def block_io(self, n_reqs, req_bytes, lbas=None, write=False, queue_policy=1, block_size=64):
         """One thread per NVMe command into cache slot tid (benchmarks/block/main.cu:99-200)."""
         _chk(self.L.bam_block_io(self.ctrl.h, self.h, n_reqs, req_bytes, _ptr(lbas), int(write), queue_policy, block_size, _stream()),

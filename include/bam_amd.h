@@ -60,6 +60,10 @@ void bam_page_cache_destroy(bam_page_cache_t* pc);
 /* out[4]: n_pages, page_size, wave_batch, staged(0/1) */
 int bam_page_cache_info(bam_page_cache_t* pc, uint64_t* out);
 int bam_page_cache_flush(bam_page_cache_t* pc);
+/* phase timers of the miss path (100 MHz ticks), non-zero only in a library built with -DBAM_PROFILE; out16[0..8]:
+ * I/O batches, commands, ticks waiting for command ids, submitting, waiting for completions, moving payload,
+ * ticks in the victim search, victim searches, lanes searching */
+int bam_page_cache_profile(bam_page_cache_t* pc, uint64_t* out16, int reset);
 int bam_range_create(bam_range_t** out, uint64_t index_start, uint64_t count, uint64_t page_start, uint64_t page_count,
                      uint64_t page_start_offset, uint64_t page_size, bam_page_cache_t* pc, uint32_t device, int dist);
 void bam_range_destroy(bam_range_t* r);

@@ -97,7 +97,12 @@ __device__ __forceinline__ uint32_t wave_slot_hash()
     return h ^ (h >> 15);
 }
 
-/* back-off: n * 64 clocks, doubling up to 32 */
+/*
+ * Back-off of a wait loop: sleep n * 64 clocks, n doubling from 1 up to 127
+ * (about 4 us).  Waits here are for I/O that takes tens of microseconds or
+ * more, and thousands of waves may be waiting at once: polling faster than
+ * that only takes memory bandwidth away from the waves that are moving data.
+ */
 __device__ __forceinline__ void backoff(uint32_t& n)
 {
     switch (n) {
@@ -106,9 +111,11 @@ __device__ __forceinline__ void backoff(uint32_t& n)
     case 4: __builtin_amdgcn_s_sleep(4); break;
     case 8: __builtin_amdgcn_s_sleep(8); break;
     case 16: __builtin_amdgcn_s_sleep(16); break;
-    default: __builtin_amdgcn_s_sleep(32); break;
+    case 32: __builtin_amdgcn_s_sleep(32); break;
+    case 64: __builtin_amdgcn_s_sleep(64); break;
+    default: __builtin_amdgcn_s_sleep(127); break;
     }
-    if (n < 32) n <<= 1;
+    if (n < 128) n <<= 1;
 }
 
 /* ---- scoped atomics on plain words ---- */
@@ -148,6 +155,7 @@ template <typename T> __device__ __forceinline__ T ld_payload(const T* p)
 
 __device__ __forceinline__ void fence_release_sys() { __builtin_amdgcn_fence(__ATOMIC_RELEASE, ""); }
 __device__ __forceinline__ void fence_acquire_sys() { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, ""); }
+__device__ __forceinline__ void fence_acquire_agent() { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent"); }
 __device__ __forceinline__ void fence_acq_rel_agent() { __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "agent"); }
 
 } // namespace bam

@@ -39,7 +39,7 @@ namespace bam {
 struct spin_t { uint32_t n = 0, slp = 1; uint64_t t0 = 0; };
 
 /*
- * One back-off step of a wait loop; true = give up.  Every 64 steps the loop
+ * One back-off step of a wait loop; true = give up.  Every 256 steps the loop
  * looks at the shared abort flag and at the wall clock (100 MHz constant
  * counter): a wait that has lasted longer than `limit_us` microseconds raises
  * the abort flag itself.  limit_us = 0 waits for ever.
@@ -47,7 +47,7 @@ struct spin_t { uint32_t n = 0, slp = 1; uint64_t t0 = 0; };
 __device__ __forceinline__ bool spin_giveup(bam_guard_t* g, uint32_t limit_us, spin_t& s)
 {
     backoff(s.slp);
-    if ((++s.n & 63u) != 0 || !g) return false;
+    if ((++s.n & 255u) != 0 || !g) return false;
     if (ld_relaxed_sys(&g->abort)) return true;
     if (!limit_us) return false;
     const uint64_t now = wall_clock64();
@@ -87,8 +87,10 @@ __device__ __forceinline__ uint32_t get_cid_group(nvm_queue_t* sq)
         const uint32_t b = t & (n_blocks - 1), shift = (uint32_t)__builtin_ctz(n_blocks);
         const uint32_t turn_mask = 0xffffffffu >> shift;
         spin_t sp;
-        while (((ld_acquire(&sq->pos_locks[b].val) - (t >> shift)) & turn_mask) != 0)
+        /* polled with plain loads: an acquire per look would invalidate this compute unit's cache every time */
+        while (((ld_relaxed(&sq->pos_locks[b].val) - (t >> shift)) & turn_mask) != 0)
             if (spin_giveup(sq, sp)) break;
+        fence_acquire_agent();
         base = b << 6;
     }
     base = bcast(base, leader);
@@ -107,15 +109,35 @@ __device__ __forceinline__ void put_cid_group(nvm_queue_t* sq, uint32_t id)
 
 __device__ __forceinline__ void cq_drain_group(nvm_queue_t* cq, nvm_queue_t* sq, uint64_t act);
 
-/* drain the completion queue if nobody else is doing so; true if this group did */
+/*
+ * Drain the completion queue if nobody else is doing so; true if this group
+ * did.  The ring may live on the far side of the interconnect, and every
+ * waiting wave comes through here, so an idle ring must cost next to nothing:
+ * the holder of head_lock first reads the one entry at the head (a single
+ * small read), and only when that entry is new does the group read a window
+ * of 64; after an empty look the queue is left alone for two microseconds
+ * (the time is kept in the otherwise unused `tail` word of the CQ descriptor).
+ */
 __device__ __forceinline__ bool try_drain_group(nvm_queue_t* cq, nvm_queue_t* sq)
 {
     const uint64_t act = active_mask();
     const uint32_t leader = first_lane(act);
     uint32_t got = 0;
-    if (lane() == leader)
-        got = ld_relaxed(&cq->head_lock) == UNLOCKED &&
-              __hip_atomic_exchange(&cq->head_lock, (uint32_t)LOCKED, __ATOMIC_ACQUIRE, BAM_AGENT) == UNLOCKED;
+    if (lane() == leader) {
+        /* the word holds the time of the next look (low 32 bits of the clock): wait only while that lies within
+         * the next two microseconds, so that a stale or never-written value can never hold anybody up */
+        const uint32_t ahead = ld_relaxed(&cq->tail) - (uint32_t)wall_clock64();
+        if (ahead - 1u >= 200u && ld_relaxed(&cq->head_lock) == UNLOCKED &&
+            __hip_atomic_exchange(&cq->head_lock, (uint32_t)LOCKED, __ATOMIC_ACQUIRE, BAM_AGENT) == UNLOCKED) {
+            const uint32_t h = ld_relaxed(&cq->head);
+            const uint32_t dw3 = ld_acquire_sys(&((nvm_cpl_t*)cq->vaddr)[h & cq->qs_minus_1].dword[3]);
+            if (((dw3 >> 16) & 1u) == ((~(h >> cq->qs_log2)) & 1u)) got = 1;
+            else {
+                st_relaxed(&cq->tail, (uint32_t)wall_clock64() + 200u);      /* nothing new: next look in 2 us */
+                st_release(&cq->head_lock, (uint32_t)UNLOCKED);
+            }
+        }
+    }
     got = bcast(got, leader);
     if (got) {
         cq_drain_group(cq, sq, act);
@@ -143,7 +165,8 @@ __device__ __forceinline__ uint32_t sq_enqueue_group(nvm_queue_t* sq, nvm_cmd_t*
     bool written = false;
     spin_t sp;
     for (;;) {
-        if (!written && ld_acquire(&sq->tickets[pos].val) == want) {
+        if (!written && ld_relaxed(&sq->tickets[pos].val) == want) {
+            fence_acquire_agent();
             uint4* dst = (uint4*)(((nvm_cmd_t*)sq->vaddr) + pos);
             const uint4* src = (const uint4*)cmd->dword;
             dst[0] = src[0]; dst[1] = src[1]; dst[2] = src[2]; dst[3] = src[3];
@@ -151,7 +174,7 @@ __device__ __forceinline__ uint32_t sq_enqueue_group(nvm_queue_t* sq, nvm_cmd_t*
             st_release_sys(&sq->tail_mark[pos].val, 1u);
             written = true;
         }
-        const uint32_t tl = ld_acquire(&sq->tail);
+        const uint32_t tl = ld_relaxed(&sq->tail);
         const bool covered = written && (int32_t)(tl - ticket) > 0;
         if (!ballot(!covered)) break;
         bool progressed = false;
@@ -247,7 +270,7 @@ __device__ __forceinline__ void cq_wait_group(nvm_queue_t* cq, nvm_queue_t* sq, 
 {
     spin_t sp;
     for (;;) {
-        const bool done = (ld_acquire(&sq->cid[cid].val) & BAM_CID_DONE) != 0;
+        const bool done = (ld_relaxed(&sq->cid[cid].val) & BAM_CID_DONE) != 0;
         if (!ballot(!done)) break;
         try_drain_group(cq, sq);
         if (spin_giveup(cq, sp)) break;

@@ -66,6 +66,7 @@ enum data_dist_t { REPLICATE = 0, STRIPE = 1 };
 #define V_NB  0x02U
 #define V_B   0x03U
 
+#define BAM_TOKEN_SLOTS 4096u
 #define BAM_STAT_SHARDS 4096
 
 struct page_cache_t;
@@ -120,6 +121,9 @@ struct page_cache_d_t {
     bool prps;
     uint64_t n_blocks_per_page;
     uint32_t wave_batch;             /* distinct pages one wave loads side by side (64: a whole wave) */
+    uint32_t* miss_tokens;           /* number of waves inside the miss path right now */
+    uint32_t miss_waves;             /* at most this many at a time per compute unit (0 = no limit) */
+    unsigned long long* prof;        /* [16] phase timers in 100 MHz ticks, filled only by builds with BAM_PROFILE */
     bam_guard_t* guard;
     uint32_t spin_limit;
 
@@ -181,7 +185,13 @@ __device__ __forceinline__ void io_group(page_cache_d_t* pc, QueuePair* qp, uint
     const uint32_t n = popc(act), rank = rank_in(act);
     const uint32_t bytes = n_blocks << qp->block_size_log;
     uint8_t* slot_addr = pc->base_addr + pc_entry * pc->page_size;
+#ifdef BAM_PROFILE
+    const uint64_t pt0 = wall_clock64();
+#endif
     const uint32_t cid = get_cid_group(&qp->sq);
+#ifdef BAM_PROFILE
+    const uint64_t pt1 = wall_clock64();
+#endif
     uint64_t prp1, prp2 = 0;
     uint8_t* stage = nullptr;
     if (qp->stage) {
@@ -203,9 +213,22 @@ __device__ __forceinline__ void io_group(page_cache_d_t* pc, QueuePair* qp, uint
     nvm_cmd_data_ptr(&cmd, prp1, prp2);
     nvm_cmd_rw_blks(&cmd, lba, (uint16_t)n_blocks);
     sq_enqueue_group(&qp->sq, &cmd);
+#ifdef BAM_PROFILE
+    const uint64_t pt2 = wall_clock64();
+#endif
     cq_wait_group(&qp->cq, &qp->sq, cid);
+#ifdef BAM_PROFILE
+    const uint64_t pt3 = wall_clock64();
+#endif
     if (stage && opcode == NVM_IO_READ) copy_pages(slot_addr, stage, bytes, act, n, rank);
     put_cid_group(&qp->sq, cid);
+#ifdef BAM_PROFILE
+    if (pc->prof && rank == 0) {
+        const uint64_t pt4 = wall_clock64();
+        atomicAdd(&pc->prof[0], 1ull); atomicAdd(&pc->prof[1], (unsigned long long)n);
+        atomicAdd(&pc->prof[2], pt1 - pt0); atomicAdd(&pc->prof[3], pt2 - pt1); atomicAdd(&pc->prof[4], pt3 - pt2); atomicAdd(&pc->prof[5], pt4 - pt3);
+    }
+#endif
 }
 
 } // namespace bam
@@ -443,7 +466,13 @@ bool range_d_t<T>::slow_step(const size_t pg, const bool write, const uint32_t q
         }
     }
     if (load_me) {
+#ifdef BAM_PROFILE
+        const uint64_t pf0 = wall_clock64();
+#endif
         const uint32_t found = cache.find_slot(pg, range_id, queue);
+#ifdef BAM_PROFILE
+        if (cache.prof && bam::lane() == bam::first_lane(bam::active_mask())) { atomicAdd(&cache.prof[6], wall_clock64() - pf0); atomicAdd(&cache.prof[7], 1ull); atomicAdd(&cache.prof[8], (unsigned long long)bam::popc(bam::active_mask())); }
+#endif
         if (found == BAM_NO_SLOT) {
             /* no evictable slot right now: hand the page back; a later pass tries again */
             __hip_atomic_fetch_and(&dp->state, DISABLE_BUSY_MASK, __ATOMIC_RELEASE, BAM_AGENT);
@@ -588,8 +617,52 @@ struct range_view {
         } else {
             /* miss path: pass after pass; groups whose page came in are served and release before the next pass */
             const uint32_t queue = wave_slot_hash();
+            const uint32_t leader = first_lane(active_mask());
             bool done = false;
             spin_t sp;
+            /*
+             * Admission: only so many waves per compute unit work on misses at a time.  Every wave in here polls
+             * queues and page states while its I/O is in flight; with all resident waves doing that at once the
+             * polling itself takes the memory system and the interconnect away from the waves that are moving
+             * payload, and throughput drops.  One counter per compute unit, 64 bytes apart: waiting waves poll
+             * their own unit's word.
+             */
+            page_cache_d_t* cache = (page_cache_d_t*)first((uint64_t)&r->cache);
+            const uint32_t limit = cache->miss_waves;
+            uint32_t* tokens = cache->miss_tokens + (cu_id() & (BAM_TOKEN_SLOTS - 1)) * 16;
+            bool admitted = limit == 0;
+            if (!admitted) {
+                uint32_t ok = 0;
+                if (me == leader) {
+                    if (__hip_atomic_fetch_add(tokens, 1u, __ATOMIC_RELAXED, BAM_AGENT) < limit) ok = 1;
+                    else __hip_atomic_fetch_add(tokens, 0u - 1u, __ATOMIC_RELAXED, BAM_AGENT);
+                }
+                admitted = bcast(ok, leader) != 0;
+            }
+            if (!admitted) {
+                /*
+                 * Queue up outside without references: a page that somebody else brings in meanwhile must stay
+                 * evictable, or the waves that wait here could pin every slot the admitted ones need.
+                 */
+                if (master == me) __hip_atomic_fetch_add(&dp->state, 0u - count, __ATOMIC_RELAXED, BAM_AGENT);
+                uint32_t ok = 0;
+                if (me == leader) {
+                    for (uint32_t i = 1;; i++) {
+                        if (ld_relaxed(tokens) < limit) {
+                            if (__hip_atomic_fetch_add(tokens, 1u, __ATOMIC_RELAXED, BAM_AGENT) < limit) { ok = 1; break; }
+                            __hip_atomic_fetch_add(tokens, 0u - 1u, __ATOMIC_RELAXED, BAM_AGENT);
+                        }
+                        __builtin_amdgcn_s_sleep(127);
+                        __builtin_amdgcn_s_sleep(127);
+                        __builtin_amdgcn_s_sleep(127);
+                        __builtin_amdgcn_s_sleep(127);
+                        /* no clock of its own: the waves inside time their waits, this one only watches for their verdict */
+                        if ((i & 63u) == 0 && cache->guard && ld_relaxed_sys(&cache->guard->abort)) break;
+                    }
+                }
+                admitted = bcast(ok, leader) != 0;
+                if (master == me) bam_try_hit(dp, count, dirty, sv, slot);     /* slow_step reads the outcome from sv */
+            }
             for (;;) {
                 bool progressed = false;
                 if (!done) {
@@ -605,8 +678,10 @@ struct range_view {
                     }
                 }
                 if (!ballot(!done)) break;
-                if (!ballot(progressed) && r->cache.spin_giveup(sp)) break;
+                if (ballot(progressed)) sp = spin_t();
+                else if (cache->spin_giveup(sp)) break;
             }
+            if (limit && admitted && me == leader) __hip_atomic_fetch_add(tokens, 0u - 1u, __ATOMIC_RELAXED, BAM_AGENT);
         }
     }
 
@@ -899,6 +974,8 @@ struct page_cache_t {
     BufferPtr page_ticket_buf;
     BufferPtr ctrl_counter_buf;
     BufferPtr extra_reads_buf;
+    BufferPtr prof_buf;
+    BufferPtr tokens_buf;
 
     uint64_t reset_stats()
     {
@@ -981,6 +1058,12 @@ struct page_cache_t {
         pdt.page_ticket = (uint32_t*)page_ticket_buf.get();
 
         pdt.wave_batch = BAM_WAVE_SIZE;
+        tokens_buf = createBuffer(BAM_TOKEN_SLOTS * 64, hipDevice);
+        pdt.miss_tokens = (uint32_t*)tokens_buf.get();
+        pdt.miss_waves = 4;
+        if (const char* e = getenv("BAM_MISS_WAVES")) pdt.miss_waves = (uint32_t)atoi(e);
+        prof_buf = createBuffer(16 * sizeof(unsigned long long), hipDevice);
+        pdt.prof = (unsigned long long*)prof_buf.get();
 
         const bool staged = ctrl.n_qps && ctrl.h_qps[0]->stage != nullptr;
         const uint64_t cache_size = ps * np;
