@@ -104,7 +104,7 @@ __global__ void k_array_write(array_d_t<uint64_t>* dr, uint64_t n_reqs, const ui
 
 // ---- cache / pattern benchmark (benchmarks/cache/main.cu:44-114): a wave streams whole pages ----
 template <int MODE>
-__global__ __launch_bounds__(256) void k_cache_stream(array_d_t<uint64_t>* dr, uint64_t n_waves, uint64_t n_pages_per_wave, const uint64_t* assignment, unsigned long long* sum)
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void k_cache_stream(array_d_t<uint64_t>* dr, uint64_t n_waves, uint64_t n_pages_per_wave, const uint64_t* assignment, unsigned long long* sum)
 {
     const uint64_t tid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const uint64_t wave = tid / BAM_WAVE_SIZE, lane = tid % BAM_WAVE_SIZE;

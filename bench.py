@@ -36,6 +36,10 @@ CACHE_PAGES = 1 << 18
 PAGE = 4096
 N_READS = 1 << 26
 HBM_PEAK_GBS = 8000.0
+# HBM bytes one launch of the page-wise streaming kernel moves over the 1 GiB cache, from the profiler's FETCH_SIZE and
+# WRITE_SIZE counters scaled by what they read for a plain 1 GiB copy (x2.0 and x1.0); figures and commands in
+# profiles/k_cache_stream_hit_path_1GiB_cache.md.  Holds for this workload only.
+HIT_STREAM_TRAFFIC_BYTES = 1084300000
 
 
 def log(*a):
@@ -51,12 +55,14 @@ def main():
     ap.add_argument("--queues", type=int, default=128)
     ap.add_argument("--depth", type=int, default=1024)
     ap.add_argument("--block", type=int, default=256, help="threads per block of the gather kernel")
-    ap.add_argument("--cpu-reads", type=int, default=1 << 22, help="size of the CPU-baseline sample (element reads)")
+    ap.add_argument("--cpu-reads", type=int, default=1 << 26, help="size of the CPU-baseline sample (element reads)")
     ap.add_argument("--cpu-threads", type=int, default=8)
     ap.add_argument("--bfs-scale", type=int, default=24, help="RMAT scale of the BFS leg (0 = skip)")
     ap.add_argument("--bfs-sources", type=int, default=8)
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--skip-block", action="store_true")
+    ap.add_argument("--only-hit", action="store_true",
+                    help="hit-path leg and a plain 1 GiB copy only (short; what the counter passes of the profiler are run on)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path runs on one GPU; --gpus %d is not supported (a GPU box here has one GPU, "
@@ -119,10 +125,22 @@ def main():
     assert st["read_io_cnt"] == 0 and st["miss_cnt"] == 0, "hit-path pass did I/O"
     roofline = {"bound": "hbm", "kernel": "k_cache_stream<2> (page-wise streaming of the resident cache)",
                 "achieved": hit["page_wise"]["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": hit["page_wise"]["GBps"] / HBM_PEAK_GBS, "traffic": None,
+                "frac": hit["page_wise"]["GBps"] / HBM_PEAK_GBS, "traffic": HIT_STREAM_TRAFFIC_BYTES,
                 "bytes_per_launch": CACHE_PAGES * PAGE, "ms_per_launch": hit["page_wise"]["ms_per_launch"],
                 "bam_ptr_kernel_GBps": hit["bam_ptr"]["GBps"]}
     log("[bench] hit path: %s" % hit)
+    if args.only_hit:
+        # a plain device copy of known size in the same process: the scale of the profiler's traffic counters
+        src = torch.empty(1 << 27, dtype=torch.int64, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        ms_c = ctypes.c_float(0)
+        for _ in range(3):
+            assert L.bam_copy_kernel(ctypes.c_void_p(src.data_ptr()), ctypes.c_void_p(dst.data_ptr()), ctypes.c_uint64(1 << 30), ctypes.byref(ms_c), stream) == 0
+        roofline["copy_1GiB_ms"] = ms_c.value
+        roofline["copy_GBps_read_plus_write"] = 2 * (1 << 30) / ms_c.value / 1e6
+        print(json.dumps({"roofline": roofline}), flush=True)
+        arr.close(); rng.close(); pc.close(); ctrl.close(); target.close()
+        return
 
     # 100 %-hit element gather (indices restricted to the resident half)
     idx_hit = gen.gather_indices(SEED, N_READS, CACHE_PAGES * 512)
@@ -269,7 +287,7 @@ def main():
         assert s == O.bo_gather_sum(SEED, SEED, 0, n_s, N_ELEMS) and cp.check() == 0, "CPU baseline checksum mismatch"
         cp.close()
         cpu = {"value": cst["read_io_cnt"] / dt, "unit": "IOPS", "cores": args.cpu_threads + 4, "kind": "port",
-               "sample": "first %d of the 2^26 reads of one step, cold cache, %d lane threads + 4 target threads; %.1f s" % (n_s, args.cpu_threads, dt),
+               "sample": "the first %d of the element reads of the timed steps (one step is 2^26), cold cache, %d lane threads + 4 target threads; %.1f s" % (n_s, args.cpu_threads, dt),
                "reads_per_s": n_s / dt}
         log("[bench] cpu baseline: %s" % cpu)
 
