@@ -78,7 +78,9 @@ struct QueuePair
         /* the ring is filled by the GPU across the interconnect and fetched by the controller from the other side:
          * have entries sealed so that one that has not fully arrived is never taken (see nvm_cmd_seal) */
         status = nvm_admin_sq_set_sealed(aq_ref, &sq);
-        if (!nvm_ok(status)) { nvm_admin_sq_delete(aq_ref, &sq, &cq); nvm_admin_cq_delete(aq_ref, &cq); delete own; throw std::runtime_error(std::string("Failed to seal submission queue: ") + nvm_strerror(status)); }
+        /* a controller that does not know the vendor command (a real device) answers with an NVMe status: the queue
+         * then runs unsealed, as the NVMe specification has it; anything else is a failed admin round trip */
+        if (!nvm_ok(status) && status > 0) { nvm_admin_sq_delete(aq_ref, &sq, &cq); nvm_admin_cq_delete(aq_ref, &cq); delete own; throw std::runtime_error(std::string("Failed to seal submission queue: ") + nvm_strerror(status)); }
 
         /* device-side protocol state */
         const uint32_t n_cids = qs < 64 ? 64 : qs;      /* handed out in blocks of 64, one block per wave */
