@@ -256,6 +256,103 @@ __global__ __launch_bounds__(128) void k_cc_coalesce_coarse_ptr_pc(array_d_t<uin
     }
 }
 
+// ---- BFS / CC by edge page: the same relaxations, work laid out along the edge array ----
+/*
+ * first[p], p = 0 .. n_pages: the vertex whose edge list holds edge p * epp (the last vertex with
+ * offsets[v] <= p * epp); first[n_pages] = V - 1.  The vertices with edges on page p are first[p] .. first[p + 1].
+ */
+__global__ void k_page_first_vertex(const uint64_t* offsets, uint64_t n_vertices, uint64_t epp, uint64_t n_pages, uint64_t* first)
+{
+    const uint64_t p = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (p > n_pages) return;
+    const uint64_t e = p * epp;
+    uint64_t lo = 0, hi = n_vertices + 1;            /* first index with offsets[idx] > e */
+    while (lo < hi) {
+        const uint64_t mid = (lo + hi) >> 1;
+        if (offsets[mid] > e) hi = mid; else lo = mid + 1;
+    }
+    uint64_t v = lo ? lo - 1 : 0;
+    if (v >= n_vertices) v = n_vertices - 1;
+    first[p] = v;
+}
+
+/*
+ * One wave, `ppw` consecutive pages of the edge array per trip (lane l looks after page l of the trip), trips
+ * handed out wave by wave along the array.  A page is wanted when one of its vertices is active; the wanted pages
+ * of a trip are taken with one acquire, so their misses go to the store as one batch of commands, and the whole
+ * wave then walks the active vertices of each page, 64 edges at a time, before the references are dropped.
+ * A wave holds at most `ppw` pages at a time; the launch keeps waves x ppw under half the cache.
+ */
+template <typename Active, typename Visit>
+__device__ __forceinline__ void graph_by_page(array_d_t<uint64_t>* da, const uint64_t* offsets, const uint64_t* first, const uint64_t n_edges,
+                                              const uint32_t ppw, Active active, Visit visit)
+{
+    const uint32_t lane = bam::lane();
+    const uint64_t wave = ((uint64_t)blockIdx.x * blockDim.x + threadIdx.x) / BAM_WAVE_SIZE;
+    const uint64_t n_waves = (uint64_t)gridDim.x * blockDim.x / BAM_WAVE_SIZE;
+    bam::range_view<uint64_t> view;
+    view.load(da->d_ranges);
+    const uint32_t epp = view.page_size / 8;
+    const uint64_t n_pages = (n_edges + epp - 1) / epp;
+    const uint64_t pso_pages = view.pso >> view.page_size_log;
+    for (uint64_t p0 = wave * ppw; p0 < n_pages; p0 += n_waves * ppw) {
+        const uint64_t p = p0 + lane;
+        const uint64_t pstart = p * epp;
+        bool want = false;
+        uint64_t va = 0, vb = 0;
+        if (lane < ppw && p < n_pages) {
+            va = first[p]; vb = first[p + 1];
+            const uint64_t pend = pstart + epp;
+            for (uint64_t v = va; v <= vb && !want; v++) want = active(v) && offsets[v] < pend && offsets[v + 1] > pstart;
+        }
+        uint32_t slot = 0;
+        if (want) {
+            auto keep = [&](uint32_t s_) { slot = s_; return false; };
+            view.acquire(p + pso_pages, false, keep, keep);
+        }
+        for (uint64_t m = bam::ballot(want); m; m &= m - 1) {
+            const uint32_t j = bam::first_lane(m);
+            const uint64_t va_j = bam::bcast(va, j), vb_j = bam::bcast(vb, j);
+            const uint64_t ps = (p0 + j) * epp, pe = ps + epp < n_edges ? ps + epp : n_edges;
+            const uint64_t* payload = (const uint64_t*)view.slot_addr(bam::bcast(slot, j));
+            for (uint64_t vbase = va_j; vbase <= vb_j; vbase += BAM_WAVE_SIZE) {
+                const uint64_t v = vbase + lane;
+                uint64_t es = 0, ee = 0;
+                if (v <= vb_j && active(v)) {
+                    es = offsets[v]; ee = offsets[v + 1];
+                    if (es < ps) es = ps;
+                    if (ee > pe) ee = pe;
+                }
+                for (uint64_t am = bam::ballot(es < ee); am; am &= am - 1) {
+                    const uint32_t k = bam::first_lane(am);
+                    const uint64_t e0 = bam::bcast(es, k), e1 = bam::bcast(ee, k), src = vbase + k;
+                    for (uint64_t i = e0 + lane; i < e1; i += BAM_WAVE_SIZE) visit(src, bam::ld_payload(payload + (i - ps)));
+                }
+            }
+        }
+        if (want) view.release(p + pso_pages, false);
+    }
+    view.flush_stats();
+}
+
+__global__ __launch_bounds__(64) void k_bfs_by_page(array_d_t<uint64_t>* da, uint32_t* label, const uint32_t level, const uint64_t* offsets,
+                                                     const uint64_t* first, uint64_t n_edges, uint32_t ppw, uint64_t* changed)
+{
+    bool any = false;
+    graph_by_page(da, offsets, first, n_edges, ppw,
+                  [&](uint64_t v) { return label[v] == level; },
+                  [&](uint64_t, uint64_t next) { if (label[next] == MYINFINITY) { label[next] = level + 1; any = true; } });
+    if (any) *changed = 1;
+}
+
+__global__ __launch_bounds__(64) void k_cc_by_page(array_d_t<uint64_t>* da, bool* curr_visit, bool* next_visit, const uint64_t* offsets,
+                                                    const uint64_t* first, uint64_t n_edges, uint32_t ppw, unsigned long long* comp, bool* changed)
+{
+    graph_by_page(da, offsets, first, n_edges, ppw,
+                  [&](uint64_t v) { return curr_visit[v]; },
+                  [&](uint64_t src, uint64_t next) { cc_compute(src, comp, next, next_visit, changed); });
+}
+
 __global__ void k_iota(unsigned long long* p, uint64_t n)
 {
     const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -676,6 +773,108 @@ int bam_cc(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, u
         hip_err_chk(hipMemcpyAsync(changed_d, &changed_h, sizeof(bool), hipMemcpyHostToDevice, st));
         hipLaunchKernelGGL(k_cc_coalesce_coarse_ptr_pc, dim3(blocks), dim3(threads), 0, st,
                            edges->a->d_array_ptr, curr, next, n_vertices, d_offsets, (unsigned long long*)d_labels, changed_d, (uint64_t)coarse);
+        hip_err_chk(hipGetLastError());
+        hip_err_chk(hipMemsetAsync(curr, 0x00, n_vertices, st));
+        bool* t = curr; curr = next; next = t;
+        iter++;
+        hip_err_chk(hipMemcpyAsync(&changed_h, changed_d, sizeof(bool), hipMemcpyDeviceToHost, st));
+        hip_err_chk(hipStreamSynchronize(st));
+    } while (changed_h);
+    if (iterations) *iterations = iter;
+    BAM_API_END
+}
+
+namespace {
+/* launch shape of the by-page graph kernels: pages per wave trip and number of waves, so that what the waves hold
+ * at any time stays under half of the cache */
+struct by_page_plan { uint64_t n_edges, n_pages; uint32_t epp, ppw, blocks; BufferPtr first; };
+
+int plan_by_page(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, hipStream_t st, by_page_plan& pl)
+{
+    array_t<uint64_t>* a = edges->a;
+    if (a->adt.n_ranges != 1) return fail(EINVAL, "by-page graph kernels take an array of one range");
+    const range_d_t<uint64_t>& r = a->h_ranges[0];
+    if (r.index_start != 0 || r.page_start_offset % r.cache.page_size) return fail(EINVAL, "by-page graph kernels need a range that starts on a page boundary");
+    pl.n_edges = a->adt.n_elems;
+    pl.epp = (uint32_t)(r.cache.page_size / 8);
+    pl.n_pages = (pl.n_edges + pl.epp - 1) / pl.epp;
+    const uint64_t budget = r.cache.n_pages / 2;               /* pages all waves together may hold */
+    if (!budget) return fail(EINVAL, "by-page graph kernels need a cache of at least two pages");
+    int dev = 0, cus = 0;
+    hip_err_chk(hipGetDevice(&dev));
+    hip_err_chk(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    const uint64_t max_waves = (uint64_t)cus * 8;              /* eight waves per compute unit */
+    uint64_t ppw = budget / max_waves;
+    if (ppw > BAM_WAVE_SIZE) ppw = BAM_WAVE_SIZE;
+    if (ppw < 1) ppw = 1;
+    uint64_t waves = budget / ppw;
+    if (waves > max_waves) waves = max_waves;
+    const uint64_t trips = (pl.n_pages + ppw - 1) / ppw;
+    if (waves > trips) waves = trips;
+    pl.ppw = (uint32_t)ppw;
+    pl.blocks = (uint32_t)waves;                               /* one wave per workgroup */
+    pl.first = createBuffer((pl.n_pages + 1) * sizeof(uint64_t), dev);
+    hipLaunchKernelGGL(k_page_first_vertex, dim3(blocks_for(pl.n_pages + 1, 256)), dim3(256), 0, st, d_offsets, n_vertices, (uint64_t)pl.epp, pl.n_pages,
+                       (uint64_t*)pl.first.get());
+    hip_err_chk(hipGetLastError());
+    return 0;
+}
+} // namespace
+
+int bam_bfs_by_page(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t src, uint32_t* d_labels,
+                    uint32_t* iterations, void* stream)
+{
+    if (!edges || !d_offsets || !d_labels) return fail(EINVAL, "bam_bfs_by_page: null argument");
+    if (src >= n_vertices) return fail(EINVAL, "bam_bfs_by_page: source out of range");
+    BAM_API_BEGIN
+    hipStream_t st = (hipStream_t)stream;
+    by_page_plan pl;
+    if (int rc = plan_by_page(edges, d_offsets, n_vertices, st, pl)) return rc;
+    BufferPtr changed_buf = createBuffer(sizeof(uint64_t), 0);
+    uint64_t* changed_d = (uint64_t*)changed_buf.get();
+    const uint32_t zero = 0;
+    hip_err_chk(hipMemsetAsync(d_labels, 0xFF, n_vertices * sizeof(uint32_t), st));
+    hip_err_chk(hipMemcpyAsync(d_labels + src, &zero, sizeof(uint32_t), hipMemcpyHostToDevice, st));
+    uint32_t level = 0, iter = 0;
+    uint64_t changed_h;
+    do {
+        changed_h = 0;
+        hip_err_chk(hipMemcpyAsync(changed_d, &changed_h, sizeof(uint64_t), hipMemcpyHostToDevice, st));
+        if (pl.n_pages)
+            hipLaunchKernelGGL(k_bfs_by_page, dim3(pl.blocks), dim3(BAM_WAVE_SIZE), 0, st, edges->a->d_array_ptr, d_labels, level, d_offsets,
+                               (const uint64_t*)pl.first.get(), pl.n_edges, pl.ppw, changed_d);
+        hip_err_chk(hipGetLastError());
+        iter++; level++;
+        hip_err_chk(hipMemcpyAsync(&changed_h, changed_d, sizeof(uint64_t), hipMemcpyDeviceToHost, st));
+        hip_err_chk(hipStreamSynchronize(st));
+    } while (changed_h);
+    if (iterations) *iterations = iter;
+    BAM_API_END
+}
+
+int bam_cc_by_page(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t* d_labels, uint32_t* iterations, void* stream)
+{
+    if (!edges || !d_offsets || !d_labels) return fail(EINVAL, "bam_cc_by_page: null argument");
+    if (!n_vertices) return fail(EINVAL, "bam_cc_by_page: empty graph");
+    BAM_API_BEGIN
+    hipStream_t st = (hipStream_t)stream;
+    by_page_plan pl;
+    if (int rc = plan_by_page(edges, d_offsets, n_vertices, st, pl)) return rc;
+    BufferPtr visit_a = createBuffer(n_vertices, 0), visit_b = createBuffer(n_vertices, 0), changed_buf = createBuffer(sizeof(uint64_t), 0);
+    bool* curr = (bool*)visit_a.get();
+    bool* next = (bool*)visit_b.get();
+    bool* changed_d = (bool*)changed_buf.get();
+    hipLaunchKernelGGL(k_iota, dim3(blocks_for(n_vertices, 256)), dim3(256), 0, st, (unsigned long long*)d_labels, n_vertices);
+    hip_err_chk(hipMemsetAsync(curr, 0x01, n_vertices, st));
+    hip_err_chk(hipMemsetAsync(next, 0x00, n_vertices, st));
+    uint32_t iter = 0;
+    bool changed_h;
+    do {
+        changed_h = false;
+        hip_err_chk(hipMemcpyAsync(changed_d, &changed_h, sizeof(bool), hipMemcpyHostToDevice, st));
+        if (pl.n_pages)
+            hipLaunchKernelGGL(k_cc_by_page, dim3(pl.blocks), dim3(BAM_WAVE_SIZE), 0, st, edges->a->d_array_ptr, curr, next, d_offsets,
+                               (const uint64_t*)pl.first.get(), pl.n_edges, pl.ppw, (unsigned long long*)d_labels, changed_d);
         hip_err_chk(hipGetLastError());
         hip_err_chk(hipMemsetAsync(curr, 0x00, n_vertices, st));
         bool* t = curr; curr = next; next = t;

@@ -206,19 +206,25 @@ class Array:
         self.stream_async(n_waves, n_pages_per_wave, s, assignment, mode)
         return int(s.item()) & MASK64
 
-    def bfs(self, offsets, src, coarse=1):
-        """Levels (uint32 as int32 bits... returned as int64-safe uint32 tensor) and launch count."""
+    def bfs(self, offsets, src, coarse=1, by_page=False):
+        """Levels (uint32 bit patterns in an int32 tensor) and launch count; by_page: the edge-page kernel."""
         n_v = offsets.numel() - 1
         labels = torch.empty(n_v, dtype=torch.int32, device=offsets.device)
         it = c_u32(0)
-        _chk(self.L.bam_bfs(self.h, _ptr(offsets), n_v, int(src), _ptr(labels), coarse, ctypes.byref(it), _stream()), "bam_bfs")
+        if by_page:
+            _chk(self.L.bam_bfs_by_page(self.h, _ptr(offsets), n_v, int(src), _ptr(labels), ctypes.byref(it), _stream()), "bam_bfs_by_page")
+        else:
+            _chk(self.L.bam_bfs(self.h, _ptr(offsets), n_v, int(src), _ptr(labels), coarse, ctypes.byref(it), _stream()), "bam_bfs")
         return labels, it.value
 
-    def cc(self, offsets, coarse=1):
+    def cc(self, offsets, coarse=1, by_page=False):
         n_v = offsets.numel() - 1
         labels = torch.empty(n_v, dtype=torch.int64, device=offsets.device)
         it = c_u32(0)
-        _chk(self.L.bam_cc(self.h, _ptr(offsets), n_v, _ptr(labels), coarse, ctypes.byref(it), _stream()), "bam_cc")
+        if by_page:
+            _chk(self.L.bam_cc_by_page(self.h, _ptr(offsets), n_v, _ptr(labels), ctypes.byref(it), _stream()), "bam_cc_by_page")
+        else:
+            _chk(self.L.bam_cc(self.h, _ptr(offsets), n_v, _ptr(labels), coarse, ctypes.byref(it), _stream()), "bam_cc")
         return labels, it.value
 
     def stats(self, reset=True):

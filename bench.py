@@ -244,29 +244,38 @@ def main():
         srcs = oracle.bfs_sources(SEED, off_h, args.bfs_sources)
         del nb
         log("[bench] bfs graph: V=2^%d E=%d cache_pages=%d (%.1fs to build)" % (args.bfs_scale, n_e, cache_pages, time.time() - t0))
-        tot_ms, tot_edges, levels_ok, iters = 0.0, 0, True, []
         nb_u = nb_h.view(np.uint64)
-        for k, src in enumerate(srcs):
-            a, b = event(), event()
-            L.bam_event_record(a, stream)
-            lv, it = ag.bfs(off, int(src), coarse=4)
-            L.bam_event_record(b, stream)
-            ms = elapsed_ms(a, b)
-            lv_h = lv.cpu().numpy().view(np.uint32)
-            if k == 0:                                                  # full-size parity against the serial oracle (timed: the CPU figure)
-                t1 = time.time()
-                ref, rit = oracle.bfs_levels(off_h, nb_u, int(src))
-                cpu_bfs_s = time.time() - t1
-                cpu_bfs_edges = O.bo_bfs_edges_scanned(len(off_h) - 1, off_h, ref)
-                levels_ok = levels_ok and np.array_equal(lv_h, ref) and it == rit
-            tot_edges += O.bo_bfs_edges_scanned(len(off_h) - 1, off_h, lv_h)
-            tot_ms += ms
-            iters.append(it)
-        assert levels_ok and not ctrl.aborted(), "BFS levels differ from the oracle"
-        st = ag.stats()
-        bfs = {"scale": args.bfs_scale, "edges": n_e, "sources": len(srcs), "GTEPS": tot_edges / tot_ms / 1e6,
-               "ms_per_source": tot_ms / len(srcs), "iterations": iters, "read_ios": st["read_io_cnt"],
-               "hit_rate": st["hit_cnt"] / max(st["access_cnt"], 1)}
+        ref = cpu_bfs_s = cpu_bfs_edges = None
+        legs = {}
+        # the edge-page kernel on every source; the reference-shaped kernel (a wave per vertex, bam_ptr per element) on the first two
+        for name, by_page, n_src in (("by_page", True, len(srcs)), ("per_vertex_bam_ptr", False, min(2, len(srcs)))):
+            tot_ms, tot_edges, levels_ok, iters = 0.0, 0, True, []
+            ag.stats()
+            for k, src in enumerate(srcs[:n_src]):
+                a, b = event(), event()
+                L.bam_event_record(a, stream)
+                lv, it = ag.bfs(off, int(src), coarse=4, by_page=by_page)
+                L.bam_event_record(b, stream)
+                ms = elapsed_ms(a, b)
+                lv_h = lv.cpu().numpy().view(np.uint32)
+                if k == 0:                                              # full-size parity against the serial oracle (timed: the CPU figure)
+                    if ref is None:
+                        t1 = time.time()
+                        ref, rit = oracle.bfs_levels(off_h, nb_u, int(src))
+                        cpu_bfs_s = time.time() - t1
+                        cpu_bfs_edges = O.bo_bfs_edges_scanned(len(off_h) - 1, off_h, ref)
+                    levels_ok = levels_ok and np.array_equal(lv_h, ref) and it == rit
+                tot_edges += O.bo_bfs_edges_scanned(len(off_h) - 1, off_h, lv_h)
+                tot_ms += ms
+                iters.append(it)
+            assert levels_ok and not ctrl.aborted(), "BFS levels differ from the oracle (%s)" % name
+            st = ag.stats()
+            legs[name] = {"sources": n_src, "GTEPS": tot_edges / tot_ms / 1e6, "ms_per_source": tot_ms / n_src, "iterations": iters,
+                          "read_ios": st["read_io_cnt"], "MIOPS": st["read_io_cnt"] / tot_ms / 1e3,
+                          "hit_rate": st["hit_cnt"] / max(st["access_cnt"], 1)}
+            log("[bench] bfs %s: %s" % (name, legs[name]))
+        bfs = {"scale": args.bfs_scale, "edges": n_e, "cache_pages": cache_pages, "GTEPS": legs["by_page"]["GTEPS"]}
+        bfs.update(legs)
         # CPU figure: the oracle's uncached in-RAM serial BFS on one core, same graph, first source
         bfs["cpu_serial_GTEPS"] = cpu_bfs_edges / cpu_bfs_s / 1e9
         log("[bench] bfs: %s" % bfs)

@@ -109,6 +109,17 @@ int bam_bfs(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, 
 int bam_cc(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t* d_labels,
            uint32_t coarse, uint32_t* iterations, void* stream);
 
+/* ---- the same two traversals, laid out along the edge array instead of along the vertices ----
+ * Same inputs, same outputs (levels / labels are unique, so they are bit-identical to bam_bfs / bam_cc).  A wave takes
+ * runs of consecutive edge pages, acquires the pages that hold edges of active vertices with one call (their misses
+ * reach the store as one batch of up to 64 commands) and relaxes those vertices' edges from the resident pages.
+ * No counterpart in the reference, whose kernels (benchmarks/bfs/main.cu:658-689, benchmarks/cc/main.cu:595-617) give
+ * one warp to one vertex and so issue one page read at a time per warp.  The array must consist of one range that
+ * starts on a page boundary. */
+int bam_bfs_by_page(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t src, uint32_t* d_labels,
+                    uint32_t* iterations, void* stream);
+int bam_cc_by_page(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t* d_labels, uint32_t* iterations, void* stream);
+
 /* ---- synthetic inputs on the device (no counterpart in the reference, which reads dataset files) ---- */
 int bam_gen_words(uint64_t seed, uint64_t first, uint64_t n, uint64_t* d_out, void* stream);                 /* out[k] = splitmix64(seed, first + k) */
 int bam_gen_mod(uint64_t seed, uint64_t first, uint64_t n, uint64_t modulus, uint64_t scale, uint64_t* d_out, void* stream); /* (splitmix64(seed, first+k) % modulus) * scale */

@@ -272,11 +272,12 @@ def test_reference_sample_graph(bam):
     nb = np.array(g["edges"], dtype=np.uint64)
     r, a = _graph_rig(bam, nb, 64)
     with r:
-        for src, exp in g["bfs"].items():
-            lv, it = a.bfs(_dev(off), int(src))
-            assert lv.cpu().numpy().view(np.uint32).tolist() == exp["levels"] and it == exp["iterations"]
-        lb, it = a.cc(_dev(off))
-        assert _u64(lb).tolist() == g["cc"]["labels"]
+        for by_page in (False, True):
+            for src, exp in g["bfs"].items():
+                lv, it = a.bfs(_dev(off), int(src), by_page=by_page)
+                assert lv.cpu().numpy().view(np.uint32).tolist() == exp["levels"] and it == exp["iterations"]
+            lb, it = a.cc(_dev(off), by_page=by_page)
+            assert _u64(lb).tolist() == g["cc"]["labels"]
 
 
 @pytest.mark.parametrize("scale,cache_pages,coarse", [(10, 4096, 1), (14, 512, 128), (16, 8192, 8)])
@@ -298,6 +299,33 @@ def test_cc_labels_uniform(bam, n_v, n_p, cache_pages, coarse):
     r, a = _graph_rig(bam, nb, cache_pages, n_queues=16, depth=256)
     with r:
         lb, it = a.cc(_dev(off), coarse=coarse)
+        ref, comps = oracle.cc_labels(off, nb)
+        assert np.array_equal(_u64(lb), ref)
+        assert len(np.unique(_u64(lb))) == comps and it >= 1
+        assert not r.c.aborted()
+
+
+@pytest.mark.parametrize("scale,cache_pages", [(10, 4096), (14, 2), (14, 64), (16, 8192), (17, 700)])
+def test_bfs_levels_rmat_by_edge_page(bam, scale, cache_pages):
+    """the edge-page kernel gives the same levels and launch counts; caches from two pages up (what a wave holds is sized from it)"""
+    off, nb = oracle.rmat_csr(SEED, scale)
+    r, a = _graph_rig(bam, nb, cache_pages, n_queues=16, depth=256)
+    with r:
+        doff = _dev(off)
+        for src in oracle.bfs_sources(SEED, off, 3):
+            lv, it = a.bfs(doff, int(src), by_page=True)
+            ref, rit = oracle.bfs_levels(off, nb, int(src))
+            assert np.array_equal(lv.cpu().numpy().view(np.uint32), ref) and it == rit
+        st = a.stats()
+        assert st["read_io_cnt"] > 0 and not r.c.aborted()
+
+
+@pytest.mark.parametrize("n_v,n_p,cache_pages", [(1 << 12, 3000, 256), (1 << 16, 1 << 18, 6), (1 << 14, 1 << 17, 4096)])
+def test_cc_labels_uniform_by_edge_page(bam, n_v, n_p, cache_pages):
+    off, nb = oracle.uniform_csr(SEED, n_v, n_p)
+    r, a = _graph_rig(bam, nb, cache_pages, n_queues=16, depth=256)
+    with r:
+        lb, it = a.cc(_dev(off), by_page=True)
         ref, comps = oracle.cc_labels(off, nb)
         assert np.array_equal(_u64(lb), ref)
         assert len(np.unique(_u64(lb))) == comps and it >= 1
