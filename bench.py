@@ -16,7 +16,8 @@ steps.  On the same JSON line:
                 with plain host clients and the interconnect ceiling for the
                 staged payload, both measured in this run
   block         raw block benchmark (2^22 reads, 128 queue pairs x 1024)
-  bfs           RMAT BFS through bam_ptr (with --bfs-scale)
+  bfs           RMAT-24 BFS through the page cache (with --bfs-scale): the edge-page kernel and the reference-shaped one
+  cc            connected components of a 2^26-vertex uniform graph, 16 GiB of edges behind an 8 GiB cache (with --cc-logv)
 
 Everything is checked against the closed-form oracle while it is measured.
 """
@@ -59,6 +60,7 @@ def main():
     ap.add_argument("--cpu-threads", type=int, default=8)
     ap.add_argument("--bfs-scale", type=int, default=24, help="RMAT scale of the BFS leg (0 = skip)")
     ap.add_argument("--bfs-sources", type=int, default=8)
+    ap.add_argument("--cc-logv", type=int, default=26, help="log2 of the vertex count of the connected-components leg (0 = skip)")
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--skip-block", action="store_true")
     ap.add_argument("--only-hit", action="store_true",
@@ -280,6 +282,48 @@ def main():
         bfs["cpu_serial_GTEPS"] = cpu_bfs_edges / cpu_bfs_s / 1e9
         log("[bench] bfs: %s" % bfs)
         ag.close(); rg.close(); pcg.close()
+        del off, nb_h, nb_u, off_h, lv, lv_h, ref
+
+    # ------------------------------------------------------------------ CC on a uniform random graph (configuration 5)
+    cc = None
+    if args.cc_logv:
+        t0 = time.time()
+        ctrl.close(); target.close()
+        n_v = 1 << args.cc_logv
+        off, nb = gen.uniform_csr(SEED, n_v, 16 * n_v)
+        n_e = nb.numel()
+        ns_bytes = (n_e * 8 + PAGE - 1) // PAGE * PAGE
+        target = bam_amd.Target("/dev/libnvm0", ns_bytes, 512, backing=True, seed=SEED, n_io_threads=args.io_threads)
+        store_words = torch.frombuffer((ctypes.c_char * (n_e * 8)).from_address(target.L.bam_target_backing(target.h)), dtype=torch.int64)
+        store_words.copy_(nb)                                           # device -> the target's host memory
+        torch.cuda.synchronize()
+        ctrl = bam_amd.Controller("/dev/libnvm0", 1, 0, queue_depth=1024, n_queues=128, spin_limit=60_000_000)
+        cache_pages = 1 << 21 if args.cc_logv == 26 else max(1 << 14, ns_bytes // PAGE // 2)        # 8 GiB at full size
+        pcc, rc_, ac = make_array(ctrl, n_e, PAGE, cache_pages)
+        log("[bench] cc graph: V=2^%d E=%d (%.1f GiB) cache_pages=%d (%.1fs to build)" % (args.cc_logv, n_e, n_e * 8 / 2**30, cache_pages, time.time() - t0))
+        a, b = event(), event()
+        L.bam_event_record(a, stream)
+        lb, it = ac.cc(off, by_page=True)
+        L.bam_event_record(b, stream)
+        ms = elapsed_ms(a, b)
+        st = ac.stats()
+        # full-size parity: the labels are the unique fixed point of min-label propagation with label[v] <= v; the same
+        # fixed point computed independently with torch gathers and scatter-min over the in-HBM copy of the graph
+        src = torch.repeat_interleave(torch.arange(n_v, device=dev), off[1:] - off[:-1])
+        ref = torch.arange(n_v, device=dev)
+        while True:
+            new = ref.clone()
+            new.scatter_reduce_(0, nb, ref[src], "amin")
+            if torch.equal(new, ref):
+                break
+            ref = new
+        assert torch.equal(ref, lb) and not ctrl.aborted(), "CC labels differ from the fixed point"
+        cc = {"log2_vertices": args.cc_logv, "edges": n_e, "cache_pages": cache_pages, "ms": ms, "iterations": it,
+              "GTEPS": it * n_e / ms / 1e6, "read_ios": st["read_io_cnt"], "MIOPS": st["read_io_cnt"] / ms / 1e3,
+              "components": int(torch.unique(lb).numel()), "kernel": "by_page"}
+        log("[bench] cc: %s" % cc)
+        del src, ref, new, nb, off, lb, store_words
+        ac.close(); rc_.close(); pcc.close()
 
     ctrl.close(); target.close()
 
@@ -310,7 +354,7 @@ def main():
                    "seed": SEED, "block_size": args.block},
         "reads_per_s": args.steps * N_READS / ms_total * 1e3,
         "hit_rate": cfg2_hit_rate,
-        "roofline": roofline, "cpu_baseline": cpu, "store": store, "hit_gather": gather_hit, "block": block, "bfs": bfs,
+        "roofline": roofline, "cpu_baseline": cpu, "store": store, "hit_gather": gather_hit, "block": block, "bfs": bfs, "cc": cc,
     }
     print(json.dumps(out), flush=True)
 

@@ -36,6 +36,10 @@
 
 namespace bam {
 
+#ifndef BAM_CQ_IDLE_TICKS
+#define BAM_CQ_IDLE_TICKS 200u          /* 100 MHz ticks between looks at an idle completion ring */
+#endif
+
 struct spin_t { uint32_t n = 0, slp = 1; uint64_t t0 = 0; };
 
 /*
@@ -127,13 +131,13 @@ __device__ __forceinline__ bool try_drain_group(nvm_queue_t* cq, nvm_queue_t* sq
         /* the word holds the time of the next look (low 32 bits of the clock): wait only while that lies within
          * the next two microseconds, so that a stale or never-written value can never hold anybody up */
         const uint32_t ahead = ld_relaxed(&cq->tail) - (uint32_t)wall_clock64();
-        if (ahead - 1u >= 200u && ld_relaxed(&cq->head_lock) == UNLOCKED &&
+        if (ahead - 1u >= BAM_CQ_IDLE_TICKS && ld_relaxed(&cq->head_lock) == UNLOCKED &&
             __hip_atomic_exchange(&cq->head_lock, (uint32_t)LOCKED, __ATOMIC_ACQUIRE, BAM_AGENT) == UNLOCKED) {
             const uint32_t h = ld_relaxed(&cq->head);
             const uint32_t dw3 = ld_acquire_sys(&((nvm_cpl_t*)cq->vaddr)[h & cq->qs_minus_1].dword[3]);
             if (((dw3 >> 16) & 1u) == ((~(h >> cq->qs_log2)) & 1u)) got = 1;
             else {
-                st_relaxed(&cq->tail, (uint32_t)wall_clock64() + 200u);      /* nothing new: next look in 2 us */
+                st_relaxed(&cq->tail, (uint32_t)wall_clock64() + BAM_CQ_IDLE_TICKS);      /* nothing new: leave the ring alone for a while */
                 st_release(&cq->head_lock, (uint32_t)UNLOCKED);
             }
         }
