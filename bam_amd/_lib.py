@@ -43,6 +43,8 @@ SIGNATURES = {
     "bam_block_checksum": (c_int, [c_vp, c_u64, c_u32, c_vp, c_vp]),
     "bam_bfs": (c_int, [c_vp, c_vp, c_u64, c_u64, c_vp, c_u32, P(c_u32), c_vp]),
     "bam_cc": (c_int, [c_vp, c_vp, c_u64, c_vp, c_u32, P(c_u32), c_vp]),
+    "bam_array_read_via": (c_int, [c_vp, c_int, c_u64, c_vp, c_u64, c_u32, c_vp, c_vp]),
+    "bam_block_io_async": (c_int, [c_vp, c_vp, c_u64, c_u32, c_u32, c_vp, c_u32, c_vp]),
     "bam_bfs_by_page": (c_int, [c_vp, c_vp, c_u64, c_u64, c_vp, P(c_u32), c_vp]),
     "bam_cc_by_page": (c_int, [c_vp, c_vp, c_u64, c_vp, P(c_u32), c_vp]),
     "bam_gen_words": (c_int, [c_u64, c_u64, c_u64, c_vp, c_vp]),

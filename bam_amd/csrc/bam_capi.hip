@@ -96,6 +96,59 @@ __global__ void k_array_read(array_d_t<uint64_t>* dr, uint64_t n_reqs, const uin
     block_accumulate(sum, v);
 }
 
+/*
+ * The same read pattern through the other access routes of array_d_t:
+ *   1  get_raw / release_raw            (the raw page handed out, lanes on one page share the references)
+ *   2  get_page_gid + acquire_page_ + release_page   (per-thread, no coalescing)
+ *   3  acquire_page / release_page      (coalesced, page kept while in use)
+ *   4  bam_ptr                          (per-thread cached page)
+ *   5  memcpy                           (wave-cooperative copy of up to `span` elements starting at the wave's index;
+ *                                        one request per wave, the copied elements are summed)
+ */
+template <int API>
+__global__ void k_array_read_via(array_d_t<uint64_t>* dr, uint64_t n_reqs, const uint64_t* assignment, uint64_t span, uint64_t* scratch, unsigned long long* sum)
+{
+    const uint64_t tid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    uint64_t v = 0;
+    if (API == 5) {
+        const uint64_t wave = tid / BAM_WAVE_SIZE;
+        if (wave < n_reqs) {
+            const uint64_t idx = assignment ? assignment[wave] : wave * span;
+            uint64_t* dst = scratch + wave * span;
+            for (uint64_t k = bam::lane(); k < span; k += BAM_WAVE_SIZE) dst[k] = 0;
+            dr->memcpy(idx, span, dst);
+            for (uint64_t k = bam::lane(); k < span; k += BAM_WAVE_SIZE) v += dst[k];
+        }
+    } else if (tid < n_reqs) {
+        const uint64_t idx = assignment ? assignment[tid] : tid * span;
+        if (API == 1) {
+            returned_cache_page_t<uint64_t> pg = dr->get_raw(idx);
+            v = bam::ld_payload(pg.addr + pg.offset);
+            dr->release_raw(idx);
+        } else if (API == 2) {
+            range_d_t<uint64_t>* r;
+            size_t page, gid, start, end;
+            data_page_t* dp;
+            dr->get_page_gid(idx, r, page, gid);
+            const uint64_t* base = (const uint64_t*)dr->acquire_page_(idx, dp, start, end, r, page);
+            if (base && idx >= start && idx < end && gid == r->get_global_address(page)) v = bam::ld_payload(base + (idx - start));
+            if (r) r->release_page(page, 1, false);
+        } else if (API == 3) {
+            size_t start, end;
+            data_page_t* dp;
+            int64_t r;
+            const uint64_t* base = (const uint64_t*)dr->acquire_page(idx, dp, start, end, r);
+            if (base) v = bam::ld_payload(base + (idx - start));
+            dr->release_page(dp, r, idx, false);
+        } else {
+            bam_ptr<uint64_t> ptr(dr);
+            const bam_ptr<uint64_t>& cptr = ptr;
+            v = cptr[idx];
+        }
+    }
+    block_accumulate(sum, v);
+}
+
 __global__ void k_array_write(array_d_t<uint64_t>* dr, uint64_t n_reqs, const uint64_t* assignment, uint64_t stride, const uint64_t* values)
 {
     const uint64_t tid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -180,6 +233,25 @@ __global__ void k_block_io(Controller** ctrls, page_cache_d_t* pc, uint32_t req_
         if (write) write_data(pc, qp, start_block, n_blocks, tid);
         else read_data(pc, qp, start_block, n_blocks, tid);
     }
+}
+
+/*
+ * Raw block reads with several commands in flight per thread (benchmarks/iodepth-block/main.cu:97-140): thread t
+ * submits its `depth` commands with access_data_async (command k of thread t reads LBA lbas[t * depth + k] into slot
+ * t * depth + k), then collects them with poll_async.  Wave w uses queue pair w mod n_qps.
+ */
+template <int DEPTH>
+__global__ void k_block_io_async(Controller** ctrls, page_cache_d_t* pc, uint32_t req_size, uint64_t n_threads, const uint64_t* lbas)
+{
+    const uint64_t tid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (tid >= n_threads) return;
+    QueuePair* qp = ctrls[0]->d_qps + (tid / BAM_WAVE_SIZE) % ctrls[0]->n_qps;
+    const uint64_t n_blocks = req_size >> qp->block_size_log;
+    uint16_t cids[DEPTH], poss[DEPTH];
+#pragma unroll
+    for (int k = 0; k < DEPTH; k++) access_data_async(pc, qp, lbas[tid * DEPTH + k], n_blocks, tid * DEPTH + k, NVM_IO_READ, cids + k, poss + k);
+#pragma unroll
+    for (int k = 0; k < DEPTH; k++) poll_async(qp, cids[k], poss[k]);
 }
 
 __global__ void k_block_checksum(page_cache_d_t* pc, uint64_t n_slots, uint32_t req_bytes, uint64_t* out)
@@ -659,6 +731,35 @@ int bam_array_read(bam_array_t* a, uint64_t n_reqs, const uint64_t* d_assignment
     BAM_API_END
 }
 
+int bam_array_read_via(bam_array_t* a, int api, uint64_t n_reqs, const uint64_t* d_assignment, uint64_t span, uint32_t block_size,
+                       uint64_t* d_sum, void* stream)
+{
+    if (!a || !d_sum) return fail(EINVAL, "bam_array_read_via: null argument");
+    if (api < 1 || api > 5) return fail(EINVAL, "bam_array_read_via: api must be 1..5");
+    if (!block_size || block_size % BAM_WAVE_SIZE || block_size > 1024) return fail(EINVAL, "bam_array_read_via: block size must be a multiple of 64, at most 1024");
+    if (!span) return fail(EINVAL, "bam_array_read_via: span must be at least 1");
+    if (!n_reqs) return 0;
+    BAM_API_BEGIN
+    hipStream_t st = (hipStream_t)stream;
+    array_d_t<uint64_t>* d = a->a->d_array_ptr;
+    unsigned long long* s = (unsigned long long*)a->partials.get();
+    const dim3 grid(blocks_for(api == 5 ? n_reqs * BAM_WAVE_SIZE : n_reqs, block_size)), block(block_size);
+    BufferPtr scratch;
+    if (api == 5) scratch = createBuffer(n_reqs * span * sizeof(uint64_t), 0);
+    uint64_t* sc = (uint64_t*)scratch.get();
+    switch (api) {
+    case 1: hipLaunchKernelGGL(k_array_read_via<1>, grid, block, 0, st, d, n_reqs, d_assignment, span, sc, s); break;
+    case 2: hipLaunchKernelGGL(k_array_read_via<2>, grid, block, 0, st, d, n_reqs, d_assignment, span, sc, s); break;
+    case 3: hipLaunchKernelGGL(k_array_read_via<3>, grid, block, 0, st, d, n_reqs, d_assignment, span, sc, s); break;
+    case 4: hipLaunchKernelGGL(k_array_read_via<4>, grid, block, 0, st, d, n_reqs, d_assignment, span, sc, s); break;
+    default: hipLaunchKernelGGL(k_array_read_via<5>, grid, block, 0, st, d, n_reqs, d_assignment, span, sc, s); break;
+    }
+    hipLaunchKernelGGL(k_fold_partials, dim3(1), dim3(1024), 0, st, s, (unsigned long long*)d_sum);
+    hip_err_chk(hipGetLastError());
+    if (api == 5) hip_err_chk(hipStreamSynchronize(st));       /* the scratch buffer goes away with this call */
+    BAM_API_END
+}
+
 int bam_array_write(bam_array_t* a, uint64_t n_reqs, const uint64_t* d_assignment, uint64_t stride, const uint64_t* d_values,
                     uint32_t block_size, void* stream)
 {
@@ -702,6 +803,36 @@ int bam_block_io(bam_ctrl_t* c, bam_page_cache_t* pc, uint64_t n_reqs, uint32_t 
     BAM_API_BEGIN
     hipLaunchKernelGGL(k_block_io, dim3(blocks_for(n_reqs, block_size)), dim3(block_size), 0, (hipStream_t)stream,
                        pc->pc->pdt.d_ctrls, pc->pc->d_pc_ptr, req_bytes, n_reqs, d_lbas, write, queue_policy);
+    hip_err_chk(hipGetLastError());
+    BAM_API_END
+}
+
+int bam_block_io_async(bam_ctrl_t* c, bam_page_cache_t* pc, uint64_t n_threads, uint32_t depth, uint32_t req_bytes, const uint64_t* d_lbas,
+                       uint32_t block_size, void* stream)
+{
+    if (!c || !pc || !d_lbas) return fail(EINVAL, "bam_block_io_async: null argument");
+    if (!block_size || block_size % BAM_WAVE_SIZE || block_size > 1024) return fail(EINVAL, "bam_block_io_async: block size must be a multiple of 64, at most 1024");
+    if (depth != 1 && depth != 2 && depth != 4 && depth != 8) return fail(EINVAL, "bam_block_io_async: depth must be 1, 2, 4 or 8");
+    if (n_threads * depth > pc->pc->pdt.n_pages) return fail(EINVAL, "bam_block_io_async: needs one cache page per command");
+    if (!req_bytes || req_bytes % c->c->blk_size || req_bytes > pc->pc->pdt.page_size) return fail(EINVAL, "bam_block_io_async: request size must be a multiple of the block size and fit a page");
+    /* a wave holds `depth` blocks of command ids of its queue pair until it has polled: all waves that can be in
+     * flight on one queue pair together must fit its blocks, or they would wait for each other's */
+    const uint64_t n_waves = (n_threads + BAM_WAVE_SIZE - 1) / BAM_WAVE_SIZE;
+    const uint64_t blocks_per_qp = (c->c->h_qps[0]->sq.cid_mask + 1u) / 64;
+    if ((n_waves + c->c->n_qps - 1) / c->c->n_qps * depth > blocks_per_qp)
+        return fail(EINVAL, "bam_block_io_async: more commands in flight per queue pair than it has command ids (waves per queue pair x depth x 64)");
+    if (!n_threads) return 0;
+    BAM_API_BEGIN
+    const dim3 grid(blocks_for(n_threads, block_size)), block(block_size);
+    hipStream_t st = (hipStream_t)stream;
+    Controller** dc = pc->pc->pdt.d_ctrls;
+    page_cache_d_t* dp = pc->pc->d_pc_ptr;
+    switch (depth) {
+    case 1: hipLaunchKernelGGL(k_block_io_async<1>, grid, block, 0, st, dc, dp, req_bytes, n_threads, d_lbas); break;
+    case 2: hipLaunchKernelGGL(k_block_io_async<2>, grid, block, 0, st, dc, dp, req_bytes, n_threads, d_lbas); break;
+    case 4: hipLaunchKernelGGL(k_block_io_async<4>, grid, block, 0, st, dc, dp, req_bytes, n_threads, d_lbas); break;
+    default: hipLaunchKernelGGL(k_block_io_async<8>, grid, block, 0, st, dc, dp, req_bytes, n_threads, d_lbas); break;
+    }
     hip_err_chk(hipGetLastError());
     BAM_API_END
 }

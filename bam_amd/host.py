@@ -134,6 +134,10 @@ class PageCache:
         _chk(self.L.bam_block_io(self.ctrl.h, self.h, n_reqs, req_bytes, _ptr(lbas), int(write), queue_policy, block_size, _stream()),
              "bam_block_io")
 
+    def block_io_async(self, n_threads, depth, req_bytes, lbas, block_size=64):
+        """`depth` commands in flight per thread (benchmarks/iodepth-block/main.cu:97-140)."""
+        _chk(self.L.bam_block_io_async(self.ctrl.h, self.h, n_threads, depth, req_bytes, _ptr(lbas), block_size, _stream()), "bam_block_io_async")
+
     def block_checksums(self, n_slots, req_bytes):
         out = torch.empty(n_slots, dtype=torch.int64, device=f"cuda:{self.device}")
         _chk(self.L.bam_block_checksum(self.h, n_slots, req_bytes, _ptr(out), _stream()), "bam_block_checksum")
@@ -193,6 +197,13 @@ class Array:
         """Sum (mod 2^64) of the elements read: thread t reads assignment[t] (or t * stride)."""
         s = self._sum_buf()
         self.read_async(n_reqs, s, assignment, stride, reqs_per_thread, block_size)
+        return int(s.item()) & MASK64
+
+    def read_via(self, api, n_reqs, assignment=None, span=1, block_size=64):
+        """The read pattern through another access route of array_d_t (1 get_raw, 2 acquire_page_, 3 acquire_page,
+        4 bam_ptr, 5 wave memcpy of up to `span` elements per request); sum of what was read."""
+        s = self._sum_buf()
+        _chk(self.L.bam_array_read_via(self.h, api, n_reqs, _ptr(assignment), span, block_size, _ptr(s), _stream()), "bam_array_read_via")
         return int(s.item()) & MASK64
 
     def write(self, n_reqs, values, assignment=None, stride=1, block_size=64):

@@ -78,6 +78,12 @@ int bam_array_stats(bam_array_t* a, uint64_t* out, int reset);
  * (mod 2^64).  The reference discards the values; the checksum is what makes the result checkable. */
 int bam_array_read(bam_array_t* a, uint64_t n_reqs, const uint64_t* d_assignment, uint64_t stride, uint64_t reqs_per_thread,
                    uint32_t block_size, uint64_t* d_sum, void* stream);
+/* The read pattern of bam_array_read (one thread per request, element d_assignment[t] or t * span) through the other
+ * access routes of array_d_t (include/page_cache.h:1240-1716, 414-485): api 1 get_raw/release_raw, 2 get_page_gid +
+ * acquire_page_ + release_page, 3 acquire_page/release_page, 4 bam_ptr, 5 memcpy (one request per wave: up to `span`
+ * elements starting at the wave's index, clipped to the page, are copied out and summed). */
+int bam_array_read_via(bam_array_t* a, int api, uint64_t n_reqs, const uint64_t* d_assignment, uint64_t span, uint32_t block_size,
+                       uint64_t* d_sum, void* stream);
 /* same request pattern through array_d_t::operator() (seq_write): element <- d_values[t] */
 int bam_array_write(bam_array_t* a, uint64_t n_reqs, const uint64_t* d_assignment, uint64_t stride, const uint64_t* d_values,
                     uint32_t block_size, void* stream);
@@ -96,6 +102,12 @@ int bam_cache_stream(bam_array_t* a, uint64_t n_waves, uint64_t n_pages_per_wave
  * queue_policy 0: queue = compute unit % n_qps (sequential kernel), 1: round-robin counter (random kernel). */
 int bam_block_io(bam_ctrl_t* c, bam_page_cache_t* pc, uint64_t n_reqs, uint32_t req_bytes, const uint64_t* d_lbas, int write,
                  int queue_policy, uint32_t block_size, void* stream);
+/* raw block reads with `depth` (1, 2, 4, 8) commands in flight per thread through access_data_async / poll_async
+ * (benchmarks/iodepth-block/main.cu:97-140): command k of thread t reads LBA d_lbas[t * depth + k] into slot
+ * t * depth + k; wave w uses queue pair w mod n_qps.  The waves of one launch that share a queue pair must fit its
+ * command ids (waves per queue pair x depth x 64 <= queue depth), checked here. */
+int bam_block_io_async(bam_ctrl_t* c, bam_page_cache_t* pc, uint64_t n_threads, uint32_t depth, uint32_t req_bytes, const uint64_t* d_lbas,
+                       uint32_t block_size, void* stream);
 /* sum of the 64-bit words of the first req_bytes of slots 0..n-1, one sum per slot */
 int bam_block_checksum(bam_page_cache_t* pc, uint64_t n_slots, uint32_t req_bytes, uint64_t* d_out, void* stream);
 

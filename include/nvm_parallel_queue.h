@@ -95,6 +95,7 @@ __device__ __forceinline__ uint32_t get_cid_group(nvm_queue_t* sq)
         while (((ld_relaxed(&sq->pos_locks[b].val) - (t >> shift)) & turn_mask) != 0)
             if (spin_giveup(sq, sp)) break;
         fence_acquire_agent();
+        st_relaxed(&sq->head_mark[b].val, popc(act));       /* ids of this block still out */
         base = b << 6;
     }
     base = bcast(base, leader);
@@ -103,12 +104,27 @@ __device__ __forceinline__ uint32_t get_cid_group(nvm_queue_t* sq)
     return id;
 }
 
-/* give the group's block of command ids back (every lane of the group that called get_cid_group) */
+/*
+ * Give command ids back.  The lanes that took a block together may return
+ * their ids in one call or in several (the asynchronous entry points are
+ * called thread by thread); the block's turn moves on when its last id is in.
+ */
 __device__ __forceinline__ void put_cid_group(nvm_queue_t* sq, uint32_t id)
 {
-    const uint64_t act = active_mask();
     st_relaxed(&sq->cid[id].val, (uint32_t)UNLOCKED);
-    if (lane() == first_lane(act)) __hip_atomic_fetch_add(&sq->pos_locks[id >> 6].val, 1u, __ATOMIC_RELEASE, BAM_AGENT);   /* next turn */
+    const uint32_t b = id >> 6;
+    for (bool done = false; !done;) {
+        const uint32_t cur = first(b);
+        if (cur == b) {
+            const uint64_t grp = active_mask();
+            if (lane() == first_lane(grp)) {
+                const uint32_t k = popc(grp);
+                if (__hip_atomic_fetch_add(&sq->head_mark[cur].val, 0u - k, __ATOMIC_RELEASE, BAM_AGENT) == k)
+                    __hip_atomic_fetch_add(&sq->pos_locks[cur].val, 1u, __ATOMIC_RELEASE, BAM_AGENT);   /* next turn */
+            }
+            done = true;
+        }
+    }
 }
 
 __device__ __forceinline__ void cq_drain_group(nvm_queue_t* cq, nvm_queue_t* sq, uint64_t act);

@@ -80,7 +80,7 @@ typedef struct
     uint32_t n_errors;   uint8_t pad5[56];  /* CQ: completions seen with a non-zero status */
 
     padded_struct*          tickets;        /* SQ [qs]: 2*lap = free for lap, odd = submitted */
-    padded_struct*          head_mark;      /* unused by the wave-cooperative engine (kept for layout parity) */
+    padded_struct*          head_mark;      /* SQ [n_cids / 64]: command ids of the block still out (the reference marks consumed CQ entries here) */
     padded_struct*          tail_mark;      /* SQ [qs]: 1 = written, waiting for the tail sweep */
     padded_struct*          cid;            /* SQ [n_cids]: per command id, 0 idle, 1 in flight, 3 in flight + completed */
     padded_struct*          pos_locks;      /* SQ [n_cids / 64]: command ids are handed out to a wave in blocks of 64; turn counter of each block */

@@ -182,16 +182,18 @@ __device__ __forceinline__ void copy_pages(uint8_t* dst, const uint8_t* src, uin
 }
 
 /*
- * One command per active lane on queue pair `qp` (wave-uniform): allocate ids,
- * build and submit the entries as one batch, wait for all completions, move
- * staged payload, recycle ids.  `pc_entry` is the cache slot the data belongs to.
+ * One command per active lane on queue pair `qp` (wave-uniform), first half:
+ * allocate ids, build the entries and submit them as one batch.  `pc_entry`
+ * is the cache slot the data belongs to.  Returns the lane's command id;
+ * `stage` is its staging page (NULL when the controller addresses the slot
+ * itself) and `pos` the submission-queue slot its entry went to.
  */
-__device__ __forceinline__ void io_group(page_cache_d_t* pc, QueuePair* qp, uint64_t lba, uint32_t n_blocks, uint64_t pc_entry, uint8_t opcode)
+__device__ __forceinline__ uint32_t io_submit_group(page_cache_d_t* pc, QueuePair* qp, uint64_t lba, uint32_t n_blocks, uint64_t pc_entry, uint8_t opcode,
+                                                    uint8_t*& stage, uint32_t& pos)
 {
     const uint64_t act = active_mask();
     const uint32_t n = popc(act), rank = rank_in(act);
     const uint32_t bytes = n_blocks << qp->block_size_log;
-    uint8_t* slot_addr = pc->base_addr + pc_entry * pc->page_size;
 #ifdef BAM_PROFILE
     const uint64_t pt0 = wall_clock64();
 #endif
@@ -200,13 +202,13 @@ __device__ __forceinline__ void io_group(page_cache_d_t* pc, QueuePair* qp, uint
     const uint64_t pt1 = wall_clock64();
 #endif
     uint64_t prp1, prp2 = 0;
-    uint8_t* stage = nullptr;
+    stage = nullptr;
     if (qp->stage) {
         stage = qp->stage + (size_t)cid * qp->stage_stride;
         prp1 = qp->stage_ioaddr + (uint64_t)cid * qp->stage_stride;
         if (bytes > qp->pageSize) prp2 = prp1 + qp->pageSize;         /* staging pages are contiguous: second controller page */
         if (opcode == NVM_IO_WRITE) {
-            copy_pages(stage, slot_addr, bytes, act, n, rank);
+            copy_pages(stage, pc->base_addr + pc_entry * pc->page_size, bytes, act, n, rank);
             fence_release_sys();
         }
     } else {
@@ -219,7 +221,24 @@ __device__ __forceinline__ void io_group(page_cache_d_t* pc, QueuePair* qp, uint
     nvm_cmd_header(&cmd, (uint16_t)cid, opcode, qp->nvmNamespace);
     nvm_cmd_data_ptr(&cmd, prp1, prp2);
     nvm_cmd_rw_blks(&cmd, lba, (uint16_t)n_blocks);
-    sq_enqueue_group(&qp->sq, &cmd);
+    pos = sq_enqueue_group(&qp->sq, &cmd);
+#ifdef BAM_PROFILE
+    if (pc->prof && rank == 0) {
+        const uint64_t pt2 = wall_clock64();
+        atomicAdd(&pc->prof[0], 1ull); atomicAdd(&pc->prof[1], (unsigned long long)n);
+        atomicAdd(&pc->prof[2], pt1 - pt0); atomicAdd(&pc->prof[3], pt2 - pt1);
+    }
+#endif
+    return cid;
+}
+
+/* the whole of one batch: submit, wait for all completions, move staged payload, recycle ids */
+__device__ __forceinline__ void io_group(page_cache_d_t* pc, QueuePair* qp, uint64_t lba, uint32_t n_blocks, uint64_t pc_entry, uint8_t opcode)
+{
+    const uint64_t act = active_mask();
+    uint8_t* stage;
+    uint32_t pos;
+    const uint32_t cid = io_submit_group(pc, qp, lba, n_blocks, pc_entry, opcode, stage, pos);
 #ifdef BAM_PROFILE
     const uint64_t pt2 = wall_clock64();
 #endif
@@ -227,14 +246,11 @@ __device__ __forceinline__ void io_group(page_cache_d_t* pc, QueuePair* qp, uint
 #ifdef BAM_PROFILE
     const uint64_t pt3 = wall_clock64();
 #endif
-    if (stage && opcode == NVM_IO_READ) copy_pages(slot_addr, stage, bytes, act, n, rank);
+    if (stage && opcode == NVM_IO_READ)
+        copy_pages(pc->base_addr + pc_entry * pc->page_size, stage, n_blocks << qp->block_size_log, act, popc(act), rank_in(act));
     put_cid_group(&qp->sq, cid);
 #ifdef BAM_PROFILE
-    if (pc->prof && rank == 0) {
-        const uint64_t pt4 = wall_clock64();
-        atomicAdd(&pc->prof[0], 1ull); atomicAdd(&pc->prof[1], (unsigned long long)n);
-        atomicAdd(&pc->prof[2], pt1 - pt0); atomicAdd(&pc->prof[3], pt2 - pt1); atomicAdd(&pc->prof[4], pt3 - pt2); atomicAdd(&pc->prof[5], pt4 - pt3);
-    }
+    if (pc->prof && lane() == first_lane(act)) { atomicAdd(&pc->prof[4], pt3 - pt2); atomicAdd(&pc->prof[5], wall_clock64() - pt3); }
 #endif
 }
 
@@ -257,6 +273,52 @@ inline __device__ void read_data(page_cache_d_t* pc, QueuePair* qp, const uint64
 inline __device__ void write_data(page_cache_d_t* pc, QueuePair* qp, const uint64_t starting_lba, const uint64_t n_blocks, const unsigned long long pc_entry)
 {
     access_data(pc, qp, starting_lba, n_blocks, pc_entry, NVM_IO_WRITE);
+}
+
+/*
+ * The two halves of access_data as separate calls (include/page_cache.h:1930-1959 of the reference): submit now,
+ * collect later, so that a thread can keep several commands in flight.  A staged read leaves its destination with
+ * the queue pair under its command id; poll_async moves the payload once the completion is in.  The threads of a
+ * wave that submit together may poll together or one by one.
+ */
+inline __device__ void access_data_async(page_cache_d_t* pc, QueuePair* qp, const uint64_t starting_lba, const uint64_t n_blocks, const unsigned long long pc_entry,
+                                         const uint8_t opcode, uint16_t* cid, uint16_t* sq_pos)
+{
+    for (bool done = false; !done;) {
+        QueuePair* cur = (QueuePair*)bam::first((uint64_t)qp);
+        page_cache_d_t* cpc = (page_cache_d_t*)bam::first((uint64_t)pc);
+        if (cur == qp && cpc == pc) {
+            uint8_t* stage;
+            uint32_t pos;
+            const uint32_t id = bam::io_submit_group(cpc, cur, starting_lba, (uint32_t)n_blocks, pc_entry, opcode, stage, pos);
+            if (stage) {
+                cur->async_dst[id] = opcode == NVM_IO_READ ? (uint64_t)(cpc->base_addr + pc_entry * cpc->page_size) : 0;
+                cur->async_len[id] = (uint32_t)n_blocks << cur->block_size_log;
+            }
+            *cid = (uint16_t)id;
+            *sq_pos = (uint16_t)pos;
+            done = true;
+        }
+    }
+}
+
+inline __device__ void poll_async(QueuePair* qp, uint16_t cid, uint16_t sq_pos)
+{
+    (void)sq_pos;
+    for (bool done = false; !done;) {
+        QueuePair* cur = (QueuePair*)bam::first((uint64_t)qp);
+        if (cur == qp) {
+            const uint64_t act = bam::active_mask();
+            bam::cq_wait_group(&cur->cq, &cur->sq, cid);
+            uint8_t* dst = nullptr;
+            uint32_t len = 0;
+            if (cur->stage) { dst = (uint8_t*)cur->async_dst[cid]; len = cur->async_len[cid]; }
+            if (bam::ballot(dst != nullptr))
+                bam::copy_pages(dst, cur->stage + (size_t)cid * cur->stage_stride, dst ? len : 0, act, bam::popc(act), bam::rank_in(act));
+            bam::put_cid_group(&cur->sq, cid);
+            done = true;
+        }
+    }
 }
 
 /* ------------------------------------------------------------------ */
@@ -810,6 +872,90 @@ struct array_d_t {
         bam::range_view<T> v;
         v.load(d_ranges + r);
         v.release(v.page_of(i), wrote);
+    }
+
+    /* range, page within the range and global page address of element i (reference :1240-1253); r_ = NULL if no range holds i */
+    __forceinline__ __device__ void get_page_gid(const uint64_t i, range_d_t<T>*& r_, size_t& pg, size_t& gid) const
+    {
+        const int64_t r = find_range(i);
+        r_ = nullptr;
+        if (r == -1) return;
+        r_ = d_ranges + r;
+        pg = r_->get_page(i);
+        gid = r_->get_global_address(pg);
+    }
+
+    /*
+     * Per-thread acquire of `page` of range `r_`, no coalescing across lanes (reference :1443-1468): one reference
+     * per calling lane.  Returns the address of the page's payload, its descriptor in `page_` and the element
+     * window [start, end) it covers.  The reference indexes the descriptor table by the cache slot here
+     * (`&r_->pages[base_master]`); this returns the descriptor of the page, which is what its callers release.
+     */
+    __forceinline__ __device__ void* acquire_page_(const size_t i, data_page_t*& page_, size_t& start, size_t& end, range_d_t<T>* r_, const size_t page) const
+    {
+        (void)i;
+        page_ = nullptr;
+        if (!r_) return nullptr;
+        const uint32_t slot = (uint32_t)r_->acquire_page(page, 1, false, 0, bam::wave_slot_hash());
+        page_ = &r_->pages[page];
+        bam::range_view<T> v;
+        v.load(r_);
+        v.window(page, start, end);
+        return (void*)(v.slot_addr(slot) + (v.byte_of(start) & (v.page_size - 1)));
+    }
+
+    /*
+     * The page holding element i, handed out raw (reference :1370-1403): address of the page's payload, its size
+     * in elements and the position of element i in it.  The references of the lanes that ask for the same page
+     * are taken with one atomic and stay taken until release_raw(i) is called by the same lanes.
+     */
+    __forceinline__ __device__ returned_cache_page_t<T> get_raw(const size_t i) const
+    {
+        returned_cache_page_t<T> ret;
+        ret.addr = nullptr; ret.size = 0; ret.offset = 0;
+        bam::range_view<T> v;
+        if (!view_of(i, v)) return ret;
+        const uint64_t byte = v.byte_of(i);
+        uint32_t slot = 0;
+        auto keep = [&](uint32_t s_) { slot = s_; return false; };
+        v.acquire(byte >> v.page_size_log, false, keep, keep);
+        v.template flush_stats<false>();
+        ret.addr = (T*)v.slot_addr(slot);
+        ret.size = v.page_size / sizeof(T);
+        ret.offset = (uint32_t)((byte & (v.page_size - 1)) / sizeof(T));
+        return ret;
+    }
+
+    __forceinline__ __device__ void release_raw(const size_t i) const
+    {
+        bam::range_view<T> v;
+        if (!view_of(i, v)) return;
+        v.release(v.page_of(i), false);
+    }
+
+    /*
+     * Wave-cooperative copy out of the cache: the active lanes, all called with the same i, copy `count` elements
+     * starting at element i to `dest`, clipped to the end of the page that holds i.  (The reference's version,
+     * :1256-1316, ignores `count` and always copies the first 512 bytes of the page.)
+     */
+    __forceinline__ __device__ void memcpy(const uint64_t i, const uint64_t count, T* dest) const
+    {
+        bam::range_view<T> v;
+        if (!view_of(i, v)) return;
+        const uint64_t byte = v.byte_of(i);
+        const uint64_t page = byte >> v.page_size_log;
+        size_t start, end;
+        v.window(page, start, end);
+        const uint64_t n = i + count < end ? count : end - i;
+        const uint64_t act = bam::active_mask();
+        const uint32_t lanes = bam::popc(act), rank = bam::rank_in(act);
+        auto copy = [&](uint32_t slot) {
+            const T* src = (const T*)(v.slot_addr(slot) + (byte & (v.page_size - 1)));
+            for (uint64_t k = rank; k < n; k += lanes) dest[k] = bam::ld_payload(src + k);
+            return true;
+        };
+        v.acquire(page, false, copy, copy);
+        v.template flush_stats<false>();
     }
 };
 

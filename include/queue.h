@@ -40,11 +40,13 @@ struct QueuePair
     uint8_t*            stage;          /* staging window (NULL: PRPs address device memory directly) */
     uint64_t            stage_ioaddr;
     uint32_t            stage_stride;   /* bytes per command id */
+    uint64_t*           async_dst;      /* [n_cids] staged asynchronous reads: destination address, 0 = none */
+    uint32_t*           async_len;      /* [n_cids] and length in bytes */
 
     /* host-side owners; a raw pointer keeps the struct trivially copyable to the device */
     struct Owners {
         DmaPtr sq_mem, cq_mem, stage_mem;
-        BufferPtr sq_tickets, sq_tail_mark, sq_cid, sq_cid_blocks;
+        BufferPtr sq_tickets, sq_tail_mark, sq_cid, sq_cid_blocks, sq_cid_left, async_dst, async_len;
     };
     Owners*             own;
     nvm_aq_ref          aq;
@@ -93,12 +95,14 @@ struct QueuePair
         sq.cid_mask = n_cids - 1;
         own->sq_cid_blocks = createBuffer((n_cids / 64) * sizeof(padded_struct), hipDevice);
         sq.pos_locks = (padded_struct*)own->sq_cid_blocks.get();
+        own->sq_cid_left = createBuffer((n_cids / 64) * sizeof(padded_struct), hipDevice);
+        sq.head_mark = (padded_struct*)own->sq_cid_left.get();
         cq.cid = sq.cid;
         cq.cid_mask = sq.cid_mask;
         sq.guard = cq.guard = guard;
         sq.spin_limit = cq.spin_limit = guard ? guard->spin_limit : 0;
 
-        stage = nullptr; stage_ioaddr = 0; stage_stride = 0;
+        stage = nullptr; stage_ioaddr = 0; stage_stride = 0; async_dst = nullptr; async_len = nullptr;
         if (stage_bytes > 2 * ctrl->page_size || (stage_bytes & (stage_bytes - 1)))
             throw std::runtime_error("QueuePair: the staging page must be a power of two of at most two controller pages (PRP1 + PRP2)");
         if (stage_bytes) {
@@ -106,6 +110,11 @@ struct QueuePair
             stage = (uint8_t*)own->stage_mem->vaddr;
             stage_ioaddr = own->stage_mem->ioaddrs[0];
             stage_stride = stage_bytes;
+            /* where the payload of a read submitted with access_data_async goes once poll_async has seen it complete */
+            own->async_dst = createBuffer(n_cids * sizeof(uint64_t), hipDevice);
+            own->async_len = createBuffer(n_cids * sizeof(uint32_t), hipDevice);
+            async_dst = (uint64_t*)own->async_dst.get();
+            async_len = (uint32_t*)own->async_len.get();
         }
     }
 

@@ -202,6 +202,39 @@ def test_page_streaming_modes(bam, mode):
         assert not r.c.aborted()
 
 
+# ---------------------------------------------------------------- the other access routes of array_d_t
+
+@pytest.mark.parametrize("api", [1, 2, 3, 4])
+def test_access_routes_give_the_same_sums(bam, api):
+    """get_raw/release_raw, get_page_gid + acquire_page_, acquire_page/release_page and bam_ptr read what operator[] reads"""
+    from bam_amd import gen
+    n_elems, n = 1 << 22, 4096                  # 8192 pages of data; 64 waves hold at most 4096 pages at a time
+    with Rig(bam, 32 << 20, n_queues=8, depth=256) as r:
+        a = r.array(n_elems, 4096, 6000)
+        for rep in range(3):                    # 3 x 4096 random pages through 6000 slots: later passes evict
+            idx = gen.gather_indices(SEED, n, n_elems, first=rep * n)
+            assert a.read_via(api, n, idx) == oracle.lib().bo_gather_sum(SEED, SEED, rep * n, n, n_elems)
+        st = a.stats()
+        assert st["access_cnt"] == 3 * n and st["read_io_cnt"] > 6000 and not r.c.aborted()
+        assert a.read_via(api, 1000, None, span=517) == int(np.sum(oracle.store(SEED, 0, n_elems)[:1000 * 517:517], dtype=np.uint64))
+
+
+def test_wave_memcpy_out_of_the_cache(bam):
+    """array_d_t::memcpy: a wave copies up to `span` elements from its index on, clipped to the page and the array"""
+    from bam_amd import gen
+    n_elems, n, span = 1 << 18, 2048, 96
+    with Rig(bam, 2 << 20) as r:
+        a = r.array(n_elems, 4096, 64)
+        idx = gen.gather_indices(SEED, n, n_elems)
+        store = oracle.store(SEED, 0, n_elems)
+        want = 0
+        for i in _u64(idx).tolist():
+            cnt = min(span, 512 - i % 512, n_elems - i)
+            want = (want + int(np.sum(store[i:i + cnt], dtype=np.uint64))) % 2**64
+        assert a.read_via(5, n, idx, span=span) == want
+        assert not r.c.aborted()
+
+
 # ---------------------------------------------------------------- raw block
 
 @pytest.mark.parametrize("req,lba,order", [(4096, 512, 0), (512, 512, 2), (4096, 4096, 1)])
@@ -223,6 +256,26 @@ def test_block_reads_payload_checksums(bam, req, lba, order):
         ts = r.t.stats()
         assert ts["read_cmds"] == 2 * n + 1000 and ts["error_cpls"] == 0 and ts["sq_doorbells"] < ts["read_cmds"]
         assert not r.c.aborted()
+        pc.close()
+
+
+@pytest.mark.parametrize("depth,n_threads", [(1, 4096), (2, 2048), (4, 1024)])
+def test_block_reads_with_several_commands_in_flight_per_thread(bam, depth, n_threads):
+    """access_data_async / poll_async: every payload arrives, ids come back (the launch can be repeated)"""
+    from bam_amd import gen
+    ns, req, lba = 1 << 30, 4096, 512
+    with Rig(bam, ns, n_queues=16, depth=256) as r:             # 4 blocks of 64 command ids per queue pair
+        n = n_threads * depth
+        pc = bam.PageCache(4096, n, 0, r.c)
+        for rep in range(3):
+            lbas = gen.block_lbas(SEED + rep, n, ns, req, lba)
+            pc.block_io_async(n_threads, depth, req, lbas)
+            cs = _u64(pc.block_checksums(n, req))
+            ref = np.array([oracle.lib().bo_block_checksum(SEED, int(x), lba, req) for x in _u64(lbas)], dtype=np.uint64)
+            assert np.array_equal(cs, ref)
+        assert r.t.stats()["read_cmds"] == 3 * n and not r.c.aborted()
+        with pytest.raises(Exception):
+            pc.block_io_async(n_threads * 2, depth * 2 if depth < 8 else 8, req, lbas)      # would not fit the command ids
         pc.close()
 
 
