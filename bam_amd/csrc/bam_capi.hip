@@ -16,6 +16,7 @@
 #include "event.h"
 #include "nvmt.h"
 #include "page_cache.h"
+#include "bafs_ptr.h"
 
 // ---------------------------------------------------------------------------
 // error plumbing
@@ -104,6 +105,8 @@ __global__ void k_array_read(array_d_t<uint64_t>* dr, uint64_t n_reqs, const uin
  *   4  bam_ptr                          (per-thread cached page)
  *   5  memcpy                           (wave-cooperative copy of up to `span` elements starting at the wave's index;
  *                                        one request per wave, the copied elements are summed)
+ *   6  bam_ptr_tlb over a 64-entry tlb in LDS, shared by the workgroup
+ *   7  bafs_ptr                         (pointer arithmetic + dereference)
  */
 template <int API>
 __global__ void k_array_read_via(array_d_t<uint64_t>* dr, uint64_t n_reqs, const uint64_t* assignment, uint64_t span, uint64_t* scratch, unsigned long long* sum)
@@ -119,9 +122,28 @@ __global__ void k_array_read_via(array_d_t<uint64_t>* dr, uint64_t n_reqs, const
             dr->memcpy(idx, span, dst);
             for (uint64_t k = bam::lane(); k < span; k += BAM_WAVE_SIZE) v += dst[k];
         }
+    } else if (API == 6) {
+        typedef tlb<uint64_t, 64, simt::thread_scope_device, SHARED_> tlb_t;
+        __shared__ tlb_t table;
+        table.init(dr);
+        __syncthreads();
+        if (tid < n_reqs) {
+            const uint64_t idx = assignment ? assignment[tid] : tid * span;
+            bam_ptr_tlb<uint64_t, 64, simt::thread_scope_device, SHARED_> ptr(dr, &table);
+            const bam_ptr_tlb<uint64_t, 64, simt::thread_scope_device, SHARED_>& cptr = ptr;
+            v = cptr[idx];
+            ptr.fini();
+        }
+        __syncthreads();
+        table.fini();
     } else if (tid < n_reqs) {
         const uint64_t idx = assignment ? assignment[tid] : tid * span;
-        if (API == 1) {
+        if (API == 7) {
+            bafs_ptr<uint64_t> p(dr, 0);
+            bafs_ptr<uint64_t> q = p + idx;
+            v = *q;
+            if (q[0] != v || !(q - idx == p)) v = 0;
+        } else if (API == 1) {
             returned_cache_page_t<uint64_t> pg = dr->get_raw(idx);
             v = bam::ld_payload(pg.addr + pg.offset);
             dr->release_raw(idx);
@@ -735,7 +757,7 @@ int bam_array_read_via(bam_array_t* a, int api, uint64_t n_reqs, const uint64_t*
                        uint64_t* d_sum, void* stream)
 {
     if (!a || !d_sum) return fail(EINVAL, "bam_array_read_via: null argument");
-    if (api < 1 || api > 5) return fail(EINVAL, "bam_array_read_via: api must be 1..5");
+    if (api < 1 || api > 7) return fail(EINVAL, "bam_array_read_via: api must be 1..7");
     if (!block_size || block_size % BAM_WAVE_SIZE || block_size > 1024) return fail(EINVAL, "bam_array_read_via: block size must be a multiple of 64, at most 1024");
     if (!span) return fail(EINVAL, "bam_array_read_via: span must be at least 1");
     if (!n_reqs) return 0;
@@ -752,7 +774,9 @@ int bam_array_read_via(bam_array_t* a, int api, uint64_t n_reqs, const uint64_t*
     case 2: hipLaunchKernelGGL(k_array_read_via<2>, grid, block, 0, st, d, n_reqs, d_assignment, span, sc, s); break;
     case 3: hipLaunchKernelGGL(k_array_read_via<3>, grid, block, 0, st, d, n_reqs, d_assignment, span, sc, s); break;
     case 4: hipLaunchKernelGGL(k_array_read_via<4>, grid, block, 0, st, d, n_reqs, d_assignment, span, sc, s); break;
-    default: hipLaunchKernelGGL(k_array_read_via<5>, grid, block, 0, st, d, n_reqs, d_assignment, span, sc, s); break;
+    case 5: hipLaunchKernelGGL(k_array_read_via<5>, grid, block, 0, st, d, n_reqs, d_assignment, span, sc, s); break;
+    case 6: hipLaunchKernelGGL(k_array_read_via<6>, grid, block, 0, st, d, n_reqs, d_assignment, span, sc, s); break;
+    default: hipLaunchKernelGGL(k_array_read_via<7>, grid, block, 0, st, d, n_reqs, d_assignment, span, sc, s); break;
     }
     hipLaunchKernelGGL(k_fold_partials, dim3(1), dim3(1024), 0, st, s, (unsigned long long*)d_sum);
     hip_err_chk(hipGetLastError());

@@ -81,7 +81,8 @@ int bam_array_read(bam_array_t* a, uint64_t n_reqs, const uint64_t* d_assignment
 /* The read pattern of bam_array_read (one thread per request, element d_assignment[t] or t * span) through the other
  * access routes of array_d_t (include/page_cache.h:1240-1716, 414-485): api 1 get_raw/release_raw, 2 get_page_gid +
  * acquire_page_ + release_page, 3 acquire_page/release_page, 4 bam_ptr, 5 memcpy (one request per wave: up to `span`
- * elements starting at the wave's index, clipped to the page, are copied out and summed). */
+ * elements starting at the wave's index, clipped to the page, are copied out and summed), 6 bam_ptr_tlb over a tlb in
+ * LDS shared by the workgroup (:127-411), 7 bafs_ptr (include/bafs_ptr.h:17-132). */
 int bam_array_read_via(bam_array_t* a, int api, uint64_t n_reqs, const uint64_t* d_assignment, uint64_t span, uint32_t block_size,
                        uint64_t* d_sum, void* stream);
 /* same request pattern through array_d_t::operator() (seq_write): element <- d_values[t] */

@@ -1081,6 +1081,170 @@ struct bam_ptr {
 };
 
 /* ------------------------------------------------------------------ */
+/* translation table in front of the cache                            */
+/* ------------------------------------------------------------------ */
+/*
+ * tlb / bam_ptr_tlb (include/page_cache.h:127-411 of the reference): a small direct-mapped table, shared by the
+ * threads of a workgroup (in LDS) or of a launch (in device memory), that keeps one reference on each page it
+ * names; threads that find their page in the table pay a count on the entry instead of an atomic on the page state.
+ *
+ * entry.state: bit 31 = entry locked, bits 29:0 = threads using the entry right now.
+ *
+ * The reference lets a thread wait on an entry that other threads are using for a different page.  In a wave the
+ * users may be lanes of the waiting lane's own wave, which cannot move while it waits; such a lane takes its page
+ * straight from the cache instead (`direct`), and so does a lane that finds the entry locked by a lane of its own
+ * wave that is in the middle of I/O.
+ */
+#define THREAD_ 0
+#define SHARED_ 1
+#define GLOBAL_ 2
+#define TLB_LOCK_  0x80000000u
+#define TLB_COUNT_ 0x3fffffffu
+
+struct tlb_entry {
+    uint64_t global_id;
+    uint32_t state;
+    uint32_t slot;
+    data_page_t* page;
+
+    __forceinline__ __host__ __device__ void init() { global_id = 0; state = 0; slot = 0; page = nullptr; }
+    /* drop the reference the entry itself holds on its page */
+    __forceinline__ __device__ void release()
+    {
+        if (page) { bam_release_refs(page, 1, false); page = nullptr; }
+    }
+    __forceinline__ __device__ void release(const uint32_t count) { __hip_atomic_fetch_add(&state, 0u - count, __ATOMIC_RELEASE, BAM_AGENT); }
+};
+
+template <typename T, size_t n = 32, simt::thread_scope _scope = simt::thread_scope_device, size_t loc = GLOBAL_>
+struct tlb {
+    tlb_entry entries[n ? n : 1];
+    array_d_t<T>* array;
+
+    /* by all threads of the workgroup (or by one thread with the others waiting), before first use */
+    __forceinline__ __device__ void init(array_d_t<T>* a)
+    {
+        const size_t tid = threadIdx.x + blockDim.x * (threadIdx.y + blockDim.y * threadIdx.z);
+        const size_t bs = (size_t)blockDim.x * blockDim.y * blockDim.z;
+        if (tid == 0) array = a;
+        for (size_t k = tid; k < n; k += bs) entries[k].init();
+    }
+    /* after the last use: the references the entries hold go back */
+    __forceinline__ __device__ void fini()
+    {
+        const size_t tid = threadIdx.x + blockDim.x * (threadIdx.y + blockDim.y * threadIdx.z);
+        const size_t bs = (size_t)blockDim.x * blockDim.y * blockDim.z;
+        for (size_t k = tid; k < n; k += bs) entries[k].release();
+    }
+
+    /*
+     * Address of the first element of the page `page_` of `range` (global id `gid`), the window it covers in
+     * [start, end), and in `direct` whether the table was bypassed; pair with release(gid, direct, range, page_).
+     */
+    __forceinline__ __device__ T* acquire(const size_t i, const size_t gid, size_t& start, size_t& end, range_d_t<T>* range, const size_t page_, bool& direct)
+    {
+        using namespace bam;
+        (void)i;
+        tlb_entry* entry = entries + (n ? gid % n : 0);
+        const uint64_t eq_mask = match_any((uint64_t)gid, (uint64_t)this);
+        const uint32_t master = first_lane(eq_mask), count = popc(eq_mask);
+        uint64_t pack = 0;                       /* slot | direct << 32 */
+        if (lane() == master) {
+            bool settled = false, go_direct = n == 0;
+            uint32_t slot = 0;
+            /* the masters of a wave come round this loop together; whoever holds an entry's lock finishes
+             * within the trip, so nobody spins on a lock held by a lane that cannot run */
+            for (uint32_t tries = 0; !settled && !go_direct; tries++) {
+                const uint32_t st = __hip_atomic_fetch_or(&entry->state, TLB_LOCK_, __ATOMIC_ACQUIRE, BAM_AGENT);
+                if ((st & TLB_LOCK_) == 0) {
+                    if (entry->page != nullptr && entry->global_id == gid) {
+                        slot = entry->slot;
+                        __hip_atomic_store(&entry->state, st + count, __ATOMIC_RELEASE, BAM_AGENT);
+                        settled = true;
+                    } else if (entry->page == nullptr || (st & TLB_COUNT_) == 0) {
+                        entry->release();
+                        slot = (uint32_t)range->acquire_page(page_, 1, false, 0, wave_slot_hash());
+                        entry->page = &range->pages[page_];
+                        entry->slot = slot;
+                        entry->global_id = gid;
+                        __hip_atomic_store(&entry->state, st + count, __ATOMIC_RELEASE, BAM_AGENT);
+                        settled = true;
+                    } else {
+                        __hip_atomic_store(&entry->state, st, __ATOMIC_RELEASE, BAM_AGENT);     /* in use for another page */
+                        go_direct = true;
+                    }
+                } else if (tries >= 8) go_direct = true;
+            }
+            if (go_direct) slot = (uint32_t)range->acquire_page(page_, count, false, 0, wave_slot_hash());
+            pack = (uint64_t)slot | ((uint64_t)go_direct << 32);
+        }
+        pack = shfl(pack, master);
+        direct = (pack >> 32) != 0;
+        range_view<T> v;
+        v.load(range);
+        v.window(page_, start, end);
+        return (T*)(v.slot_addr((uint32_t)pack) + (v.byte_of(start) & (v.page_size - 1)));
+    }
+
+    __forceinline__ __device__ void release(const size_t gid, const bool direct, range_d_t<T>* range, const size_t page_)
+    {
+        using namespace bam;
+        const uint64_t eq_mask = match_any((uint64_t)gid, (uint64_t)this ^ (direct ? 1ull : 0ull));
+        if (lane() != first_lane(eq_mask)) return;
+        if (direct) range->release_page(page_, popc(eq_mask), false);
+        else entries[n ? gid % n : 0].release(popc(eq_mask));
+    }
+};
+
+template <typename T, size_t n = 32, simt::thread_scope _scope = simt::thread_scope_device, size_t loc = GLOBAL_>
+struct bam_ptr_tlb {
+    tlb<T, n, _scope, loc>* tlb_ = nullptr;
+    array_d_t<T>* array = nullptr;
+    range_d_t<T>* range = nullptr;
+    size_t page = 0;
+    size_t start = 0;
+    size_t end = 0;
+    size_t gid = 0;
+    T* addr = nullptr;
+    bool direct = false;
+
+    __forceinline__ __device__ bam_ptr_tlb(array_d_t<T>* a, tlb<T, n, _scope, loc>* t) { init(a, t); }
+    __forceinline__ __device__ ~bam_ptr_tlb() { fini(); }
+    __forceinline__ __device__ void init(array_d_t<T>* a, tlb<T, n, _scope, loc>* t) { array = a; tlb_ = t; }
+
+    __forceinline__ __device__ void fini(void)
+    {
+        if (addr) {
+            tlb_->release(gid, direct, range, page);
+            addr = nullptr;
+            start = end = 0;
+        }
+    }
+
+    __forceinline__ __device__ void update_page(const size_t i)
+    {
+        fini();
+        array->get_page_gid(i, range, page, gid);
+        if (range) addr = tlb_->acquire(i, gid, start, end, range, page, direct);
+    }
+
+    __forceinline__ __device__ T operator[](const size_t i) const
+    {
+        bam_ptr_tlb* self = const_cast<bam_ptr_tlb*>(this);
+        if (i < start || i >= end) self->update_page(i);
+        return bam::ld_payload(self->addr + (i - start));
+    }
+
+    /* address of element i for the caller to write through: the page is marked dirty */
+    __forceinline__ __device__ T* memref(const size_t i)
+    {
+        if (i < start || i >= end) update_page(i);
+        range->mark_page_dirty(page);
+        return addr + (i - start);
+    }
+};
+
+/* ------------------------------------------------------------------ */
 /* host side                                                          */
 /* ------------------------------------------------------------------ */
 

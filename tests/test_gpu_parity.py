@@ -204,9 +204,9 @@ def test_page_streaming_modes(bam, mode):
 
 # ---------------------------------------------------------------- the other access routes of array_d_t
 
-@pytest.mark.parametrize("api", [1, 2, 3, 4])
+@pytest.mark.parametrize("api", [1, 2, 3, 4, 6, 7])
 def test_access_routes_give_the_same_sums(bam, api):
-    """get_raw/release_raw, get_page_gid + acquire_page_, acquire_page/release_page and bam_ptr read what operator[] reads"""
+    """get_raw/release_raw, get_page_gid + acquire_page_, acquire_page/release_page, bam_ptr, bam_ptr_tlb and bafs_ptr read what operator[] reads"""
     from bam_amd import gen
     n_elems, n = 1 << 22, 4096                  # 8192 pages of data; 64 waves hold at most 4096 pages at a time
     with Rig(bam, 32 << 20, n_queues=8, depth=256) as r:
@@ -215,8 +215,10 @@ def test_access_routes_give_the_same_sums(bam, api):
             idx = gen.gather_indices(SEED, n, n_elems, first=rep * n)
             assert a.read_via(api, n, idx) == oracle.lib().bo_gather_sum(SEED, SEED, rep * n, n, n_elems)
         st = a.stats()
-        assert st["access_cnt"] == 3 * n and st["read_io_cnt"] > 6000 and not r.c.aborted()
+        assert st["access_cnt"] == 3 * n * (2 if api == 7 else 1) and st["read_io_cnt"] > 6000 and not r.c.aborted()      # route 7 dereferences twice
         assert a.read_via(api, 1000, None, span=517) == int(np.sum(oracle.store(SEED, 0, n_elems)[:1000 * 517:517], dtype=np.uint64))
+        # neighbouring elements: the lanes of a wave share pages (and, through a tlb, entries)
+        assert a.read_via(api, 50000, None, span=3, block_size=256) == int(np.sum(oracle.store(SEED, 0, n_elems)[:150000:3], dtype=np.uint64))
 
 
 def test_wave_memcpy_out_of_the_cache(bam):
