@@ -45,6 +45,8 @@ SIGNATURES = {
     "bam_cc": (c_int, [c_vp, c_vp, c_u64, c_vp, c_u32, P(c_u32), c_vp]),
     "bam_array_read_via": (c_int, [c_vp, c_int, c_u64, c_vp, c_u64, c_u32, c_vp, c_vp]),
     "bam_block_io_async": (c_int, [c_vp, c_vp, c_u64, c_u32, c_u32, c_vp, c_u32, c_vp]),
+    "bam_store_write_file": (c_int, [c_vp, c_vp, ctypes.c_char_p, c_u64, c_u64, c_u64, P(c_u64)]),
+    "bam_store_read_file": (c_int, [c_vp, c_vp, ctypes.c_char_p, c_u64, c_u64]),
     "bam_bfs_by_page": (c_int, [c_vp, c_vp, c_u64, c_u64, c_vp, P(c_u32), c_vp]),
     "bam_cc_by_page": (c_int, [c_vp, c_vp, c_u64, c_vp, P(c_u32), c_vp]),
     "bam_gen_words": (c_int, [c_u64, c_u64, c_u64, c_vp, c_vp]),
@@ -52,6 +54,8 @@ SIGNATURES = {
     "bam_gen_rmat": (c_int, [c_u64, c_u32, c_u64, c_u64, c_vp, c_vp, c_vp]),
     "bam_gen_uniform": (c_int, [c_u64, c_u64, c_u64, c_u64, c_vp, c_vp, c_vp]),
     "bam_copy_kernel": (c_int, [c_vp, c_vp, c_u64, P(ctypes.c_float), c_vp]),
+    "bam_read_kernel": (c_int, [c_vp, c_u64, P(ctypes.c_float), c_vp]),
+    "bam_gather_kernel": (c_int, [c_vp, c_vp, c_u64, P(ctypes.c_float), c_vp]),
     "bam_host_read_ceiling": (c_int, [c_u64, c_u32, P(ctypes.c_float)]),
     "bam_event_create": (c_int, [P(c_vp)]),
     "bam_event_record": (c_int, [c_vp, c_vp]),

@@ -5,6 +5,11 @@
 #include "bam_amd.h"
 
 #include <hip/hip_runtime.h>
+#include <fcntl.h>
+#include <sys/mman.h>
+#include <sys/stat.h>
+#include <unistd.h>
+#include <algorithm>
 #include <cerrno>
 #include <cstdlib>
 #include <cstring>
@@ -30,6 +35,7 @@ static thread_local std::string g_err;
       catch (...) { g_err = "unknown error"; return EIO; }
 
 static int fail(int code, const char* msg) { g_err = msg; return code; }
+static int fail(int code, const std::string& msg) { g_err = msg; return code; }
 
 struct bam_target {
     nvmt_t* t = nullptr;
@@ -276,6 +282,20 @@ __global__ void k_block_io_async(Controller** ctrls, page_cache_d_t* pc, uint32_
     for (int k = 0; k < DEPTH; k++) poll_async(qp, cids[k], poss[k]);
 }
 
+// ---- readwrite benchmark (benchmarks/readwrite/main.cu:73-116): cache slots <-> consecutive pages of the store ----
+__global__ void k_sequential_access(Controller** ctrls, page_cache_d_t* pc, uint32_t req_size, uint64_t n_slots, uint64_t store_byte, int write)
+{
+    const uint64_t tid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const uint64_t n_threads = (uint64_t)gridDim.x * blockDim.x;
+    QueuePair* qp = ctrls[0]->d_qps + (tid / BAM_WAVE_SIZE) % ctrls[0]->n_qps;
+    const uint64_t n_blocks = req_size >> qp->block_size_log;
+    for (uint64_t t = tid; t < n_slots; t += n_threads) {
+        const uint64_t start_block = (store_byte + t * req_size) >> qp->block_size_log;
+        if (write) write_data(pc, qp, start_block, n_blocks, t);
+        else read_data(pc, qp, start_block, n_blocks, t);
+    }
+}
+
 __global__ void k_block_checksum(page_cache_d_t* pc, uint64_t n_slots, uint32_t req_bytes, uint64_t* out)
 {
     /* one wave per slot */
@@ -493,6 +513,29 @@ __global__ void k_gen_uniform(uint64_t seed, uint64_t n_vertices, uint64_t first
 __global__ void k_copy16(const uint4* __restrict__ src, uint4* __restrict__ dst, uint64_t n16)
 {
     for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (uint64_t)gridDim.x * blockDim.x) dst[i] = src[i];
+}
+/* plain streaming read of device memory, 16 bytes per lane per load, eight loads in flight: what the memory system gives a
+ * reader that does nothing else (the practical ceiling under the hit-path figure) */
+__global__ __launch_bounds__(256) void k_read16(const uint4* __restrict__ src, uint64_t n16, unsigned long long* partials)
+{
+    uint64_t a = 0;
+    const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+    uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    for (; i + 7 * stride < n16; i += 8 * stride) {
+        uint4 x[8];
+#pragma unroll
+        for (int k = 0; k < 8; k++) x[k] = src[i + k * stride];
+#pragma unroll
+        for (int k = 0; k < 8; k++) a += (uint64_t)x[k].x + x[k].y + x[k].z + x[k].w;
+    }
+    for (; i < n16; i += stride) { const uint4 x = src[i]; a += (uint64_t)x.x + x.y + x.z + x.w; }
+    block_accumulate(partials, a);
+}
+/* plain random gather of 8-byte words from device memory: the ceiling of that access pattern without any cache protocol */
+__global__ void k_gather8(const uint64_t* __restrict__ src, const uint64_t* __restrict__ idx, uint64_t n, unsigned long long* partials)
+{
+    const uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    block_accumulate(partials, t < n ? src[idx[t]] : 0);
 }
 /* every wave pulls whole chunks of host-pinned memory into device memory, 16 bytes per lane per load */
 __global__ void k_host_pull(const uint4* __restrict__ host, uint4* __restrict__ dev, uint64_t n_chunks, uint32_t chunk16, uint64_t host_chunks)
@@ -861,6 +904,98 @@ int bam_block_io_async(bam_ctrl_t* c, bam_page_cache_t* pc, uint64_t n_threads, 
     BAM_API_END
 }
 
+namespace {
+/* a file mapped read-only, or created and mapped for writing */
+struct mapped_file {
+    int fd = -1;
+    uint8_t* p = nullptr;
+    size_t size = 0;
+    int open_ro(const char* path)
+    {
+        fd = ::open(path, O_RDONLY);
+        if (fd < 0) return errno;
+        struct stat sb;
+        if (fstat(fd, &sb)) return errno;
+        size = (size_t)sb.st_size;
+        if (size) { void* m = mmap(nullptr, size, PROT_READ, MAP_PRIVATE, fd, 0); if (m == MAP_FAILED) return errno; p = (uint8_t*)m; }
+        return 0;
+    }
+    int create_rw(const char* path, size_t bytes)
+    {
+        fd = ::open(path, O_RDWR | O_CREAT | O_TRUNC, 0644);
+        if (fd < 0) return errno;
+        if (ftruncate(fd, (off_t)bytes)) return errno;
+        size = bytes;
+        if (size) { void* m = mmap(nullptr, size, PROT_READ | PROT_WRITE, MAP_SHARED, fd, 0); if (m == MAP_FAILED) return errno; p = (uint8_t*)m; }
+        return 0;
+    }
+    ~mapped_file() { if (p) munmap(p, size); if (fd >= 0) ::close(fd); }
+};
+
+int check_store_span(bam_ctrl_t* c, bam_page_cache_t* pc, uint64_t store_offset, uint64_t n_bytes, const char* who)
+{
+    const uint64_t ps = pc->pc->pdt.page_size;
+    if (store_offset % ps) return fail(EINVAL, std::string(who) + ": the store offset must be a multiple of the page size");
+    const uint64_t ns_bytes = (uint64_t)c->c->ns.size * c->c->blk_size;
+    const uint64_t padded = (n_bytes + ps - 1) / ps * ps;
+    if (store_offset > ns_bytes || padded > ns_bytes - store_offset) return fail(ERANGE, std::string(who) + ": past the end of the namespace");
+    return 0;
+}
+} // namespace
+
+int bam_store_write_file(bam_ctrl_t* c, bam_page_cache_t* pc, const char* path, uint64_t file_offset, uint64_t store_offset, uint64_t n_bytes,
+                         uint64_t* bytes_done)
+{
+    if (!c || !pc || !path) return fail(EINVAL, "bam_store_write_file: null argument");
+    BAM_API_BEGIN
+    mapped_file in;
+    if (int rc = in.open_ro(path)) return fail(rc, std::string("bam_store_write_file: ") + path + ": " + strerror(rc));
+    if (file_offset > in.size) return fail(ERANGE, "bam_store_write_file: offset past the end of the file");
+    if (!n_bytes) n_bytes = in.size - file_offset;
+    if (n_bytes > in.size - file_offset) return fail(ERANGE, "bam_store_write_file: more bytes than the file holds");
+    if (int rc = check_store_span(c, pc, store_offset, n_bytes, "bam_store_write_file")) return rc;
+    const uint64_t ps = pc->pc->pdt.page_size, cache_bytes = ps * pc->pc->pdt.n_pages;
+    uint64_t done = 0;
+    while (done < n_bytes) {
+        const uint64_t chunk = std::min(cache_bytes, n_bytes - done);
+        const uint64_t n_slots = (chunk + ps - 1) / ps;
+        hip_err_chk(hipMemcpy(pc->pc->pdt.base_addr, in.p + file_offset + done, chunk, hipMemcpyHostToDevice));
+        if (chunk % ps) hip_err_chk(hipMemset(pc->pc->pdt.base_addr + chunk, 0, n_slots * ps - chunk));      /* the tail of the last page */
+        hipLaunchKernelGGL(k_sequential_access, dim3(blocks_for(std::min<uint64_t>(n_slots, 1u << 18), 64)), dim3(64), 0, 0,
+                           pc->pc->pdt.d_ctrls, pc->pc->d_pc_ptr, (uint32_t)ps, n_slots, store_offset + done, 1);
+        hip_err_chk(hipGetLastError());
+        hip_err_chk(hipDeviceSynchronize());
+        if (c->c->aborted()) return fail(EIO, "bam_store_write_file: a device-side wait gave up");
+        done += chunk;
+    }
+    if (bytes_done) *bytes_done = done;
+    BAM_API_END
+}
+
+int bam_store_read_file(bam_ctrl_t* c, bam_page_cache_t* pc, const char* path, uint64_t store_offset, uint64_t n_bytes)
+{
+    if (!c || !pc || !path || !n_bytes) return fail(EINVAL, "bam_store_read_file: null argument or nothing to read");
+    BAM_API_BEGIN
+    if (int rc = check_store_span(c, pc, store_offset, n_bytes, "bam_store_read_file")) return rc;
+    mapped_file out;
+    if (int rc = out.create_rw(path, n_bytes)) return fail(rc, std::string("bam_store_read_file: ") + path + ": " + strerror(rc));
+    const uint64_t ps = pc->pc->pdt.page_size, cache_bytes = ps * pc->pc->pdt.n_pages;
+    uint64_t done = 0;
+    while (done < n_bytes) {
+        const uint64_t chunk = std::min(cache_bytes, n_bytes - done);
+        const uint64_t n_slots = (chunk + ps - 1) / ps;
+        hipLaunchKernelGGL(k_sequential_access, dim3(blocks_for(std::min<uint64_t>(n_slots, 1u << 18), 64)), dim3(64), 0, 0,
+                           pc->pc->pdt.d_ctrls, pc->pc->d_pc_ptr, (uint32_t)ps, n_slots, store_offset + done, 0);
+        hip_err_chk(hipGetLastError());
+        hip_err_chk(hipDeviceSynchronize());
+        if (c->c->aborted()) return fail(EIO, "bam_store_read_file: a device-side wait gave up");
+        hip_err_chk(hipMemcpy(out.p + done, pc->pc->pdt.base_addr, chunk, hipMemcpyDeviceToHost));
+        done += chunk;
+    }
+    if (msync(out.p, out.size, MS_SYNC)) return fail(errno, "bam_store_read_file: msync failed");
+    BAM_API_END
+}
+
 int bam_block_checksum(bam_page_cache_t* pc, uint64_t n_slots, uint32_t req_bytes, uint64_t* d_out, void* stream)
 {
     if (!pc || !d_out) return fail(EINVAL, "bam_block_checksum: null argument");
@@ -1088,6 +1223,34 @@ int bam_copy_kernel(const void* d_src, void* d_dst, uint64_t n_bytes, float* ms,
     hipStream_t st = (hipStream_t)stream;
     Event a(st);
     hipLaunchKernelGGL(k_copy16, dim3(256 * 16), dim3(256), 0, st, (const uint4*)d_src, (uint4*)d_dst, n_bytes / 16);
+    hip_err_chk(hipGetLastError());
+    Event b(st);
+    if (ms) *ms = (float)((b - a) / 1e3);
+    BAM_API_END
+}
+
+int bam_read_kernel(const void* d_src, uint64_t n_bytes, float* ms, void* stream)
+{
+    if (!d_src || n_bytes % 16) return fail(EINVAL, "bam_read_kernel: bad argument");
+    BAM_API_BEGIN
+    hipStream_t st = (hipStream_t)stream;
+    BufferPtr partials = createBuffer(BAM_SUM_PARTIALS * sizeof(unsigned long long), 0);
+    Event a(st);
+    hipLaunchKernelGGL(k_read16, dim3(256 * 16), dim3(256), 0, st, (const uint4*)d_src, n_bytes / 16, (unsigned long long*)partials.get());
+    hip_err_chk(hipGetLastError());
+    Event b(st);
+    if (ms) *ms = (float)((b - a) / 1e3);
+    BAM_API_END
+}
+
+int bam_gather_kernel(const uint64_t* d_src, const uint64_t* d_idx, uint64_t n, float* ms, void* stream)
+{
+    if (!d_src || !d_idx || !n) return fail(EINVAL, "bam_gather_kernel: bad argument");
+    BAM_API_BEGIN
+    hipStream_t st = (hipStream_t)stream;
+    BufferPtr partials = createBuffer(BAM_SUM_PARTIALS * sizeof(unsigned long long), 0);
+    Event a(st);
+    hipLaunchKernelGGL(k_gather8, dim3(blocks_for(n, 256)), dim3(256), 0, st, d_src, d_idx, n, (unsigned long long*)partials.get());
     hip_err_chk(hipGetLastError());
     Event b(st);
     if (ms) *ms = (float)((b - a) / 1e3);

@@ -8,6 +8,7 @@ buffers are torch tensors on the handle's device; 64-bit unsigned data travels
 as int64 tensors (same bits).
 """
 import ctypes
+import os
 
 import torch
 
@@ -137,6 +138,17 @@ class PageCache:
     def block_io_async(self, n_threads, depth, req_bytes, lbas, block_size=64):
         """`depth` commands in flight per thread (benchmarks/iodepth-block/main.cu:97-140)."""
         _chk(self.L.bam_block_io_async(self.ctrl.h, self.h, n_threads, depth, req_bytes, _ptr(lbas), block_size, _stream()), "bam_block_io_async")
+
+    def write_file(self, path, file_offset=0, store_offset=0, n_bytes=0):
+        """file -> store through the cache slots (benchmarks/readwrite, write mode); returns the bytes written."""
+        done = c_u64(0)
+        _chk(self.L.bam_store_write_file(self.ctrl.h, self.h, os.fsencode(path), file_offset, store_offset, n_bytes, ctypes.byref(done)),
+             "bam_store_write_file")
+        return done.value
+
+    def read_file(self, path, store_offset, n_bytes):
+        """store -> a new file (benchmarks/readwrite, read mode)"""
+        _chk(self.L.bam_store_read_file(self.ctrl.h, self.h, os.fsencode(path), store_offset, n_bytes), "bam_store_read_file")
 
     def block_checksums(self, n_slots, req_bytes):
         out = torch.empty(n_slots, dtype=torch.int64, device=f"cuda:{self.device}")

@@ -109,6 +109,14 @@ int bam_block_io(bam_ctrl_t* c, bam_page_cache_t* pc, uint64_t n_reqs, uint32_t 
  * command ids (waves per queue pair x depth x 64 <= queue depth), checked here. */
 int bam_block_io_async(bam_ctrl_t* c, bam_page_cache_t* pc, uint64_t n_threads, uint32_t depth, uint32_t req_bytes, const uint64_t* d_lbas,
                        uint32_t block_size, void* stream);
+/* ---- readwrite benchmark (benchmarks/readwrite/main.cu:73-116, host loops :283-316 and :317-391) ----
+ * Copy n_bytes (0 = to the end) of the file from file_offset on to the store from byte store_offset on (a multiple of
+ * the page size), one pass of the cache at a time: file -> cache slots -> one NVMe write per slot.  This is how a
+ * dataset, e.g. the payload of a graph's .dst file (file_offset 16, see bel.h), is placed on the store.  The tail of
+ * the last page is zero-filled.  read_file is the inverse: store -> cache slots -> a new file of n_bytes. */
+int bam_store_write_file(bam_ctrl_t* c, bam_page_cache_t* pc, const char* path, uint64_t file_offset, uint64_t store_offset, uint64_t n_bytes,
+                         uint64_t* bytes_done);
+int bam_store_read_file(bam_ctrl_t* c, bam_page_cache_t* pc, const char* path, uint64_t store_offset, uint64_t n_bytes);
 /* sum of the 64-bit words of the first req_bytes of slots 0..n-1, one sum per slot */
 int bam_block_checksum(bam_page_cache_t* pc, uint64_t n_slots, uint32_t req_bytes, uint64_t* d_out, void* stream);
 
@@ -144,6 +152,10 @@ int bam_gen_uniform(uint64_t seed, uint64_t n_vertices, uint64_t first_pair, uin
  * GPU (the interconnect ceiling of staged transfers); both return elapsed milliseconds measured with HIP events. */
 int bam_copy_kernel(const void* d_src, void* d_dst, uint64_t n_bytes, float* ms, void* stream);
 int bam_host_read_ceiling(uint64_t n_bytes, uint32_t chunk_bytes, float* ms);
+/* what the memory system gives plain kernels with the access patterns of the hit path, no cache protocol: a streaming
+ * read of n bytes, and a gather of n 8-byte words at d_idx[] from d_src; elapsed milliseconds */
+int bam_read_kernel(const void* d_src, uint64_t n_bytes, float* ms, void* stream);
+int bam_gather_kernel(const uint64_t* d_src, const uint64_t* d_idx, uint64_t n, float* ms, void* stream);
 /* time a callback-free region: record/elapsed on the stream the kernels above were launched on */
 int bam_event_create(void** ev);
 int bam_event_record(void* ev, void* stream);

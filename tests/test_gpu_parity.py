@@ -387,6 +387,48 @@ def test_cc_labels_uniform_by_edge_page(bam, n_v, n_p, cache_pages):
         assert not r.c.aborted()
 
 
+# ---------------------------------------------------------------- dataset placement (readwrite) and graph files
+
+def test_graph_file_to_store_then_traverse(bam, tmp_path):
+    """.bel pair on disk -> payload of .dst written to the store at a page-aligned offset through the cache slots ->
+    BFS and CC over an array that starts at that offset -> the store read back into a file"""
+    from bam_amd import bel
+    off, nb = oracle.rmat_csr(SEED, 12)
+    prefix = str(tmp_path / "rmat12.bel")
+    bel.write(prefix, off, nb)
+    n_off, n_e = bel.info(prefix)
+    assert n_off == len(off) and n_e == len(nb)
+    loffset = 3 << 20                                           # --loffset of the reference's graph benchmarks
+    ns_bytes = 16 << 20
+    with Rig(bam, ns_bytes, backing=True, n_queues=8, depth=256) as r:
+        store = r.backing(ns_bytes // 8)
+        store[:] = 0x5a5a5a5a5a5a5a5a
+        loader = bam.PageCache(4096, 100, 0, r.c)              # smaller than the file: several passes, ragged last page
+        assert loader.write_file(prefix + ".dst", file_offset=bel.HEADER_BYTES, store_offset=loffset) == n_e * 8
+        first = loffset // 8
+        assert np.array_equal(store[first:first + n_e], nb)
+        pad = (-n_e) % 512
+        assert not store[first + n_e:first + n_e + pad].any() and store[first + n_e + pad] == 0x5a5a5a5a5a5a5a5a and store[first - 1] == 0x5a5a5a5a5a5a5a5a
+        back = str(tmp_path / "back.bin")
+        loader.read_file(back, loffset, n_e * 8)
+        assert np.array_equal(np.fromfile(back, dtype=np.uint64), nb)
+        with pytest.raises(Exception):
+            loader.write_file(prefix + ".dst", file_offset=16, store_offset=loffset + 512)      # not page aligned
+        with pytest.raises(Exception):
+            loader.write_file(prefix + ".dst", file_offset=16, store_offset=ns_bytes - 4096)    # past the end
+        loader.close()
+        a = r.array(n_e, 4096, 64, disk_offset=loffset)
+        doff = _dev(bel.read_offsets(prefix))
+        for by_page in (False, True):
+            for src in oracle.bfs_sources(SEED, off, 2):
+                lv, it = a.bfs(doff, int(src), coarse=2, by_page=by_page)
+                ref, rit = oracle.bfs_levels(off, nb, int(src))
+                assert np.array_equal(lv.cpu().numpy().view(np.uint32), ref) and it == rit
+            lb, _ = a.cc(doff, coarse=2, by_page=by_page)
+            assert np.array_equal(_u64(lb), oracle.cc_labels(off, nb)[0])
+        assert r.t.stats()["write_cmds"] == (n_e * 8 + 4095) // 4096 and not r.c.aborted()
+
+
 # ---------------------------------------------------------------- failure handling
 
 def test_lost_completion_ends_the_kernel_with_the_abort_flag(bam):
