@@ -185,7 +185,7 @@ __global__ void k_array_write(array_d_t<uint64_t>* dr, uint64_t n_reqs, const ui
 
 // ---- cache / pattern benchmark (benchmarks/cache/main.cu:44-114): a wave streams whole pages ----
 template <int MODE>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void k_cache_stream(array_d_t<uint64_t>* dr, uint64_t n_waves, uint64_t n_pages_per_wave, const uint64_t* assignment, unsigned long long* sum)
+__device__ __forceinline__ void cache_stream_body(array_d_t<uint64_t>* dr, uint64_t n_waves, uint64_t n_pages_per_wave, const uint64_t* assignment, unsigned long long* sum)
 {
     const uint64_t tid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const uint64_t wave = tid / BAM_WAVE_SIZE, lane = tid % BAM_WAVE_SIZE;
@@ -198,7 +198,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void k
             /*
              * Descriptor read once.  Pages are taken sixteen at a time: lane l of the wave asks for page l of the
              * batch, so the sixteen reference counts go out as one vector atomic; then the whole wave streams the
-             * sixteen pages, eight loads in flight per lane, and the sixteen references are dropped together.
+             * sixteen pages, eight 8-byte loads in flight per lane, and the sixteen references are dropped together.
              */
             bam::range_view<uint64_t> view;
             view.load(r0);
@@ -210,7 +210,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void k
                 const uint64_t page = view.page_of((start_page + p0 + (lane < nb ? lane : 0)) * epp);
                 if (lane < nb) {
                     auto keep = [&](uint32_t s_) { slot = s_; return false; };
-                    view.acquire(page, false, keep, keep);
+                    view.acquire<true>(page, false, keep, keep);
                 }
                 for (uint32_t k = 0; k < nb; k++) {
                     const uint64_t* base = (const uint64_t*)view.slot_addr(bam::bcast(slot, k));
@@ -238,6 +238,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void k
         }
     }
     block_accumulate(sum, v);
+}
+
+/*
+ * One kernel per mode, each with the register budget that suits it: the two per-element kernels live on occupancy
+ * (every page change is a dependent chain of atomics and loads) and are held at four waves per SIMD; the page-wise
+ * kernel keeps sixty-four bytes per lane in flight and runs best with the registers it asks for.
+ */
+template <int MODE>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void k_cache_stream(array_d_t<uint64_t>* dr, uint64_t n_waves, uint64_t n_pages_per_wave, const uint64_t* assignment, unsigned long long* sum)
+{
+    cache_stream_body<MODE>(dr, n_waves, n_pages_per_wave, assignment, sum);
+}
+__global__ __launch_bounds__(256) void k_cache_stream_pages(array_d_t<uint64_t>* dr, uint64_t n_waves, uint64_t n_pages_per_wave, const uint64_t* assignment, unsigned long long* sum)
+{
+    cache_stream_body<2>(dr, n_waves, n_pages_per_wave, assignment, sum);
 }
 
 // ---- raw block benchmark (benchmarks/block/main.cu:99-200) ----
@@ -853,7 +868,7 @@ int bam_cache_stream(bam_array_t* a, uint64_t n_waves, uint64_t n_pages_per_wave
     unsigned long long* s = (unsigned long long*)a->partials.get();
     if (mode == 0) hipLaunchKernelGGL(k_cache_stream<0>, grid, block, 0, (hipStream_t)stream, d, n_waves, n_pages_per_wave, d_assignment, s);
     else if (mode == 1) hipLaunchKernelGGL(k_cache_stream<1>, grid, block, 0, (hipStream_t)stream, d, n_waves, n_pages_per_wave, d_assignment, s);
-    else hipLaunchKernelGGL(k_cache_stream<2>, grid, block, 0, (hipStream_t)stream, d, n_waves, n_pages_per_wave, d_assignment, s);
+    else hipLaunchKernelGGL(k_cache_stream_pages, grid, block, 0, (hipStream_t)stream, d, n_waves, n_pages_per_wave, d_assignment, s);
     hipLaunchKernelGGL(k_fold_partials, dim3(1), dim3(1024), 0, (hipStream_t)stream, s, (unsigned long long*)d_sum);
     hip_err_chk(hipGetLastError());
     BAM_API_END

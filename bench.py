@@ -37,6 +37,7 @@ CACHE_PAGES = 1 << 18
 PAGE = 4096
 N_READS = 1 << 26
 HBM_PEAK_GBS = 8000.0
+STREAM_PAGES_PER_WAVE = 16      # one acquire batch of the page-wise streaming kernel
 # HBM bytes one launch of the page-wise streaming kernel moves over the 1 GiB cache, from the profiler's FETCH_SIZE and
 # WRITE_SIZE counters scaled by what they read for a plain 1 GiB copy (x2.0 and x1.0); figures and commands in
 # profiles/k_cache_stream_hit_path_1GiB_cache.md.  Holds for this workload only.
@@ -105,21 +106,21 @@ def main():
     log("[bench] set-up %.1fs: %s %s" % (time.time() - t0, ctrl.info(), pc.info()))
 
     # ------------------------------------------------------------------ hit path (roofline): stream the resident cache
-    arr.stream(CACHE_PAGES // 4, 4, mode=2)             # cold pass fills the cache with pages 0 .. CACHE_PAGES-1
+    arr.stream(CACHE_PAGES // STREAM_PAGES_PER_WAVE, STREAM_PAGES_PER_WAVE, mode=2)             # cold pass fills the cache with pages 0 .. CACHE_PAGES-1
     arr.stats()
     ref_stream = O.bo_store_sum(SEED, 0, 1, 1 << 24)
     assert arr.stream((1 << 24) // 512 // 4, 4, mode=2) == ref_stream, "hit-path checksum mismatch"
     hit_reps = 20
     s_hit = torch.zeros(1, dtype=torch.int64, device=dev)
     for mode, name in ((2, "page_wise"), (1, "bam_ptr")):
-        arr.stream_async(CACHE_PAGES // 4, 4, s_hit, mode=mode)
+        arr.stream_async(CACHE_PAGES // STREAM_PAGES_PER_WAVE, STREAM_PAGES_PER_WAVE, s_hit, mode=mode)
     torch.cuda.synchronize()
     hit = {}
     for mode, name in ((2, "page_wise"), (1, "bam_ptr")):
         a, b = event(), event()
         L.bam_event_record(a, stream)
         for _ in range(hit_reps):
-            arr.stream_async(CACHE_PAGES // 4, 4, s_hit, mode=mode)
+            arr.stream_async(CACHE_PAGES // STREAM_PAGES_PER_WAVE, STREAM_PAGES_PER_WAVE, s_hit, mode=mode)
         L.bam_event_record(b, stream)
         ms = elapsed_ms(a, b) / hit_reps
         hit[name] = {"ms_per_launch": ms, "GBps": CACHE_PAGES * PAGE / ms / 1e6}
@@ -129,7 +130,15 @@ def main():
                 "achieved": hit["page_wise"]["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": hit["page_wise"]["GBps"] / HBM_PEAK_GBS, "traffic": HIT_STREAM_TRAFFIC_BYTES,
                 "bytes_per_launch": CACHE_PAGES * PAGE, "ms_per_launch": hit["page_wise"]["ms_per_launch"],
-                "bam_ptr_kernel_GBps": hit["bam_ptr"]["GBps"]}
+                "bam_ptr_kernel_GBps": hit["bam_ptr"]["GBps"], "pages_per_wave": STREAM_PAGES_PER_WAVE}
+    # what the memory system gives a plain kernel that only reads (no cache protocol): the practical ceiling under `peak`
+    probe = torch.empty(1 << 27, dtype=torch.int64, device=dev).fill_(1)
+    ms_c = ctypes.c_float(0)
+    best = 1e9
+    for _ in range(5):
+        assert L.bam_read_kernel(ctypes.c_void_p(probe.data_ptr()), ctypes.c_uint64(1 << 30), ctypes.byref(ms_c), stream) == 0
+        best = min(best, ms_c.value)
+    roofline["plain_read_kernel_GBps"] = (1 << 30) / best / 1e6
     log("[bench] hit path: %s" % hit)
     if args.only_hit:
         # a plain device copy of known size in the same process: the scale of the profiler's traffic counters
@@ -155,6 +164,10 @@ def main():
     ms = elapsed_ms(a, b)
     assert int(s_hit.item()) & (2**64 - 1) == O.bo_gather_sum(SEED, SEED, 0, N_READS, CACHE_PAGES * 512), "hit gather checksum mismatch"
     gather_hit = {"reads_per_s": N_READS / ms * 1e3, "GBps_of_u64": N_READS * 8 / ms / 1e6, "ms": ms}
+    for _ in range(2):      # the same index pattern as a plain gather from a flat 1 GiB array, no cache protocol
+        assert L.bam_gather_kernel(ctypes.c_void_p(probe.data_ptr()), ctypes.c_void_p(idx_hit.data_ptr()), ctypes.c_uint64(N_READS), ctypes.byref(ms_c), stream) == 0
+    gather_hit["plain_gather_reads_per_s"] = N_READS / ms_c.value * 1e3
+    del probe
     arr.stats()
     del idx_hit
     log("[bench] hit gather: %s" % gather_hit)

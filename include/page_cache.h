@@ -180,6 +180,18 @@ __device__ __forceinline__ void copy_pages(uint8_t* dst, const uint8_t* src, uin
         for (; i < nb; i += movers) d[i] = s[i];
     }
 }
+/*
+ * The same with helpers: called by all active lanes, of which those with `mine` have payload to move; the others
+ * lend their load slots.  A wave that loads one page for all of its lanes (a bam_ptr walking an edge list) moves it
+ * in one trip of 64 lanes instead of sixty-four trips of one.
+ */
+__device__ __forceinline__ void copy_pages_helped(uint8_t* dst, const uint8_t* src, uint32_t bytes, bool mine)
+{
+    const uint64_t owners = ballot(mine);
+    if (!owners) return;
+    const uint64_t all = active_mask();
+    copy_pages(dst, src, mine ? bytes : 0u, owners, popc(all), rank_in(all));
+}
 
 /*
  * One command per active lane on queue pair `qp` (wave-uniform), first half:
@@ -262,6 +274,35 @@ inline __device__ void access_data(page_cache_d_t* pc, QueuePair* qp, const uint
         QueuePair* cur = (QueuePair*)bam::first((uint64_t)qp);
         page_cache_d_t* cpc = (page_cache_d_t*)bam::first((uint64_t)pc);
         if (cur == qp && cpc == pc) { bam::io_group(cpc, cur, starting_lba, (uint32_t)n_blocks, pc_entry, opcode); done = true; }
+    }
+}
+
+/* read_data in two halves: submitted and completed, payload still in `stage` (NULL: already in the slot) | ids handed back */
+inline __device__ void read_begin(page_cache_d_t* pc, QueuePair* qp, const uint64_t starting_lba, const uint64_t n_blocks, const unsigned long long pc_entry,
+                                  uint32_t& cid, uint8_t*& stage)
+{
+    for (bool done = false; !done;) {
+        QueuePair* cur = (QueuePair*)bam::first((uint64_t)qp);
+        page_cache_d_t* cpc = (page_cache_d_t*)bam::first((uint64_t)pc);
+        if (cur == qp && cpc == pc) {
+            uint32_t pos;
+            cid = bam::io_submit_group(cpc, cur, starting_lba, (uint32_t)n_blocks, pc_entry, NVM_IO_READ, stage, pos);
+#ifdef BAM_PROFILE
+            const uint64_t pt2 = wall_clock64();
+#endif
+            bam::cq_wait_group(&cur->cq, &cur->sq, cid);
+#ifdef BAM_PROFILE
+            if (cpc->prof && bam::lane() == bam::first_lane(bam::active_mask())) atomicAdd(&cpc->prof[4], wall_clock64() - pt2);
+#endif
+            done = true;
+        }
+    }
+}
+inline __device__ void read_end(QueuePair* qp, const uint32_t cid)
+{
+    for (bool done = false; !done;) {
+        QueuePair* cur = (QueuePair*)bam::first((uint64_t)qp);
+        if (cur == qp) { bam::put_cid_group(&cur->sq, cid); done = true; }
     }
 }
 
@@ -440,7 +481,8 @@ struct range_d_t {
     __forceinline__ __device__ uint64_t acquire_page(const size_t pg, const uint32_t count, const bool write, const uint32_t ctrl, const uint32_t queue);
     /* spread by workgroup so that no counter word is shared by more than a few waves at a time */
     __forceinline__ __device__ bam_stat_shard_t* shard() const { return stats + (((blockIdx.x + blockIdx.y * gridDim.x) * 0x9E3779B1u) >> 20) % BAM_STAT_SHARDS; }
-    __forceinline__ __device__ bool slow_step(const size_t pg, const bool write, const uint32_t queue, uint64_t& sv, uint32_t& slot, bool& was_hit, bool& progressed);
+    __forceinline__ __device__ bool slow_step(const size_t pg, const bool write, const uint32_t queue, uint64_t& sv, uint32_t& slot, bool& was_hit, bool& progressed, const bool take_part = true,
+                                              const bool may_load = true, bool* wants_load = nullptr);
 };
 
 /*
@@ -515,55 +557,117 @@ __device__ __forceinline__ void stat_add(unsigned long long* ctr, uint32_t v)
  */
 template <typename T>
 __forceinline__ __device__
-bool range_d_t<T>::slow_step(const size_t pg, const bool write, const uint32_t queue, uint64_t& sv, uint32_t& slot, bool& was_hit, bool& progressed)
+bool range_d_t<T>::slow_step(const size_t pg, const bool write, const uint32_t queue, uint64_t& sv, uint32_t& slot, bool& was_hit, bool& progressed, const bool take_part,
+                             const bool may_load, bool* wants_load)
 {
     using namespace bam;
     data_page_t* dp = &pages[pg];
     bool load_me = false, resolved = false;
     const uint32_t s = (uint32_t)sv, st = s >> (CNT_SHIFT + 1);
     progressed = false;
-    if (st == V_NB) {
+    if (!take_part) {
+        /* here only to help move payload */
+    } else if (st == V_NB) {
         if (write && (s & DIRTY) == 0) __hip_atomic_fetch_or(&dp->state, DIRTY, __ATOMIC_RELAXED, BAM_AGENT);
         slot = (uint32_t)(sv >> 32);
         was_hit = true;
         resolved = true;
     } else if (st == NV_NB) {
-        const uint32_t o = __hip_atomic_fetch_or(&dp->state, BUSY, __ATOMIC_ACQUIRE, BAM_AGENT);
-        if ((o & BUSY) == 0) {
-            if ((o >> (CNT_SHIFT + 1)) == NV_NB) load_me = true;
-            else __hip_atomic_fetch_and(&dp->state, DISABLE_BUSY_MASK, __ATOMIC_RELEASE, BAM_AGENT);  /* became valid meanwhile */
+        if (!may_load) {
+            *wants_load = true;                 /* the caller has to be admitted to the miss path first */
+        } else {
+            const uint32_t o = __hip_atomic_fetch_or(&dp->state, BUSY, __ATOMIC_ACQUIRE, BAM_AGENT);
+            if ((o & BUSY) == 0) {
+                if ((o >> (CNT_SHIFT + 1)) == NV_NB) load_me = true;
+                else __hip_atomic_fetch_and(&dp->state, DISABLE_BUSY_MASK, __ATOMIC_RELEASE, BAM_AGENT);  /* became valid meanwhile */
+            }
         }
     }
+    uint32_t found = BAM_NO_SLOT, cid = 0;
+    uint8_t* stage = nullptr;
+    QueuePair* qp = nullptr;
     if (load_me) {
 #ifdef BAM_PROFILE
         const uint64_t pf0 = wall_clock64();
 #endif
-        const uint32_t found = cache.find_slot(pg, range_id, queue);
+        found = cache.find_slot(pg, range_id, queue);
 #ifdef BAM_PROFILE
         if (cache.prof && bam::lane() == bam::first_lane(bam::active_mask())) { atomicAdd(&cache.prof[6], wall_clock64() - pf0); atomicAdd(&cache.prof[7], 1ull); atomicAdd(&cache.prof[8], (unsigned long long)bam::popc(bam::active_mask())); }
 #endif
         if (found == BAM_NO_SLOT) {
             /* no evictable slot right now: hand the page back; a later pass tries again */
             __hip_atomic_fetch_and(&dp->state, DISABLE_BUSY_MASK, __ATOMIC_RELEASE, BAM_AGENT);
+            load_me = false;
         } else {
             uint64_t c = get_backing_ctrl(pg);
             if (c == ALL_CTRLS) c = cache.n_ctrls == 1 ? 0 : cache.ctrl_counter->fetch_add(1, simt::memory_order_relaxed) % cache.n_ctrls;
             Controller* ctl = cache.d_ctrls[c];
             stat_add((unsigned long long*)&ctl->access_counter, 1);
             stat_add(&shard()->read_io_cnt, 1);
-            read_data(&cache, ctl->d_qps + (queue % ctl->n_qps), get_backing_page(pg) * cache.n_blocks_per_page, cache.n_blocks_per_page, found);
-            st_relaxed(&dp->offset, found);
-            if (write) __hip_atomic_fetch_or(&dp->state, DIRTY, __ATOMIC_RELAXED, BAM_AGENT);
-            /* BUSY -> 0 and VALID -> 1 in one step; publishes the payload and the offset */
-            __hip_atomic_fetch_xor(&dp->state, DISABLE_BUSY_ENABLE_VALID, __ATOMIC_RELEASE, BAM_AGENT);
-            slot = found;
-            was_hit = false;
-            resolved = true;
-            progressed = true;
+            qp = ctl->d_qps + (queue % ctl->n_qps);
+            read_begin(&cache, qp, get_backing_page(pg) * cache.n_blocks_per_page, cache.n_blocks_per_page, found, cid, stage);
         }
     }
-    if (!resolved) sv = __hip_atomic_load((uint64_t*)dp, __ATOMIC_RELAXED, BAM_AGENT);
+    /* staged payload is moved by every lane that came in, whether it loaded a page itself or not */
+#ifdef BAM_PROFILE
+    const uint64_t pc0 = wall_clock64();
+#endif
+    copy_pages_helped(cache.base_addr + (uint64_t)found * cache.page_size, stage, (uint32_t)cache.page_size, load_me && stage != nullptr);
+#ifdef BAM_PROFILE
+    if (cache.prof && bam::ballot(load_me) && bam::lane() == bam::first_lane(bam::active_mask())) atomicAdd(&cache.prof[5], wall_clock64() - pc0);
+#endif
+    if (load_me) {
+        read_end(qp, cid);
+        st_relaxed(&dp->offset, found);
+        if (write) __hip_atomic_fetch_or(&dp->state, DIRTY, __ATOMIC_RELAXED, BAM_AGENT);
+        /* BUSY -> 0 and VALID -> 1 in one step; publishes the payload and the offset */
+        __hip_atomic_fetch_xor(&dp->state, DISABLE_BUSY_ENABLE_VALID, __ATOMIC_RELEASE, BAM_AGENT);
+        slot = found;
+        was_hit = false;
+        resolved = true;
+        progressed = true;
+    }
+    if (take_part && !resolved) sv = __hip_atomic_load((uint64_t*)dp, __ATOMIC_RELAXED, BAM_AGENT);
     return resolved;
+}
+
+/*
+ * slow_step as a function of its own, values in and values out.  It holds everything that is heavy in registers
+ * (victim search, command submission, completion handling, payload copy); kept out of line, the callers' path for
+ * resident pages stays lean, and what has to be saved around the call is saved on the miss path only.
+ */
+struct bam_pass_t { uint64_t sv; uint32_t slot; uint32_t flags; };
+#define BAM_PASS_RESOLVED   1u
+#define BAM_PASS_HIT        2u
+#define BAM_PASS_PROGRESSED 4u
+#define BAM_PASS_WANTS      8u
+#define BAM_PASS_WRITE      16u     /* in: */
+#define BAM_PASS_TAKE_PART  32u
+#define BAM_PASS_MAY_LOAD   64u
+template <typename T>
+__forceinline__ __device__ bam_pass_t bam_slow_pass_inline(range_d_t<T>* r, const uint64_t pg, const uint32_t queue, uint64_t sv, uint32_t slot, const uint32_t in)
+{
+    bool hit = false, progressed = false, wants = false;
+    const bool resolved = r->slow_step(pg, (in & BAM_PASS_WRITE) != 0, queue, sv, slot, hit, progressed, (in & BAM_PASS_TAKE_PART) != 0,
+                                       (in & BAM_PASS_MAY_LOAD) != 0, &wants);
+    bam_pass_t out;
+    out.sv = sv;
+    out.slot = slot;
+    out.flags = (resolved ? BAM_PASS_RESOLVED : 0u) | (hit ? BAM_PASS_HIT : 0u) | (progressed ? BAM_PASS_PROGRESSED : 0u) | (wants ? BAM_PASS_WANTS : 0u);
+    return out;
+}
+template <typename T>
+__attribute__((noinline)) __device__ bam_pass_t bam_slow_pass_call(range_d_t<T>* r, const uint64_t pg, const uint32_t queue, uint64_t sv, uint32_t slot, const uint32_t in)
+{
+    return bam_slow_pass_inline(r, pg, queue, sv, slot, in);
+}
+/* OUTLINE: as a call (measured best for kernels that are mostly misses: one thread per random element) or expanded in
+ * place (best where the caller is mostly hits and would otherwise carry the callee's register budget) */
+template <bool OUTLINE, typename T>
+__forceinline__ __device__ bam_pass_t bam_slow_pass(range_d_t<T>* r, const uint64_t pg, const uint32_t queue, uint64_t sv, uint32_t slot, const uint32_t in)
+{
+    if constexpr (OUTLINE) return bam_slow_pass_call(r, pg, queue, sv, slot, in);
+    else return bam_slow_pass_inline(r, pg, queue, sv, slot, in);
 }
 
 /* the reference's entry point: references + slot, and the access is accounted in the range's counters */
@@ -580,8 +684,10 @@ uint64_t range_d_t<T>::acquire_page(const size_t pg, const uint32_t count, const
         bool resolved = false;
         bam::spin_t sp;
         for (;;) {
-            bool progressed = false;
-            if (!resolved) resolved = slow_step(pg, write, queue, sv, slot, hit, progressed);
+            /* resolved lanes go in too: they help move payload */
+            const bam_pass_t ps = bam_slow_pass<false>(this, pg, queue, sv, slot, (write ? BAM_PASS_WRITE : 0u) | (resolved ? 0u : BAM_PASS_TAKE_PART) | BAM_PASS_MAY_LOAD);
+            const bool progressed = (ps.flags & BAM_PASS_PROGRESSED) != 0;
+            if (!resolved) { sv = ps.sv; slot = ps.slot; hit = (ps.flags & BAM_PASS_HIT) != 0; resolved = (ps.flags & BAM_PASS_RESOLVED) != 0; }
             if (!bam::ballot(!resolved)) break;
             if (!bam::ballot(progressed) && cache.spin_giveup(sp)) { if (!resolved) slot = 0; break; }
         }
@@ -666,7 +772,7 @@ struct range_view {
      * wave that waits for I/O holds no reference on anything but the pages it
      * is loading.  `on_miss(slot)` runs for those lanes once their page is in.
      */
-    template <typename FH, typename FM>
+    template <bool OUTLINE = false, typename FH, typename FM>
     __forceinline__ __device__ void acquire(const uint64_t page, const bool write, FH&& on_hit, FM&& on_miss)
     {
         const uint32_t me = lane();
@@ -678,11 +784,12 @@ struct range_view {
         uint32_t slot = 0;
         if (master == me) { const bool h = bam_try_hit(dp, count, dirty, sv, slot); pack = (uint64_t)slot | ((uint64_t)h << 63); }
         pack = shfl(pack, master);
-        if (pack >> 63) {
+        if (__builtin_expect((pack >> 63) != 0, 1)) {          /* resident: the path to keep lean; register spills, if any, belong in the other branch */
             account(true);
             const bool drop = on_hit((uint32_t)pack);
-            __builtin_amdgcn_wave_barrier();
-            if (drop && master == me) bam_release_refs(dp, count, dirty);
+            /* the lanes of a group may answer differently (one keeps the page, another only touched it) */
+            const uint32_t n_drop = popc(ballot(drop) & eq_mask);
+            if (n_drop && master == me) bam_release_refs(dp, n_drop, dirty);
         } else {
             /* miss path: pass after pass; groups whose page came in are served and release before the next pass */
             const uint32_t queue = wave_slot_hash();
@@ -690,65 +797,80 @@ struct range_view {
             bool done = false;
             spin_t sp;
             /*
-             * Admission: only so many waves per compute unit work on misses at a time.  Every wave in here polls
-             * queues and page states while its I/O is in flight; with all resident waves doing that at once the
-             * polling itself takes the memory system and the interconnect away from the waves that are moving
-             * payload, and throughput drops.  One counter per compute unit, 64 bytes apart: waiting waves poll
-             * their own unit's word.
+             * Admission: only so many waves per compute unit load pages at a time.  Every wave that has I/O in
+             * flight polls queues and command words; with all resident waves doing that at once the polling itself
+             * takes the memory system and the interconnect away from the waves that are moving payload, and
+             * throughput drops.  A wave asks for admission when one of its pages is there to be loaded, and steps
+             * out again whenever it finds itself only waiting for pages that other waves are loading.  One counter
+             * per compute unit, 64 bytes apart: waiting waves poll their own unit's word.
              */
             page_cache_d_t* cache = (page_cache_d_t*)first((uint64_t)&r->cache);
             const uint32_t limit = cache->miss_waves;
             uint32_t* tokens = cache->miss_tokens + (cu_id() & (BAM_TOKEN_SLOTS - 1)) * 16;
             bool admitted = limit == 0;
-            if (!admitted) {
-                uint32_t ok = 0;
-                if (me == leader) {
-                    if (__hip_atomic_fetch_add(tokens, 1u, __ATOMIC_RELAXED, BAM_AGENT) < limit) ok = 1;
-                    else __hip_atomic_fetch_add(tokens, 0u - 1u, __ATOMIC_RELAXED, BAM_AGENT);
-                }
-                admitted = bcast(ok, leader) != 0;
-            }
-            if (!admitted) {
-                /*
-                 * Queue up outside without references: a page that somebody else brings in meanwhile must stay
-                 * evictable, or the waves that wait here could pin every slot the admitted ones need.
-                 */
-                if (master == me) __hip_atomic_fetch_add(&dp->state, 0u - count, __ATOMIC_RELAXED, BAM_AGENT);
-                uint32_t ok = 0;
-                if (me == leader) {
-                    for (uint32_t i = 1;; i++) {
-                        if (ld_relaxed(tokens) < limit) {
-                            if (__hip_atomic_fetch_add(tokens, 1u, __ATOMIC_RELAXED, BAM_AGENT) < limit) { ok = 1; break; }
-                            __hip_atomic_fetch_add(tokens, 0u - 1u, __ATOMIC_RELAXED, BAM_AGENT);
-                        }
-                        __builtin_amdgcn_s_sleep(127);
-                        __builtin_amdgcn_s_sleep(127);
-                        __builtin_amdgcn_s_sleep(127);
-                        __builtin_amdgcn_s_sleep(127);
-                        /* no clock of its own: the waves inside time their waits, this one only watches for their verdict */
-                        if ((i & 63u) == 0 && cache->guard && ld_relaxed_sys(&cache->guard->abort)) break;
-                    }
-                }
-                admitted = bcast(ok, leader) != 0;
-                if (master == me) bam_try_hit(dp, count, dirty, sv, slot);     /* slow_step reads the outcome from sv */
-            }
             for (;;) {
-                bool progressed = false;
+                /* every lane of the miss branch goes in: the masters that still wait for their page take part, the rest help move payload */
+                const bool part = !done && master == me;
+                const bam_pass_t ps = bam_slow_pass<OUTLINE>(r, page, queue, sv, slot,
+                                                    (dirty ? BAM_PASS_WRITE : 0u) | (part ? BAM_PASS_TAKE_PART : 0u) | (admitted ? BAM_PASS_MAY_LOAD : 0u));
+                const bool progressed = (ps.flags & BAM_PASS_PROGRESSED) != 0, wants = (ps.flags & BAM_PASS_WANTS) != 0;
+                if (part) {
+                    sv = ps.sv;
+                    pack = (uint64_t)ps.slot | ((uint64_t)((ps.flags & BAM_PASS_HIT) != 0) << 63) | ((uint64_t)((ps.flags & BAM_PASS_RESOLVED) != 0) << 62);
+                }
                 if (!done) {
-                    bool hit = false, resolved = false;
-                    if (master == me) { resolved = r->slow_step(page, dirty, queue, sv, slot, hit, progressed); pack = (uint64_t)slot | ((uint64_t)hit << 63) | ((uint64_t)resolved << 62); }
                     pack = shfl(pack, master);
                     if ((pack >> 62) & 1) {
                         account((pack >> 63) != 0);
                         const bool drop = on_miss((uint32_t)pack);
-                        __builtin_amdgcn_wave_barrier();
-                        if (drop && master == me) bam_release_refs(dp, count, dirty);
+                        const uint32_t n_drop = popc(ballot(drop) & eq_mask);
+                        if (n_drop && master == me) bam_release_refs(dp, n_drop, dirty);
                         done = true;
                     }
                 }
                 if (!ballot(!done)) break;
+                if (!admitted && ballot(wants)) {
+                    const bool holder = !done && master == me;                 /* lanes that hold their group's references */
+                    uint32_t ok = 0;
+                    if (me == leader) {
+                        if (__hip_atomic_fetch_add(tokens, 1u, __ATOMIC_RELAXED, BAM_AGENT) < limit) ok = 1;
+                        else __hip_atomic_fetch_add(tokens, 0u - 1u, __ATOMIC_RELAXED, BAM_AGENT);
+                    }
+                    if (!bcast(ok, leader)) {
+                        /*
+                         * Queue up without references: a page that somebody else brings in meanwhile must stay
+                         * evictable, or the waves that wait here could pin every slot the admitted ones need.
+                         */
+                        if (holder) __hip_atomic_fetch_add(&dp->state, 0u - count, __ATOMIC_RELAXED, BAM_AGENT);
+                        if (me == leader) {
+                            for (uint32_t i = 1;; i++) {
+                                if (ld_relaxed(tokens) < limit) {
+                                    if (__hip_atomic_fetch_add(tokens, 1u, __ATOMIC_RELAXED, BAM_AGENT) < limit) { ok = 1; break; }
+                                    __hip_atomic_fetch_add(tokens, 0u - 1u, __ATOMIC_RELAXED, BAM_AGENT);
+                                }
+                                __builtin_amdgcn_s_sleep(127);
+                                __builtin_amdgcn_s_sleep(127);
+                                __builtin_amdgcn_s_sleep(127);
+                                __builtin_amdgcn_s_sleep(127);
+                                /* no clock of its own: the waves inside time their waits, this one only watches for their verdict */
+                                if ((i & 15u) == 0 && cache->guard && ld_relaxed_sys(&cache->guard->abort)) break;
+                            }
+                        }
+                        if (holder) bam_try_hit(dp, count, dirty, sv, slot);   /* the next pass reads the outcome from sv */
+                    }
+                    admitted = bcast(ok, leader) != 0;
+                    if (!admitted) break;                                      /* only an abort ends the wait without admission */
+                    continue;
+                }
                 if (ballot(progressed)) sp = spin_t();
-                else if (cache->spin_giveup(sp)) break;
+                else {
+                    /* only waiting for pages other waves are loading: make room for a wave that has something to load */
+                    if (limit && admitted) {
+                        if (me == leader) __hip_atomic_fetch_add(tokens, 0u - 1u, __ATOMIC_RELAXED, BAM_AGENT);
+                        admitted = false;
+                    }
+                    if (cache->spin_giveup(sp)) break;
+                }
             }
             if (limit && admitted && me == leader) __hip_atomic_fetch_add(tokens, 0u - 1u, __ATOMIC_RELAXED, BAM_AGENT);
         }
@@ -817,7 +939,7 @@ struct array_d_t {
         if (!view_of(i, v)) return;
         const uint64_t byte = v.byte_of(i);
         auto use = [&](uint32_t slot) { fn((T*)(v.slot_addr(slot) + (byte & (v.page_size - 1)))); return true; };
-        v.acquire(byte >> v.page_size_log, write, use, use);
+        v.template acquire<true>(byte >> v.page_size_log, write, use, use);
         v.template flush_stats<false>();
     }
 
