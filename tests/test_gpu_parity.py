@@ -176,6 +176,24 @@ def test_large_pages_through_bigger_staging(bam):
         assert r.t.stats()["bytes_read"] == a.stats()["read_io_cnt"] * 8192
 
 
+def test_direct_placement_without_staging(bam):
+    """stage_bytes = 0: PRPs name the cache slots themselves and the controller writes the payload into device memory"""
+    from bam_amd import gen
+    n_elems, n = 1 << 22, 1 << 18
+    with Rig(bam, 32 << 20, n_queues=8, depth=256, stage_bytes=0, backing=True) as r:
+        a = r.array(n_elems, 4096, 1024)
+        assert r.objs[0][2].info()["staged"] == 0
+        for rep in range(2):
+            idx = gen.gather_indices(SEED, n, n_elems, first=rep * n)
+            assert a.read(n, idx, block_size=128) == oracle.lib().bo_gather_sum(SEED, SEED, rep * n, n, n_elems)
+        # the write path the other way: dirty pages are read by the controller out of device memory
+        vals = np.arange(1 << 16, dtype=np.uint64) * np.uint64(7) + np.uint64(3)
+        a.write(1 << 16, _dev(vals), block_size=64)
+        r.objs[0][2].flush()
+        assert np.array_equal(r.backing(1 << 16), vals)
+        assert a.stats()["read_io_cnt"] > 0 and not r.c.aborted()
+
+
 # ---------------------------------------------------------------- cache / pattern streaming
 
 @pytest.mark.parametrize("mode", [0, 1, 2])
