@@ -712,7 +712,8 @@ int bam_page_cache_info(bam_page_cache_t* pc, uint64_t* out)
     out[0] = pc->pc->pdt.n_pages;
     out[1] = pc->pc->pdt.page_size;
     out[2] = pc->pc->pdt.wave_batch;
-    out[3] = pc->pc->pdt.prp1 == nullptr;
+    out[3] = pc->ctrl->n_qps && pc->ctrl->h_qps[0]->stage != nullptr;
+    out[4] = pc->pc->pdt.direct_share;
     return 0;
 }
 

@@ -116,9 +116,9 @@ class PageCache:
         _chk(self.L.bam_page_cache_create(ctypes.byref(self.h), page_size, n_pages, device, ctrl.h, max_range), "bam_page_cache_create")
 
     def info(self):
-        out = (c_u64 * 4)()
+        out = (c_u64 * 5)()
         _chk(self.L.bam_page_cache_info(self.h, out), "bam_page_cache_info")
-        return dict(zip(("n_pages", "page_size", "wave_batch", "staged"), list(out)))
+        return dict(zip(("n_pages", "page_size", "wave_batch", "staged", "direct_share"), list(out)))
 
     def flush(self):
         _chk(self.L.bam_page_cache_flush(self.h), "bam_page_cache_flush")

@@ -57,7 +57,7 @@ int bam_ctrl_aborted(bam_ctrl_t* c, int clear);
 /* ---- page_cache_t / range_t<uint64_t> / array_t<uint64_t> (include/page_cache.h:697-875, 984-1030, 1754-1772) ---- */
 int bam_page_cache_create(bam_page_cache_t** out, uint64_t page_size, uint64_t n_pages, uint32_t device, bam_ctrl_t* ctrl, uint64_t max_range);
 void bam_page_cache_destroy(bam_page_cache_t* pc);
-/* out[4]: n_pages, page_size, wave_batch, staged(0/1) */
+/* out[5]: n_pages, page_size, wave_batch, staged(0/1), of every 8 read batches how many bypass the staging pages */
 int bam_page_cache_info(bam_page_cache_t* pc, uint64_t* out);
 int bam_page_cache_flush(bam_page_cache_t* pc);
 /* phase timers of the miss path (100 MHz ticks), non-zero only in a library built with -DBAM_PROFILE; out16[0..8]:
