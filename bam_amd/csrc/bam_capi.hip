@@ -385,7 +385,7 @@ __global__ __launch_bounds__(128) void k_cc_coalesce_coarse_ptr_pc(array_d_t<uin
     }
 }
 
-// ---- BFS / CC by edge page: the same relaxations, work laid out along the edge array ----
+// ---- BFS / CC by edge page (benchmarks/bfs/main.cu:1074-1140 kernel_optimized_ptr_pc, first-vertex table :122-181) ----
 /*
  * first[p], p = 0 .. n_pages: the vertex whose edge list holds edge p * epp (the last vertex with
  * offsets[v] <= p * epp); first[n_pages] = V - 1.  The vertices with edges on page p are first[p] .. first[p + 1].

@@ -131,12 +131,13 @@ int bam_cc(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, u
            uint32_t coarse, uint32_t* iterations, void* stream);
 
 /* ---- the same two traversals, laid out along the edge array instead of along the vertices ----
- * Same inputs, same outputs (levels / labels are unique, so they are bit-identical to bam_bfs / bam_cc).  A wave takes
- * runs of consecutive edge pages, acquires the pages that hold edges of active vertices with one call (their misses
- * reach the store as one batch of up to 64 commands) and relaxes those vertices' edges from the resident pages.
- * No counterpart in the reference, whose kernels (benchmarks/bfs/main.cu:658-689, benchmarks/cc/main.cu:595-617) give
- * one warp to one vertex and so issue one page read at a time per warp.  The array must consist of one range that
- * starts on a page boundary. */
+ * The reference's page-tiled variant (benchmarks/bfs/main.cu:1074-1140 kernel_optimized_ptr_pc, with the table of the
+ * first vertex of every page built by kernel_first_vertex_step1/2, :122-181; the same in benchmarks/cc): one warp per
+ * page of the edge array, which it walks vertex by vertex.  Here a wave takes a run of up to 64 consecutive pages,
+ * acquires those that hold edges of active vertices with one call (their misses reach the store as one batch of
+ * commands) and relaxes those vertices' edges from the resident pages; the table is built by binary search.
+ * Same inputs, same outputs as bam_bfs / bam_cc (levels and labels are unique, so they are bit-identical).
+ * The array must consist of one range that starts on a page boundary. */
 int bam_bfs_by_page(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t src, uint32_t* d_labels,
                     uint32_t* iterations, void* stream);
 int bam_cc_by_page(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t* d_labels, uint32_t* iterations, void* stream);
