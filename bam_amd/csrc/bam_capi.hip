@@ -45,7 +45,7 @@ struct bam_target {
     nvmt_config_t cfg{};
 };
 struct bam_ctrl { Controller* c; };
-struct bam_page_cache { page_cache_t* pc; Controller* ctrl; };
+struct bam_page_cache { page_cache_t* pc; Controller* ctrl; };      /* ctrl: the first controller of the cache */
 struct bam_range { range_t<uint64_t>* r; };
 #define BAM_SUM_PARTIALS 4096
 struct bam_array { array_t<uint64_t>* a; BufferPtr partials; };      /* partials: [BAM_SUM_PARTIALS] checksum shards, zero between launches */
@@ -240,13 +240,9 @@ __device__ __forceinline__ void cache_stream_body(array_d_t<uint64_t>* dr, uint6
     block_accumulate(sum, v);
 }
 
-/*
- * One kernel per mode, each with the register budget that suits it: the two per-element kernels live on occupancy
- * (every page change is a dependent chain of atomics and loads) and are held at four waves per SIMD; the page-wise
- * kernel keeps sixty-four bytes per lane in flight and runs best with the registers it asks for.
- */
+/* one kernel per mode; the page-wise one has a name of its own because it is the one the hit-path roofline is quoted on */
 template <int MODE>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void k_cache_stream(array_d_t<uint64_t>* dr, uint64_t n_waves, uint64_t n_pages_per_wave, const uint64_t* assignment, unsigned long long* sum)
+__global__ __launch_bounds__(256) void k_cache_stream(array_d_t<uint64_t>* dr, uint64_t n_waves, uint64_t n_pages_per_wave, const uint64_t* assignment, unsigned long long* sum)
 {
     cache_stream_body<MODE>(dr, n_waves, n_pages_per_wave, assignment, sum);
 }
@@ -696,6 +692,22 @@ int bam_page_cache_create(bam_page_cache_t** out, uint64_t page_size, uint64_t n
     std::vector<Controller*> ctrls{ctrl->c};
     page_cache_t* pc = new page_cache_t(page_size, n_pages, device, *ctrl->c, max_range, ctrls);
     *out = new bam_page_cache{pc, ctrl->c};
+    BAM_API_END
+}
+
+int bam_page_cache_create_multi(bam_page_cache_t** out, uint64_t page_size, uint64_t n_pages, uint32_t device, bam_ctrl_t** ctrls, uint32_t n_ctrls,
+                                uint64_t max_range)
+{
+    if (!out || !ctrls || !n_ctrls) return fail(EINVAL, "bam_page_cache_create_multi: null argument");
+    *out = nullptr;
+    std::vector<Controller*> cs;
+    for (uint32_t i = 0; i < n_ctrls; i++) {
+        if (!ctrls[i]) return fail(EINVAL, "bam_page_cache_create_multi: null controller");
+        cs.push_back(ctrls[i]->c);
+    }
+    BAM_API_BEGIN
+    page_cache_t* pc = new page_cache_t(page_size, n_pages, device, *cs[0], max_range, cs);
+    *out = new bam_page_cache{pc, cs[0]};
     BAM_API_END
 }
 

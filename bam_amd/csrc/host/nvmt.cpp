@@ -283,7 +283,14 @@ void serve_sq(nvmt* t, IoThread* me, Sq& sq)
                 std::atomic_thread_fence(std::memory_order_acquire);
                 if (!nvm_cmd_seal_ok(&batch[got], sq.fetched + got)) break;
             }
-            if (got < n && !sq.retry_counted) { st_.bump(st_.sqe_retries); sq.retry_counted = true; }
+            if (got < n && !sq.retry_counted) {
+                st_.bump(st_.sqe_retries); sq.retry_counted = true;
+                if (getenv("NVMT_DEBUG_SEAL")) {
+                    const nvm_cmd_t& e = batch[got];
+                    fprintf(stderr, "[nvmt %p] sq %u slot %u: want ticket %u, entry dw0 %08x dw2 %08x dw3 %08x (seal %08x) slba %u head %u tail %u\n", (void*)t, sq.id,
+                            (sq.head + got) & mask, sq.fetched + got, e.dword[0], e.dword[2], e.dword[3], nvm_cmd_seal_value(&e, sq.fetched + got), e.dword[10], sq.head, tail);
+                }
+            }
             if (!got) return;
             sq.retry_counted = false;
             n = got;

@@ -111,9 +111,15 @@ class PageCache:
     def __init__(self, page_size, n_pages, device, ctrl, max_range=64):
         self.L = _lib.load()
         self.h = c_vp()
-        self.ctrl = ctrl
+        self.ctrls = list(ctrl) if isinstance(ctrl, (list, tuple)) else [ctrl]
+        self.ctrl = self.ctrls[0]
         self.device = device
-        _chk(self.L.bam_page_cache_create(ctypes.byref(self.h), page_size, n_pages, device, ctrl.h, max_range), "bam_page_cache_create")
+        if len(self.ctrls) == 1:
+            _chk(self.L.bam_page_cache_create(ctypes.byref(self.h), page_size, n_pages, device, self.ctrl.h, max_range), "bam_page_cache_create")
+        else:
+            arr = (c_vp * len(self.ctrls))(*[c.h for c in self.ctrls])
+            _chk(self.L.bam_page_cache_create_multi(ctypes.byref(self.h), page_size, n_pages, device, arr, len(self.ctrls), max_range),
+                 "bam_page_cache_create_multi")
 
     def info(self):
         out = (c_u64 * 5)()

@@ -56,6 +56,11 @@ int bam_ctrl_aborted(bam_ctrl_t* c, int clear);
 
 /* ---- page_cache_t / range_t<uint64_t> / array_t<uint64_t> (include/page_cache.h:697-875, 984-1030, 1754-1772) ---- */
 int bam_page_cache_create(bam_page_cache_t** out, uint64_t page_size, uint64_t n_pages, uint32_t device, bam_ctrl_t* ctrl, uint64_t max_range);
+/* one cache in front of several controllers (the `ctrls` vector of page_cache_t, include/page_cache.h:697-705): ranges
+ * created with dist = 1 (STRIPE) put page p on controller p % n at page p / n, ranges with dist = 0 (REPLICATE) expect
+ * the same data on every controller and spread their reads over them (:556-582) */
+int bam_page_cache_create_multi(bam_page_cache_t** out, uint64_t page_size, uint64_t n_pages, uint32_t device, bam_ctrl_t** ctrls, uint32_t n_ctrls,
+                                uint64_t max_range);
 void bam_page_cache_destroy(bam_page_cache_t* pc);
 /* out[5]: n_pages, page_size, wave_batch, staged(0/1), of every 8 read batches how many bypass the staging pages */
 int bam_page_cache_info(bam_page_cache_t* pc, uint64_t* out);

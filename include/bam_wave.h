@@ -23,7 +23,18 @@ namespace bam {
 
 __device__ __forceinline__ uint32_t lane() { return __lane_id(); }
 __device__ __forceinline__ uint64_t ballot(bool p) { return __builtin_amdgcn_ballot_w64(p); }
-__device__ __forceinline__ uint64_t active_mask() { return __builtin_amdgcn_ballot_w64(true); }
+/*
+ * The lanes executing right now, read from the execution mask itself.  A ballot of `true` says the same, but the
+ * compiler may move such a ballot out of a branch it sits in (it has no operands that tie it there), and the mask
+ * of the enclosing region is not the mask of the branch: inside "for each distinct queue of the wave: if (mine) {...}"
+ * that hands the group of one queue the lanes of all of them.
+ */
+__device__ __forceinline__ uint64_t active_mask()
+{
+    uint64_t m;
+    asm volatile("s_mov_b64 %0, exec" : "=s"(m));
+    return m;
+}
 __device__ __forceinline__ uint32_t popc(uint64_t m) { return (uint32_t)__builtin_popcountll(m); }
 __device__ __forceinline__ uint32_t first_lane(uint64_t m) { return (uint32_t)__builtin_ctzll(m); }
 __device__ __forceinline__ uint64_t lanes_below(uint32_t l) { return (1ull << l) - 1ull; }
@@ -76,6 +87,34 @@ __device__ __forceinline__ uint64_t match_any(uint64_t key_a, uint64_t key_b)
         if (eq) { mine = grp; done = true; }
     }
     return mine;
+}
+
+/*
+ * Run `body` once for each distinct key among the active lanes, with exactly the lanes that hold that key active.
+ *
+ * The loop is driven by a wave-uniform set of lanes still to be served, so every lane makes every trip and the
+ * branch around the body is the only place where the lanes part.  (Written the obvious way, "pick the first lane's
+ * key; the lanes that match do the work and leave the loop", the work sits right before a lane's loop exit, and the
+ * compiler is free to move it behind the loop, where all lanes are back together: group operations in the body,
+ * ballots, lane counts, elections of a leader, would then see the lanes of every key at once.)
+ */
+template <typename F>
+__device__ __forceinline__ void for_each_group(const uint64_t key_a, const uint64_t key_b, F&& body)
+{
+    uint64_t todo = active_mask();
+    while (todo) {
+        const uint32_t l = first_lane(todo);
+        const uint64_t a = bcast(key_a, l), b = bcast(key_b, l);
+        const bool mine = key_a == a && key_b == b;
+        const uint64_t grp = ballot(mine);
+        if (mine) body(a, b);
+        todo &= ~grp;
+    }
+}
+template <typename F>
+__device__ __forceinline__ void for_each_group(const uint64_t key, F&& body)
+{
+    for_each_group(key, 0, [&](uint64_t a, uint64_t) { body(a); });
 }
 
 /* compute-unit identity across the whole device: XCC, shader engine and CU bits */

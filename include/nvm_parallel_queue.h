@@ -112,19 +112,14 @@ __device__ __forceinline__ uint32_t get_cid_group(nvm_queue_t* sq)
 __device__ __forceinline__ void put_cid_group(nvm_queue_t* sq, uint32_t id)
 {
     st_relaxed(&sq->cid[id].val, (uint32_t)UNLOCKED);
-    const uint32_t b = id >> 6;
-    for (bool done = false; !done;) {
-        const uint32_t cur = first(b);
-        if (cur == b) {
-            const uint64_t grp = active_mask();
-            if (lane() == first_lane(grp)) {
-                const uint32_t k = popc(grp);
-                if (__hip_atomic_fetch_add(&sq->head_mark[cur].val, 0u - k, __ATOMIC_RELEASE, BAM_AGENT) == k)
-                    __hip_atomic_fetch_add(&sq->pos_locks[cur].val, 1u, __ATOMIC_RELEASE, BAM_AGENT);   /* next turn */
-            }
-            done = true;
+    for_each_group((uint64_t)(id >> 6), [&](uint64_t b) {
+        const uint64_t grp = active_mask();
+        if (lane() == first_lane(grp)) {
+            const uint32_t k = popc(grp);
+            if (__hip_atomic_fetch_add(&sq->head_mark[b].val, 0u - k, __ATOMIC_RELEASE, BAM_AGENT) == k)
+                __hip_atomic_fetch_add(&sq->pos_locks[b].val, 1u, __ATOMIC_RELEASE, BAM_AGENT);   /* next turn */
         }
-    }
+    });
 }
 
 __device__ __forceinline__ void cq_drain_group(nvm_queue_t* cq, nvm_queue_t* sq, uint64_t act);
@@ -306,30 +301,21 @@ __device__ __forceinline__ void cq_wait_group(nvm_queue_t* cq, nvm_queue_t* sq, 
 inline __device__ uint16_t get_cid(nvm_queue_t* sq)
 {
     uint32_t id = 0;
-    for (bool done = false; !done;) {
-        nvm_queue_t* cur = (nvm_queue_t*)bam::first((uint64_t)sq);
-        if (cur == sq) { id = bam::get_cid_group(cur); done = true; }
-    }
+    bam::for_each_group((uint64_t)sq, [&](uint64_t q) { id = bam::get_cid_group((nvm_queue_t*)q); });
     return (uint16_t)id;
 }
 
-/* to be called by the same lanes that called get_cid together */
+/* to be called by the same lanes that called get_cid together, all at once or in parts */
 inline __device__ void put_cid(nvm_queue_t* sq, uint16_t id)
 {
-    for (bool done = false; !done;) {
-        nvm_queue_t* cur = (nvm_queue_t*)bam::first((uint64_t)sq);
-        if (cur == sq) { bam::put_cid_group(cur, id); done = true; }
-    }
+    bam::for_each_group((uint64_t)sq, [&](uint64_t q) { bam::put_cid_group((nvm_queue_t*)q, id); });
 }
 
 /* returns the SQ slot used */
 inline __device__ uint16_t sq_enqueue(nvm_queue_t* sq, nvm_cmd_t* cmd)
 {
     uint32_t pos = 0;
-    for (bool done = false; !done;) {
-        nvm_queue_t* cur = (nvm_queue_t*)bam::first((uint64_t)sq);
-        if (cur == sq) { pos = bam::sq_enqueue_group(cur, cmd); done = true; }
-    }
+    bam::for_each_group((uint64_t)sq, [&](uint64_t q) { pos = bam::sq_enqueue_group((nvm_queue_t*)q, cmd); });
     return (uint16_t)pos;
 }
 
@@ -342,10 +328,7 @@ inline __device__ uint16_t sq_enqueue(nvm_queue_t* sq, nvm_cmd_t* cmd)
  */
 inline __device__ uint32_t cq_poll(nvm_queue_t* cq, uint16_t search_cid, uint32_t* loc_ = nullptr, uint32_t* cq_head = nullptr)
 {
-    for (bool done = false; !done;) {
-        nvm_queue_t* cur = (nvm_queue_t*)bam::first((uint64_t)cq);
-        if (cur == cq) { bam::cq_wait_group(cur, (nvm_queue_t*)cur->pair, search_cid); done = true; }
-    }
+    bam::for_each_group((uint64_t)cq, [&](uint64_t q) { bam::cq_wait_group((nvm_queue_t*)q, (nvm_queue_t*)((nvm_queue_t*)q)->pair, search_cid); });
     uint32_t h = bam::ld_relaxed(&cq->head);
     if (loc_) *loc_ = h;
     if (cq_head) *cq_head = h;

@@ -278,40 +278,48 @@ __device__ __forceinline__ void io_group(page_cache_d_t* pc, QueuePair* qp, uint
 
 inline __device__ void access_data(page_cache_d_t* pc, QueuePair* qp, const uint64_t starting_lba, const uint64_t n_blocks, const unsigned long long pc_entry, const uint8_t opcode)
 {
-    for (bool done = false; !done;) {
-        QueuePair* cur = (QueuePair*)bam::first((uint64_t)qp);
-        page_cache_d_t* cpc = (page_cache_d_t*)bam::first((uint64_t)pc);
-        if (cur == qp && cpc == pc) { bam::io_group(cpc, cur, starting_lba, (uint32_t)n_blocks, pc_entry, opcode); done = true; }
-    }
+    bam::for_each_group((uint64_t)qp, (uint64_t)pc, [&](uint64_t q, uint64_t c) {
+        bam::io_group((page_cache_d_t*)c, (QueuePair*)q, starting_lba, (uint32_t)n_blocks, pc_entry, opcode);
+    });
 }
 
-/* read_data in two halves: submitted and completed, payload still in `stage` (NULL: already in the slot) | ids handed back */
+/*
+ * read_data in two halves: submitted and completed, payload still in `stage` (NULL: already in the slot) | ids handed
+ * back.  The split exists so that between the halves every lane of the wave can help move the payload.  It is only
+ * taken when the calling lanes form one group (one queue pair, one cache): a wave that holds the command ids of one
+ * queue while it waits for ids of another could end up waiting for a wave that does the same the other way round, so
+ * with several groups each one runs its whole transfer before the next starts, and `held` comes back false.
+ */
 inline __device__ void read_begin(page_cache_d_t* pc, QueuePair* qp, const uint64_t starting_lba, const uint64_t n_blocks, const unsigned long long pc_entry,
-                                  uint32_t& cid, uint8_t*& stage)
+                                  uint32_t& cid, uint8_t*& stage, bool& held)
 {
-    for (bool done = false; !done;) {
-        QueuePair* cur = (QueuePair*)bam::first((uint64_t)qp);
-        page_cache_d_t* cpc = (page_cache_d_t*)bam::first((uint64_t)pc);
-        if (cur == qp && cpc == pc) {
-            uint32_t pos;
-            cid = bam::io_submit_group(cpc, cur, starting_lba, (uint32_t)n_blocks, pc_entry, NVM_IO_READ, stage, pos);
-#ifdef BAM_PROFILE
-            const uint64_t pt2 = wall_clock64();
-#endif
-            bam::cq_wait_group(&cur->cq, &cur->sq, cid);
-#ifdef BAM_PROFILE
-            if (cpc->prof && bam::lane() == bam::first_lane(bam::active_mask())) atomicAdd(&cpc->prof[4], wall_clock64() - pt2);
-#endif
-            done = true;
-        }
+    const uint64_t all = bam::active_mask();
+    const bool one_group = bam::ballot(qp == (QueuePair*)bam::first((uint64_t)qp) && pc == (page_cache_d_t*)bam::first((uint64_t)pc)) == all;
+    held = one_group;
+    stage = nullptr;
+    cid = 0;
+    if (!one_group) {
+        bam::for_each_group((uint64_t)qp, (uint64_t)pc, [&](uint64_t q, uint64_t c) {
+            bam::io_group((page_cache_d_t*)c, (QueuePair*)q, starting_lba, (uint32_t)n_blocks, pc_entry, NVM_IO_READ);
+        });
+        return;
     }
+    QueuePair* cur = (QueuePair*)bam::first((uint64_t)qp);
+    page_cache_d_t* cpc = (page_cache_d_t*)bam::first((uint64_t)pc);
+    uint32_t pos;
+    cid = bam::io_submit_group(cpc, cur, starting_lba, (uint32_t)n_blocks, pc_entry, NVM_IO_READ, stage, pos);
+#ifdef BAM_PROFILE
+    const uint64_t pt2 = wall_clock64();
+#endif
+    bam::cq_wait_group(&cur->cq, &cur->sq, cid);
+#ifdef BAM_PROFILE
+    if (cpc->prof && bam::lane() == bam::first_lane(all)) atomicAdd(&cpc->prof[4], wall_clock64() - pt2);
+#endif
 }
+/* for the lanes of a read_begin that came back with `held`: one queue pair */
 inline __device__ void read_end(QueuePair* qp, const uint32_t cid)
 {
-    for (bool done = false; !done;) {
-        QueuePair* cur = (QueuePair*)bam::first((uint64_t)qp);
-        if (cur == qp) { bam::put_cid_group(&cur->sq, cid); done = true; }
-    }
+    bam::put_cid_group(&((QueuePair*)bam::first((uint64_t)qp))->sq, cid);
 }
 
 inline __device__ void read_data(page_cache_d_t* pc, QueuePair* qp, const uint64_t starting_lba, const uint64_t n_blocks, const unsigned long long pc_entry)
@@ -333,41 +341,35 @@ inline __device__ void write_data(page_cache_d_t* pc, QueuePair* qp, const uint6
 inline __device__ void access_data_async(page_cache_d_t* pc, QueuePair* qp, const uint64_t starting_lba, const uint64_t n_blocks, const unsigned long long pc_entry,
                                          const uint8_t opcode, uint16_t* cid, uint16_t* sq_pos)
 {
-    for (bool done = false; !done;) {
-        QueuePair* cur = (QueuePair*)bam::first((uint64_t)qp);
-        page_cache_d_t* cpc = (page_cache_d_t*)bam::first((uint64_t)pc);
-        if (cur == qp && cpc == pc) {
-            uint8_t* stage;
-            uint32_t pos;
-            const uint32_t id = bam::io_submit_group(cpc, cur, starting_lba, (uint32_t)n_blocks, pc_entry, opcode, stage, pos);
-            if (stage) {
-                cur->async_dst[id] = opcode == NVM_IO_READ ? (uint64_t)(cpc->base_addr + pc_entry * cpc->page_size) : 0;
-                cur->async_len[id] = (uint32_t)n_blocks << cur->block_size_log;
-            }
-            *cid = (uint16_t)id;
-            *sq_pos = (uint16_t)pos;
-            done = true;
+    bam::for_each_group((uint64_t)qp, (uint64_t)pc, [&](uint64_t q, uint64_t c) {
+        QueuePair* cur = (QueuePair*)q;
+        page_cache_d_t* cpc = (page_cache_d_t*)c;
+        uint8_t* stage;
+        uint32_t pos;
+        const uint32_t id = bam::io_submit_group(cpc, cur, starting_lba, (uint32_t)n_blocks, pc_entry, opcode, stage, pos);
+        if (stage) {
+            cur->async_dst[id] = opcode == NVM_IO_READ ? (uint64_t)(cpc->base_addr + pc_entry * cpc->page_size) : 0;
+            cur->async_len[id] = (uint32_t)n_blocks << cur->block_size_log;
         }
-    }
+        *cid = (uint16_t)id;
+        *sq_pos = (uint16_t)pos;
+    });
 }
 
 inline __device__ void poll_async(QueuePair* qp, uint16_t cid, uint16_t sq_pos)
 {
     (void)sq_pos;
-    for (bool done = false; !done;) {
-        QueuePair* cur = (QueuePair*)bam::first((uint64_t)qp);
-        if (cur == qp) {
-            const uint64_t act = bam::active_mask();
-            bam::cq_wait_group(&cur->cq, &cur->sq, cid);
-            uint8_t* dst = nullptr;
-            uint32_t len = 0;
-            if (cur->stage) { dst = (uint8_t*)cur->async_dst[cid]; len = cur->async_len[cid]; }
-            if (bam::ballot(dst != nullptr))
-                bam::copy_pages(dst, cur->stage + (size_t)cid * cur->stage_stride, dst ? len : 0, act, bam::popc(act), bam::rank_in(act));
-            bam::put_cid_group(&cur->sq, cid);
-            done = true;
-        }
-    }
+    bam::for_each_group((uint64_t)qp, [&](uint64_t q) {
+        QueuePair* cur = (QueuePair*)q;
+        const uint64_t act = bam::active_mask();
+        bam::cq_wait_group(&cur->cq, &cur->sq, cid);
+        uint8_t* dst = nullptr;
+        uint32_t len = 0;
+        if (cur->stage) { dst = (uint8_t*)cur->async_dst[cid]; len = cur->async_len[cid]; }
+        if (bam::ballot(dst != nullptr))
+            bam::copy_pages(dst, cur->stage + (size_t)cid * cur->stage_stride, dst ? len : 0, act, bam::popc(act), bam::rank_in(act));
+        bam::put_cid_group(&cur->sq, cid);
+    });
 }
 
 /* ------------------------------------------------------------------ */
@@ -533,17 +535,13 @@ namespace bam {
 template <int BITS = 7>
 __device__ __forceinline__ void stat_add(unsigned long long* ctr, uint32_t v)
 {
-    for (bool done = false; !done;) {
-        const uint64_t a0 = first((uint64_t)ctr);
-        if ((uint64_t)ctr == a0) {
-            unsigned long long total = 0;
+    for_each_group((uint64_t)ctr, [&](uint64_t a0) {
+        unsigned long long total = 0;
 #pragma unroll
-            for (uint32_t b = 0; b < BITS; b++) total += (unsigned long long)popc(ballot((v >> b) & 1u)) << b;
-            if (lane() == first_lane(active_mask()) && total)
-                __hip_atomic_fetch_add((unsigned long long*)a0, total, __ATOMIC_RELAXED, BAM_AGENT);
-            done = true;
-        }
-    }
+        for (uint32_t b = 0; b < BITS; b++) total += (unsigned long long)popc(ballot((v >> b) & 1u)) << b;
+        if (lane() == first_lane(active_mask()) && total)
+            __hip_atomic_fetch_add((unsigned long long*)a0, total, __ATOMIC_RELAXED, BAM_AGENT);
+    });
 }
 } // namespace bam
 
@@ -594,6 +592,7 @@ bool range_d_t<T>::slow_step(const size_t pg, const bool write, const uint32_t q
     uint32_t found = BAM_NO_SLOT, cid = 0;
     uint8_t* stage = nullptr;
     QueuePair* qp = nullptr;
+    bool held = false;
     if (load_me) {
 #ifdef BAM_PROFILE
         const uint64_t pf0 = wall_clock64();
@@ -613,7 +612,7 @@ bool range_d_t<T>::slow_step(const size_t pg, const bool write, const uint32_t q
             stat_add((unsigned long long*)&ctl->access_counter, 1);
             stat_add(&shard()->read_io_cnt, 1);
             qp = ctl->d_qps + (queue % ctl->n_qps);
-            read_begin(&cache, qp, get_backing_page(pg) * cache.n_blocks_per_page, cache.n_blocks_per_page, found, cid, stage);
+            read_begin(&cache, qp, get_backing_page(pg) * cache.n_blocks_per_page, cache.n_blocks_per_page, found, cid, stage, held);
         }
     }
     /* staged payload is moved by every lane that came in, whether it loaded a page itself or not */
@@ -625,7 +624,7 @@ bool range_d_t<T>::slow_step(const size_t pg, const bool write, const uint32_t q
     if (cache.prof && bam::ballot(load_me) && bam::lane() == bam::first_lane(bam::active_mask())) atomicAdd(&cache.prof[5], wall_clock64() - pc0);
 #endif
     if (load_me) {
-        read_end(qp, cid);
+        if (held) read_end(qp, cid);
         st_relaxed(&dp->offset, found);
         if (write) __hip_atomic_fetch_or(&dp->state, DIRTY, __ATOMIC_RELAXED, BAM_AGENT);
         /* BUSY -> 0 and VALID -> 1 in one step; publishes the payload and the offset */
@@ -1166,7 +1165,7 @@ struct bam_ptr {
         const uint64_t pg = view.page_of(i);
         uint32_t slot = 0;
         auto keep = [&](uint32_t s_) { slot = s_; return false; };
-        view.acquire(pg, false, keep, keep);
+        view.template acquire<true>(pg, false, keep, keep);
         page = view.pages + pg;
         view.window(pg, start, end);
         addr = (T*)(view.slot_addr(slot) + (view.byte_of(start) & (view.page_size - 1)));

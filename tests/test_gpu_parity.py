@@ -176,6 +176,70 @@ def test_large_pages_through_bigger_staging(bam):
         assert r.t.stats()["bytes_read"] == a.stats()["read_io_cnt"] * 8192
 
 
+def test_array_of_several_ranges(bam):
+    """three ranges of one array, placed apart on the store, the third starting in the middle of a page (range_t's
+    page_start / page_start_offset, include/page_cache.h:984-1030 of the reference)"""
+    from bam_amd import gen
+    per = 1 << 16
+    with Rig(bam, 16 << 20, n_queues=8, depth=256) as r:
+        pc = bam.PageCache(4096, 256, 0, r.c)
+        layout = [(0, 0), (1000, 0), (300, 1024)]                    # (first page on the store, byte offset of the first element in it)
+        ranges = [bam.Range(k * per, (k + 1) * per, ps, (per * 8 + pso + 4095) // 4096, pso, 4096, pc, 0) for k, (ps, pso) in enumerate(layout)]
+        a = bam.Array(3 * per, 0, ranges, 0)
+        store = oracle.store(SEED, 0, 2 << 20)
+        flat = np.concatenate([store[ps * 512 + pso // 8: ps * 512 + pso // 8 + per] for ps, pso in layout])
+        assert a.read(3 * per) == int(np.sum(flat, dtype=np.uint64))
+        idx = gen.gather_indices(SEED, 1 << 17, 3 * per)
+        assert a.read(1 << 17, idx, block_size=256) == int(np.sum(flat[_u64(idx)], dtype=np.uint64))
+        # bam_ptr crosses ranges too (every lane keeps the page it points into: few enough threads for the slots there are)
+        assert a.read_via(4, 64, idx) == int(np.sum(flat[_u64(idx)[:64]], dtype=np.uint64))
+        seams = np.concatenate([np.arange(k * per - 1024, k * per + 1024, dtype=np.uint64) for k in (1, 2)])
+        assert a.read_via(4, len(seams), _dev(seams)) == int(np.sum(flat[seams], dtype=np.uint64))
+        st = a.stats()
+        assert st["access_cnt"] == 3 * per + (1 << 17) + 64 + len(seams) and not r.c.aborted()
+        a.close()
+        for x in ranges:
+            x.close()
+        pc.close()
+
+
+@pytest.mark.parametrize("dist", [0, 1])
+def test_two_controllers_behind_one_cache(bam, dist):
+    """REPLICATE: the same data on both, reads spread over them; STRIPE: page p on controller p % 2 at page p / 2
+    (get_backing_page_ / get_backing_ctrl_, include/page_cache.h:556-582 of the reference)"""
+    from bam_amd import gen
+    n_elems, n = 1 << 20, 1 << 17
+    seeds = (SEED, SEED) if dist == 0 else (11, 22)
+    paths = [_path(), _path()]
+    ts = [bam.Target(p, 16 << 20, 512, seed=sd, n_io_threads=2) for p, sd in zip(paths, seeds)]
+    cs = [bam.Controller(p, 1, 0, queue_depth=256, n_queues=4, spin_limit=LIMIT_US) for p in paths]
+    try:
+        pc = bam.PageCache(4096, 256, 0, cs)
+        rg = bam.Range(0, n_elems, 0, n_elems // 512, 0, 4096, pc, 0, dist=dist)
+        a = bam.Array(n_elems, 0, [rg], 0)
+        if dist == 0:
+            flat = oracle.store(SEED, 0, n_elems)
+        else:
+            pages = [oracle.store(sd, 0, n_elems // 2).reshape(-1, 512) for sd in seeds]
+            flat = np.empty((n_elems // 512, 512), dtype=np.uint64)
+            flat[0::2] = pages[0]
+            flat[1::2] = pages[1]
+            flat = flat.reshape(-1)
+        idx = gen.gather_indices(SEED, n, n_elems)
+        for _ in range(2):
+            assert a.read(n, idx, block_size=128) == int(np.sum(flat[_u64(idx)], dtype=np.uint64))
+        assert a.read(n_elems, block_size=256) == int(np.sum(flat, dtype=np.uint64))
+        reads = [t.stats()["read_cmds"] for t in ts]
+        assert min(reads) > 0.3 * max(reads) and sum(reads) == a.stats()["read_io_cnt"]
+        assert not cs[0].aborted() and not cs[1].aborted()
+        a.close(); rg.close(); pc.close()
+    finally:
+        for c in cs:
+            c.close()
+        for t in ts:
+            t.close()
+
+
 def test_direct_placement_without_staging(bam):
     """stage_bytes = 0: PRPs name the cache slots themselves and the controller writes the payload into device memory"""
     from bam_amd import gen
