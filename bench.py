@@ -40,8 +40,8 @@ HBM_PEAK_GBS = 8000.0
 STREAM_PAGES_PER_WAVE = 16      # one acquire batch of the page-wise streaming kernel
 # HBM bytes one launch of the page-wise streaming kernel moves over the 1 GiB cache, from the profiler's FETCH_SIZE and
 # WRITE_SIZE counters scaled by what they read for a plain 1 GiB copy (x2.0 and x1.0); figures and commands in
-# profiles/k_cache_stream_hit_path_1GiB_cache.md.  Holds for this workload only.
-HIT_STREAM_TRAFFIC_BYTES = 1084300000
+# profiles/k_cache_stream_pages_hit_path_1GiB_cache.md.  Holds for this workload only.
+HIT_STREAM_TRAFFIC_BYTES = 1079621517
 
 
 def log(*a):
@@ -126,7 +126,7 @@ def main():
         hit[name] = {"ms_per_launch": ms, "GBps": CACHE_PAGES * PAGE / ms / 1e6}
     st = arr.stats()
     assert st["read_io_cnt"] == 0 and st["miss_cnt"] == 0, "hit-path pass did I/O"
-    roofline = {"bound": "hbm", "kernel": "k_cache_stream<2> (page-wise streaming of the resident cache)",
+    roofline = {"bound": "hbm", "kernel": "k_cache_stream_pages (page-wise streaming of the resident cache)",
                 "achieved": hit["page_wise"]["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": hit["page_wise"]["GBps"] / HBM_PEAK_GBS, "traffic": HIT_STREAM_TRAFFIC_BYTES,
                 "bytes_per_launch": CACHE_PAGES * PAGE, "ms_per_launch": hit["page_wise"]["ms_per_launch"],
