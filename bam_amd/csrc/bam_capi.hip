@@ -48,7 +48,9 @@ struct bam_ctrl { Controller* c; };
 struct bam_page_cache { page_cache_t* pc; Controller* ctrl; };      /* ctrl: the first controller of the cache */
 struct bam_range { range_t<uint64_t>* r; };
 #define BAM_SUM_PARTIALS 4096
-struct bam_array { array_t<uint64_t>* a; BufferPtr partials; };      /* partials: [BAM_SUM_PARTIALS] checksum shards, zero between launches */
+struct bam_array { array_t<uint64_t>* a; BufferPtr partials; };
+struct bam_range32 { range_t<uint32_t>* r; };
+struct bam_array32 { array_t<uint32_t>* a; BufferPtr partials; };      /* partials: [BAM_SUM_PARTIALS] checksum shards, zero between launches */
 
 // ---------------------------------------------------------------------------
 // device helpers
@@ -476,6 +478,50 @@ __global__ __launch_bounds__(64) void k_cc_by_page(array_d_t<uint64_t>* da, bool
     graph_by_page(da, offsets, first, n_edges, ppw,
                   [&](uint64_t v) { return curr_visit[v]; },
                   [&](uint64_t src, uint64_t next) { cc_compute(src, comp, next, next_visit, changed); });
+}
+
+// ---- SSSP (benchmarks/sssp/main.cu:174-201 kernel_coalesce_pc, :282-292 update): 32-bit costs, weights in their own array ----
+__global__ __launch_bounds__(128) void k_sssp_coalesce_pc(array_d_t<uint64_t>* de, array_d_t<uint32_t>* dw, bool* label, uint32_t* newCostList,
+                                                          const uint64_t vertex_count, const uint64_t* vertexList)
+{
+    const uint64_t tid = (uint64_t)blockDim.x * blockIdx.x + threadIdx.x;
+    const uint64_t v = tid / BAM_WAVE_SIZE, laneIdx = tid % BAM_WAVE_SIZE;
+    if (v < vertex_count && label[v]) {
+        const uint64_t start = vertexList[v];
+        const uint64_t shift_start = start & 0xFFFFFFFFFFFFFFF0ull;
+        const uint64_t end = vertexList[v + 1];
+        const uint32_t cost = newCostList[v];
+        for (uint64_t i = shift_start + laneIdx; i < end; i += BAM_WAVE_SIZE) {
+            /* somebody found a cheaper way to v meanwhile: the update step flags v again and the next round starts over from it */
+            if (__hip_atomic_load(&newCostList[v], __ATOMIC_RELAXED, BAM_AGENT) != cost) break;
+            if (i >= start) {
+                const uint64_t next = de->seq_read(i);
+                const uint32_t weight = dw->seq_read(i);
+                if (__hip_atomic_load(&newCostList[next], __ATOMIC_RELAXED, BAM_AGENT) > cost + weight) atomicMin(&newCostList[next], cost + weight);
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+        label[v] = false;
+    }
+}
+
+__global__ void k_sssp_update(bool* label, uint32_t* costList, const uint32_t* newCostList, const uint64_t vertex_count, bool* changed)
+{
+    const uint64_t tid = (uint64_t)blockDim.x * blockIdx.x + threadIdx.x;
+    if (tid < vertex_count && newCostList[tid] < costList[tid]) {
+        costList[tid] = newCostList[tid];
+        label[tid] = true;
+        *changed = true;
+    }
+}
+
+/* one thread per request over an array of 32-bit elements: sum of the values read */
+__global__ void k_array32_read(array_d_t<uint32_t>* dr, uint64_t n_reqs, const uint64_t* assignment, uint64_t stride, unsigned long long* sum)
+{
+    const uint64_t tid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    uint64_t v = 0;
+    if (tid < n_reqs) v = (*dr)[assignment ? assignment[tid] : tid * stride];
+    block_accumulate(sum, v);
 }
 
 __global__ void k_iota(unsigned long long* p, uint64_t n)
@@ -1196,6 +1242,109 @@ int bam_cc_by_page(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_ver
         hip_err_chk(hipGetLastError());
         hip_err_chk(hipMemsetAsync(curr, 0x00, n_vertices, st));
         bool* t = curr; curr = next; next = t;
+        iter++;
+        hip_err_chk(hipMemcpyAsync(&changed_h, changed_d, sizeof(bool), hipMemcpyDeviceToHost, st));
+        hip_err_chk(hipStreamSynchronize(st));
+    } while (changed_h);
+    if (iterations) *iterations = iter;
+    BAM_API_END
+}
+
+// ---- arrays of 32-bit elements and SSSP ----
+int bam_range32_create(bam_range32_t** out, uint64_t index_start, uint64_t count, uint64_t page_start, uint64_t page_count,
+                       uint64_t page_start_offset, uint64_t page_size, bam_page_cache_t* pc, uint32_t device, int dist)
+{
+    if (!out || !pc) return fail(EINVAL, "bam_range32_create: null argument");
+    *out = nullptr;
+    if (dist != REPLICATE && dist != STRIPE) return fail(EINVAL, "bam_range32_create: unknown distribution");
+    if (page_size != pc->pc->pdt.page_size) return fail(EINVAL, "bam_range32_create: page size differs from the cache's");
+    if (page_start_offset >= page_size || page_start_offset % sizeof(uint32_t) || count <= index_start || page_count == 0)
+        return fail(EINVAL, "bam_range32_create: empty or misaligned range");
+    if (((count - index_start) * sizeof(uint32_t) + page_start_offset + page_size - 1) / page_size > page_count)
+        return fail(EINVAL, "bam_range32_create: page_count does not cover the elements");
+    BAM_API_BEGIN
+    *out = new bam_range32{new range_t<uint32_t>(index_start, count, page_start, page_count, page_start_offset, page_size, pc->pc, device, (data_dist_t)dist)};
+    BAM_API_END
+}
+
+void bam_range32_destroy(bam_range32_t* r)
+{
+    if (!r) return;
+    delete r->r;
+    delete r;
+}
+
+int bam_array32_create(bam_array32_t** out, uint64_t n_elems, uint64_t disk_start_offset, bam_range32_t** ranges, uint32_t n_ranges, uint32_t device)
+{
+    if (!out || !ranges || !n_ranges) return fail(EINVAL, "bam_array32_create: null argument");
+    *out = nullptr;
+    BAM_API_BEGIN
+    std::vector<range_t<uint32_t>*> rs;
+    for (uint32_t i = 0; i < n_ranges; i++) rs.push_back(ranges[i]->r);
+    *out = new bam_array32{new array_t<uint32_t>(n_elems, disk_start_offset, rs, device), createBuffer(BAM_SUM_PARTIALS * sizeof(uint64_t), device)};
+    BAM_API_END
+}
+
+void bam_array32_destroy(bam_array32_t* a)
+{
+    if (!a) return;
+    delete a->a;
+    delete a;
+}
+
+int bam_array32_stats(bam_array32_t* a, uint64_t* out)
+{
+    if (!a || !out) return fail(EINVAL, "bam_array32_stats: null argument");
+    BAM_API_BEGIN
+    hip_err_chk(hipDeviceSynchronize());
+    bam_array_counters t = a->a->reset_stats();
+    out[0] = t.read_io_cnt; out[1] = t.access_cnt; out[2] = t.miss_cnt; out[3] = t.hit_cnt;
+    BAM_API_END
+}
+
+int bam_array32_read(bam_array32_t* a, uint64_t n_reqs, const uint64_t* d_assignment, uint64_t stride, uint32_t block_size, uint64_t* d_sum, void* stream)
+{
+    if (!a || !d_sum) return fail(EINVAL, "bam_array32_read: null argument");
+    if (!block_size || block_size % BAM_WAVE_SIZE || block_size > 1024) return fail(EINVAL, "bam_array32_read: block size must be a multiple of 64, at most 1024");
+    if (!n_reqs) return 0;
+    BAM_API_BEGIN
+    hipLaunchKernelGGL(k_array32_read, dim3(blocks_for(n_reqs, block_size)), dim3(block_size), 0, (hipStream_t)stream,
+                       a->a->d_array_ptr, n_reqs, d_assignment, stride, (unsigned long long*)a->partials.get());
+    hipLaunchKernelGGL(k_fold_partials, dim3(1), dim3(1024), 0, (hipStream_t)stream, (unsigned long long*)a->partials.get(), (unsigned long long*)d_sum);
+    hip_err_chk(hipGetLastError());
+    BAM_API_END
+}
+
+int bam_sssp(bam_array_t* edges, bam_array32_t* weights, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t src, uint32_t* d_costs,
+             uint32_t* iterations, void* stream)
+{
+    if (!edges || !weights || !d_offsets || !d_costs) return fail(EINVAL, "bam_sssp: null argument");
+    if (src >= n_vertices) return fail(EINVAL, "bam_sssp: source out of range");
+    if (edges->a->adt.n_elems != weights->a->adt.n_elems) return fail(EINVAL, "bam_sssp: one weight per edge");
+    BAM_API_BEGIN
+    hipStream_t st = (hipStream_t)stream;
+    BufferPtr new_cost = createBuffer(n_vertices * sizeof(uint32_t), 0), label = createBuffer(n_vertices, 0), changed_buf = createBuffer(sizeof(uint64_t), 0);
+    uint32_t* new_d = (uint32_t*)new_cost.get();
+    bool* label_d = (bool*)label.get();
+    bool* changed_d = (bool*)changed_buf.get();
+    const uint32_t zero = 0;
+    const bool one = true;
+    hip_err_chk(hipMemsetAsync(d_costs, 0xFF, n_vertices * sizeof(uint32_t), st));
+    hip_err_chk(hipMemsetAsync(new_d, 0xFF, n_vertices * sizeof(uint32_t), st));
+    hip_err_chk(hipMemsetAsync(label_d, 0, n_vertices, st));
+    hip_err_chk(hipMemcpyAsync(label_d + src, &one, sizeof(bool), hipMemcpyHostToDevice, st));
+    hip_err_chk(hipMemcpyAsync(d_costs + src, &zero, sizeof(uint32_t), hipMemcpyHostToDevice, st));
+    hip_err_chk(hipMemcpyAsync(new_d + src, &zero, sizeof(uint32_t), hipMemcpyHostToDevice, st));
+    const uint32_t threads = 128;
+    uint32_t iter = 0;
+    bool changed_h;
+    do {
+        changed_h = false;
+        hip_err_chk(hipMemcpyAsync(changed_d, &changed_h, sizeof(bool), hipMemcpyHostToDevice, st));
+        hipLaunchKernelGGL(k_sssp_coalesce_pc, dim3(blocks_for(n_vertices * BAM_WAVE_SIZE, threads)), dim3(threads), 0, st,
+                           edges->a->d_array_ptr, weights->a->d_array_ptr, label_d, new_d, n_vertices, d_offsets);
+        hipLaunchKernelGGL(k_sssp_update, dim3(blocks_for(n_vertices, 256)), dim3(256), 0, st, label_d, d_costs, new_d, n_vertices, changed_d);
+        hip_err_chk(hipGetLastError());
         iter++;
         hip_err_chk(hipMemcpyAsync(&changed_h, changed_d, sizeof(bool), hipMemcpyDeviceToHost, st));
         hip_err_chk(hipStreamSynchronize(st));

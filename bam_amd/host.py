@@ -273,6 +273,70 @@ class Array:
             pass
 
 
+class Range32:
+    """range_t<uint32_t>: same arguments as Range"""
+
+    def __init__(self, index_start, count, page_start, page_count, page_start_offset, page_size, cache, device, dist=0):
+        self.L = _lib.load()
+        self.h = c_vp()
+        self.cache = cache
+        _chk(self.L.bam_range32_create(ctypes.byref(self.h), index_start, count, page_start, page_count, page_start_offset,
+                                       page_size, cache.h, device, dist), "bam_range32_create")
+
+    def close(self):
+        if self.h:
+            self.L.bam_range32_destroy(self.h)
+            self.h = c_vp()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class Array32:
+    """array_t<uint32_t>"""
+
+    def __init__(self, n_elems, disk_start_offset, ranges, device):
+        self.L = _lib.load()
+        self.h = c_vp()
+        self.ranges = list(ranges)
+        self.device = device
+        arr = (c_vp * len(ranges))(*[r.h for r in ranges])
+        _chk(self.L.bam_array32_create(ctypes.byref(self.h), n_elems, disk_start_offset, arr, len(ranges), device), "bam_array32_create")
+
+    def read(self, n_reqs, assignment=None, stride=1, block_size=64):
+        s = torch.zeros(1, dtype=torch.int64, device=f"cuda:{self.device}")
+        _chk(self.L.bam_array32_read(self.h, n_reqs, _ptr(assignment), stride, block_size, _ptr(s), _stream()), "bam_array32_read")
+        return int(s.item()) & MASK64
+
+    def stats(self):
+        out = (c_u64 * 4)()
+        _chk(self.L.bam_array32_stats(self.h, out), "bam_array32_stats")
+        return dict(zip(("read_io_cnt", "access_cnt", "miss_cnt", "hit_cnt"), list(out)))
+
+    def close(self):
+        if self.h:
+            self.L.bam_array32_destroy(self.h)
+            self.h = c_vp()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def sssp(edges, weights, offsets, src):
+    """Costs (uint32 bit patterns in an int32 tensor) of the cheapest paths from src, and the number of rounds."""
+    n_v = offsets.numel() - 1
+    costs = torch.empty(n_v, dtype=torch.int32, device=offsets.device)
+    it = c_u32(0)
+    _chk(edges.L.bam_sssp(edges.h, weights.h, _ptr(offsets), n_v, int(src), _ptr(costs), ctypes.byref(it), _stream()), "bam_sssp")
+    return costs, it.value
+
+
 def make_array(ctrl, n_elems, page_size, cache_pages, device=0, disk_offset_bytes=0, max_range=64):
     """page cache + one range + array over n_elems u64 stored from byte disk_offset_bytes (page aligned)."""
     pc = PageCache(page_size, cache_pages, device, ctrl, max_range)

@@ -22,6 +22,8 @@ typedef struct bam_ctrl bam_ctrl_t;           /* Controller */
 typedef struct bam_page_cache bam_page_cache_t;
 typedef struct bam_range bam_range_t;         /* range_t<uint64_t> */
 typedef struct bam_array bam_array_t;         /* array_t<uint64_t> */
+typedef struct bam_range32 bam_range32_t;     /* range_t<uint32_t> */
+typedef struct bam_array32 bam_array32_t;     /* array_t<uint32_t> */
 
 const char* bam_last_error(void);
 /* 1 when the library was built with the gfx950 device path and a HIP device is present */
@@ -146,6 +148,26 @@ int bam_cc(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, u
 int bam_bfs_by_page(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t src, uint32_t* d_labels,
                     uint32_t* iterations, void* stream);
 int bam_cc_by_page(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t* d_labels, uint32_t* iterations, void* stream);
+
+/* ---- arrays of 32-bit elements (the weight arrays of the reference's weighted-graph benchmarks are array_t<WeightT>,
+ * WeightT = uint32_t, benchmarks/sssp/main.cu:69, 640-661) ----
+ * Same arguments as the 64-bit handles; ranges of both element sizes may share one page cache. */
+int bam_range32_create(bam_range32_t** out, uint64_t index_start, uint64_t count, uint64_t page_start, uint64_t page_count,
+                       uint64_t page_start_offset, uint64_t page_size, bam_page_cache_t* pc, uint32_t device, int dist);
+void bam_range32_destroy(bam_range32_t* r);
+int bam_array32_create(bam_array32_t** out, uint64_t n_elems, uint64_t disk_start_offset, bam_range32_t** ranges, uint32_t n_ranges, uint32_t device);
+void bam_array32_destroy(bam_array32_t* a);
+/* out[4]: read_io_cnt, access_cnt, miss_cnt, hit_cnt since the last call */
+int bam_array32_stats(bam_array32_t* a, uint64_t* out);
+/* thread t reads element d_assignment[t] (or t * stride); the values read are summed into *d_sum */
+int bam_array32_read(bam_array32_t* a, uint64_t n_reqs, const uint64_t* d_assignment, uint64_t stride, uint32_t block_size, uint64_t* d_sum, void* stream);
+
+/* ---- SSSP (benchmarks/sssp/main.cu:174-201 kernel_coalesce_pc, :282-292 update, host loop :663-725) ----
+ * Rounds of relax + update from src until nothing changes: neighbour ids through `edges`, one 32-bit weight per CSR
+ * entry through `weights`; d_costs[V] receives the cost of the cheapest path to every vertex (0xFFFFFFFF =
+ * unreachable).  *iterations = rounds. */
+int bam_sssp(bam_array_t* edges, bam_array32_t* weights, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t src, uint32_t* d_costs,
+             uint32_t* iterations, void* stream);
 
 /* ---- synthetic inputs on the device (no counterpart in the reference, which reads dataset files) ---- */
 int bam_gen_words(uint64_t seed, uint64_t first, uint64_t n, uint64_t* d_out, void* stream);                 /* out[k] = splitmix64(seed, first + k) */

@@ -52,6 +52,9 @@ def lib():
         "bo_cc_labels": (u64, [u64, _p64, _p64, _p64]),
         "bo_cc_labels_sweep": (u64, [u64, _p64, _p64, _p64, ctypes.POINTER(u32)]),
         "bo_bfs_edges_scanned": (u64, [u64, _p64, _p32]),
+        "bo_edge_weights": (None, [u64, u64, u64, _p32]),
+        "bo_sssp_costs": (None, [u64, _p64, _p64, _p32, u64, _p32]),
+        "bo_sssp_costs_sweep": (u32, [u64, _p64, _p64, _p32, u64, _p32]),
         "bo_cmd_rw": (None, [_p32, ctypes.c_uint16, ctypes.c_uint8, u32, u64, u64, u64, ctypes.c_uint16]),
     }
     for name, (res, args) in sig.items():
@@ -127,6 +130,23 @@ def cc_labels(offsets, neigh, sweep=False):
         return lb, comps, it.value
     comps = lib().bo_cc_labels(len(offsets) - 1, offsets, nb, lb)
     return lb, comps
+
+
+def edge_weights(seed, n, first=0):
+    out = np.empty(max(n, 1), dtype=np.uint32)
+    lib().bo_edge_weights(seed, first, n, out)
+    return out[:n]
+
+
+def sssp_costs(offsets, neigh, weights, src, sweep=False):
+    costs = np.empty(len(offsets) - 1, dtype=np.uint32)
+    nb = neigh if len(neigh) else np.zeros(1, dtype=np.uint64)
+    w = weights if len(weights) else np.zeros(1, dtype=np.uint32)
+    if sweep:
+        rounds = lib().bo_sssp_costs_sweep(len(offsets) - 1, offsets, nb, w, int(src), costs)
+        return costs, rounds
+    lib().bo_sssp_costs(len(offsets) - 1, offsets, nb, w, int(src), costs)
+    return costs
 
 
 # ---- CPU restatement of the page-cache + queue protocol (cpu_path.c) -------

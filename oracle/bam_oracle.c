@@ -262,3 +262,80 @@ void bo_cmd_rw(uint32_t dword[16], uint16_t cid, uint8_t opcode, uint32_t nsid, 
     dword[10] = (uint32_t)slba;  dword[11] = (uint32_t)(slba >> 32);
     dword[12] = (uint32_t)((n_blocks - 1) & 0xffff);
 }
+
+/* ---- weighted graphs: single-source shortest paths ---- */
+void bo_edge_weights(uint64_t seed, uint64_t first, uint64_t n, uint32_t* out)
+{
+    for (uint64_t k = 0; k < n; k++) out[k] = 1u + (uint32_t)(bo_splitmix64(seed ^ 0x3e16ull, first + k) % 255u);
+}
+
+typedef struct { uint64_t cost; uint64_t v; } heap_item;
+
+static void heap_push(heap_item* h, uint64_t* n, heap_item x)
+{
+    uint64_t i = (*n)++;
+    while (i) {
+        uint64_t p = (i - 1) / 2;
+        if (h[p].cost <= x.cost) break;
+        h[i] = h[p];
+        i = p;
+    }
+    h[i] = x;
+}
+
+static heap_item heap_pop(heap_item* h, uint64_t* n)
+{
+    heap_item top = h[0], last = h[--(*n)];
+    uint64_t i = 0;
+    for (;;) {
+        uint64_t c = 2 * i + 1;
+        if (c >= *n) break;
+        if (c + 1 < *n && h[c + 1].cost < h[c].cost) c++;
+        if (last.cost <= h[c].cost) break;
+        h[i] = h[c];
+        i = c;
+    }
+    h[i] = last;
+    return top;
+}
+
+void bo_sssp_costs(uint64_t n_vertices, const uint64_t* offsets, const uint64_t* neigh, const uint32_t* weights, uint64_t src, uint32_t* costs)
+{
+    for (uint64_t v = 0; v < n_vertices; v++) costs[v] = BO_INF32;
+    /* lazy deletion: at most one heap entry per relaxation */
+    heap_item* heap = (heap_item*)malloc((offsets[n_vertices] + 1) * sizeof(heap_item));
+    uint64_t n = 0;
+    costs[src] = 0;
+    heap_push(heap, &n, (heap_item){0, src});
+    while (n) {
+        heap_item it = heap_pop(heap, &n);
+        if (it.cost != costs[it.v]) continue;
+        for (uint64_t e = offsets[it.v]; e < offsets[it.v + 1]; e++) {
+            uint64_t c = it.cost + weights[e];
+            if (c < costs[neigh[e]]) {
+                costs[neigh[e]] = (uint32_t)c;
+                heap_push(heap, &n, (heap_item){c, neigh[e]});
+            }
+        }
+    }
+    free(heap);
+}
+
+uint32_t bo_sssp_costs_sweep(uint64_t n_vertices, const uint64_t* offsets, const uint64_t* neigh, const uint32_t* weights, uint64_t src, uint32_t* costs)
+{
+    for (uint64_t v = 0; v < n_vertices; v++) costs[v] = BO_INF32;
+    costs[src] = 0;
+    uint32_t rounds = 0;
+    for (int changed = 1; changed;) {
+        changed = 0;
+        for (uint64_t v = 0; v < n_vertices; v++) {
+            if (costs[v] == BO_INF32) continue;
+            for (uint64_t e = offsets[v]; e < offsets[v + 1]; e++) {
+                uint64_t c = (uint64_t)costs[v] + weights[e];
+                if (c < costs[neigh[e]]) { costs[neigh[e]] = (uint32_t)c; changed = 1; }
+            }
+        }
+        rounds += changed;
+    }
+    return rounds;
+}

@@ -13,6 +13,7 @@
  *   bo_bfs_levels            reference sample graph (bfs/main.cu:1262-1263) + scipy BFS
  *   bo_cc_labels             reference sample graph + scipy connected_components
  *   bo_rmat_edges/bo_uniform_edges/bo_build_csr   independent numpy restatement
+ *   bo_sssp_costs            hand-computed weighted graph + scipy dijkstra + the independent sweep bo_sssp_costs_sweep
  *   cpu path (cpu_path.c)    closed-form sums + counter invariants of the
  *                            reference logs; simt::atomic semantics: parity unpinned
  */
@@ -47,6 +48,14 @@ uint32_t bo_bfs_levels_sweep(uint64_t n_vertices, const uint64_t* offsets, const
 uint64_t bo_cc_labels(uint64_t n_vertices, const uint64_t* offsets, const uint64_t* neigh, uint64_t* labels);
 uint64_t bo_cc_labels_sweep(uint64_t n_vertices, const uint64_t* offsets, const uint64_t* neigh, uint64_t* labels, uint32_t* iters);
 uint64_t bo_bfs_edges_scanned(uint64_t n_vertices, const uint64_t* offsets, const uint32_t* levels);
+
+/* edge weights of the synthetic weighted graphs: weight of CSR entry e = 1 + splitmix64(seed ^ 0x3e16, e) mod 255 */
+void     bo_edge_weights(uint64_t seed, uint64_t first, uint64_t n, uint32_t* out);
+/* single-source shortest paths, 32-bit costs (benchmarks/sssp/main.cu:69, 174-201, 282-292: the fixed point of its
+ * relax + update rounds); unreachable = BO_INF32.  Dijkstra with a binary heap; the sweep is plain Bellman-Ford rounds
+ * and returns how many rounds changed something. */
+void     bo_sssp_costs(uint64_t n_vertices, const uint64_t* offsets, const uint64_t* neigh, const uint32_t* weights, uint64_t src, uint32_t* costs);
+uint32_t bo_sssp_costs_sweep(uint64_t n_vertices, const uint64_t* offsets, const uint64_t* neigh, const uint32_t* weights, uint64_t src, uint32_t* costs);
 
 void     bo_cmd_rw(uint32_t dword[16], uint16_t cid, uint8_t opcode, uint32_t nsid, uint64_t prp1, uint64_t prp2, uint64_t slba, uint16_t n_blocks);
 

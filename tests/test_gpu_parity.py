@@ -469,6 +469,35 @@ def test_cc_labels_uniform_by_edge_page(bam, n_v, n_p, cache_pages):
         assert not r.c.aborted()
 
 
+@pytest.mark.parametrize("scale,cache_pages", [(10, 2048), (13, 160)])
+def test_sssp_costs_two_arrays_in_one_cache(bam, scale, cache_pages):
+    """neighbour ids (64-bit) and weights (32-bit) as two arrays behind one page cache; costs against Dijkstra"""
+    off, nb = oracle.rmat_csr(SEED, scale)
+    w = oracle.edge_weights(SEED, len(nb))
+    e_pages = (len(nb) * 8 + 4095) // 4096
+    w_pages = (len(w) * 4 + 4095) // 4096
+    with Rig(bam, (e_pages + w_pages + 1) * 4096, backing=True, n_queues=8, depth=256) as r:
+        store = r.backing((e_pages + w_pages + 1) * 512)
+        store[:len(nb)] = nb
+        store[e_pages * 512:].view(np.uint32)[:len(w)] = w
+        pc = bam.PageCache(4096, cache_pages, 0, r.c)
+        re_ = bam.Range(0, len(nb), 0, e_pages, 0, 4096, pc, 0)
+        rw = bam.Range32(0, len(w), e_pages, w_pages, 0, 4096, pc, 0)
+        edges = bam.Array(len(nb), 0, [re_], 0)
+        weights = bam.Array32(len(w), e_pages * 4096, [rw], 0)
+        # the 32-bit array by itself first
+        assert weights.read(len(w)) == int(np.sum(w, dtype=np.uint64))
+        assert weights.read(1000, stride=7, block_size=128) == int(np.sum(w[:7000:7], dtype=np.uint64))
+        ws = weights.stats()
+        assert ws["access_cnt"] == len(w) + 1000 and ws["read_io_cnt"] >= w_pages
+        doff = _dev(off)
+        for src in oracle.bfs_sources(SEED, off, 3):
+            costs, rounds = bam.sssp(edges, weights, doff, int(src))
+            assert np.array_equal(costs.cpu().numpy().view(np.uint32), oracle.sssp_costs(off, nb, w, int(src))) and rounds >= 2
+        assert edges.stats()["read_io_cnt"] > 0 and weights.stats()["access_cnt"] > 0 and not r.c.aborted()
+        edges.close(); weights.close(); re_.close(); rw.close(); pc.close()
+
+
 # ---------------------------------------------------------------- dataset placement (readwrite) and graph files
 
 def test_graph_file_to_store_then_traverse(bam, tmp_path):

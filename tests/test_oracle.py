@@ -151,3 +151,43 @@ def test_cc_against_scipy(n_v, n_p):
     mins = np.full(ncomp, n_v, dtype=np.int64)
     np.minimum.at(mins, lab, np.arange(n_v))
     assert np.array_equal(lb.astype(np.int64), mins[lab])
+
+
+# ---------------------------------------------------------------- weighted graphs (single-source shortest paths)
+
+def test_edge_weights_definition():
+    w = oracle.edge_weights(42, 1000, first=7)
+    want = np.array([1 + onp.splitmix64(42 ^ 0x3e16, 7 + k) % 255 for k in range(1000)], dtype=np.uint32)
+    assert np.array_equal(w, want) and w.min() >= 1 and w.max() <= 255
+
+
+def test_sssp_hand_computed_graph():
+    """a six-vertex graph worked out by hand: the cheap route 0-1-2-3 beats the direct edge 0-3; vertex 5 is unreachable;
+    edge weights are per direction (2->1 costs more than 1->2)"""
+    #        0:(1,w2)(3,w10)   1:(0,w2)(2,w3)   2:(1,w9)(3,w1)(4,w7)   3:(0,w10)(2,w1)   4:(2,w7)   5:-
+    off = np.array([0, 2, 4, 7, 9, 10, 10], dtype=np.uint64)
+    nb = np.array([1, 3, 0, 2, 1, 3, 4, 0, 2, 2], dtype=np.uint64)
+    w = np.array([2, 10, 2, 3, 9, 1, 7, 10, 1, 7], dtype=np.uint32)
+    inf = 0xFFFFFFFF
+    assert oracle.sssp_costs(off, nb, w, 0).tolist() == [0, 2, 5, 6, 12, inf]
+    assert oracle.sssp_costs(off, nb, w, 3).tolist() == [10, 10, 1, 0, 8, inf]
+    assert oracle.sssp_costs(off, nb, w, 5).tolist() == [inf] * 5 + [0]
+    costs, rounds = oracle.sssp_costs(off, nb, w, 0, sweep=True)
+    assert costs.tolist() == [0, 2, 5, 6, 12, inf] and rounds >= 1
+
+
+@pytest.mark.parametrize("seed,scale", [(42, 8), (0, 10), (7, 12)])
+def test_sssp_against_scipy_and_the_sweep(seed, scale):
+    off, nb = oracle.rmat_csr(seed, scale)
+    w = oracle.edge_weights(seed, len(nb))
+    n = len(off) - 1
+    m = sp.csr_matrix((w.astype(np.float64), nb.astype(np.int64), off.astype(np.int64)), shape=(n, n))
+    for src in oracle.bfs_sources(seed, off, 3):
+        got = oracle.sssp_costs(off, nb, w, int(src))
+        ref = csg.dijkstra(m, directed=True, indices=int(src))
+        want = np.where(np.isinf(ref), 0xFFFFFFFF, ref).astype(np.uint64).astype(np.uint32)
+        assert np.array_equal(got, want)
+        swept, _ = oracle.sssp_costs(off, nb, w, int(src), sweep=True)
+        assert np.array_equal(swept, got)
+        # unreachable exactly where BFS does not reach
+        assert np.array_equal(got == 0xFFFFFFFF, oracle.bfs_levels(off, nb, int(src))[0] == 0xFFFFFFFF)
