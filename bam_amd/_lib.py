@@ -50,6 +50,7 @@ SIGNATURES = {
     "bam_store_read_file": (c_int, [c_vp, c_vp, ctypes.c_char_p, c_u64, c_u64]),
     "bam_bfs_by_page": (c_int, [c_vp, c_vp, c_u64, c_u64, c_vp, P(c_u32), c_vp]),
     "bam_cc_by_page": (c_int, [c_vp, c_vp, c_u64, c_vp, P(c_u32), c_vp]),
+    "bam_vectoradd": (c_int, [c_vp, c_vp, c_vp, c_u64, c_vp]),
     "bam_range32_create": (c_int, [P(c_vp), c_u64, c_u64, c_u64, c_u64, c_u64, c_u64, c_vp, c_u32, c_int]),
     "bam_range32_destroy": (None, [c_vp]),
     "bam_array32_create": (c_int, [P(c_vp), c_u64, c_u64, P(c_vp), c_u32, c_u32]),

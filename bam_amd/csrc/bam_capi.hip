@@ -480,6 +480,18 @@ __global__ __launch_bounds__(64) void k_cc_by_page(array_d_t<uint64_t>* da, bool
                   [&](uint64_t src, uint64_t next) { cc_compute(src, comp, next, next_visit, changed); });
 }
 
+// ---- vectoradd (benchmarks/vectoradd/main.cu:102-117 kernel_baseline_ptr_pc): C[i] = A[i] + B[i], all three behind the cache ----
+__global__ __launch_bounds__(64) void k_vectoradd_ptr_pc(array_d_t<uint64_t>* da, array_d_t<uint64_t>* db, uint64_t n_elems, array_d_t<uint64_t>* dc)
+{
+    const uint64_t tid = (uint64_t)blockDim.x * blockIdx.x + threadIdx.x;
+    bam_ptr<uint64_t> Aptr(da);
+    bam_ptr<uint64_t> Bptr(db);
+    bam_ptr<uint64_t> Cptr(dc);
+    const bam_ptr<uint64_t>& A = Aptr;
+    const bam_ptr<uint64_t>& B = Bptr;
+    if (tid < n_elems) Cptr[tid] = A[tid] + B[tid];
+}
+
 // ---- SSSP (benchmarks/sssp/main.cu:174-201 kernel_coalesce_pc, :282-292 update): 32-bit costs, weights in their own array ----
 __global__ __launch_bounds__(128) void k_sssp_coalesce_pc(array_d_t<uint64_t>* de, array_d_t<uint32_t>* dw, bool* label, uint32_t* newCostList,
                                                           const uint64_t vertex_count, const uint64_t* vertexList)
@@ -1247,6 +1259,18 @@ int bam_cc_by_page(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_ver
         hip_err_chk(hipStreamSynchronize(st));
     } while (changed_h);
     if (iterations) *iterations = iter;
+    BAM_API_END
+}
+
+int bam_vectoradd(bam_array_t* a, bam_array_t* b, bam_array_t* c, uint64_t n_elems, void* stream)
+{
+    if (!a || !b || !c) return fail(EINVAL, "bam_vectoradd: null argument");
+    if (n_elems > a->a->adt.n_elems || n_elems > b->a->adt.n_elems || n_elems > c->a->adt.n_elems) return fail(EINVAL, "bam_vectoradd: more elements than the arrays hold");
+    if (!n_elems) return 0;
+    BAM_API_BEGIN
+    hipLaunchKernelGGL(k_vectoradd_ptr_pc, dim3(blocks_for(n_elems, 64)), dim3(64), 0, (hipStream_t)stream,
+                       a->a->d_array_ptr, b->a->d_array_ptr, n_elems, c->a->d_array_ptr);
+    hip_err_chk(hipGetLastError());
     BAM_API_END
 }
 

@@ -328,6 +328,11 @@ class Array32:
             pass
 
 
+def vectoradd(a, b, c, n_elems):
+    """c[i] = a[i] + b[i] through the cache (benchmarks/vectoradd)"""
+    _chk(a.L.bam_vectoradd(a.h, b.h, c.h, n_elems, _stream()), "bam_vectoradd")
+
+
 def sssp(edges, weights, offsets, src):
     """Costs (uint32 bit patterns in an int32 tensor) of the cheapest paths from src, and the number of rounds."""
     n_v = offsets.numel() - 1

@@ -149,6 +149,11 @@ int bam_bfs_by_page(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_ve
                     uint32_t* iterations, void* stream);
 int bam_cc_by_page(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t* d_labels, uint32_t* iterations, void* stream);
 
+/* ---- vectoradd (benchmarks/vectoradd/main.cu:102-117 kernel_baseline_ptr_pc) ----
+ * c[i] = a[i] + b[i] for i < n_elems, one thread per element, all three arrays read and written through bam_ptr; the
+ * results reach the store when their pages are evicted or the cache is flushed (bam_page_cache_flush). */
+int bam_vectoradd(bam_array_t* a, bam_array_t* b, bam_array_t* c, uint64_t n_elems, void* stream);
+
 /* ---- arrays of 32-bit elements (the weight arrays of the reference's weighted-graph benchmarks are array_t<WeightT>,
  * WeightT = uint32_t, benchmarks/sssp/main.cu:69, 640-661) ----
  * Same arguments as the 64-bit handles; ranges of both element sizes may share one page cache. */

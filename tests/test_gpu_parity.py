@@ -393,6 +393,33 @@ def test_array_write_eviction_write_back_and_flush(bam):
         assert r.t.stats()["write_cmds"] >= 128 and not r.c.aborted()
 
 
+def test_vectoradd_three_arrays_write_back(bam):
+    """C = A + B with all three arrays behind one cache (three ranges): the results reach the store with the flush.
+    Every lane keeps a page of each array while it works, so the cache has to hold what the waves in flight can pin:
+    here all 768 pages."""
+    n = 1 << 17                                                  # 256 pages per array
+    pages = n // 512
+    with Rig(bam, 3 * n * 8, backing=True, n_queues=8, depth=256) as r:
+        store = r.backing(3 * n)
+        a_h = oracle.store(SEED, 0, n)
+        b_h = oracle.store(SEED + 1, 0, n)
+        store[:n] = a_h
+        store[n:2 * n] = b_h
+        store[2 * n:] = 0
+        pc = bam.PageCache(4096, 800, 0, r.c)
+        rs = [bam.Range(0, n, k * pages, pages, 0, 4096, pc, 0) for k in range(3)]
+        arrs = [bam.Array(n, k * n * 8, [rs[k]], 0) for k in range(3)]
+        bam.vectoradd(arrs[0], arrs[1], arrs[2], n)
+        pc.flush()
+        assert np.array_equal(store[2 * n:], a_h + b_h)
+        assert np.array_equal(store[:n], a_h) and np.array_equal(store[n:2 * n], b_h)      # inputs untouched
+        assert r.t.stats()["write_cmds"] >= pages and not r.c.aborted()
+        assert arrs[2].read(n) == int(np.sum(a_h + b_h, dtype=np.uint64))
+        for x in arrs + rs:
+            x.close()
+        pc.close()
+
+
 # ---------------------------------------------------------------- graphs
 
 def _graph_rig(bam, nb, cache_pages, **kw):
