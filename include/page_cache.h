@@ -220,9 +220,11 @@ __device__ __forceinline__ uint32_t io_submit_group(page_cache_d_t* pc, QueuePai
      * Staged or direct.  Staged payload is pulled by the GPU (reads of host memory), direct payload is pushed by the
      * controller (writes into device memory): the two use opposite directions of the interconnect, so sending a
      * share of the read batches each way carries more than either alone.  Small reads stay staged: pushed in
-     * pieces of a few hundred bytes they cost the controller more than they save.
+     * pieces of a few hundred bytes they cost the controller more than they save.  Transfers larger than a staging
+     * page (cache pages above two controller pages) always go direct, through their PRP lists.
      */
-    const bool staged = qp->stage && !(opcode == NVM_IO_READ && bytes >= 2048 && pc->prp1 && ((cid >> 6) & 7u) < pc->direct_share);
+    const bool direct = pc->prp1 && (bytes > qp->stage_stride || (opcode == NVM_IO_READ && bytes >= 2048 && ((cid >> 6) & 7u) < pc->direct_share));
+    const bool staged = qp->stage && !direct;
     if (staged) {
         stage = qp->stage + (size_t)cid * qp->stage_stride;
         prp1 = qp->stage_ioaddr + (uint64_t)cid * qp->stage_stride;
@@ -1515,8 +1517,8 @@ struct page_cache_t {
         const uint64_t cache_size = ps * np;
         pdt.direct_share = 3;        /* measured best on the random-gather workload: 12.1M 4 KiB reads/s against 11.4M all staged, 10.4M all direct */
         if (const char* e = getenv("BAM_DIRECT_SHARE")) pdt.direct_share = (uint32_t)atoi(e);
-        if (!staged || ps > 2 * ctrl.ctrl->page_size) pdt.direct_share = 0;
-        if (staged && ps > ctrl.h_qps[0]->stage_stride) throw error(string("page_cache_t: page size exceeds the staging window of the queue pairs"));
+        if (!staged) pdt.direct_share = 0;
+        if (staged && ps > ctrl.h_qps[0]->stage_stride) pdt.direct_share = 8;      /* pages that do not fit a staging page: all direct */
         if (staged && pdt.direct_share == 0) {
             /* the controller never addresses the cache: plain device memory, no PRP tables */
             pages_buf = createBuffer(cache_size, hipDevice);

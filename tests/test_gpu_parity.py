@@ -258,6 +258,25 @@ def test_direct_placement_without_staging(bam):
         assert a.stats()["read_io_cnt"] > 0 and not r.c.aborted()
 
 
+@pytest.mark.parametrize("page,stage", [(16384, 0), (65536, 0), (16384, 4096)])
+def test_pages_above_two_controller_pages_use_prp_lists(bam, page, stage):
+    """cache pages of 4 and 16 controller pages: PRP1 + a PRP list per slot (include/page_cache.h:826-867 of the
+    reference), placed directly; with staging pages configured they are too small for such a page and are bypassed"""
+    from bam_amd import gen
+    n_elems, n = 1 << 22, 1 << 16
+    with Rig(bam, 32 << 20, n_queues=8, depth=256, stage_bytes=stage, backing=True) as r:
+        a = r.array(n_elems, page, 40)
+        idx = gen.gather_indices(SEED, n, n_elems)
+        assert a.read(n, idx, block_size=128) == oracle.lib().bo_gather_sum(SEED, SEED, 0, n, n_elems)
+        assert a.read(1 << 18, stride=16) == oracle.lib().bo_store_sum(SEED, 0, 16, 1 << 18)
+        st = a.stats()
+        assert r.t.stats()["bytes_read"] == r.c.info()["ssd_accesses"] * page and st["read_io_cnt"] > 40 and not r.c.aborted()
+        vals = np.arange(1 << 15, dtype=np.uint64) * np.uint64(5) + np.uint64(9)
+        a.write(1 << 15, _dev(vals), block_size=64)               # dirty large pages go back the same way
+        r.objs[0][2].flush()
+        assert np.array_equal(r.backing(1 << 15), vals) and not r.c.aborted()
+
+
 # ---------------------------------------------------------------- cache / pattern streaming
 
 @pytest.mark.parametrize("mode", [0, 1, 2])
