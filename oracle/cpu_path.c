@@ -422,7 +422,7 @@ void bo_cpu_path_stats(bo_cpu_path_t* p, uint64_t out[4], int reset)
     if (reset) { atomic_store(&p->read_io_cnt, 0); atomic_store(&p->access_cnt, 0); atomic_store(&p->miss_cnt, 0); atomic_store(&p->hit_cnt, 0); }
 }
 
-/* invariants at quiescence (SURVEY of the state machine): every state is INVALID or VALID with no references,
+/* invariants of the page state machine at quiescence: every state is INVALID or VALID with no references,
  * every valid page's slot translates back to it, no two valid pages share a slot.  0 = all hold. */
 int bo_cpu_path_check(bo_cpu_path_t* p)
 {
