@@ -412,7 +412,7 @@ __global__ void k_page_first_vertex(const uint64_t* offsets, uint64_t n_vertices
  */
 template <typename Active, typename Visit>
 __device__ __forceinline__ void graph_by_page(array_d_t<uint64_t>* da, const uint64_t* offsets, const uint64_t* first, const uint64_t n_edges,
-                                              const uint32_t ppw, Active active, Visit visit)
+                                              const uint32_t ppw, const bool backwards, Active active, Visit visit)
 {
     const uint32_t lane = bam::lane();
     const uint64_t wave = ((uint64_t)blockIdx.x * blockDim.x + threadIdx.x) / BAM_WAVE_SIZE;
@@ -422,7 +422,10 @@ __device__ __forceinline__ void graph_by_page(array_d_t<uint64_t>* da, const uin
     const uint32_t epp = view.page_size / 8;
     const uint64_t n_pages = (n_edges + epp - 1) / epp;
     const uint64_t pso_pages = view.pso >> view.page_size_log;
-    for (uint64_t p0 = wave * ppw; p0 < n_pages; p0 += n_waves * ppw) {
+    const uint64_t n_trips = (n_pages + ppw - 1) / ppw;
+    for (uint64_t t = wave; t < n_trips; t += n_waves) {
+        /* every other sweep runs from the far end: what the last sweep left in the cache is what this one asks for first */
+        const uint64_t p0 = (backwards ? n_trips - 1 - t : t) * ppw;
         const uint64_t p = p0 + lane;
         const uint64_t pstart = p * epp;
         bool want = false;
@@ -466,16 +469,16 @@ __global__ __launch_bounds__(64) void k_bfs_by_page(array_d_t<uint64_t>* da, uin
                                                      const uint64_t* first, uint64_t n_edges, uint32_t ppw, uint64_t* changed)
 {
     bool any = false;
-    graph_by_page(da, offsets, first, n_edges, ppw,
+    graph_by_page(da, offsets, first, n_edges, ppw, (level & 1u) != 0,
                   [&](uint64_t v) { return label[v] == level; },
                   [&](uint64_t, uint64_t next) { if (label[next] == MYINFINITY) { label[next] = level + 1; any = true; } });
     if (any) *changed = 1;
 }
 
 __global__ __launch_bounds__(64) void k_cc_by_page(array_d_t<uint64_t>* da, bool* curr_visit, bool* next_visit, const uint64_t* offsets,
-                                                    const uint64_t* first, uint64_t n_edges, uint32_t ppw, unsigned long long* comp, bool* changed)
+                                                    const uint64_t* first, uint64_t n_edges, uint32_t ppw, uint32_t sweep, unsigned long long* comp, bool* changed)
 {
-    graph_by_page(da, offsets, first, n_edges, ppw,
+    graph_by_page(da, offsets, first, n_edges, ppw, (sweep & 1u) != 0,
                   [&](uint64_t v) { return curr_visit[v]; },
                   [&](uint64_t src, uint64_t next) { cc_compute(src, comp, next, next_visit, changed); });
 }
@@ -1250,7 +1253,7 @@ int bam_cc_by_page(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_ver
         hip_err_chk(hipMemcpyAsync(changed_d, &changed_h, sizeof(bool), hipMemcpyHostToDevice, st));
         if (pl.n_pages)
             hipLaunchKernelGGL(k_cc_by_page, dim3(pl.blocks), dim3(BAM_WAVE_SIZE), 0, st, edges->a->d_array_ptr, curr, next, d_offsets,
-                               (const uint64_t*)pl.first.get(), pl.n_edges, pl.ppw, (unsigned long long*)d_labels, changed_d);
+                               (const uint64_t*)pl.first.get(), pl.n_edges, pl.ppw, iter, (unsigned long long*)d_labels, changed_d);
         hip_err_chk(hipGetLastError());
         hip_err_chk(hipMemsetAsync(curr, 0x00, n_vertices, st));
         bool* t = curr; curr = next; next = t;
