@@ -495,6 +495,156 @@ __global__ __launch_bounds__(64) void k_vectoradd_ptr_pc(array_d_t<uint64_t>* da
     if (tid < n_elems) Cptr[tid] = A[tid] + B[tid];
 }
 
+// ---- reduction (benchmarks/reduction/main.cu:166-195 kernel_reduce_baseline_ptr_pc): output[b] = sum of the 2 x blockDim elements of block b ----
+__global__ void k_reduce_ptr_pc(array_d_t<uint64_t>* da, unsigned long long* output, uint64_t len)
+{
+    __shared__ uint64_t wave_total[1024 / BAM_WAVE_SIZE];
+    const uint64_t tid = threadIdx.x, start = 2ull * blockDim.x * blockIdx.x;
+    uint64_t v = 0;
+    {
+        bam_ptr<uint64_t> in_ptr(da);
+        const bam_ptr<uint64_t>& input = in_ptr;
+        if (start + tid < len) v = input[start + tid];
+        if (blockDim.x + start + tid < len) v += input[blockDim.x + start + tid];
+    }
+    v = wave_sum(v);
+    if (bam::lane() == 0) wave_total[tid / BAM_WAVE_SIZE] = v;
+    __syncthreads();
+    if (tid < BAM_WAVE_SIZE) {
+        v = wave_sum(tid < blockDim.x / BAM_WAVE_SIZE ? wave_total[tid] : 0);
+        if (tid == 0) output[blockIdx.x] = v;
+    }
+}
+
+// ---- scan (benchmarks/scan/main.cu:147-190 kernel_scan_baseline_ptr_pc, :89-100 finalsum) ----
+/* inclusive sums over the 64 lanes of a wave (all lanes active) */
+__device__ __forceinline__ uint64_t wave_inclusive_sum(uint64_t v)
+{
+    const uint32_t lane = bam::lane();
+#pragma unroll
+    for (uint32_t o = 1; o < BAM_WAVE_SIZE; o <<= 1) {
+        const uint64_t u = bam::shfl(v, lane >= o ? lane - o : lane);
+        if (lane >= o) v += u;
+    }
+    return v;
+}
+
+/*
+ * Block b scans its 2 x blockDim elements: output[i] = sum of the block's elements up to and including i,
+ * intermediate[b] = the block's total.  The elements are read as the reference reads them (thread t takes t and
+ * t + blockDim, so a wave reads consecutive elements through one page reference); the scan itself runs over wave
+ * shuffles on pairs of neighbours rather than the two tree passes over shared memory.
+ */
+__global__ void k_scan_ptr_pc(array_d_t<uint64_t>* da, unsigned long long* output, unsigned long long* intermediate, uint64_t len)
+{
+    extern __shared__ uint64_t scan_mem[];                      /* 2 x blockDim elements, then one total per wave */
+    const uint32_t B = blockDim.x, t = threadIdx.x;
+    uint64_t* wave_total = scan_mem + 2 * B;
+    const uint64_t idx = 2ull * blockIdx.x * B + t;
+    {
+        bam_ptr<uint64_t> in_ptr(da);
+        const bam_ptr<uint64_t>& ptr = in_ptr;
+        scan_mem[t] = idx < len ? ptr[idx] : 0;
+        scan_mem[t + B] = idx + B < len ? ptr[idx + B] : 0;
+    }
+    __syncthreads();
+    const uint64_t a = scan_mem[2 * t], b = a + scan_mem[2 * t + 1];
+    const uint64_t s = wave_inclusive_sum(b);
+    if (bam::lane() == BAM_WAVE_SIZE - 1) wave_total[t / BAM_WAVE_SIZE] = s;
+    __syncthreads();
+    uint64_t before = s - b;
+    for (uint32_t w = 0; w < t / BAM_WAVE_SIZE; w++) before += wave_total[w];
+    scan_mem[2 * t] = before + a;
+    scan_mem[2 * t + 1] = before + b;
+    __syncthreads();
+    if (idx < len) output[idx] = scan_mem[t];
+    if (idx + B < len) output[idx + B] = scan_mem[t + B];
+    if (intermediate && t == B - 1) intermediate[blockIdx.x] = before + b;
+}
+
+/* one block: v[i] = v[0] + ... + v[i] in place (the reference calls cub::DeviceScan::InclusiveSum here, scan/main.cu:416-418) */
+__global__ void k_scan_block_totals(unsigned long long* v, uint64_t n)
+{
+    __shared__ uint64_t wave_total[1024 / BAM_WAVE_SIZE];
+    __shared__ uint64_t carry_s;
+    const uint32_t t = threadIdx.x;
+    if (t == 0) carry_s = 0;
+    __syncthreads();
+    for (uint64_t base = 0; base < n; base += blockDim.x) {
+        const uint64_t x = base + t < n ? v[base + t] : 0;
+        const uint64_t s = wave_inclusive_sum(x);
+        if (bam::lane() == BAM_WAVE_SIZE - 1) wave_total[t / BAM_WAVE_SIZE] = s;
+        __syncthreads();
+        uint64_t r = carry_s + s;
+        for (uint32_t w = 0; w < t / BAM_WAVE_SIZE; w++) r += wave_total[w];
+        if (base + t < n) v[base + t] = r;
+        __syncthreads();
+        if (t == blockDim.x - 1) carry_s = r;
+        __syncthreads();
+    }
+}
+
+__global__ void k_scan_finalsum(const unsigned long long* scanned_totals, unsigned long long* output, uint64_t len)
+{
+    if (blockIdx.x == 0) return;
+    const uint64_t B = blockDim.x, idx = 2ull * blockIdx.x * B + threadIdx.x;
+    const uint64_t add = scanned_totals[blockIdx.x - 1];
+    if (idx < len) output[idx] += add;
+    if (idx + B < len) output[idx + B] += add;
+}
+
+// ---- PageRank by residual pushes (benchmarks/pagerank/main.cu:107-115 initialize, :252-273 kernel_coalesce_pc, :412-421 update) ----
+__global__ void k_pr_initialize(bool* label, float* delta, float* residual, float* value, const uint64_t vertex_count, const uint64_t* vertexList, float alpha)
+{
+    const uint64_t tid = (uint64_t)blockDim.x * blockIdx.x + threadIdx.x;
+    if (tid < vertex_count) {
+        value[tid] = 1.0f - alpha;
+        delta[tid] = (1.0f - alpha) * alpha / (vertexList[tid + 1] - vertexList[tid]);
+        residual[tid] = 0.0f;
+        label[tid] = true;
+    }
+}
+
+/* one wave per vertex: every neighbour of a flagged vertex receives the vertex's delta */
+__global__ __launch_bounds__(128) void k_pr_coalesce_pc(array_d_t<uint64_t>* da, bool* label, const float* delta, float* residual,
+                                                        const uint64_t vertex_count, const uint64_t* vertexList)
+{
+    const uint64_t tid = (uint64_t)blockDim.x * blockIdx.x + threadIdx.x;
+    const uint64_t v = tid / BAM_WAVE_SIZE, laneIdx = tid % BAM_WAVE_SIZE;
+    if (v < vertex_count && label[v]) {
+        const uint64_t start = vertexList[v];
+        const uint64_t shift_start = start & 0xFFFFFFFFFFFFFFF0ull;
+        const uint64_t end = vertexList[v + 1];
+        const float d = delta[v];
+        for (uint64_t i = shift_start + laneIdx; i < end; i += BAM_WAVE_SIZE)
+            if (i >= start) unsafeAtomicAdd(&residual[da->seq_read(i)], d);
+        __builtin_amdgcn_wave_barrier();
+        label[v] = false;
+    }
+}
+
+/* the same pushes taken page by page of the edge array; the flags are cleared by the host loop after the sweep */
+__global__ __launch_bounds__(64) void k_pr_by_page(array_d_t<uint64_t>* da, const bool* label, const float* delta, float* residual, const uint64_t* offsets,
+                                                    const uint64_t* first, uint64_t n_edges, uint32_t ppw, uint32_t sweep)
+{
+    graph_by_page(da, offsets, first, n_edges, ppw, (sweep & 1u) != 0,
+                  [&](uint64_t v) { return label[v]; },
+                  [&](uint64_t src, uint64_t next) { unsafeAtomicAdd(&residual[next], delta[src]); });
+}
+
+__global__ void k_pr_update(bool* label, float* delta, float* residual, float* value, const uint64_t vertex_count, const uint64_t* vertexList,
+                            float tolerance, float alpha, bool* changed)
+{
+    const uint64_t tid = (uint64_t)blockDim.x * blockIdx.x + threadIdx.x;
+    if (tid < vertex_count && residual[tid] > tolerance) {
+        value[tid] += residual[tid];
+        delta[tid] = residual[tid] * alpha / (vertexList[tid + 1] - vertexList[tid]);
+        residual[tid] = 0.0f;
+        label[tid] = true;
+        *changed = true;
+    }
+}
+
 // ---- SSSP (benchmarks/sssp/main.cu:174-201 kernel_coalesce_pc, :282-292 update): 32-bit costs, weights in their own array ----
 __global__ __launch_bounds__(128) void k_sssp_coalesce_pc(array_d_t<uint64_t>* de, array_d_t<uint32_t>* dw, bool* label, uint32_t* newCostList,
                                                           const uint64_t vertex_count, const uint64_t* vertexList)
@@ -1274,6 +1424,84 @@ int bam_vectoradd(bam_array_t* a, bam_array_t* b, bam_array_t* c, uint64_t n_ele
     hipLaunchKernelGGL(k_vectoradd_ptr_pc, dim3(blocks_for(n_elems, 64)), dim3(64), 0, (hipStream_t)stream,
                        a->a->d_array_ptr, b->a->d_array_ptr, n_elems, c->a->d_array_ptr);
     hip_err_chk(hipGetLastError());
+    BAM_API_END
+}
+
+int bam_reduce(bam_array_t* a, uint64_t n_elems, uint32_t block_size, uint64_t* d_partials, void* stream)
+{
+    if (!a || !d_partials) return fail(EINVAL, "bam_reduce: null argument");
+    if (!block_size || block_size % BAM_WAVE_SIZE || block_size > 1024) return fail(EINVAL, "bam_reduce: block size must be a multiple of 64, at most 1024");
+    if (n_elems > a->a->adt.n_elems) return fail(EINVAL, "bam_reduce: more elements than the array holds");
+    if (!n_elems) return 0;
+    BAM_API_BEGIN
+    hipLaunchKernelGGL(k_reduce_ptr_pc, dim3(blocks_for(n_elems, 2ull * block_size)), dim3(block_size), 0, (hipStream_t)stream,
+                       a->a->d_array_ptr, (unsigned long long*)d_partials, n_elems);
+    hip_err_chk(hipGetLastError());
+    BAM_API_END
+}
+
+int bam_scan(bam_array_t* a, uint64_t n_elems, uint32_t block_size, uint64_t* d_result, void* stream)
+{
+    if (!a || !d_result) return fail(EINVAL, "bam_scan: null argument");
+    if (!block_size || block_size % BAM_WAVE_SIZE || block_size > 1024) return fail(EINVAL, "bam_scan: block size must be a multiple of 64, at most 1024");
+    if (n_elems > a->a->adt.n_elems) return fail(EINVAL, "bam_scan: more elements than the array holds");
+    BAM_API_BEGIN
+    hipStream_t st = (hipStream_t)stream;
+    hip_err_chk(hipMemsetAsync(d_result, 0, sizeof(uint64_t), st));
+    if (n_elems) {
+        const uint64_t n_blocks = blocks_for(n_elems, 2ull * block_size);
+        BufferPtr totals = createBuffer(n_blocks * sizeof(uint64_t), 0);
+        unsigned long long* out = (unsigned long long*)d_result + 1;
+        const size_t lds = (2 * block_size + 1024 / BAM_WAVE_SIZE) * sizeof(uint64_t);
+        hipLaunchKernelGGL(k_scan_ptr_pc, dim3(n_blocks), dim3(block_size), lds, st, a->a->d_array_ptr, out, (unsigned long long*)totals.get(), n_elems);
+        hipLaunchKernelGGL(k_scan_block_totals, dim3(1), dim3(1024), 0, st, (unsigned long long*)totals.get(), n_blocks);
+        hipLaunchKernelGGL(k_scan_finalsum, dim3(n_blocks), dim3(block_size), 0, st, (const unsigned long long*)totals.get(), out, n_elems);
+        hip_err_chk(hipGetLastError());
+        hip_err_chk(hipStreamSynchronize(st));         /* `totals` is released on return */
+    }
+    BAM_API_END
+}
+
+int bam_pagerank(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, float alpha, float tolerance, uint32_t max_iterations,
+                 int by_page, float* d_value, uint32_t* iterations, void* stream)
+{
+    if (!edges || !d_offsets || !d_value) return fail(EINVAL, "bam_pagerank: null argument");
+    if (iterations) *iterations = 0;
+    if (!n_vertices) return 0;
+    BAM_API_BEGIN
+    hipStream_t st = (hipStream_t)stream;
+    BufferPtr delta = createBuffer(n_vertices * sizeof(float), 0), residual = createBuffer(n_vertices * sizeof(float), 0),
+              label = createBuffer(n_vertices, 0), changed_buf = createBuffer(sizeof(uint64_t), 0);
+    float* delta_d = (float*)delta.get();
+    float* residual_d = (float*)residual.get();
+    bool* label_d = (bool*)label.get();
+    bool* changed_d = (bool*)changed_buf.get();
+    by_page_plan pl{};
+    if (by_page)
+        if (int rc = plan_by_page(edges, d_offsets, n_vertices, st, pl)) return rc;
+    const uint32_t upd_blocks = blocks_for(n_vertices, 256);
+    hipLaunchKernelGGL(k_pr_initialize, dim3(upd_blocks), dim3(256), 0, st, label_d, delta_d, residual_d, d_value, n_vertices, d_offsets, alpha);
+    uint32_t iter = 0;
+    bool changed_h;
+    do {
+        changed_h = false;
+        hip_err_chk(hipMemcpyAsync(changed_d, &changed_h, sizeof(bool), hipMemcpyHostToDevice, st));
+        if (by_page) {
+            if (pl.n_pages)
+                hipLaunchKernelGGL(k_pr_by_page, dim3(pl.blocks), dim3(BAM_WAVE_SIZE), 0, st, edges->a->d_array_ptr, label_d, delta_d, residual_d, d_offsets,
+                                   (const uint64_t*)pl.first.get(), pl.n_edges, pl.ppw, iter);
+            hip_err_chk(hipMemsetAsync(label_d, 0, n_vertices, st));
+        } else {
+            hipLaunchKernelGGL(k_pr_coalesce_pc, dim3(blocks_for(n_vertices * BAM_WAVE_SIZE, 128)), dim3(128), 0, st, edges->a->d_array_ptr, label_d, delta_d,
+                               residual_d, n_vertices, d_offsets);
+        }
+        iter++;
+        hipLaunchKernelGGL(k_pr_update, dim3(upd_blocks), dim3(256), 0, st, label_d, delta_d, residual_d, d_value, n_vertices, d_offsets, tolerance, alpha, changed_d);
+        hip_err_chk(hipGetLastError());
+        hip_err_chk(hipMemcpyAsync(&changed_h, changed_d, sizeof(bool), hipMemcpyDeviceToHost, st));
+        hip_err_chk(hipStreamSynchronize(st));
+    } while (changed_h && iter < max_iterations);
+    if (iterations) *iterations = iter;
     BAM_API_END
 }
 

@@ -256,6 +256,28 @@ class Array:
             _chk(self.L.bam_cc(self.h, _ptr(offsets), n_v, _ptr(labels), coarse, ctypes.byref(it), _stream()), "bam_cc")
         return labels, it.value
 
+    def reduce(self, n_elems, block_size=64):
+        """Per-workgroup sums of 2 * block_size consecutive elements (benchmarks/reduction); int64 tensor of bit patterns."""
+        n_blocks = (n_elems + 2 * block_size - 1) // (2 * block_size)
+        out = torch.zeros(n_blocks, dtype=torch.int64, device=f"cuda:{self.device}")
+        _chk(self.L.bam_reduce(self.h, n_elems, block_size, _ptr(out), _stream()), "bam_reduce")
+        return out
+
+    def scan(self, n_elems, block_size=64):
+        """n_elems + 1 running sums, the first 0 and the last the total (benchmarks/scan); int64 tensor of bit patterns."""
+        out = torch.empty(n_elems + 1, dtype=torch.int64, device=f"cuda:{self.device}")
+        _chk(self.L.bam_scan(self.h, n_elems, block_size, _ptr(out), _stream()), "bam_scan")
+        return out
+
+    def pagerank(self, offsets, alpha=0.85, tolerance=0.001, max_iterations=100, by_page=False):
+        """PageRank values (float32) by residual pushes over the CSR whose neighbour ids this array holds, and the sweeps taken."""
+        n_v = offsets.numel() - 1
+        value = torch.empty(n_v, dtype=torch.float32, device=offsets.device)
+        it = c_u32(0)
+        _chk(self.L.bam_pagerank(self.h, _ptr(offsets), n_v, alpha, tolerance, max_iterations, int(by_page), _ptr(value),
+                                 ctypes.byref(it), _stream()), "bam_pagerank")
+        return value, it.value
+
     def stats(self, reset=True):
         out = (c_u64 * 4)()
         _chk(self.L.bam_array_stats(self.h, out, int(reset)), "bam_array_stats")

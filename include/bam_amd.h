@@ -154,6 +154,32 @@ int bam_cc_by_page(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_ver
  * results reach the store when their pages are evicted or the cache is flushed (bam_page_cache_flush). */
 int bam_vectoradd(bam_array_t* a, bam_array_t* b, bam_array_t* c, uint64_t n_elems, void* stream);
 
+/* ---- reduction (benchmarks/reduction/main.cu:166-195 kernel_reduce_baseline_ptr_pc, launch :476) ----
+ * Workgroup b of block_size threads sums elements [2 b block_size, 2 (b + 1) block_size) of the array, read through
+ * bam_ptr, into d_partials[b]; ceil(n_elems / (2 block_size)) partial sums, which the caller adds up as the reference's
+ * main() does (:507-511).  The reference's "optimized" variant (:198-237) overwrites one shared buffer from every warp of
+ * a block and is not reproduced. */
+int bam_reduce(bam_array_t* a, uint64_t n_elems, uint32_t block_size, uint64_t* d_partials, void* stream);
+
+/* ---- scan (benchmarks/scan/main.cu:147-190 kernel_scan_baseline_ptr_pc, :89-100 finalsum, host :413-420) ----
+ * d_result[0] = 0, d_result[i + 1] = a[0] + ... + a[i] (mod 2^64) for i < n_elems: n_elems + 1 words, the total last,
+ * as the reference lays its result out (:370-373, 405).  Per-block scans of 2 block_size elements read through bam_ptr,
+ * a scan of the block totals, and the pass that adds them back. */
+int bam_scan(bam_array_t* a, uint64_t n_elems, uint32_t block_size, uint64_t* d_result, void* stream);
+
+/* ---- PageRank (benchmarks/pagerank/main.cu: initialize :107-115, kernel_coalesce_pc :252-273, update :412-421,
+ * host loop :704-768; the reference runs alpha = 0.85, tolerance = 0.001, at most 100 iterations, :476-477) ----
+ * Residual pushes in single precision: every flagged vertex adds its delta to the residual of each neighbour (atomic
+ * float adds, neighbour ids through the cache), then every vertex whose residual exceeds `tolerance` moves it into its
+ * value and is flagged with delta = residual * alpha / degree.  d_value[V] receives the values; *iterations = sweeps.
+ * by_page = 0: one wave per vertex as the reference; 1: along the pages of the edge array as bam_bfs_by_page.
+ * The order of the float adds is not fixed (neither is it in the reference), so values agree between runs only to
+ * rounding, and a residual that lands within rounding of `tolerance` may be moved one sweep earlier or later;
+ * whatever the order, on return 0 <= x - value <= x * tolerance / (1 - alpha) up to rounding, x the exact solution of
+ * x = (1 - alpha) + alpha * sum over in-neighbours u of x_u / degree(u). */
+int bam_pagerank(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, float alpha, float tolerance, uint32_t max_iterations,
+                 int by_page, float* d_value, uint32_t* iterations, void* stream);
+
 /* ---- arrays of 32-bit elements (the weight arrays of the reference's weighted-graph benchmarks are array_t<WeightT>,
  * WeightT = uint32_t, benchmarks/sssp/main.cu:69, 640-661) ----
  * Same arguments as the 64-bit handles; ranges of both element sizes may share one page cache. */

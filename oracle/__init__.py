@@ -16,6 +16,8 @@ u64 = ctypes.c_uint64
 u32 = ctypes.c_uint32
 _p64 = np.ctypeslib.ndpointer(dtype=np.uint64, flags="C_CONTIGUOUS")
 _p32 = np.ctypeslib.ndpointer(dtype=np.uint32, flags="C_CONTIGUOUS")
+_pf32 = np.ctypeslib.ndpointer(dtype=np.float32, flags="C_CONTIGUOUS")
+_pf64 = np.ctypeslib.ndpointer(dtype=np.float64, flags="C_CONTIGUOUS")
 
 
 def build(force=False):
@@ -55,6 +57,10 @@ def lib():
         "bo_edge_weights": (None, [u64, u64, u64, _p32]),
         "bo_sssp_costs": (None, [u64, _p64, _p64, _p32, u64, _p32]),
         "bo_sssp_costs_sweep": (u32, [u64, _p64, _p64, _p32, u64, _p32]),
+        "bo_reduce_blocks": (None, [_p64, u64, u32, _p64]),
+        "bo_scan": (None, [_p64, u64, _p64]),
+        "bo_pagerank": (u32, [u64, _p64, _p64, ctypes.c_float, ctypes.c_float, u32, _pf32]),
+        "bo_pagerank_limit": (None, [u64, _p64, _p64, ctypes.c_double, u32, _pf64]),
         "bo_cmd_rw": (None, [_p32, ctypes.c_uint16, ctypes.c_uint8, u32, u64, u64, u64, ctypes.c_uint16]),
     }
     for name, (res, args) in sig.items():
@@ -147,6 +153,35 @@ def sssp_costs(offsets, neigh, weights, src, sweep=False):
         return costs, rounds
     lib().bo_sssp_costs(len(offsets) - 1, offsets, nb, w, int(src), costs)
     return costs
+
+
+def reduce_blocks(a, block):
+    a = np.ascontiguousarray(a, dtype=np.uint64)
+    per = 2 * block
+    out = np.empty(max((len(a) + per - 1) // per, 1), dtype=np.uint64)
+    lib().bo_reduce_blocks(a if len(a) else np.zeros(1, dtype=np.uint64), len(a), block, out)
+    return out[:(len(a) + per - 1) // per]
+
+
+def scan(a):
+    a = np.ascontiguousarray(a, dtype=np.uint64)
+    out = np.empty(len(a) + 1, dtype=np.uint64)
+    lib().bo_scan(a if len(a) else np.zeros(1, dtype=np.uint64), len(a), out)
+    return out
+
+
+def pagerank(offsets, neigh, alpha=0.85, tolerance=0.001, max_iterations=100):
+    value = np.empty(len(offsets) - 1, dtype=np.float32)
+    nb = neigh if len(neigh) else np.zeros(1, dtype=np.uint64)
+    it = lib().bo_pagerank(len(offsets) - 1, offsets, nb, alpha, tolerance, max_iterations, value)
+    return value, it
+
+
+def pagerank_limit(offsets, neigh, alpha=0.85, sweeps=300):
+    x = np.empty(len(offsets) - 1, dtype=np.float64)
+    nb = neigh if len(neigh) else np.zeros(1, dtype=np.uint64)
+    lib().bo_pagerank_limit(len(offsets) - 1, offsets, nb, alpha, sweeps, x)
+    return x
 
 
 # ---- CPU restatement of the page-cache + queue protocol (cpu_path.c) -------

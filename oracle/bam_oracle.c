@@ -321,6 +321,84 @@ void bo_sssp_costs(uint64_t n_vertices, const uint64_t* offsets, const uint64_t*
     free(heap);
 }
 
+/* benchmarks/reduction/main.cu:166-195: block b of `block` threads sums elements [2 b block, 2 (b + 1) block) */
+void bo_reduce_blocks(const uint64_t* a, uint64_t n, uint32_t block, uint64_t* out)
+{
+    const uint64_t per = 2ull * block, n_blocks = (n + per - 1) / per;
+    for (uint64_t b = 0; b < n_blocks; b++) {
+        uint64_t s = 0;
+        for (uint64_t i = b * per; i < (b + 1) * per && i < n; i++) s += a[i];
+        out[b] = s;
+    }
+}
+
+/* benchmarks/scan/main.cu:370-373, 413-420: result[0] = 0, result[i + 1] = a[0] + ... + a[i] */
+void bo_scan(const uint64_t* a, uint64_t n, uint64_t* out)
+{
+    out[0] = 0;
+    for (uint64_t i = 0; i < n; i++) out[i + 1] = out[i] + a[i];
+}
+
+/*
+ * benchmarks/pagerank/main.cu: initialize :107-115, push :252-273 (every neighbour of a flagged vertex receives the
+ * vertex's delta), update :412-421, host loop :704-768.  Single precision as the reference (ValueT = float, :78);
+ * the pushes of one sweep are added in vertex order here, in no fixed order on a GPU.
+ */
+uint32_t bo_pagerank(uint64_t n_vertices, const uint64_t* offsets, const uint64_t* neigh, float alpha, float tolerance, uint32_t max_iterations,
+                     float* value)
+{
+    float* delta = (float*)malloc(n_vertices * sizeof(float));
+    float* residual = (float*)malloc(n_vertices * sizeof(float));
+    uint8_t* label = (uint8_t*)malloc(n_vertices);
+    for (uint64_t v = 0; v < n_vertices; v++) {
+        value[v] = 1.0f - alpha;
+        delta[v] = (1.0f - alpha) * alpha / (offsets[v + 1] - offsets[v]);
+        residual[v] = 0.0f;
+        label[v] = 1;
+    }
+    uint32_t iter = 0;
+    int changed;
+    do {
+        changed = 0;
+        for (uint64_t v = 0; v < n_vertices; v++) {
+            if (!label[v]) continue;
+            for (uint64_t e = offsets[v]; e < offsets[v + 1]; e++) residual[neigh[e]] += delta[v];
+            label[v] = 0;
+        }
+        iter++;
+        for (uint64_t v = 0; v < n_vertices; v++) {
+            if (residual[v] > tolerance) {
+                value[v] += residual[v];
+                delta[v] = residual[v] * alpha / (offsets[v + 1] - offsets[v]);
+                residual[v] = 0.0f;
+                label[v] = 1;
+                changed = 1;
+            }
+        }
+    } while (changed && iter < max_iterations);
+    free(delta); free(residual); free(label);
+    return iter;
+}
+
+/* what the pushes converge to as tolerance -> 0: x = (1 - alpha) + alpha * sum over in-neighbours u of x_u / degree(u),
+ * by `sweeps` Jacobi steps in double precision (error <= alpha^sweeps * max x) */
+void bo_pagerank_limit(uint64_t n_vertices, const uint64_t* offsets, const uint64_t* neigh, double alpha, uint32_t sweeps, double* x)
+{
+    double* y = (double*)malloc(n_vertices * sizeof(double));
+    for (uint64_t v = 0; v < n_vertices; v++) x[v] = 1.0 - alpha;
+    for (uint32_t k = 0; k < sweeps; k++) {
+        for (uint64_t v = 0; v < n_vertices; v++) y[v] = 1.0 - alpha;
+        for (uint64_t u = 0; u < n_vertices; u++) {
+            const uint64_t deg = offsets[u + 1] - offsets[u];
+            if (!deg) continue;
+            const double share = alpha * x[u] / (double)deg;
+            for (uint64_t e = offsets[u]; e < offsets[u + 1]; e++) y[neigh[e]] += share;
+        }
+        memcpy(x, y, n_vertices * sizeof(double));
+    }
+    free(y);
+}
+
 uint32_t bo_sssp_costs_sweep(uint64_t n_vertices, const uint64_t* offsets, const uint64_t* neigh, const uint32_t* weights, uint64_t src, uint32_t* costs)
 {
     for (uint64_t v = 0; v < n_vertices; v++) costs[v] = BO_INF32;

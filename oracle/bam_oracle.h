@@ -14,6 +14,10 @@
  *   bo_cc_labels             reference sample graph + scipy connected_components
  *   bo_rmat_edges/bo_uniform_edges/bo_build_csr   independent numpy restatement
  *   bo_sssp_costs            hand-computed weighted graph + scipy dijkstra + the independent sweep bo_sssp_costs_sweep
+ *   bo_reduce_blocks/bo_scan numpy sums and cumsum, closed form n(n+1)/2 on 0..n-1, wrap-around mod 2^64
+ *   bo_pagerank              hand-computed first sweeps on a 3-vertex path; sparse solve of (I - alpha P^T) x = (1 - alpha)
+ *                            (scipy, double) with the bound 0 <= x - value <= x tolerance / (1 - alpha); bo_pagerank_limit
+ *                            against the same solve
  *   cpu path (cpu_path.c)    closed-form sums + counter invariants of the
  *                            reference logs; simt::atomic semantics: parity unpinned
  */
@@ -56,6 +60,16 @@ void     bo_edge_weights(uint64_t seed, uint64_t first, uint64_t n, uint32_t* ou
  * and returns how many rounds changed something. */
 void     bo_sssp_costs(uint64_t n_vertices, const uint64_t* offsets, const uint64_t* neigh, const uint32_t* weights, uint64_t src, uint32_t* costs);
 uint32_t bo_sssp_costs_sweep(uint64_t n_vertices, const uint64_t* offsets, const uint64_t* neigh, const uint32_t* weights, uint64_t src, uint32_t* costs);
+
+/* benchmarks/reduction/main.cu:166-195 and benchmarks/scan/main.cu:147-190, 89-100: per-block sums; running sums with a
+ * leading zero (out holds n + 1 words) */
+void     bo_reduce_blocks(const uint64_t* a, uint64_t n, uint32_t block, uint64_t* out);
+void     bo_scan(const uint64_t* a, uint64_t n, uint64_t* out);
+/* PageRank by residual pushes in single precision (benchmarks/pagerank/main.cu:107-115, 252-273, 412-421, 704-768);
+ * returns the sweeps taken.  bo_pagerank_limit: the solution the pushes approach as the tolerance goes to 0. */
+uint32_t bo_pagerank(uint64_t n_vertices, const uint64_t* offsets, const uint64_t* neigh, float alpha, float tolerance, uint32_t max_iterations,
+                     float* value);
+void     bo_pagerank_limit(uint64_t n_vertices, const uint64_t* offsets, const uint64_t* neigh, double alpha, uint32_t sweeps, double* x);
 
 void     bo_cmd_rw(uint32_t dword[16], uint16_t cid, uint8_t opcode, uint32_t nsid, uint64_t prp1, uint64_t prp2, uint64_t slba, uint16_t n_blocks);
 

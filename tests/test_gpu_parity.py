@@ -439,6 +439,24 @@ def test_vectoradd_three_arrays_write_back(bam):
         pc.close()
 
 
+@pytest.mark.parametrize("n,block,cache_pages", [(1, 64, 8), (1000, 64, 8), (1 << 16, 256, 32), ((1 << 18) + 77, 1024, 128), (1 << 18, 512, 1024)])
+def test_reduction_and_scan_through_bam_ptr(bam, n, block, cache_pages):
+    """benchmarks/reduction and benchmarks/scan: per-workgroup sums, and running sums with the total last; unsigned 64-bit
+    arithmetic, so bit-exact whatever the order of the adds"""
+    pad = (-n) % 512
+    with Rig(bam, (n + pad) * 8, backing=True, n_queues=8, depth=256) as r:
+        vals = oracle.store(SEED, 11, n)
+        r.backing(n + pad)[:n] = vals
+        a = r.array(n, 4096, cache_pages)
+        assert np.array_equal(_u64(a.reduce(n, block)), oracle.reduce_blocks(vals, block))
+        assert np.array_equal(_u64(a.scan(n, block)), oracle.scan(vals))
+        # a prefix of the array only: the tail must not leak in
+        m = n - n // 3
+        assert np.array_equal(_u64(a.scan(m, block)), oracle.scan(vals[:m]))
+        assert int(_u64(a.reduce(m, block)).sum(dtype=np.uint64)) == int(oracle.scan(vals[:m])[-1])
+        assert a.stats()["access_cnt"] > 0 and not r.c.aborted()
+
+
 # ---------------------------------------------------------------- graphs
 
 def _graph_rig(bam, nb, cache_pages, **kw):
@@ -542,6 +560,34 @@ def test_sssp_costs_two_arrays_in_one_cache(bam, scale, cache_pages):
             assert np.array_equal(costs.cpu().numpy().view(np.uint32), oracle.sssp_costs(off, nb, w, int(src))) and rounds >= 2
         assert edges.stats()["read_io_cnt"] > 0 and weights.stats()["access_cnt"] > 0 and not r.c.aborted()
         edges.close(); weights.close(); re_.close(); rw.close(); pc.close()
+
+
+@pytest.mark.parametrize("scale,cache_pages,tol", [(10, 2048, 1e-3), (13, 96, 1e-3), (14, 512, 1e-4)])
+@pytest.mark.parametrize("by_page", [False, True])
+def test_pagerank_values(bam, scale, cache_pages, tol, by_page):
+    """benchmarks/pagerank, single precision with atomic float adds in no fixed order (as in the reference), so no two
+    runs need agree bit for bit.  Tolerance, stated: with x the exact solution (double-precision limit of the pushes),
+    every value must satisfy x (1 - tol / (1 - alpha)) - 1e-5 x <= value <= x + 1e-5 x (what is left unpushed is at most
+    `tol` per vertex; 1e-5 x covers float rounding of a few hundred adds), and therefore lies within
+    x tol / (1 - alpha) + 2e-5 x of the oracle's serial run of the same algorithm."""
+    alpha = 0.85
+    off, nb = oracle.rmat_csr(SEED, scale)
+    x = oracle.pagerank_limit(off, nb, alpha)
+    want, want_it = oracle.pagerank(off, nb, alpha, tol, 1000)
+    r, a = _graph_rig(bam, nb, cache_pages, n_queues=16, depth=256)
+    with r:
+        v, it = a.pagerank(_dev(off), alpha, tol, 1000, by_page=by_page)
+        v = v.cpu().numpy().astype(np.float64)
+        assert 1 < it < 1000 and abs(it - want_it) <= 3
+        assert np.all(v <= x * (1 + 1e-5)) and np.all(v >= x * (1 - tol / (1 - alpha) - 1e-5))
+        assert np.all(np.abs(v - want) <= x * (tol / (1 - alpha) + 2e-5))
+        deg = np.diff(off.astype(np.int64))
+        assert np.all(v[deg == 0] == np.float32(1) - np.float32(alpha))
+        # a capped run stops at the cap
+        v1, it1 = a.pagerank(_dev(off), alpha, tol, 1, by_page=by_page)
+        w1, _ = oracle.pagerank(off, nb, alpha, tol, 1)
+        assert it1 == 1 and np.allclose(v1.cpu().numpy(), w1, rtol=1e-5)
+        assert a.stats()["read_io_cnt"] > 0 and not r.c.aborted()
 
 
 # ---------------------------------------------------------------- dataset placement (readwrite) and graph files

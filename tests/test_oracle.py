@@ -191,3 +191,72 @@ def test_sssp_against_scipy_and_the_sweep(seed, scale):
         assert np.array_equal(swept, got)
         # unreachable exactly where BFS does not reach
         assert np.array_equal(got == 0xFFFFFFFF, oracle.bfs_levels(off, nb, int(src))[0] == 0xFFFFFFFF)
+
+
+# ---------------------------------------------------------------- reduction and scan
+
+@pytest.mark.parametrize("n,block", [(0, 64), (1, 64), (127, 64), (128, 64), (129, 64), (5000, 256), (4096, 1024)])
+def test_reduce_blocks_and_scan_against_numpy(n, block):
+    a = oracle.store(42, 3, n) if n else np.zeros(0, dtype=np.uint64)
+    per = 2 * block
+    want = [int(a[b * per:(b + 1) * per].sum(dtype=np.uint64)) for b in range((n + per - 1) // per)]
+    assert oracle.reduce_blocks(a, block).tolist() == want
+    s = oracle.scan(a)
+    assert len(s) == n + 1 and s[0] == 0
+    assert np.array_equal(s[1:], np.cumsum(a, dtype=np.uint64))
+    if n:
+        assert int(s[-1]) == int(oracle.reduce_blocks(a, block).sum(dtype=np.uint64))
+
+
+def test_scan_closed_form_and_wrap_around():
+    n = 100000
+    s = oracle.scan(np.arange(n, dtype=np.uint64))
+    assert s.tolist() == [i * (i - 1) // 2 for i in range(n + 1)]
+    big = np.full(5, 2**63, dtype=np.uint64)                       # sums leave 64 bits: kept mod 2^64
+    assert oracle.scan(big).tolist() == [0, 2**63, 0, 2**63, 0, 2**63]
+    assert oracle.reduce_blocks(big, 64).tolist() == [2**63]
+
+
+# ---------------------------------------------------------------- PageRank
+
+def _pagerank_solve(off, nb, alpha):
+    """x = (1 - alpha) + alpha * P^T x, P = D^-1 A, solved directly in double precision"""
+    import scipy.sparse.linalg as spl
+    n = len(off) - 1
+    deg = np.diff(off.astype(np.int64)).astype(np.float64)
+    a = sp.csr_matrix((np.ones(len(nb)), nb.astype(np.int64), off.astype(np.int64)), shape=(n, n))
+    inv = np.divide(1.0, deg, out=np.zeros(n), where=deg > 0)
+    p_t = (sp.diags(inv) @ a).T.tocsc()
+    return spl.spsolve(sp.identity(n, format="csc") - alpha * p_t, np.full(n, 1.0 - alpha))
+
+
+def test_pagerank_first_sweeps_by_hand():
+    """path 0 - 1 - 2, alpha 0.85: after one sweep every vertex has taken what its neighbours pushed from the initial
+    deltas 0.1275, 0.06375, 0.1275; after two, the deltas made from those residuals"""
+    off = np.array([0, 1, 3, 4], dtype=np.uint64)
+    nb = np.array([1, 0, 2, 1], dtype=np.uint64)
+    v, it = oracle.pagerank(off, nb, 0.85, 0.001, max_iterations=1)
+    assert it == 1 and np.allclose(v, [0.21375, 0.405, 0.21375], rtol=1e-6)
+    v, it = oracle.pagerank(off, nb, 0.85, 0.001, max_iterations=2)
+    assert it == 2 and np.allclose(v, [0.322125, 0.513375, 0.322125], rtol=1e-6)
+    # the limit, worked out from x0 = 0.15 + 0.425 x1, x1 = 0.15 + 1.7 x0
+    x = oracle.pagerank_limit(off, nb, 0.85)
+    assert np.allclose(x, [0.21375 / 0.2775, 0.15 + 1.7 * 0.21375 / 0.2775, 0.21375 / 0.2775], rtol=1e-12)
+    v, it = oracle.pagerank(off, nb, 0.85, 1e-6, max_iterations=1000)
+    assert it < 1000 and np.allclose(v, x, rtol=2e-5)
+
+
+@pytest.mark.parametrize("seed,scale,tol", [(42, 8, 1e-3), (0, 10, 1e-3), (7, 12, 1e-4)])
+def test_pagerank_against_a_direct_solve(seed, scale, tol):
+    off, nb = oracle.rmat_csr(seed, scale)
+    alpha = 0.85
+    x = _pagerank_solve(off, nb, alpha)
+    assert np.allclose(oracle.pagerank_limit(off, nb, alpha), x, rtol=1e-10)
+    deg = np.diff(off.astype(np.int64))
+    assert abs(x[deg > 0].sum() - (deg > 0).sum()) < 1e-6 * len(x)      # no dangling vertices among the connected: mass is kept
+    assert np.allclose(x[deg == 0], 1 - alpha)
+    v, it = oracle.pagerank(off, nb, alpha, tol, max_iterations=1000)
+    assert it < 1000
+    # whatever is left unpushed is at most `tol` per vertex: 0 <= x - value <= x * tol / (1 - alpha), up to float rounding
+    slack = 1e-5 * x
+    assert np.all(v <= x + slack) and np.all(v >= x * (1 - tol / (1 - alpha)) - slack)
