@@ -324,30 +324,182 @@ __global__ void k_block_checksum(page_cache_d_t* pc, uint64_t n_slots, uint32_t 
 
 // ---- BFS: wave per `coarse` vertices, edges through bam_ptr (benchmarks/bfs/main.cu:658-689) ----
 #define MYINFINITY 0xFFFFFFFFu
-__global__ __launch_bounds__(128) void k_bfs_coalesce_coarse_ptr_pc(array_d_t<uint64_t>* da, uint32_t* label, const uint32_t level, const uint64_t vertex_count,
-                                                                   const uint64_t* vertexList, uint64_t* changed, uint64_t coarse)
+/*
+ * Read-ahead for a wave that walks one vertex's edge list through bam_ptr.  Left to itself the walk meets the
+ * pages of the list one after the other and pays one full trip to the store for each; the list of a hub of a
+ * power-law graph covers hundreds of pages, and the one wave that has it then decides how long the whole level
+ * takes.  Whenever the walk is about to enter pages it has not asked for yet, the lanes touch the next pages of
+ * the list (one each, taken and dropped again): those that are not resident are loaded as one batch of commands,
+ * and the walk that follows finds them there.  Nothing is held, so a page that is evicted again before the walk
+ * gets to it is simply read once more; results do not depend on it.  Arrays of one range only, and the reach
+ * scales with the cache (a 64th of its pages, at most one page per lane).
+ */
+template <typename T>
+struct list_read_ahead {
+    bam::range_view<T> view;
+    uint64_t asked_to = 0, last_page = 0;
+    uint32_t reach = 0;
+    bool long_list = false;
+    __device__ __forceinline__ void init(array_d_t<T>* da)
+    {
+        if (da->n_ranges != 1) return;
+        view.load(da->d_ranges);
+        const uint64_t r = da->d_ranges[0].cache.n_pages >> 6;
+        reach = r > BAM_WAVE_SIZE ? BAM_WAVE_SIZE : (uint32_t)r;
+    }
+    /* lanes with `act` are about to have the list of their vertex `v` walked: touch the first page of each list */
+    __device__ __forceinline__ void group(const uint64_t* vertexList, const bool act, const uint64_t v)
+    {
+        if (reach < 2) return;
+        bool want = false;
+        uint64_t pg = 0;
+        if (act) {
+            const uint64_t s = vertexList[v];
+            if (vertexList[v + 1] > s) { want = true; pg = view.page_of(s); }
+        }
+        if (bam::popc(bam::ballot(want)) < 2) return;          /* a single list: its walk does the same */
+        if (want) {
+            auto touch = [](uint32_t) { return true; };
+            view.acquire(pg, false, touch, touch);
+        }
+        view.n_access = view.n_hit = 0;
+    }
+    /* wave-uniform: the list is elements [start, end) */
+    __device__ __forceinline__ void begin(const uint64_t start, const uint64_t end)
+    {
+        long_list = false;
+        if (reach < 2 || end <= start) return;
+        last_page = view.page_of(end - 1);
+        long_list = last_page > view.page_of(start);
+        asked_to = 0;
+    }
+    /* wave-uniform: the walk is about to read from element `at` on */
+    __device__ __forceinline__ void step(const uint64_t at)
+    {
+        if (!long_list) return;
+        const uint64_t pg = view.page_of(at);
+        if (pg < asked_to) return;
+        const uint64_t p = pg + bam::lane();
+        if (bam::lane() < reach && p <= last_page) {
+            auto touch = [](uint32_t) { return true; };
+            view.acquire(p, false, touch, touch);
+        }
+        asked_to = pg + reach;
+        view.n_access = view.n_hit = 0;         /* not accesses of the kernel's own: kept out of the counters */
+    }
+};
+
+/*
+ * The traversal of the reference's coarsened per-vertex kernels (bfs/main.cu:658-689, cc/main.cu:123-144): wave w
+ * looks after vertices [w coarse, (w + 1) coarse) and walks the edge list of each active one, 64 entries per step
+ * through bam_ptr, the first access aligned to 128 bytes.  Around that walk, for the store's sake: the vertices'
+ * flags are read 64 at a time (one load and a ballot instead of `coarse` loads one after the other), the first
+ * page of every active vertex of such a group is touched before the first list is walked (what is not resident
+ * comes in as one batch of commands, not one trip per vertex), and long lists are read ahead (list_read_ahead).
+ * The larger `coarse`, the more distinct pages the resident waves ask for at a time: consecutive vertices share
+ * pages, so with one vertex per wave dozens of waves wait for the same page.
+ */
+/*
+ * A list of BAM_HEAVY_EDGES entries or more is not walked by the wave that finds it: it is cut into pieces of that
+ * size, which are queued and walked by a wave each in a second launch (walk_heavy_pieces).  The hubs of a power-law
+ * graph have lists of hundreds of pages; walked by one wave, a single hub takes longer than all other vertices of
+ * its level together.
+ */
+#define BAM_HEAVY_EDGES 4096u
+struct heavy_piece_t { uint64_t v, first, last; };      /* entries [first, last) of the list of vertex v */
+
+template <typename Active, typename Visit>
+__device__ __forceinline__ void walk_vertex_groups(array_d_t<uint64_t>* da, const uint64_t* vertexList, const uint64_t vertex_count, const uint64_t coarse,
+                                                   heavy_piece_t* heavy, unsigned long long* n_heavy, Active active, Visit visit)
 {
     const uint64_t tid = (uint64_t)blockDim.x * blockIdx.x + threadIdx.x;
     const uint64_t waveIdx = tid / BAM_WAVE_SIZE, laneIdx = tid % BAM_WAVE_SIZE;
+    const uint64_t first = waveIdx * coarse;
+    if (first >= vertex_count) return;
     bam_ptr<uint64_t> ptr(da);
-    bool any = false;
-    for (uint64_t j = 0; j < coarse; j++) {
-        const uint64_t v = waveIdx * coarse + j;
-        if (v < vertex_count && label[v] == level) {
+    list_read_ahead<uint64_t> ahead;
+    bool ready = false;
+#ifdef BAM_PROFILE
+    const uint64_t wt0 = wall_clock64();
+#endif
+    for (uint64_t b = 0; b < coarse; b += BAM_WAVE_SIZE) {
+        const uint64_t mine = first + b + laneIdx;
+        const bool act = b + laneIdx < coarse && mine < vertex_count && active(mine);
+        uint64_t m = bam::ballot(act);
+        if (!m) continue;
+        if (!ready) { ahead.init(da); ready = true; }
+        ahead.group(vertexList, act, mine);
+        for (; m; m &= m - 1) {
+            const uint64_t v = first + b + bam::first_lane(m);
             const uint64_t start = vertexList[v];
             const uint64_t shift_start = start & 0xFFFFFFFFFFFFFFF0ull;      /* 128-byte aligned first access */
             const uint64_t end = vertexList[v + 1];
-            for (uint64_t i = shift_start + laneIdx; i < end; i += BAM_WAVE_SIZE) {
-                if (i >= start) {
-                    const uint64_t next = ptr[i];
-                    if (label[next] == MYINFINITY) {
-                        label[next] = level + 1;
-                        any = true;
-                    }
+            if (end - start >= BAM_HEAVY_EDGES) {
+                const uint64_t pieces = (end - start + BAM_HEAVY_EDGES - 1) / BAM_HEAVY_EDGES;
+                unsigned long long at = 0;
+                if (laneIdx == 0) at = atomicAdd(n_heavy, (unsigned long long)pieces);
+                at = bam::bcast((uint64_t)at, 0);
+                for (uint64_t k = laneIdx; k < pieces; k += BAM_WAVE_SIZE) {
+                    const uint64_t f = start + k * BAM_HEAVY_EDGES;
+                    heavy[at + k] = heavy_piece_t{v, f, f + BAM_HEAVY_EDGES < end ? f + BAM_HEAVY_EDGES : end};
                 }
+                continue;
+            }
+            ahead.begin(start, end);
+            for (uint64_t i = shift_start + laneIdx; i < end; i += BAM_WAVE_SIZE) {
+                ahead.step(i - laneIdx > start ? i - laneIdx : start);
+                if (i >= start) visit(v, ptr[i]);
             }
         }
     }
+#ifdef BAM_PROFILE
+    unsigned long long* prof = da->d_ranges[0].cache.prof;
+    if (prof && ready && laneIdx == 0) {
+        const unsigned long long dt = wall_clock64() - wt0;
+        atomicAdd(&prof[9], dt); atomicAdd(&prof[10], 1ull); atomicMax(&prof[11], dt);
+        if (dt > 100000ull) { atomicAdd(&prof[12], dt); atomicAdd(&prof[13], 1ull); }      /* waves that ran for more than a millisecond */
+    }
+#endif
+}
+
+/* the queued pieces, one wave at a time each: the same walk through bam_ptr, read ahead over the piece */
+template <typename Visit>
+__device__ __forceinline__ void walk_heavy_pieces(array_d_t<uint64_t>* da, const heavy_piece_t* heavy, const unsigned long long* n_heavy, Visit visit)
+{
+    const uint64_t tid = (uint64_t)blockDim.x * blockIdx.x + threadIdx.x;
+    const uint64_t waveIdx = tid / BAM_WAVE_SIZE, laneIdx = tid % BAM_WAVE_SIZE;
+    const uint64_t n_waves = (uint64_t)gridDim.x * blockDim.x / BAM_WAVE_SIZE;
+    const uint64_t n = *n_heavy;
+    if (waveIdx >= n) return;
+    bam_ptr<uint64_t> ptr(da);
+    list_read_ahead<uint64_t> ahead;
+    ahead.init(da);
+    for (uint64_t k = waveIdx; k < n; k += n_waves) {
+        const heavy_piece_t pc = heavy[k];
+        ahead.begin(pc.first, pc.last);
+        for (uint64_t i = (pc.first & 0xFFFFFFFFFFFFFFF0ull) + laneIdx; i < pc.last; i += BAM_WAVE_SIZE) {
+            ahead.step(i - laneIdx > pc.first ? i - laneIdx : pc.first);
+            if (i >= pc.first) visit(pc.v, ptr[i]);
+        }
+    }
+}
+
+__global__ __launch_bounds__(128) void k_bfs_coalesce_coarse_ptr_pc(array_d_t<uint64_t>* da, uint32_t* label, const uint32_t level, const uint64_t vertex_count,
+                                                                   const uint64_t* vertexList, uint64_t* changed, uint64_t coarse,
+                                                                   heavy_piece_t* heavy, unsigned long long* n_heavy)
+{
+    bool any = false;
+    walk_vertex_groups(da, vertexList, vertex_count, coarse, heavy, n_heavy,
+                       [&](uint64_t v) { return label[v] == level; },
+                       [&](uint64_t, uint64_t next) { if (label[next] == MYINFINITY) { label[next] = level + 1; any = true; } });
+    if (any) *changed = 1;
+}
+
+__global__ __launch_bounds__(128) void k_bfs_heavy_ptr_pc(array_d_t<uint64_t>* da, uint32_t* label, const uint32_t level, uint64_t* changed,
+                                                         const heavy_piece_t* heavy, const unsigned long long* n_heavy)
+{
+    bool any = false;
+    walk_heavy_pieces(da, heavy, n_heavy, [&](uint64_t, uint64_t next) { if (label[next] == MYINFINITY) { label[next] = level + 1; any = true; } });
     if (any) *changed = 1;
 }
 
@@ -366,21 +518,18 @@ __device__ __forceinline__ void cc_compute(uint64_t cid, unsigned long long* com
 }
 
 __global__ __launch_bounds__(128) void k_cc_coalesce_coarse_ptr_pc(array_d_t<uint64_t>* da, bool* curr_visit, bool* next_visit, uint64_t vertex_count,
-                                                                  const uint64_t* vertexList, unsigned long long* comp, bool* changed, uint64_t coarse)
+                                                                  const uint64_t* vertexList, unsigned long long* comp, bool* changed, uint64_t coarse,
+                                                                  heavy_piece_t* heavy, unsigned long long* n_heavy)
 {
-    const uint64_t tid = (uint64_t)blockDim.x * blockIdx.x + threadIdx.x;
-    const uint64_t waveIdx = tid / BAM_WAVE_SIZE, laneIdx = tid % BAM_WAVE_SIZE;
-    bam_ptr<uint64_t> ptr(da);
-    for (uint64_t j = 0; j < coarse; j++) {
-        const uint64_t v = waveIdx * coarse + j;
-        if (v < vertex_count && curr_visit[v] == true) {
-            const uint64_t start = vertexList[v];
-            const uint64_t shift_start = start & 0xFFFFFFFFFFFFFFF0ull;
-            const uint64_t end = vertexList[v + 1];
-            for (uint64_t i = shift_start + laneIdx; i < end; i += BAM_WAVE_SIZE)
-                if (i >= start) cc_compute(v, comp, ptr[i], next_visit, changed);
-        }
-    }
+    walk_vertex_groups(da, vertexList, vertex_count, coarse, heavy, n_heavy,
+                       [&](uint64_t v) { return curr_visit[v]; },
+                       [&](uint64_t v, uint64_t next) { cc_compute(v, comp, next, next_visit, changed); });
+}
+
+__global__ __launch_bounds__(128) void k_cc_heavy_ptr_pc(array_d_t<uint64_t>* da, bool* next_visit, unsigned long long* comp, bool* changed,
+                                                        const heavy_piece_t* heavy, const unsigned long long* n_heavy)
+{
+    walk_heavy_pieces(da, heavy, n_heavy, [&](uint64_t v, uint64_t next) { cc_compute(v, comp, next, next_visit, changed); });
 }
 
 // ---- BFS / CC by edge page (benchmarks/bfs/main.cu:1074-1140 kernel_optimized_ptr_pc, first-vertex table :122-181) ----
@@ -616,8 +765,13 @@ __global__ __launch_bounds__(128) void k_pr_coalesce_pc(array_d_t<uint64_t>* da,
         const uint64_t shift_start = start & 0xFFFFFFFFFFFFFFF0ull;
         const uint64_t end = vertexList[v + 1];
         const float d = delta[v];
-        for (uint64_t i = shift_start + laneIdx; i < end; i += BAM_WAVE_SIZE)
+        list_read_ahead<uint64_t> ahead;
+        ahead.init(da);
+        ahead.begin(start, end);
+        for (uint64_t i = shift_start + laneIdx; i < end; i += BAM_WAVE_SIZE) {
+            ahead.step(i - laneIdx > start ? i - laneIdx : start);
             if (i >= start) unsafeAtomicAdd(&residual[da->seq_read(i)], d);
+        }
         __builtin_amdgcn_wave_barrier();
         label[v] = false;
     }
@@ -1247,6 +1401,27 @@ int bam_block_checksum(bam_page_cache_t* pc, uint64_t n_slots, uint32_t req_byte
     BAM_API_END
 }
 
+namespace {
+/* queue of the pieces of long edge lists, refilled in every sweep of the per-vertex graph kernels: a list of d >= BAM_HEAVY_EDGES
+ * entries makes at most d / BAM_HEAVY_EDGES + 1 <= 2 d / BAM_HEAVY_EDGES pieces */
+struct heavy_queue {
+    BufferPtr buf, cnt;
+    heavy_piece_t* pieces;
+    unsigned long long* count;
+    uint32_t blocks;
+    explicit heavy_queue(uint64_t n_edges)
+    {
+        const uint64_t cap = 2 * (n_edges / BAM_HEAVY_EDGES) + 1;
+        buf = createBuffer(cap * sizeof(heavy_piece_t), 0);
+        cnt = createBuffer(sizeof(unsigned long long), 0);
+        pieces = (heavy_piece_t*)buf.get();
+        count = (unsigned long long*)cnt.get();
+        const uint64_t waves = cap < 4096 ? cap : 4096;          /* the pieces are shared out over this many waves */
+        blocks = (uint32_t)((waves + 1) / 2);                   /* two waves per workgroup */
+    }
+};
+} // namespace
+
 int bam_bfs(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t src, uint32_t* d_labels,
             uint32_t coarse, uint32_t* iterations, void* stream)
 {
@@ -1262,13 +1437,16 @@ int bam_bfs(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, 
     const uint32_t threads = 128;
     const uint64_t n_waves = (n_vertices + coarse - 1) / coarse;
     const uint32_t blocks = blocks_for(n_waves * BAM_WAVE_SIZE, threads);
+    heavy_queue hq(edges->a->adt.n_elems);
     uint32_t level = 0, iter = 0;
     uint64_t changed_h;
     do {
         changed_h = 0;
         hip_err_chk(hipMemcpyAsync(changed_d, &changed_h, sizeof(uint64_t), hipMemcpyHostToDevice, st));
+        hip_err_chk(hipMemsetAsync(hq.count, 0, sizeof(unsigned long long), st));
         hipLaunchKernelGGL(k_bfs_coalesce_coarse_ptr_pc, dim3(blocks), dim3(threads), 0, st,
-                           edges->a->d_array_ptr, d_labels, level, n_vertices, d_offsets, changed_d, (uint64_t)coarse);
+                           edges->a->d_array_ptr, d_labels, level, n_vertices, d_offsets, changed_d, (uint64_t)coarse, hq.pieces, hq.count);
+        hipLaunchKernelGGL(k_bfs_heavy_ptr_pc, dim3(hq.blocks), dim3(threads), 0, st, edges->a->d_array_ptr, d_labels, level, changed_d, hq.pieces, hq.count);
         hip_err_chk(hipGetLastError());
         iter++; level++;
         hip_err_chk(hipMemcpyAsync(&changed_h, changed_d, sizeof(uint64_t), hipMemcpyDeviceToHost, st));
@@ -1295,13 +1473,17 @@ int bam_cc(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, u
     const uint32_t threads = 128;
     const uint64_t n_waves = (n_vertices + coarse - 1) / coarse;
     const uint32_t blocks = blocks_for(n_waves * BAM_WAVE_SIZE, threads);
+    heavy_queue hq(edges->a->adt.n_elems);
     uint32_t iter = 0;
     bool changed_h;
     do {
         changed_h = false;
         hip_err_chk(hipMemcpyAsync(changed_d, &changed_h, sizeof(bool), hipMemcpyHostToDevice, st));
+        hip_err_chk(hipMemsetAsync(hq.count, 0, sizeof(unsigned long long), st));
         hipLaunchKernelGGL(k_cc_coalesce_coarse_ptr_pc, dim3(blocks), dim3(threads), 0, st,
-                           edges->a->d_array_ptr, curr, next, n_vertices, d_offsets, (unsigned long long*)d_labels, changed_d, (uint64_t)coarse);
+                           edges->a->d_array_ptr, curr, next, n_vertices, d_offsets, (unsigned long long*)d_labels, changed_d, (uint64_t)coarse, hq.pieces, hq.count);
+        hipLaunchKernelGGL(k_cc_heavy_ptr_pc, dim3(hq.blocks), dim3(threads), 0, st, edges->a->d_array_ptr, next, (unsigned long long*)d_labels, changed_d,
+                           hq.pieces, hq.count);
         hip_err_chk(hipGetLastError());
         hip_err_chk(hipMemsetAsync(curr, 0x00, n_vertices, st));
         bool* t = curr; curr = next; next = t;

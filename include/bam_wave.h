@@ -192,6 +192,19 @@ template <typename T> __device__ __forceinline__ T ld_payload(const T* p)
     } else { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent"); return *p; }
 }
 
+/*
+ * Ordering among words that are only ever touched with agent-scope atomics (the bookkeeping of the queues and of
+ * the cache: tickets, marks, locks, page states) and stores to uncached host memory (submission entries,
+ * doorbells).  Such accesses are performed at the device's point of coherence whatever the caches hold, so a
+ * hand-over needs one thing only: the wave's earlier accesses have completed before its later ones are issued.
+ * That is a wait on the wave's own memory counters.  A release or acquire at agent scope does the same wait and
+ * also writes back or invalidates the caches of the whole compute-unit cluster, which only payload moved with
+ * plain loads and stores needs; at several such operations per command, and with the L2 full of other waves'
+ * dirty lines, those write-backs were most of the latency of a single command.
+ */
+__device__ __forceinline__ void fence_meta() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory"); }
+template <typename T> __device__ __forceinline__ void st_publish(T* p, T v) { fence_meta(); __hip_atomic_store(p, v, __ATOMIC_RELAXED, BAM_AGENT); }
+
 __device__ __forceinline__ void fence_release_sys() { __builtin_amdgcn_fence(__ATOMIC_RELEASE, ""); }
 __device__ __forceinline__ void fence_acquire_sys() { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, ""); }
 __device__ __forceinline__ void fence_acquire_agent() { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent"); }

@@ -94,7 +94,7 @@ __device__ __forceinline__ uint32_t get_cid_group(nvm_queue_t* sq)
         /* polled with plain loads: an acquire per look would invalidate this compute unit's cache every time */
         while (((ld_relaxed(&sq->pos_locks[b].val) - (t >> shift)) & turn_mask) != 0)
             if (spin_giveup(sq, sp)) break;
-        fence_acquire_agent();
+        fence_meta();
         st_relaxed(&sq->head_mark[b].val, popc(act));       /* ids of this block still out */
         base = b << 6;
     }
@@ -112,12 +112,13 @@ __device__ __forceinline__ uint32_t get_cid_group(nvm_queue_t* sq)
 __device__ __forceinline__ void put_cid_group(nvm_queue_t* sq, uint32_t id)
 {
     st_relaxed(&sq->cid[id].val, (uint32_t)UNLOCKED);
+    fence_meta();                    /* whatever the lanes did with their ids and staging pages is over */
     for_each_group((uint64_t)(id >> 6), [&](uint64_t b) {
         const uint64_t grp = active_mask();
         if (lane() == first_lane(grp)) {
             const uint32_t k = popc(grp);
-            if (__hip_atomic_fetch_add(&sq->head_mark[b].val, 0u - k, __ATOMIC_RELEASE, BAM_AGENT) == k)
-                __hip_atomic_fetch_add(&sq->pos_locks[b].val, 1u, __ATOMIC_RELEASE, BAM_AGENT);   /* next turn */
+            if (__hip_atomic_fetch_add(&sq->head_mark[b].val, 0u - k, __ATOMIC_RELAXED, BAM_AGENT) == k)
+                __hip_atomic_fetch_add(&sq->pos_locks[b].val, 1u, __ATOMIC_RELAXED, BAM_AGENT);   /* next turn */
         }
     });
 }
@@ -143,20 +144,21 @@ __device__ __forceinline__ bool try_drain_group(nvm_queue_t* cq, nvm_queue_t* sq
          * the next two microseconds, so that a stale or never-written value can never hold anybody up */
         const uint32_t ahead = ld_relaxed(&cq->tail) - (uint32_t)wall_clock64();
         if (ahead - 1u >= BAM_CQ_IDLE_TICKS && ld_relaxed(&cq->head_lock) == UNLOCKED &&
-            __hip_atomic_exchange(&cq->head_lock, (uint32_t)LOCKED, __ATOMIC_ACQUIRE, BAM_AGENT) == UNLOCKED) {
+            __hip_atomic_exchange(&cq->head_lock, (uint32_t)LOCKED, __ATOMIC_RELAXED, BAM_AGENT) == UNLOCKED) {
+            fence_meta();
             const uint32_t h = ld_relaxed(&cq->head);
-            const uint32_t dw3 = ld_acquire_sys(&((nvm_cpl_t*)cq->vaddr)[h & cq->qs_minus_1].dword[3]);
+            const uint32_t dw3 = ld_relaxed_sys(&((nvm_cpl_t*)cq->vaddr)[h & cq->qs_minus_1].dword[3]);
             if (((dw3 >> 16) & 1u) == ((~(h >> cq->qs_log2)) & 1u)) got = 1;
             else {
                 st_relaxed(&cq->tail, (uint32_t)wall_clock64() + BAM_CQ_IDLE_TICKS);      /* nothing new: leave the ring alone for a while */
-                st_release(&cq->head_lock, (uint32_t)UNLOCKED);
+                st_publish(&cq->head_lock, (uint32_t)UNLOCKED);
             }
         }
     }
     got = bcast(got, leader);
     if (got) {
         cq_drain_group(cq, sq, act);
-        if (lane() == leader) st_release(&cq->head_lock, (uint32_t)UNLOCKED);
+        if (lane() == leader) st_publish(&cq->head_lock, (uint32_t)UNLOCKED);
     }
     return got != 0;
 }
@@ -181,12 +183,14 @@ __device__ __forceinline__ uint32_t sq_enqueue_group(nvm_queue_t* sq, nvm_cmd_t*
     spin_t sp;
     for (;;) {
         if (!written && ld_relaxed(&sq->tickets[pos].val) == want) {
-            fence_acquire_agent();
-            uint4* dst = (uint4*)(((nvm_cmd_t*)sq->vaddr) + pos);
-            const uint4* src = (const uint4*)cmd->dword;
-            dst[0] = src[0]; dst[1] = src[1]; dst[2] = src[2]; dst[3] = src[3];
-            /* the entry must be visible to the controller before the mark can be swept into a doorbell */
-            st_release_sys(&sq->tail_mark[pos].val, 1u);
+            fence_meta();
+            /* written through to the ring, which may be host memory the L2 would otherwise hold on to */
+            uint64_t* dst = (uint64_t*)(((nvm_cmd_t*)sq->vaddr) + pos);
+            const uint64_t* src = (const uint64_t*)cmd->dword;
+#pragma unroll
+            for (int i = 0; i < 8; i++) __hip_atomic_store(dst + i, src[i], __ATOMIC_RELAXED, BAM_SYSTEM);
+            /* the entry must have left for the controller before the mark can be swept into a doorbell */
+            st_publish(&sq->tail_mark[pos].val, 1u);
             written = true;
         }
         const uint32_t tl = ld_relaxed(&sq->tail);
@@ -198,28 +202,29 @@ __device__ __forceinline__ uint32_t sq_enqueue_group(nvm_queue_t* sq, nvm_cmd_t*
             uint32_t got = 0;
             if (lane() == leader)
                 got = ld_relaxed(&sq->tail_lock) == UNLOCKED &&
-                      __hip_atomic_exchange(&sq->tail_lock, (uint32_t)LOCKED, __ATOMIC_ACQUIRE, BAM_AGENT) == UNLOCKED;
+                      __hip_atomic_exchange(&sq->tail_lock, (uint32_t)LOCKED, __ATOMIC_RELAXED, BAM_AGENT) == UNLOCKED;
             got = bcast(got, leader);
             if (got) {
+                fence_meta();
                 const uint32_t cur = ld_relaxed(&sq->tail);
                 /* never let tail + 1 == head (mod qs): at most qs - 1 entries outstanding */
-                const uint32_t room = ld_acquire(&sq->head) + sq->qs - 1u - cur;
+                const uint32_t room = ld_relaxed(&sq->head) + sq->qs - 1u - cur;
                 uint32_t total = 0;
                 for (;;) {
                     const uint32_t k = total + rank;
-                    const bool m = k < room && ld_acquire(&sq->tail_mark[(cur + k) & mask].val) == 1u;
+                    const bool m = k < room && ld_relaxed(&sq->tail_mark[(cur + k) & mask].val) == 1u;
                     const uint32_t run = leading_run(act, ballot(m));
                     if (rank < run) st_relaxed(&sq->tail_mark[(cur + k) & mask].val, 0u);
                     total += run;
                     if (run < n) break;
                 }
+                fence_meta();                /* the marks read and cleared above: before the doorbell and the unlock */
                 if (lane() == leader) {
                     if (total) {
-                        fence_release_sys();
                         st_relaxed_sys(sq->db, (cur + total) & mask);     /* one doorbell for the whole run */
-                        st_release(&sq->tail, cur + total);
+                        st_relaxed(&sq->tail, cur + total);
                     }
-                    st_release(&sq->tail_lock, (uint32_t)UNLOCKED);
+                    st_publish(&sq->tail_lock, (uint32_t)UNLOCKED);
                 }
                 progressed = total != 0;
             }
@@ -249,12 +254,13 @@ __device__ __forceinline__ void cq_drain_group(nvm_queue_t* cq, nvm_queue_t* sq,
     for (;;) {
         const uint32_t idx = h + moved + rank, loc = idx & mask;
         const uint32_t phase = (~(idx >> cq->qs_log2)) & 1u;          /* first lap carries phase 1 */
-        const uint32_t dw3 = ld_acquire_sys(&ring[loc].dword[3]);
+        const uint32_t dw3 = ld_relaxed_sys(&ring[loc].dword[3]);
+        fence_meta();
         const bool valid = ((dw3 >> 16) & 1u) == phase && moved + rank < mask;
         const uint32_t run = leading_run(act, ballot(valid));
         if (rank < run) {
             if (dw3 >> 17) __hip_atomic_fetch_add(&cq->n_errors, 1u, __ATOMIC_RELAXED, BAM_AGENT);
-            st_release(&sq->cid[dw3 & sq->cid_mask].val, (uint32_t)LOCKED | BAM_CID_DONE);
+            st_relaxed(&sq->cid[dw3 & sq->cid_mask].val, (uint32_t)LOCKED | BAM_CID_DONE);
         }
         if (run) {
             uint32_t v = 0;
@@ -270,12 +276,13 @@ __device__ __forceinline__ void cq_drain_group(nvm_queue_t* cq, nvm_queue_t* sq,
         const uint32_t smask = sq->qs_minus_1;
         const uint32_t sh = ld_relaxed(&sq->head);
         const uint32_t freed = (sqhd - sh) & smask;
+        fence_meta();
         for (uint32_t i = rank; i < freed; i += n)
-            __hip_atomic_fetch_add(&sq->tickets[(sh + i) & smask].val, 2u, __ATOMIC_RELEASE, BAM_AGENT);
+            __hip_atomic_fetch_add(&sq->tickets[(sh + i) & smask].val, 2u, __ATOMIC_RELAXED, BAM_AGENT);
         if (lane() == leader) {
-            if (freed) st_release(&sq->head, sh + freed);
+            if (freed) st_relaxed(&sq->head, sh + freed);
             st_relaxed_sys(cq->db, (h + moved) & mask);                /* one doorbell for the whole run */
-            st_release(&cq->head, h + moved);
+            st_relaxed(&cq->head, h + moved);
         }
     }
 }

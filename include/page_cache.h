@@ -207,6 +207,10 @@ __device__ __forceinline__ uint32_t io_submit_group(page_cache_d_t* pc, QueuePai
     const uint64_t act = active_mask();
     const uint32_t n = popc(act), rank = rank_in(act);
     const uint32_t bytes = n_blocks << qp->block_size_log;
+    /* payload on its way out was written with plain stores, maybe by other compute units (which made it visible
+     * when they dropped their references): nothing stale may be read when it is copied to a staging page, and
+     * what this wave wrote itself must have reached memory before the controller fetches it */
+    if (opcode == NVM_IO_WRITE) __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "");
 #ifdef BAM_PROFILE
     const uint64_t pt0 = wall_clock64();
 #endif
@@ -231,7 +235,7 @@ __device__ __forceinline__ uint32_t io_submit_group(page_cache_d_t* pc, QueuePai
         if (bytes > qp->pageSize) prp2 = prp1 + qp->pageSize;         /* staging pages are contiguous: second controller page */
         if (opcode == NVM_IO_WRITE) {
             copy_pages(stage, pc->base_addr + pc_entry * pc->page_size, bytes, act, n, rank);
-            fence_release_sys();
+            fence_release_sys();             /* plain stores to host memory: written back before the command goes out */
         }
     } else {
         prp1 = pc->prp1[pc_entry];
@@ -411,19 +415,20 @@ uint32_t page_cache_d_t::find_slot(uint64_t address, uint64_t range_id, const ui
             cache_page_t* cp = &cache_pages[p];
             uint32_t v = ld_relaxed(&cp->page_take_lock);
             if (v == FREE) {
-                if (__hip_atomic_compare_exchange_strong(&cp->page_take_lock, &v, (uint32_t)LOCKED, __ATOMIC_ACQUIRE, __ATOMIC_RELAXED, BAM_AGENT)) {
-                    cp->page_translation = global_address;
-                    st_release(&cp->page_take_lock, (uint32_t)UNLOCKED);
+                if (__hip_atomic_compare_exchange_strong(&cp->page_take_lock, &v, (uint32_t)LOCKED, __ATOMIC_RELAXED, __ATOMIC_RELAXED, BAM_AGENT)) {
+                    st_relaxed(&cp->page_translation, global_address);
+                    st_publish(&cp->page_take_lock, (uint32_t)UNLOCKED);
                     page = p; looking = false;
                 }
             } else if (v == UNLOCKED) {
-                if (__hip_atomic_compare_exchange_strong(&cp->page_take_lock, &v, (uint32_t)LOCKED, __ATOMIC_ACQUIRE, __ATOMIC_RELAXED, BAM_AGENT)) {
-                    const uint64_t prev = cp->page_translation;
+                if (__hip_atomic_compare_exchange_strong(&cp->page_take_lock, &v, (uint32_t)LOCKED, __ATOMIC_RELAXED, __ATOMIC_RELAXED, BAM_AGENT)) {
+                    fence_meta();
+                    const uint64_t prev = ld_relaxed(&cp->page_translation);
                     const uint64_t prev_range = prev & n_ranges_mask, prev_page = prev >> n_ranges_bits;
                     data_page_t* victim = &ranges[prev_range][prev_page];
                     const uint32_t e = ld_relaxed(&victim->state);
                     if ((e & CNT_MASK) == 0 && (e & BUSY) == 0) {
-                        const uint32_t o = __hip_atomic_fetch_or(&victim->state, BUSY, __ATOMIC_ACQUIRE, BAM_AGENT);
+                        const uint32_t o = __hip_atomic_fetch_or(&victim->state, BUSY, __ATOMIC_RELAXED, BAM_AGENT);
                         if ((o & BUSY) == 0) {
                             if ((o & CNT_MASK) == 0) {
                                 if (o & DIRTY) {
@@ -437,15 +442,16 @@ uint32_t page_cache_d_t::find_slot(uint64_t address, uint64_t range_id, const ui
                                     }
                                 }
                                 /* -> INVALID; references taken meanwhile stay counted and their owners reload */
-                                __hip_atomic_fetch_and(&victim->state, CNT_MASK, __ATOMIC_RELEASE, BAM_AGENT);
-                                cp->page_translation = global_address;
+                                fence_meta();
+                                __hip_atomic_fetch_and(&victim->state, CNT_MASK, __ATOMIC_RELAXED, BAM_AGENT);
+                                st_relaxed(&cp->page_translation, global_address);
                                 page = p; looking = false;
                             } else {
-                                __hip_atomic_fetch_and(&victim->state, DISABLE_BUSY_MASK, __ATOMIC_RELEASE, BAM_AGENT);
+                                __hip_atomic_fetch_and(&victim->state, DISABLE_BUSY_MASK, __ATOMIC_RELAXED, BAM_AGENT);
                             }
                         }
                     }
-                    st_release(&cp->page_take_lock, (uint32_t)UNLOCKED);
+                    st_publish(&cp->page_take_lock, (uint32_t)UNLOCKED);
                 }
             }
             if (looking && tries + 1 >= BAM_FIND_SLOT_TRIES) looking = false;
@@ -584,10 +590,10 @@ bool range_d_t<T>::slow_step(const size_t pg, const bool write, const uint32_t q
         if (!may_load) {
             *wants_load = true;                 /* the caller has to be admitted to the miss path first */
         } else {
-            const uint32_t o = __hip_atomic_fetch_or(&dp->state, BUSY, __ATOMIC_ACQUIRE, BAM_AGENT);
+            const uint32_t o = __hip_atomic_fetch_or(&dp->state, BUSY, __ATOMIC_RELAXED, BAM_AGENT);
             if ((o & BUSY) == 0) {
                 if ((o >> (CNT_SHIFT + 1)) == NV_NB) load_me = true;
-                else __hip_atomic_fetch_and(&dp->state, DISABLE_BUSY_MASK, __ATOMIC_RELEASE, BAM_AGENT);  /* became valid meanwhile */
+                else __hip_atomic_fetch_and(&dp->state, DISABLE_BUSY_MASK, __ATOMIC_RELAXED, BAM_AGENT);  /* became valid meanwhile */
             }
         }
     }
@@ -605,7 +611,7 @@ bool range_d_t<T>::slow_step(const size_t pg, const bool write, const uint32_t q
 #endif
         if (found == BAM_NO_SLOT) {
             /* no evictable slot right now: hand the page back; a later pass tries again */
-            __hip_atomic_fetch_and(&dp->state, DISABLE_BUSY_MASK, __ATOMIC_RELEASE, BAM_AGENT);
+            __hip_atomic_fetch_and(&dp->state, DISABLE_BUSY_MASK, __ATOMIC_RELAXED, BAM_AGENT);
             load_me = false;
         } else {
             uint64_t c = get_backing_ctrl(pg);
@@ -629,8 +635,12 @@ bool range_d_t<T>::slow_step(const size_t pg, const bool write, const uint32_t q
         if (held) read_end(qp, cid);
         st_relaxed(&dp->offset, found);
         if (write) __hip_atomic_fetch_or(&dp->state, DIRTY, __ATOMIC_RELAXED, BAM_AGENT);
+        /* payload this wave (helpers included) moved in with plain stores has to be written back for the other
+         * compute units before the page shows as valid; payload the controller placed is in memory already */
+        if (bam::ballot(stage != nullptr || !held)) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+        else fence_meta();
         /* BUSY -> 0 and VALID -> 1 in one step; publishes the payload and the offset */
-        __hip_atomic_fetch_xor(&dp->state, DISABLE_BUSY_ENABLE_VALID, __ATOMIC_RELEASE, BAM_AGENT);
+        __hip_atomic_fetch_xor(&dp->state, DISABLE_BUSY_ENABLE_VALID, __ATOMIC_RELAXED, BAM_AGENT);
         slot = found;
         was_hit = false;
         resolved = true;

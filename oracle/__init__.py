@@ -113,6 +113,11 @@ def _csr(n_v, u, v):
     return off, nb[:e].copy()
 
 
+def csr_from_pairs(n_vertices, u, v):
+    """symmetrized, sorted, deduplicated CSR of the pairs (u[k], v[k]), self loops dropped"""
+    return _csr(n_vertices, np.ascontiguousarray(u, dtype=np.uint64), np.ascontiguousarray(v, dtype=np.uint64))
+
+
 def bfs_sources(seed, offsets, n_src=8):
     out = np.empty(n_src, dtype=np.uint64)
     lib().bo_bfs_sources(seed, len(offsets) - 1, offsets, n_src, out)

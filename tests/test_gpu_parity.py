@@ -533,6 +533,31 @@ def test_cc_labels_uniform_by_edge_page(bam, n_v, n_p, cache_pages):
         assert not r.c.aborted()
 
 
+@pytest.mark.parametrize("cache_pages,coarse", [(24, 1), (256, 4), (4096, 64), (4096, 200)])
+def test_hub_lists_are_cut_into_pieces(bam, cache_pages, coarse):
+    """two hubs with lists of 9000 and 4096 entries (18 and 8 pages) on top of a sparse random graph: the per-vertex
+    kernels queue such lists in pieces for a second launch; levels and labels must not notice.  The hubs sit in
+    different components until an edge of the random part joins them."""
+    n_v = 20000
+    pu = np.empty(6000, dtype=np.uint64); pv = np.empty(6000, dtype=np.uint64)
+    oracle.lib().bo_uniform_edges(SEED, n_v, 0, 6000, pu, pv)
+    hub_a = np.full(9000, 7, dtype=np.uint64); leaves_a = np.arange(100, 9100, dtype=np.uint64)
+    hub_b = np.full(4096, 15000, dtype=np.uint64); leaves_b = np.arange(9100, 9100 + 4096, dtype=np.uint64)
+    off, nb = oracle.csr_from_pairs(n_v, np.concatenate([pu, hub_a, hub_b]), np.concatenate([pv, leaves_a, leaves_b]))
+    deg = np.diff(off.astype(np.int64))
+    assert deg[7] >= 9000 and deg[15000] >= 4096
+    r, a = _graph_rig(bam, nb, cache_pages, n_queues=8, depth=256)
+    with r:
+        doff = _dev(off)
+        for src in (7, 15000, 100, int(oracle.bfs_sources(SEED, off, 1)[0])):
+            lv, it = a.bfs(doff, src, coarse=coarse)
+            want, want_it = oracle.bfs_levels(off, nb, src)
+            assert np.array_equal(lv.cpu().numpy().view(np.uint32), want) and it == want_it
+        lb, _ = a.cc(doff, coarse=coarse)
+        assert np.array_equal(_u64(lb), oracle.cc_labels(off, nb)[0])
+        assert not r.c.aborted()
+
+
 @pytest.mark.parametrize("scale,cache_pages", [(10, 2048), (13, 160)])
 def test_sssp_costs_two_arrays_in_one_cache(bam, scale, cache_pages):
     """neighbour ids (64-bit) and weights (32-bit) as two arrays behind one page cache; costs against Dijkstra"""
