@@ -269,13 +269,14 @@ def main():
         ref = cpu_bfs_s = cpu_bfs_edges = None
         legs = {}
         # the edge-page kernel on every source; the reference-shaped kernel (a wave per vertex, bam_ptr per element) on the first two
-        for name, by_page, n_src in (("by_page", True, len(srcs)), ("per_vertex_bam_ptr", False, min(2, len(srcs)))):
+        # (64 vertices per wave: consecutive vertices share pages, so the more vertices a wave has, the more distinct pages are asked for at a time)
+        for name, by_page, n_src, coarse in (("by_page", True, len(srcs), 1), ("per_vertex_bam_ptr", False, min(4, len(srcs)), 64)):
             tot_ms, tot_edges, levels_ok, iters = 0.0, 0, True, []
             ag.stats()
             for k, src in enumerate(srcs[:n_src]):
                 a, b = event(), event()
                 L.bam_event_record(a, stream)
-                lv, it = ag.bfs(off, int(src), coarse=4, by_page=by_page)
+                lv, it = ag.bfs(off, int(src), coarse=coarse, by_page=by_page)
                 L.bam_event_record(b, stream)
                 ms = elapsed_ms(a, b)
                 lv_h = lv.cpu().numpy().view(np.uint32)
@@ -291,7 +292,7 @@ def main():
                 iters.append(it)
             assert levels_ok and not ctrl.aborted(), "BFS levels differ from the oracle (%s)" % name
             st = ag.stats()
-            legs[name] = {"sources": n_src, "GTEPS": tot_edges / tot_ms / 1e6, "ms_per_source": tot_ms / n_src, "iterations": iters,
+            legs[name] = {"sources": n_src, "coarse": coarse, "GTEPS": tot_edges / tot_ms / 1e6, "ms_per_source": tot_ms / n_src, "iterations": iters,
                           "read_ios": st["read_io_cnt"], "MIOPS": st["read_io_cnt"] / tot_ms / 1e3,
                           "hit_rate": st["hit_cnt"] / max(st["access_cnt"], 1)}
             log("[bench] bfs %s: %s" % (name, legs[name]))
