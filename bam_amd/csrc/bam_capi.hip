@@ -347,21 +347,17 @@ struct list_read_ahead {
         const uint64_t r = da->d_ranges[0].cache.n_pages >> 6;
         reach = r > BAM_WAVE_SIZE ? BAM_WAVE_SIZE : (uint32_t)r;
     }
-    /* lanes with `act` are about to have the list of their vertex `v` walked: touch the first page of each list */
-    __device__ __forceinline__ void group(const uint64_t* vertexList, const bool act, const uint64_t v)
+    /* every lane's elements [es, ee) (empty for lanes without any) are about to be read: touch the first and the last page
+     * of each run, so that what is not resident comes in as one batch or two, not one trip to the store per run */
+    __device__ __forceinline__ void group(const uint64_t es, const uint64_t ee)
     {
         if (reach < 2) return;
-        bool want = false;
-        uint64_t pg = 0;
-        if (act) {
-            const uint64_t s = vertexList[v];
-            if (vertexList[v + 1] > s) { want = true; pg = view.page_of(s); }
-        }
-        if (bam::popc(bam::ballot(want)) < 2) return;          /* a single list: its walk does the same */
-        if (want) {
-            auto touch = [](uint32_t) { return true; };
-            view.acquire(pg, false, touch, touch);
-        }
+        const bool want = ee > es;
+        if (!bam::ballot(want)) return;
+        auto touch = [](uint32_t) { return true; };
+        const uint64_t pf = want ? view.page_of(es) : 0, pl = want ? view.page_of(ee - 1) : 0;
+        if (want) view.acquire(pf, false, touch, touch);
+        if (want && pl != pf) view.acquire(pl, false, touch, touch);
         view.n_access = view.n_hit = 0;
     }
     /* wave-uniform: the list is elements [start, end) */
@@ -390,14 +386,50 @@ struct list_read_ahead {
 };
 
 /*
- * The traversal of the reference's coarsened per-vertex kernels (bfs/main.cu:658-689, cc/main.cu:123-144): wave w
- * looks after vertices [w coarse, (w + 1) coarse) and walks the edge list of each active one, 64 entries per step
- * through bam_ptr, the first access aligned to 128 bytes.  Around that walk, for the store's sake: the vertices'
- * flags are read 64 at a time (one load and a ballot instead of `coarse` loads one after the other), the first
- * page of every active vertex of such a group is touched before the first list is walked (what is not resident
- * comes in as one batch of commands, not one trip per vertex), and long lists are read ahead (list_read_ahead).
- * The larger `coarse`, the more distinct pages the resident waves ask for at a time: consecutive vertices share
- * pages, so with one vertex per wave dozens of waves wait for the same page.
+ * Every lane brings a run of elements [es, ee) (possibly empty, each shorter than 2^20) and the vertex `src` the run
+ * belongs to; the wave visits all elements of all runs, 64 per step, consecutive lanes taking consecutive elements
+ * across the ends of the runs.  With lists of a dozen edges, walking one list per step leaves most lanes idle and
+ * pays the whole chain of dependent loads (offsets, payload, label) once per vertex; packed, it is paid once per 64
+ * edges.  A lane finds the run its element belongs to by binary search in the running sums of the run lengths
+ * (six shuffles).  `read(i)` fetches element i, `visit(src, value)` consumes it.
+ */
+template <typename Read, typename Visit>
+__device__ __forceinline__ void walk_packed(const uint64_t es, const uint64_t ee, const uint64_t src, Read read, Visit visit)
+{
+    const uint32_t lane = bam::lane();
+    const uint32_t len = (uint32_t)(ee - es);
+    uint32_t incl = len;
+#pragma unroll
+    for (uint32_t o = 1; o < BAM_WAVE_SIZE; o <<= 1) {
+        const uint32_t u = bam::shfl(incl, lane >= o ? lane - o : lane);
+        if (lane >= o) incl += u;
+    }
+    const uint32_t total = bam::shfl(incl, BAM_WAVE_SIZE - 1), excl = incl - len;
+    for (uint32_t base = 0; base < total; base += BAM_WAVE_SIZE) {
+        const uint32_t k = base + lane;
+        uint32_t j = 0;                                          /* number of runs that end at or before k */
+#pragma unroll
+        for (uint32_t step = BAM_WAVE_SIZE / 2; step; step >>= 1)
+            if (bam::shfl(incl, j + step - 1) <= k) j += step;
+        j &= BAM_WAVE_SIZE - 1;                                  /* lanes past the end: any valid lane, they do not visit */
+        const uint64_t i = bam::shfl(es, j) + (k - bam::shfl(excl, j));
+        const uint64_t s = bam::shfl(src, j);
+        if (k < total) visit(s, read(i));
+    }
+}
+
+/*
+ * The traversal of the reference's coarsened per-vertex kernels (bfs/main.cu:658-689, cc/main.cu:123-144): the
+ * vertices are handed out in groups of `coarse`, and the edge list of every active vertex is read through bam_ptr.
+ * What differs, for the store's and the memory system's sake:
+ *  - the launch has as many waves as the device holds at a time, and a wave takes the next group when it is done
+ *    with its last one (one atomic per group).  One group per wave of a large grid leaves most of the device idle
+ *    here: groups differ in length by orders of magnitude, and workgroups are started in order;
+ *  - the flags and offsets of 64 vertices are read at a time, one vertex per lane, and the lists of those vertices
+ *    are walked packed (walk_packed): 64 edges per step whichever vertices they belong to;
+ *  - before the walk the first and last page of every list are touched, so that what is not resident comes in as
+ *    one batch of commands or two, not one trip to the store per vertex;
+ *  - lists of BAM_HEAVY_EDGES entries and more are queued in pieces for a second launch (below).
  */
 /*
  * A list of BAM_HEAVY_EDGES entries or more is not walked by the wave that finds it: it is cut into pieces of that
@@ -405,36 +437,36 @@ struct list_read_ahead {
  * graph have lists of hundreds of pages; walked by one wave, a single hub takes longer than all other vertices of
  * its level together.
  */
-#define BAM_HEAVY_EDGES 4096u
+#define BAM_HEAVY_EDGES 1024u
 struct heavy_piece_t { uint64_t v, first, last; };      /* entries [first, last) of the list of vertex v */
 
 template <typename Active, typename Visit>
 __device__ __forceinline__ void walk_vertex_groups(array_d_t<uint64_t>* da, const uint64_t* vertexList, const uint64_t vertex_count, const uint64_t coarse,
                                                    heavy_piece_t* heavy, unsigned long long* n_heavy, Active active, Visit visit)
 {
-    const uint64_t tid = (uint64_t)blockDim.x * blockIdx.x + threadIdx.x;
-    const uint64_t waveIdx = tid / BAM_WAVE_SIZE, laneIdx = tid % BAM_WAVE_SIZE;
-    const uint64_t first = waveIdx * coarse;
-    if (first >= vertex_count) return;
+    const uint64_t laneIdx = threadIdx.x % BAM_WAVE_SIZE;
+    unsigned long long* next_group = n_heavy + 1;
+    const uint64_t n_groups = (vertex_count + coarse - 1) / coarse;
     bam_ptr<uint64_t> ptr(da);
     list_read_ahead<uint64_t> ahead;
     bool ready = false;
-#ifdef BAM_PROFILE
-    const uint64_t wt0 = wall_clock64();
-#endif
-    for (uint64_t b = 0; b < coarse; b += BAM_WAVE_SIZE) {
-        const uint64_t mine = first + b + laneIdx;
-        const bool act = b + laneIdx < coarse && mine < vertex_count && active(mine);
-        uint64_t m = bam::ballot(act);
-        if (!m) continue;
-        if (!ready) { ahead.init(da); ready = true; }
-        ahead.group(vertexList, act, mine);
-        for (; m; m &= m - 1) {
-            const uint64_t v = first + b + bam::first_lane(m);
-            const uint64_t start = vertexList[v];
-            const uint64_t shift_start = start & 0xFFFFFFFFFFFFFFF0ull;      /* 128-byte aligned first access */
-            const uint64_t end = vertexList[v + 1];
-            if (end - start >= BAM_HEAVY_EDGES) {
+    for (;;) {
+        unsigned long long g = 0;
+        if (laneIdx == 0) g = atomicAdd(next_group, 1ull);
+        g = bam::bcast((uint64_t)g, 0);
+        if (g >= n_groups) break;
+        const uint64_t first = g * coarse;
+        for (uint64_t b = 0; b < coarse; b += BAM_WAVE_SIZE) {
+            const uint64_t mine = first + b + laneIdx;
+            const bool act = b + laneIdx < coarse && mine < vertex_count && active(mine);
+            if (!bam::ballot(act)) continue;
+            if (!ready) { ahead.init(da); ready = true; }
+            uint64_t es = 0, ee = 0;
+            if (act) { es = vertexList[mine]; ee = vertexList[mine + 1]; }
+            /* long lists go to the queue, in pieces */
+            for (uint64_t hm = bam::ballot(ee - es >= BAM_HEAVY_EDGES); hm; hm &= hm - 1) {
+                const uint32_t j = bam::first_lane(hm);
+                const uint64_t start = bam::bcast(es, j), end = bam::bcast(ee, j), v = first + b + j;
                 const uint64_t pieces = (end - start + BAM_HEAVY_EDGES - 1) / BAM_HEAVY_EDGES;
                 unsigned long long at = 0;
                 if (laneIdx == 0) at = atomicAdd(n_heavy, (unsigned long long)pieces);
@@ -443,23 +475,12 @@ __device__ __forceinline__ void walk_vertex_groups(array_d_t<uint64_t>* da, cons
                     const uint64_t f = start + k * BAM_HEAVY_EDGES;
                     heavy[at + k] = heavy_piece_t{v, f, f + BAM_HEAVY_EDGES < end ? f + BAM_HEAVY_EDGES : end};
                 }
-                continue;
             }
-            ahead.begin(start, end);
-            for (uint64_t i = shift_start + laneIdx; i < end; i += BAM_WAVE_SIZE) {
-                ahead.step(i - laneIdx > start ? i - laneIdx : start);
-                if (i >= start) visit(v, ptr[i]);
-            }
+            if (ee - es >= BAM_HEAVY_EDGES) ee = es;
+            ahead.group(es, ee);
+            walk_packed(es, ee, mine, [&](uint64_t i) { return ptr.read(i); }, visit);
         }
     }
-#ifdef BAM_PROFILE
-    unsigned long long* prof = da->d_ranges[0].cache.prof;
-    if (prof && ready && laneIdx == 0) {
-        const unsigned long long dt = wall_clock64() - wt0;
-        atomicAdd(&prof[9], dt); atomicAdd(&prof[10], 1ull); atomicMax(&prof[11], dt);
-        if (dt > 100000ull) { atomicAdd(&prof[12], dt); atomicAdd(&prof[13], 1ull); }      /* waves that ran for more than a millisecond */
-    }
-#endif
 }
 
 /* the queued pieces, one wave at a time each: the same walk through bam_ptr, read ahead over the piece */
@@ -602,11 +623,8 @@ __device__ __forceinline__ void graph_by_page(array_d_t<uint64_t>* da, const uin
                     if (es < ps) es = ps;
                     if (ee > pe) ee = pe;
                 }
-                for (uint64_t am = bam::ballot(es < ee); am; am &= am - 1) {
-                    const uint32_t k = bam::first_lane(am);
-                    const uint64_t e0 = bam::bcast(es, k), e1 = bam::bcast(ee, k), src = vbase + k;
-                    for (uint64_t i = e0 + lane; i < e1; i += BAM_WAVE_SIZE) visit(src, bam::ld_payload(payload + (i - ps)));
-                }
+                if (ee < es) ee = es;
+                walk_packed(es, ee, v, [&](uint64_t i) { return bam::ld_payload(payload + (i - ps)); }, visit);
             }
         }
         if (want) view.release(p + pso_pages, false);
@@ -1407,18 +1425,28 @@ namespace {
 struct heavy_queue {
     BufferPtr buf, cnt;
     heavy_piece_t* pieces;
-    unsigned long long* count;
-    uint32_t blocks;
-    explicit heavy_queue(uint64_t n_edges)
+    unsigned long long* count;       /* [0] pieces queued in this sweep, [1] next group of vertices to hand out */
+    uint32_t blocks;                 /* launch of the piece walk */
+    uint64_t group;                  /* vertices handed to a wave at a time */
+    uint32_t group_blocks;           /* launch of the group walk: what the device holds at a time */
+    heavy_queue(uint64_t n_edges, uint64_t n_vertices, uint32_t coarse)
     {
         const uint64_t cap = 2 * (n_edges / BAM_HEAVY_EDGES) + 1;
         buf = createBuffer(cap * sizeof(heavy_piece_t), 0);
-        cnt = createBuffer(sizeof(unsigned long long), 0);
+        cnt = createBuffer(2 * sizeof(unsigned long long), 0);
         pieces = (heavy_piece_t*)buf.get();
         count = (unsigned long long*)cnt.get();
         const uint64_t waves = cap < 4096 ? cap : 4096;          /* the pieces are shared out over this many waves */
         blocks = (uint32_t)((waves + 1) / 2);                   /* two waves per workgroup */
+        /* one atomic per group on one word: a few hundred vertices per group keep that word out of the way */
+        group = coarse > 256 ? coarse : 256;
+        int dev = 0, cus = 0;
+        hip_err_chk(hipGetDevice(&dev));
+        hip_err_chk(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+        const uint64_t n_groups = (n_vertices + group - 1) / group, resident = (uint64_t)cus * 16;      /* waves */
+        group_blocks = (uint32_t)(((n_groups < resident ? n_groups : resident) + 1) / 2);
     }
+    void reset(hipStream_t st) { hip_err_chk(hipMemsetAsync(count, 0, 2 * sizeof(unsigned long long), st)); }
 };
 } // namespace
 
@@ -1435,17 +1463,15 @@ int bam_bfs(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, 
     hip_err_chk(hipMemsetAsync(d_labels, 0xFF, n_vertices * sizeof(uint32_t), st));
     hip_err_chk(hipMemcpyAsync(d_labels + src, &zero, sizeof(uint32_t), hipMemcpyHostToDevice, st));
     const uint32_t threads = 128;
-    const uint64_t n_waves = (n_vertices + coarse - 1) / coarse;
-    const uint32_t blocks = blocks_for(n_waves * BAM_WAVE_SIZE, threads);
-    heavy_queue hq(edges->a->adt.n_elems);
+    heavy_queue hq(edges->a->adt.n_elems, n_vertices, coarse);
     uint32_t level = 0, iter = 0;
     uint64_t changed_h;
     do {
         changed_h = 0;
         hip_err_chk(hipMemcpyAsync(changed_d, &changed_h, sizeof(uint64_t), hipMemcpyHostToDevice, st));
-        hip_err_chk(hipMemsetAsync(hq.count, 0, sizeof(unsigned long long), st));
-        hipLaunchKernelGGL(k_bfs_coalesce_coarse_ptr_pc, dim3(blocks), dim3(threads), 0, st,
-                           edges->a->d_array_ptr, d_labels, level, n_vertices, d_offsets, changed_d, (uint64_t)coarse, hq.pieces, hq.count);
+        hq.reset(st);
+        hipLaunchKernelGGL(k_bfs_coalesce_coarse_ptr_pc, dim3(hq.group_blocks), dim3(threads), 0, st,
+                           edges->a->d_array_ptr, d_labels, level, n_vertices, d_offsets, changed_d, hq.group, hq.pieces, hq.count);
         hipLaunchKernelGGL(k_bfs_heavy_ptr_pc, dim3(hq.blocks), dim3(threads), 0, st, edges->a->d_array_ptr, d_labels, level, changed_d, hq.pieces, hq.count);
         hip_err_chk(hipGetLastError());
         iter++; level++;
@@ -1471,17 +1497,15 @@ int bam_cc(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, u
     hip_err_chk(hipMemsetAsync(curr, 0x01, n_vertices, st));
     hip_err_chk(hipMemsetAsync(next, 0x00, n_vertices, st));
     const uint32_t threads = 128;
-    const uint64_t n_waves = (n_vertices + coarse - 1) / coarse;
-    const uint32_t blocks = blocks_for(n_waves * BAM_WAVE_SIZE, threads);
-    heavy_queue hq(edges->a->adt.n_elems);
+    heavy_queue hq(edges->a->adt.n_elems, n_vertices, coarse);
     uint32_t iter = 0;
     bool changed_h;
     do {
         changed_h = false;
         hip_err_chk(hipMemcpyAsync(changed_d, &changed_h, sizeof(bool), hipMemcpyHostToDevice, st));
-        hip_err_chk(hipMemsetAsync(hq.count, 0, sizeof(unsigned long long), st));
-        hipLaunchKernelGGL(k_cc_coalesce_coarse_ptr_pc, dim3(blocks), dim3(threads), 0, st,
-                           edges->a->d_array_ptr, curr, next, n_vertices, d_offsets, (unsigned long long*)d_labels, changed_d, (uint64_t)coarse, hq.pieces, hq.count);
+        hq.reset(st);
+        hipLaunchKernelGGL(k_cc_coalesce_coarse_ptr_pc, dim3(hq.group_blocks), dim3(threads), 0, st,
+                           edges->a->d_array_ptr, curr, next, n_vertices, d_offsets, (unsigned long long*)d_labels, changed_d, hq.group, hq.pieces, hq.count);
         hipLaunchKernelGGL(k_cc_heavy_ptr_pc, dim3(hq.blocks), dim3(threads), 0, st, edges->a->d_array_ptr, next, (unsigned long long*)d_labels, changed_d,
                            hq.pieces, hq.count);
         hip_err_chk(hipGetLastError());

@@ -133,8 +133,7 @@ class PageCache:
         """Miss-path phase timers (only a library built with -DBAM_PROFILE fills them)."""
         out = (c_u64 * 16)()
         _chk(self.L.bam_page_cache_profile(self.h, out, int(reset)), "bam_page_cache_profile")
-        keys = ("batches", "commands", "t_cid", "t_submit", "t_wait", "t_copy", "t_find_slot", "find_slot_calls", "find_slot_lanes",
-                "t_waves", "waves", "t_wave_max", "t_long_waves", "long_waves")
+        keys = ("batches", "commands", "t_cid", "t_submit", "t_wait", "t_copy", "t_find_slot", "find_slot_calls", "find_slot_lanes")
         return dict(zip(keys, list(out)))
 
     def block_io(self, n_reqs, req_bytes, lbas=None, write=False, queue_policy=1, block_size=64):
