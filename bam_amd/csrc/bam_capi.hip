@@ -356,8 +356,9 @@ struct list_read_ahead {
         if (!bam::ballot(want)) return;
         auto touch = [](uint32_t) { return true; };
         const uint64_t pf = want ? view.page_of(es) : 0, pl = want ? view.page_of(ee - 1) : 0;
-        if (want) view.acquire(pf, false, touch, touch);
-        if (want && pl != pf) view.acquire(pl, false, touch, touch);
+        /* all lanes go in: those without a page of their own help move what the others load */
+        view.acquire_helped(pf, want, false, touch, touch);
+        if (bam::ballot(want && pl != pf)) view.acquire_helped(pl, want && pl != pf, false, touch, touch);
         view.n_access = view.n_hit = 0;
     }
     /* wave-uniform: the list is elements [start, end) */
@@ -376,10 +377,8 @@ struct list_read_ahead {
         const uint64_t pg = view.page_of(at);
         if (pg < asked_to) return;
         const uint64_t p = pg + bam::lane();
-        if (bam::lane() < reach && p <= last_page) {
-            auto touch = [](uint32_t) { return true; };
-            view.acquire(p, false, touch, touch);
-        }
+        auto touch = [](uint32_t) { return true; };
+        view.acquire_helped(p, bam::lane() < reach && p <= last_page, false, touch, touch);
         asked_to = pg + reach;
         view.n_access = view.n_hit = 0;         /* not accesses of the kernel's own: kept out of the counters */
     }
@@ -606,9 +605,10 @@ __device__ __forceinline__ void graph_by_page(array_d_t<uint64_t>* da, const uin
             for (uint64_t v = va; v <= vb && !want; v++) want = active(v) && offsets[v] < pend && offsets[v + 1] > pstart;
         }
         uint32_t slot = 0;
-        if (want) {
+        if (bam::ballot(want)) {
+            /* the lanes without a page of their own come along and help move what the others load */
             auto keep = [&](uint32_t s_) { slot = s_; return false; };
-            view.acquire(p + pso_pages, false, keep, keep);
+            view.acquire_helped(p + pso_pages, want, false, keep, keep);
         }
         for (uint64_t m = bam::ballot(want); m; m &= m - 1) {
             const uint32_t j = bam::first_lane(m);

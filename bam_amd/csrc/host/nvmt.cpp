@@ -331,16 +331,32 @@ void serve_sq(nvmt* t, IoThread* me, Sq& sq)
 void io_loop(nvmt* t, IoThread* me)
 {
     uint32_t idle = 0;
+    const bool dbg = getenv("NVMT_DEBUG_LOOP") != nullptr;
+    uint64_t d_sweeps = 0, d_busy_sweeps = 0, d_visits = 0, d_cmds = 0, d_busy_ns = 0, d_max_sweep_ns = 0, d_t_first = 0, d_t_last = 0;
     while (!t->stop.load(std::memory_order_relaxed)) {
         bool any = false;
         {
             std::lock_guard<std::mutex> g(me->mu);
+            const auto s0 = dbg ? std::chrono::steady_clock::now() : std::chrono::steady_clock::time_point();
             for (uint16_t id : me->sqs) {
                 Sq& sq = t->sqs[id];
                 if (!sq.valid) continue;
                 uint32_t before = sq.head;
                 serve_sq(t, me, sq);
                 any |= before != sq.head;
+                if (dbg && before != sq.head) { d_visits++; d_cmds += (sq.head - before) & (sq.qs - 1); }
+            }
+            if (dbg) {
+                const uint64_t ns = (uint64_t)std::chrono::duration_cast<std::chrono::nanoseconds>(std::chrono::steady_clock::now() - s0).count();
+                d_sweeps++;
+                if (any) {
+                    d_busy_sweeps++;
+                    d_busy_ns += ns;
+                    if (ns > d_max_sweep_ns) d_max_sweep_ns = ns;
+                    const uint64_t now = (uint64_t)std::chrono::duration_cast<std::chrono::nanoseconds>(s0.time_since_epoch()).count();
+                    if (!d_t_first) d_t_first = now;
+                    d_t_last = now + ns;
+                }
             }
             if (me->sqs.empty()) idle = 1u << 20;
         }
@@ -348,6 +364,10 @@ void io_loop(nvmt* t, IoThread* me)
         else if (++idle > 4096) std::this_thread::sleep_for(std::chrono::microseconds(idle > (1u << 19) ? 200 : 20));
         else cpu_relax();
     }
+    if (dbg && d_cmds)
+        fprintf(stderr, "[nvmt loop] queues %zu: busy sweeps %llu of %llu, busy time %.1f ms over a span of %.1f ms, max sweep %.1f us, visits with work %llu, cmds %llu (%.2f per visit, %.2f us per cmd)\n",
+                me->sqs.size(), (unsigned long long)d_busy_sweeps, (unsigned long long)d_sweeps, d_busy_ns / 1e6, (d_t_last - d_t_first) / 1e6, d_max_sweep_ns / 1e3,
+                (unsigned long long)d_visits, (unsigned long long)d_cmds, (double)d_cmds / d_visits, d_busy_ns / 1e3 / d_cmds);
 }
 
 // ---- admin side ----

@@ -794,14 +794,31 @@ struct range_view {
     template <bool OUTLINE = false, typename FH, typename FM>
     __forceinline__ __device__ void acquire(const uint64_t page, const bool write, FH&& on_hit, FM&& on_miss)
     {
+        acquire_<OUTLINE, false>(page, write, on_hit, on_miss, true);
+    }
+    /*
+     * The same for callers of which only some lanes want a page (`take`): the others come along to help.  A wave that
+     * touches two or three pages ahead of its work would otherwise have each staged page moved by the two or three
+     * lanes that asked, sixty-four round trips over the interconnect per page instead of one.
+     */
+    template <bool OUTLINE = false, typename FH, typename FM>
+    __forceinline__ __device__ void acquire_helped(const uint64_t page, const bool take, const bool write, FH&& on_hit, FM&& on_miss)
+    {
+        acquire_<OUTLINE, true>(page, write, on_hit, on_miss, take);
+    }
+    template <bool OUTLINE, bool HELPERS, typename FH, typename FM>
+    __forceinline__ __device__ void acquire_(const uint64_t page_, const bool write, FH&& on_hit, FM&& on_miss, const bool take)
+    {
         const uint32_t me = lane();
+        /* helpers form a group of their own on a page number no range has; they take nothing */
+        const uint64_t page = HELPERS && !take ? ~0ull : page_;
         const uint64_t eq_mask = match_any(page, (uint64_t)r);
         const uint32_t master = first_lane(eq_mask), count = popc(eq_mask);
         const bool dirty = (ballot(write) & eq_mask) != 0;
         data_page_t* dp = pages + page;
         uint64_t sv = 0, pack = 0;
         uint32_t slot = 0;
-        if (master == me) { const bool h = bam_try_hit(dp, count, dirty, sv, slot); pack = (uint64_t)slot | ((uint64_t)h << 63); }
+        if (master == me && (!HELPERS || take)) { const bool h = bam_try_hit(dp, count, dirty, sv, slot); pack = (uint64_t)slot | ((uint64_t)h << 63); }
         pack = shfl(pack, master);
         if (__builtin_expect((pack >> 63) != 0, 1)) {          /* resident: the path to keep lean; register spills, if any, belong in the other branch */
             account(true);
@@ -813,7 +830,7 @@ struct range_view {
             /* miss path: pass after pass; groups whose page came in are served and release before the next pass */
             const uint32_t queue = wave_slot_hash();
             const uint32_t leader = first_lane(active_mask());
-            bool done = false;
+            bool done = HELPERS && !take;
             spin_t sp;
             /*
              * Admission: only so many waves per compute unit load pages at a time.  Every wave that has I/O in
@@ -827,6 +844,7 @@ struct range_view {
             const uint32_t limit = cache->miss_waves;
             uint32_t* tokens = cache->miss_tokens + (cu_id() & (BAM_TOKEN_SLOTS - 1)) * 16;
             bool admitted = limit == 0;
+            if (!HELPERS || ballot(!done))          /* helpers alone: nobody missed, nothing to help with */
             for (;;) {
                 /* every lane of the miss branch goes in: the masters that still wait for their page take part, the rest help move payload */
                 const bool part = !done && master == me;
