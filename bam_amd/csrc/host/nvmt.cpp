@@ -227,7 +227,7 @@ uint16_t do_rw(nvmt* t, Stats& st_, const nvm_cmd_t& c, bool write)
         done += len;
     });
     if (!ok) return ST_INVALID_FIELD;
-    if (!write) copy_out_fence();       /* streaming stores are weakly ordered: drain them before the completion is posted */
+    /* streaming stores are weakly ordered: the caller drains them (copy_out_fence) before it posts completions */
     if (write) { st_.bump(st_.write_cmds); st_.bump(st_.bytes_written, bytes); }
     else       { st_.bump(st_.read_cmds);  st_.bump(st_.bytes_read, bytes); }
     return ST_OK;
@@ -239,7 +239,9 @@ bool post_cpl(nvmt* t, Stats& st_, Cq& cq, uint16_t sqid, uint16_t sqhd, uint16_
     // tail is an index in [0, qs); admin queues need not be powers of two
     const uint32_t next = cq.tail + 1 == cq.qs ? 0 : cq.tail + 1;
     bool stalled = false;
-    for (;;) {
+    // the head doorbell is written by the consumer, so reading it is a cache miss every time it has moved: it is
+    // looked at only when the ring is full as far as this side knows
+    while (next == cq.head_seen) {
         // the consumer can only have acknowledged entries that were posted: a doorbell value outside
         // [head_seen, tail] is an old one that arrived late, and is ignored
         const uint32_t hd = ld<uint32_t>(cq.head_db) % cq.qs;
@@ -307,14 +309,19 @@ void serve_sq(nvmt* t, IoThread* me, Sq& sq)
                 uint32_t j = (uint32_t)(me->rng % i), x = order[i - 1];
                 order[i - 1] = order[j]; order[j] = x;
             }
+        // all commands of the batch first, then one drain of the streaming stores, then their completions
+        uint16_t statuses[64];
+        bool dropped[64];
         for (uint32_t k = 0; k < n; k++) {
             const nvm_cmd_t& c = batch[order[k]];
             uint8_t op = c.dword[0] & 0xff;
-            uint16_t cid = c.dword[0] >> 16, status;
+            uint16_t status;
             const bool inject = t->cfg.drop_every || t->cfg.fail_every;
             const uint64_t seq = inject ? ++t->cmd_seq : 0;       // a shared counter only when fault injection needs one
             st_.bump(st_.io_cmds);
-            if (t->cfg.drop_every && seq % t->cfg.drop_every == 0) { st_.bump(st_.dropped); continue; }
+            dropped[k] = false;
+            statuses[k] = ST_OK;
+            if (t->cfg.drop_every && seq % t->cfg.drop_every == 0) { st_.bump(st_.dropped); dropped[k] = true; continue; }
             if (t->cfg.fail_every && seq % t->cfg.fail_every == 0) status = ST_DATA_XFER_ERROR;
             else if (op == NVM_IO_READ) status = do_rw(t, st_, c, false);
             else if (op == NVM_IO_WRITE) status = do_rw(t, st_, c, true);
@@ -323,7 +330,13 @@ void serve_sq(nvmt* t, IoThread* me, Sq& sq)
             if (status && t->trace_errors.load(std::memory_order_relaxed) > 0 && t->trace_errors.fetch_sub(1) > 0)
                 fprintf(stderr, "[nvmt] sq %u status %#x: dw0 %08x nsid %u prp1 %08x%08x prp2 %08x%08x slba %08x%08x dw12 %08x (sq head %u)\n",
                         sq.id, status, c.dword[0], c.dword[1], c.dword[7], c.dword[6], c.dword[9], c.dword[8], c.dword[11], c.dword[10], c.dword[12], sq.head);
-            if (!post_cpl(t, st_, cq, sq.id, (uint16_t)sq.head, cid, status, 0)) return;
+            statuses[k] = status;
+        }
+        copy_out_fence();
+        for (uint32_t k = 0; k < n; k++) {
+            if (dropped[k]) continue;
+            const uint16_t cid = batch[order[k]].dword[0] >> 16;
+            if (!post_cpl(t, st_, cq, sq.id, (uint16_t)sq.head, cid, statuses[k], 0)) return;
         }
     }
 }
