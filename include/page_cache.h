@@ -505,14 +505,20 @@ struct range_d_t {
 
 /*
  * Drop `count` references of a page.  A reader only has to have its loads of
- * the page returned before the count drops (a wave-level wait); only a writer
- * must also make its stores visible to the other compute units before an
- * evictor may write the page back, which costs an L2 write-back.
+ * the page returned before the count drops (a wait on the wave's own memory
+ * counters); only a writer must also make its stores visible to the other
+ * compute units before an evictor may write the page back, which costs an L2
+ * write-back.  The wait is spelt out: a release fence at workgroup scope
+ * compiles to a wait for LDS and scalar operations only (within a workgroup
+ * vector memory is ordered by the hardware), so a payload load could still be
+ * in flight when the count reached zero, and with a cache so small that a slot
+ * is evicted and refilled within that load's latency it returned the next
+ * page's data.
  */
 __forceinline__ __device__ void bam_release_refs(data_page_t* dp, const uint32_t count, const bool wrote)
 {
     if (bam::ballot(wrote)) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-    else __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    else bam::fence_meta();
     __hip_atomic_fetch_add(&dp->state, 0u - count, __ATOMIC_RELAXED, BAM_AGENT);
 }
 

@@ -457,6 +457,26 @@ def test_reduction_and_scan_through_bam_ptr(bam, n, block, cache_pages):
         assert a.stats()["access_cnt"] > 0 and not r.c.aborted()
 
 
+@pytest.mark.parametrize("direct_share", ["8", "3", "0"])
+def test_program_written_against_the_cpp_surface(bam, direct_share):
+    """bam_amd/examples/array_sum: an ordinary HIP program that includes page_cache.h and ctrl.h, builds the host objects
+    itself and launches its own kernels (operator[] and bam_ptr), as a benchmark of the reference does.  4096 waves, each
+    reading one page, share 256 cache slots: a slot is evicted and refilled within microseconds of its last read, which
+    is what once let a payload load that was still in flight when its reference was dropped return the next page's data
+    (most readily with payload placed directly by the target, hence the three placements)."""
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "bam_amd", "examples", "array_sum")
+    assert os.path.exists(exe), "bam_amd/examples/array_sum is built by make -C bam_amd/csrc"
+    n_elems, cache_pages, stride = 1 << 21, 256, 8                       # 4096 pages of data behind 256 cached pages
+    want = oracle.lib().bo_store_sum(SEED, 0, stride, n_elems // stride)
+    env = dict(os.environ, BAM_DIRECT_SHARE=direct_share)
+    for _ in range(3):
+        r = subprocess.run([exe, str(n_elems), str(cache_pages), str(stride), str(SEED)], capture_output=True, text=True, timeout=110, env=env)
+        assert r.returncode == 0, r.stdout + r.stderr
+        out = dict(line.split(None, 1) for line in r.stdout.splitlines() if line.startswith(("sum_by", "aborted")))
+        assert int(out["sum_by_index"], 16) == want and int(out["sum_by_ptr"], 16) == want and out["aborted"].strip() == "0"
+
+
 # ---------------------------------------------------------------- graphs
 
 def _graph_rig(bam, nb, cache_pages, **kw):
