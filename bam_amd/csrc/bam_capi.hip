@@ -390,7 +390,7 @@ struct list_read_ahead {
  * across the ends of the runs.  With lists of a dozen edges, walking one list per step leaves most lanes idle and
  * pays the whole chain of dependent loads (offsets, payload, label) once per vertex; packed, it is paid once per 64
  * edges.  A lane finds the run its element belongs to by binary search in the running sums of the run lengths
- * (six shuffles).  `read(i)` fetches element i, `visit(src, value)` consumes it.
+ * (six shuffles).  `read(i)` fetches element i, `visit(src, value, i)` consumes it.
  */
 template <typename Read, typename Visit>
 __device__ __forceinline__ void walk_packed(const uint64_t es, const uint64_t ee, const uint64_t src, Read read, Visit visit)
@@ -413,7 +413,7 @@ __device__ __forceinline__ void walk_packed(const uint64_t es, const uint64_t ee
         j &= BAM_WAVE_SIZE - 1;                                  /* lanes past the end: any valid lane, they do not visit */
         const uint64_t i = bam::shfl(es, j) + (k - bam::shfl(excl, j));
         const uint64_t s = bam::shfl(src, j);
-        if (k < total) visit(s, read(i));
+        if (k < total) visit(s, read(i), i);
     }
 }
 
@@ -499,7 +499,7 @@ __device__ __forceinline__ void walk_heavy_pieces(array_d_t<uint64_t>* da, const
         ahead.begin(pc.first, pc.last);
         for (uint64_t i = (pc.first & 0xFFFFFFFFFFFFFFF0ull) + laneIdx; i < pc.last; i += BAM_WAVE_SIZE) {
             ahead.step(i - laneIdx > pc.first ? i - laneIdx : pc.first);
-            if (i >= pc.first) visit(pc.v, ptr[i]);
+            if (i >= pc.first) visit(pc.v, ptr.read(i), i);
         }
     }
 }
@@ -511,7 +511,7 @@ __global__ __launch_bounds__(128) void k_bfs_coalesce_coarse_ptr_pc(array_d_t<ui
     bool any = false;
     walk_vertex_groups(da, vertexList, vertex_count, coarse, heavy, n_heavy,
                        [&](uint64_t v) { return label[v] == level; },
-                       [&](uint64_t, uint64_t next) { if (label[next] == MYINFINITY) { label[next] = level + 1; any = true; } });
+                       [&](uint64_t, uint64_t next, uint64_t) { if (label[next] == MYINFINITY) { label[next] = level + 1; any = true; } });
     if (any) *changed = 1;
 }
 
@@ -519,7 +519,7 @@ __global__ __launch_bounds__(128) void k_bfs_heavy_ptr_pc(array_d_t<uint64_t>* d
                                                          const heavy_piece_t* heavy, const unsigned long long* n_heavy)
 {
     bool any = false;
-    walk_heavy_pieces(da, heavy, n_heavy, [&](uint64_t, uint64_t next) { if (label[next] == MYINFINITY) { label[next] = level + 1; any = true; } });
+    walk_heavy_pieces(da, heavy, n_heavy, [&](uint64_t, uint64_t next, uint64_t) { if (label[next] == MYINFINITY) { label[next] = level + 1; any = true; } });
     if (any) *changed = 1;
 }
 
@@ -543,13 +543,13 @@ __global__ __launch_bounds__(128) void k_cc_coalesce_coarse_ptr_pc(array_d_t<uin
 {
     walk_vertex_groups(da, vertexList, vertex_count, coarse, heavy, n_heavy,
                        [&](uint64_t v) { return curr_visit[v]; },
-                       [&](uint64_t v, uint64_t next) { cc_compute(v, comp, next, next_visit, changed); });
+                       [&](uint64_t v, uint64_t next, uint64_t) { cc_compute(v, comp, next, next_visit, changed); });
 }
 
 __global__ __launch_bounds__(128) void k_cc_heavy_ptr_pc(array_d_t<uint64_t>* da, bool* next_visit, unsigned long long* comp, bool* changed,
                                                         const heavy_piece_t* heavy, const unsigned long long* n_heavy)
 {
-    walk_heavy_pieces(da, heavy, n_heavy, [&](uint64_t v, uint64_t next) { cc_compute(v, comp, next, next_visit, changed); });
+    walk_heavy_pieces(da, heavy, n_heavy, [&](uint64_t v, uint64_t next, uint64_t) { cc_compute(v, comp, next, next_visit, changed); });
 }
 
 // ---- BFS / CC by edge page (benchmarks/bfs/main.cu:1074-1140 kernel_optimized_ptr_pc, first-vertex table :122-181) ----
@@ -638,7 +638,7 @@ __global__ __launch_bounds__(64) void k_bfs_by_page(array_d_t<uint64_t>* da, uin
     bool any = false;
     graph_by_page(da, offsets, first, n_edges, ppw, (level & 1u) != 0,
                   [&](uint64_t v) { return label[v] == level; },
-                  [&](uint64_t, uint64_t next) { if (label[next] == MYINFINITY) { label[next] = level + 1; any = true; } });
+                  [&](uint64_t, uint64_t next, uint64_t) { if (label[next] == MYINFINITY) { label[next] = level + 1; any = true; } });
     if (any) *changed = 1;
 }
 
@@ -647,7 +647,7 @@ __global__ __launch_bounds__(64) void k_cc_by_page(array_d_t<uint64_t>* da, bool
 {
     graph_by_page(da, offsets, first, n_edges, ppw, (sweep & 1u) != 0,
                   [&](uint64_t v) { return curr_visit[v]; },
-                  [&](uint64_t src, uint64_t next) { cc_compute(src, comp, next, next_visit, changed); });
+                  [&](uint64_t src, uint64_t next, uint64_t) { cc_compute(src, comp, next, next_visit, changed); });
 }
 
 // ---- vectoradd (benchmarks/vectoradd/main.cu:102-117 kernel_baseline_ptr_pc): C[i] = A[i] + B[i], all three behind the cache ----
@@ -772,27 +772,21 @@ __global__ void k_pr_initialize(bool* label, float* delta, float* residual, floa
     }
 }
 
-/* one wave per vertex: every neighbour of a flagged vertex receives the vertex's delta */
-__global__ __launch_bounds__(128) void k_pr_coalesce_pc(array_d_t<uint64_t>* da, bool* label, const float* delta, float* residual,
-                                                        const uint64_t vertex_count, const uint64_t* vertexList)
+/* every neighbour of a flagged vertex receives the vertex's delta: the group walk of the per-vertex graph kernels; the flags
+ * are cleared by the host loop after the sweep */
+__global__ __launch_bounds__(128) void k_pr_coalesce_pc(array_d_t<uint64_t>* da, const bool* label, const float* delta, float* residual,
+                                                        const uint64_t vertex_count, const uint64_t* vertexList, uint64_t group,
+                                                        heavy_piece_t* heavy, unsigned long long* n_heavy)
 {
-    const uint64_t tid = (uint64_t)blockDim.x * blockIdx.x + threadIdx.x;
-    const uint64_t v = tid / BAM_WAVE_SIZE, laneIdx = tid % BAM_WAVE_SIZE;
-    if (v < vertex_count && label[v]) {
-        const uint64_t start = vertexList[v];
-        const uint64_t shift_start = start & 0xFFFFFFFFFFFFFFF0ull;
-        const uint64_t end = vertexList[v + 1];
-        const float d = delta[v];
-        list_read_ahead<uint64_t> ahead;
-        ahead.init(da);
-        ahead.begin(start, end);
-        for (uint64_t i = shift_start + laneIdx; i < end; i += BAM_WAVE_SIZE) {
-            ahead.step(i - laneIdx > start ? i - laneIdx : start);
-            if (i >= start) unsafeAtomicAdd(&residual[da->seq_read(i)], d);
-        }
-        __builtin_amdgcn_wave_barrier();
-        label[v] = false;
-    }
+    walk_vertex_groups(da, vertexList, vertex_count, group, heavy, n_heavy,
+                       [&](uint64_t v) { return label[v]; },
+                       [&](uint64_t src, uint64_t next, uint64_t) { unsafeAtomicAdd(&residual[next], delta[src]); });
+}
+
+__global__ __launch_bounds__(128) void k_pr_heavy_pc(array_d_t<uint64_t>* da, const float* delta, float* residual, const heavy_piece_t* heavy,
+                                                     const unsigned long long* n_heavy)
+{
+    walk_heavy_pieces(da, heavy, n_heavy, [&](uint64_t src, uint64_t next, uint64_t) { unsafeAtomicAdd(&residual[next], delta[src]); });
 }
 
 /* the same pushes taken page by page of the edge array; the flags are cleared by the host loop after the sweep */
@@ -801,7 +795,7 @@ __global__ __launch_bounds__(64) void k_pr_by_page(array_d_t<uint64_t>* da, cons
 {
     graph_by_page(da, offsets, first, n_edges, ppw, (sweep & 1u) != 0,
                   [&](uint64_t v) { return label[v]; },
-                  [&](uint64_t src, uint64_t next) { unsafeAtomicAdd(&residual[next], delta[src]); });
+                  [&](uint64_t src, uint64_t next, uint64_t) { unsafeAtomicAdd(&residual[next], delta[src]); });
 }
 
 __global__ void k_pr_update(bool* label, float* delta, float* residual, float* value, const uint64_t vertex_count, const uint64_t* vertexList,
@@ -818,28 +812,29 @@ __global__ void k_pr_update(bool* label, float* delta, float* residual, float* v
 }
 
 // ---- SSSP (benchmarks/sssp/main.cu:174-201 kernel_coalesce_pc, :282-292 update): 32-bit costs, weights in their own array ----
-__global__ __launch_bounds__(128) void k_sssp_coalesce_pc(array_d_t<uint64_t>* de, array_d_t<uint32_t>* dw, bool* label, uint32_t* newCostList,
-                                                          const uint64_t vertex_count, const uint64_t* vertexList)
+/* relaxation of the edges of the flagged vertices with the cost each has at the time (any cost a vertex holds is the cost of a
+ * path to it); the group walk of the per-vertex graph kernels, the weight of entry i read through a bam_ptr of its own */
+__device__ __forceinline__ void sssp_relax(uint32_t* newCostList, const bam_ptr<uint32_t>& weights, uint64_t src, uint64_t next, uint64_t i)
 {
-    const uint64_t tid = (uint64_t)blockDim.x * blockIdx.x + threadIdx.x;
-    const uint64_t v = tid / BAM_WAVE_SIZE, laneIdx = tid % BAM_WAVE_SIZE;
-    if (v < vertex_count && label[v]) {
-        const uint64_t start = vertexList[v];
-        const uint64_t shift_start = start & 0xFFFFFFFFFFFFFFF0ull;
-        const uint64_t end = vertexList[v + 1];
-        const uint32_t cost = newCostList[v];
-        for (uint64_t i = shift_start + laneIdx; i < end; i += BAM_WAVE_SIZE) {
-            /* somebody found a cheaper way to v meanwhile: the update step flags v again and the next round starts over from it */
-            if (__hip_atomic_load(&newCostList[v], __ATOMIC_RELAXED, BAM_AGENT) != cost) break;
-            if (i >= start) {
-                const uint64_t next = de->seq_read(i);
-                const uint32_t weight = dw->seq_read(i);
-                if (__hip_atomic_load(&newCostList[next], __ATOMIC_RELAXED, BAM_AGENT) > cost + weight) atomicMin(&newCostList[next], cost + weight);
-            }
-        }
-        __builtin_amdgcn_wave_barrier();
-        label[v] = false;
-    }
+    const uint32_t cost = __hip_atomic_load(&newCostList[src], __ATOMIC_RELAXED, BAM_AGENT) + weights[i];
+    if (__hip_atomic_load(&newCostList[next], __ATOMIC_RELAXED, BAM_AGENT) > cost) atomicMin(&newCostList[next], cost);
+}
+
+__global__ __launch_bounds__(128) void k_sssp_coalesce_pc(array_d_t<uint64_t>* de, array_d_t<uint32_t>* dw, const bool* label, uint32_t* newCostList,
+                                                          const uint64_t vertex_count, const uint64_t* vertexList, uint64_t group,
+                                                          heavy_piece_t* heavy, unsigned long long* n_heavy)
+{
+    bam_ptr<uint32_t> wptr(dw);
+    walk_vertex_groups(de, vertexList, vertex_count, group, heavy, n_heavy,
+                       [&](uint64_t v) { return label[v]; },
+                       [&](uint64_t src, uint64_t next, uint64_t i) { sssp_relax(newCostList, wptr, src, next, i); });
+}
+
+__global__ __launch_bounds__(128) void k_sssp_heavy_pc(array_d_t<uint64_t>* de, array_d_t<uint32_t>* dw, uint32_t* newCostList, const heavy_piece_t* heavy,
+                                                       const unsigned long long* n_heavy)
+{
+    bam_ptr<uint32_t> wptr(dw);
+    walk_heavy_pieces(de, heavy, n_heavy, [&](uint64_t src, uint64_t next, uint64_t i) { sssp_relax(newCostList, wptr, src, next, i); });
 }
 
 __global__ void k_sssp_update(bool* label, uint32_t* costList, const uint32_t* newCostList, const uint64_t vertex_count, bool* changed)
@@ -1686,6 +1681,7 @@ int bam_pagerank(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_verti
     if (by_page)
         if (int rc = plan_by_page(edges, d_offsets, n_vertices, st, pl)) return rc;
     const uint32_t upd_blocks = blocks_for(n_vertices, 256);
+    heavy_queue hq(edges->a->adt.n_elems, n_vertices, 1);
     hipLaunchKernelGGL(k_pr_initialize, dim3(upd_blocks), dim3(256), 0, st, label_d, delta_d, residual_d, d_value, n_vertices, d_offsets, alpha);
     uint32_t iter = 0;
     bool changed_h;
@@ -1698,8 +1694,11 @@ int bam_pagerank(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_verti
                                    (const uint64_t*)pl.first.get(), pl.n_edges, pl.ppw, iter);
             hip_err_chk(hipMemsetAsync(label_d, 0, n_vertices, st));
         } else {
-            hipLaunchKernelGGL(k_pr_coalesce_pc, dim3(blocks_for(n_vertices * BAM_WAVE_SIZE, 128)), dim3(128), 0, st, edges->a->d_array_ptr, label_d, delta_d,
-                               residual_d, n_vertices, d_offsets);
+            hq.reset(st);
+            hipLaunchKernelGGL(k_pr_coalesce_pc, dim3(hq.group_blocks), dim3(128), 0, st, edges->a->d_array_ptr, label_d, delta_d, residual_d, n_vertices,
+                               d_offsets, hq.group, hq.pieces, hq.count);
+            hipLaunchKernelGGL(k_pr_heavy_pc, dim3(hq.blocks), dim3(128), 0, st, edges->a->d_array_ptr, delta_d, residual_d, hq.pieces, hq.count);
+            hip_err_chk(hipMemsetAsync(label_d, 0, n_vertices, st));
         }
         iter++;
         hipLaunchKernelGGL(k_pr_update, dim3(upd_blocks), dim3(256), 0, st, label_d, delta_d, residual_d, d_value, n_vertices, d_offsets, tolerance, alpha, changed_d);
@@ -1797,13 +1796,17 @@ int bam_sssp(bam_array_t* edges, bam_array32_t* weights, const uint64_t* d_offse
     hip_err_chk(hipMemcpyAsync(d_costs + src, &zero, sizeof(uint32_t), hipMemcpyHostToDevice, st));
     hip_err_chk(hipMemcpyAsync(new_d + src, &zero, sizeof(uint32_t), hipMemcpyHostToDevice, st));
     const uint32_t threads = 128;
+    heavy_queue hq(edges->a->adt.n_elems, n_vertices, 1);
     uint32_t iter = 0;
     bool changed_h;
     do {
         changed_h = false;
         hip_err_chk(hipMemcpyAsync(changed_d, &changed_h, sizeof(bool), hipMemcpyHostToDevice, st));
-        hipLaunchKernelGGL(k_sssp_coalesce_pc, dim3(blocks_for(n_vertices * BAM_WAVE_SIZE, threads)), dim3(threads), 0, st,
-                           edges->a->d_array_ptr, weights->a->d_array_ptr, label_d, new_d, n_vertices, d_offsets);
+        hq.reset(st);
+        hipLaunchKernelGGL(k_sssp_coalesce_pc, dim3(hq.group_blocks), dim3(threads), 0, st, edges->a->d_array_ptr, weights->a->d_array_ptr, label_d, new_d,
+                           n_vertices, d_offsets, hq.group, hq.pieces, hq.count);
+        hipLaunchKernelGGL(k_sssp_heavy_pc, dim3(hq.blocks), dim3(threads), 0, st, edges->a->d_array_ptr, weights->a->d_array_ptr, new_d, hq.pieces, hq.count);
+        hip_err_chk(hipMemsetAsync(label_d, 0, n_vertices, st));
         hipLaunchKernelGGL(k_sssp_update, dim3(blocks_for(n_vertices, 256)), dim3(256), 0, st, label_d, d_costs, new_d, n_vertices, changed_d);
         hip_err_chk(hipGetLastError());
         iter++;

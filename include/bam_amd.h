@@ -129,7 +129,11 @@ int bam_block_checksum(bam_page_cache_t* pc, uint64_t n_slots, uint32_t req_byte
 
 /* ---- BFS (benchmarks/bfs/main.cu:658-689 kernel_coalesce_coarse_ptr_pc, host loop :1557-1566, 1577-1736) ----
  * Level-synchronous BFS from src: d_offsets[V+1] in device memory, neighbour ids read through the array,
- * d_labels[V] receives the level of every vertex (0xFFFFFFFF = unreachable).  *iterations = kernel launches. */
+ * d_labels[V] receives the level of every vertex (0xFFFFFFFF = unreachable).  *iterations = levels swept.
+ * The vertices are handed out in groups of max(coarse, 256) to as many waves as the device holds; the lists of 64
+ * vertices at a time are read through bam_ptr, 64 entries per step across list ends, and lists of 1024 entries and
+ * more are cut into pieces that a second launch per level walks with a wave each (the same for bam_cc, bam_sssp and
+ * bam_pagerank without by_page). */
 int bam_bfs(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t src, uint32_t* d_labels,
             uint32_t coarse, uint32_t* iterations, void* stream);
 /* ---- CC (benchmarks/cc/main.cu:123-144 cc_compute, :595-617 kernel, host loop :1410-1425, 1515-1521) ----
@@ -172,7 +176,8 @@ int bam_scan(bam_array_t* a, uint64_t n_elems, uint32_t block_size, uint64_t* d_
  * Residual pushes in single precision: every flagged vertex adds its delta to the residual of each neighbour (atomic
  * float adds, neighbour ids through the cache), then every vertex whose residual exceeds `tolerance` moves it into its
  * value and is flagged with delta = residual * alpha / degree.  d_value[V] receives the values; *iterations = sweeps.
- * by_page = 0: one wave per vertex as the reference; 1: along the pages of the edge array as bam_bfs_by_page.
+ * by_page = 0: vertex by vertex as the reference (the group walk of bam_bfs); 1: along the pages of the edge array as
+ * bam_bfs_by_page.
  * The order of the float adds is not fixed (neither is it in the reference), so values agree between runs only to
  * rounding, and a residual that lands within rounding of `tolerance` may be moved one sweep earlier or later;
  * whatever the order, on return 0 <= x - value <= x * tolerance / (1 - alpha) up to rounding, x the exact solution of

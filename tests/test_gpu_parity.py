@@ -575,6 +575,11 @@ def test_hub_lists_are_cut_into_pieces(bam, cache_pages, coarse):
             assert np.array_equal(lv.cpu().numpy().view(np.uint32), want) and it == want_it
         lb, _ = a.cc(doff, coarse=coarse)
         assert np.array_equal(_u64(lb), oracle.cc_labels(off, nb)[0])
+        # PageRank pushes over the same lists (tolerance as in test_pagerank_values)
+        x = oracle.pagerank_limit(off, nb, 0.85)
+        v, it = a.pagerank(doff, 0.85, 1e-3, 1000)
+        v = v.cpu().numpy().astype(np.float64)
+        assert 1 < it < 1000 and np.all(v <= x * (1 + 1e-5)) and np.all(v >= x * (1 - 1e-3 / 0.15 - 1e-5))
         assert not r.c.aborted()
 
 
