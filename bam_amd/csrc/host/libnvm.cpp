@@ -14,7 +14,6 @@
 #include "nvm_queue.h"
 #include "nvm_types.h"
 #include "nvm_util.h"
-#include "nvmt.h"
 
 #include <cerrno>
 #include <chrono>
@@ -37,7 +36,6 @@ struct CtrlBox {
 struct DmaBox {
     CtrlBox* ctrl;
     void* owned;            // memory allocated by nvm_dma_create (freed on unmap)
-    size_t device_size;     // non-zero: device memory, made known to the software targets (nvmt_device_range)
     nvm_dma_t map;          // flexible tail: must stay last
 };
 
@@ -385,15 +383,7 @@ static int map_identity(nvm_dma_t** map, const nvm_ctrl_t* ctrl, void* vaddr, si
 }
 
 int nvm_dma_map_host(nvm_dma_t** map, const nvm_ctrl_t* ctrl, void* vaddr, size_t size) { return map_identity(map, ctrl, vaddr, size); }
-int nvm_dma_map_device(nvm_dma_t** map, const nvm_ctrl_t* ctrl, void* devptr, size_t size)
-{
-    int err = map_identity(map, ctrl, devptr, size);
-    if (!err) {
-        box_of(*map)->device_size = size;
-        nvmt_device_range(devptr, size, 1);
-    }
-    return err;
-}
+int nvm_dma_map_device(nvm_dma_t** map, const nvm_ctrl_t* ctrl, void* devptr, size_t size) { return map_identity(map, ctrl, devptr, size); }
 
 int nvm_dma_create(nvm_dma_t** map, const nvm_ctrl_t* ctrl, size_t size)
 {
@@ -422,7 +412,6 @@ void nvm_dma_unmap(nvm_dma_t* map)
 {
     if (!map) return;
     DmaBox* b = box_of(map);
-    if (b->device_size) nvmt_device_range(map->vaddr, b->device_size, 0);
     ctrl_put(b->ctrl);
     free(b->owned);
     free(b);

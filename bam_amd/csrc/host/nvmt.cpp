@@ -111,25 +111,6 @@ struct nvmt {
 
 namespace {
 
-// Ranges of device memory that have been mapped for DMA (nvm_dma_map_device).  What the target stores there travels
-// as posted writes over the interconnect, and neither a store fence nor the completion that follows (a store to host
-// memory, which the device reads from there) waits for them to arrive: the device has been seen to read a completion
-// up to tens of microseconds before the payload it announces had landed.  A load from the device is ordered behind the
-// posted writes that precede it, so the target reads back the end of the last payload it placed in device memory before
-// it posts the completions of a batch.
-constexpr int kMaxDevRanges = 64;
-std::atomic<uintptr_t> g_dev_lo[kMaxDevRanges], g_dev_hi[kMaxDevRanges];
-std::atomic<int> g_dev_n{0};
-inline bool in_device_memory(uintptr_t a)
-{
-    const int n = g_dev_n.load(std::memory_order_acquire);
-    for (int i = 0; i < n; i++) {
-        const uintptr_t hi = g_dev_hi[i].load(std::memory_order_acquire);
-        if (hi && a >= g_dev_lo[i].load(std::memory_order_relaxed) && a < hi) return true;
-    }
-    return false;
-}
-
 // Walk the PRP entries of a command: fn(bus_addr, length) for every contiguous piece.
 template <typename F>
 bool for_each_prp(const nvmt* t, const nvm_cmd_t& c, uint64_t bytes, F&& fn)
@@ -218,7 +199,7 @@ gen_words_fn pick_gen_words()
 }
 const gen_words_fn gen_words = pick_gen_words();
 
-uint16_t do_rw(nvmt* t, Stats& st_, const nvm_cmd_t& c, bool write, uintptr_t& last_in_device)
+uint16_t do_rw(nvmt* t, Stats& st_, const nvm_cmd_t& c, bool write)
 {
     const uint32_t lba = t->cfg.lba_bytes;
     uint64_t slba = ((uint64_t)c.dword[11] << 32) | c.dword[10];
@@ -243,7 +224,6 @@ uint16_t do_rw(nvmt* t, Stats& st_, const nvm_cmd_t& c, bool write, uintptr_t& l
                 copy_out(p + k, tmp, n);
             }
         }
-        if (!write && in_device_memory((uintptr_t)addr)) last_in_device = (uintptr_t)addr + len - 8;
         done += len;
     });
     if (!ok) return ST_INVALID_FIELD;
@@ -332,7 +312,6 @@ void serve_sq(nvmt* t, IoThread* me, Sq& sq)
         // all commands of the batch first, then one drain of the streaming stores, then their completions
         uint16_t statuses[64];
         bool dropped[64];
-        uintptr_t last_in_device = 0;
         for (uint32_t k = 0; k < n; k++) {
             const nvm_cmd_t& c = batch[order[k]];
             uint8_t op = c.dword[0] & 0xff;
@@ -344,8 +323,8 @@ void serve_sq(nvmt* t, IoThread* me, Sq& sq)
             statuses[k] = ST_OK;
             if (t->cfg.drop_every && seq % t->cfg.drop_every == 0) { st_.bump(st_.dropped); dropped[k] = true; continue; }
             if (t->cfg.fail_every && seq % t->cfg.fail_every == 0) status = ST_DATA_XFER_ERROR;
-            else if (op == NVM_IO_READ) status = do_rw(t, st_, c, false, last_in_device);
-            else if (op == NVM_IO_WRITE) status = do_rw(t, st_, c, true, last_in_device);
+            else if (op == NVM_IO_READ) status = do_rw(t, st_, c, false);
+            else if (op == NVM_IO_WRITE) status = do_rw(t, st_, c, true);
             else if (op == NVM_IO_FLUSH) status = ST_OK;
             else status = ST_INVALID_OPCODE;
             if (status && t->trace_errors.load(std::memory_order_relaxed) > 0 && t->trace_errors.fetch_sub(1) > 0)
@@ -354,7 +333,6 @@ void serve_sq(nvmt* t, IoThread* me, Sq& sq)
             statuses[k] = status;
         }
         copy_out_fence();
-        if (last_in_device) (void)ld<uint64_t>((const void*)last_in_device);      /* pushes the posted writes ahead of it */
         for (uint32_t k = 0; k < n; k++) {
             if (dropped[k]) continue;
             const uint16_t cid = batch[order[k]].dword[0] >> 16;
@@ -669,23 +647,3 @@ void nvmt_reset_stats(nvmt_t* t)
 void nvmt_fill_words(uint64_t seed, uint64_t first_word, uint64_t n, uint64_t* out) { gen_words(seed, first_word, n, out); }
 
 } // extern "C"
-
-void nvmt_device_range(const void* base, size_t size, int add)
-{
-    static std::mutex mu;
-    std::lock_guard<std::mutex> g(mu);
-    const uintptr_t lo = (uintptr_t)base;
-    if (add) {
-        int i = 0;
-        const int n = g_dev_n.load(std::memory_order_relaxed);
-        while (i < n && g_dev_hi[i].load(std::memory_order_relaxed)) i++;
-        if (i == kMaxDevRanges) return;                 /* no room: such a range is treated as host memory */
-        g_dev_lo[i].store(lo, std::memory_order_relaxed);
-        g_dev_hi[i].store(lo + size, std::memory_order_release);
-        if (i == n) g_dev_n.store(n + 1, std::memory_order_release);
-    } else {
-        const int n = g_dev_n.load(std::memory_order_relaxed);
-        for (int i = 0; i < n; i++)
-            if (g_dev_hi[i].load(std::memory_order_relaxed) && g_dev_lo[i].load(std::memory_order_relaxed) == lo) g_dev_hi[i].store(0, std::memory_order_release);
-    }
-}

@@ -78,13 +78,6 @@ void     nvmt_reset_stats(nvmt_t* t);
 int      nvmt_publish(const char* path, nvmt_t* t);
 nvmt_t*  nvmt_lookup(const char* path);
 const nvmt_config_t* nvmt_config(nvmt_t* t);
-/*
- * Tells the targets of this process that [base, base + size) is device memory mapped for DMA (add != 0) or no longer
- * is (add == 0; base as it was added).  Payload a target places there is pushed over the interconnect; before it
- * posts the completions of a batch the target reads back the end of the last such payload, which cannot return
- * before the writes ahead of it have arrived.  Called by nvm_dma_map_device / nvm_dma_unmap.
- */
-void     nvmt_device_range(const void* base, size_t size, int add);
 /* procedural content: fills out[0..n) with words first_word.. of a namespace with this seed */
 void     nvmt_fill_words(uint64_t seed, uint64_t first_word, uint64_t n, uint64_t* out);
 /*
