@@ -412,6 +412,31 @@ def test_array_write_eviction_write_back_and_flush(bam):
         assert r.t.stats()["write_cmds"] >= 128 and not r.c.aborted()
 
 
+@pytest.mark.parametrize("cache_pages,direct_share", [(24, None), (96, None), (96, "8"), (96, "0")])
+def test_random_writes_and_reads_against_a_model_of_the_store(bam, cache_pages, direct_share, monkeypatch):
+    """rounds of scattered writes (distinct elements per round, many per page) and scattered reads through a cache far
+    smaller than the data: dirty pages are evicted, written back and read again all the time; a numpy array plays the
+    store.  Reads of a round see the writes of all rounds before it, whatever the cache did with the pages in between."""
+    if direct_share is not None:
+        monkeypatch.setenv("BAM_DIRECT_SHARE", direct_share)
+    n_elems = 1 << 19                                                # 1024 pages of data
+    rng = np.random.default_rng(SEED + cache_pages)
+    with Rig(bam, n_elems * 8, backing=True, n_queues=16, depth=256) as r:
+        model = r.backing(n_elems).copy()
+        a = r.array(n_elems, 4096, cache_pages)
+        for rnd in range(6):
+            widx = rng.permutation(n_elems)[:1 << 15].astype(np.uint64)
+            wval = (widx * np.uint64(0x9E3779B97F4A7C15) + np.uint64(rnd + 1)).astype(np.uint64)
+            a.write(len(widx), _dev(wval), assignment=_dev(widx), block_size=64)
+            model[widx] = wval
+            ridx = rng.integers(0, n_elems, 1 << 16).astype(np.uint64)
+            assert a.read(len(ridx), _dev(ridx), block_size=256) == int(np.sum(model[ridx], dtype=np.uint64)), "round %d" % rnd
+        r.objs[0][2].flush()
+        assert np.array_equal(r.backing(n_elems), model)
+        assert a.read(n_elems) == int(np.sum(model, dtype=np.uint64))
+        assert r.t.stats()["write_cmds"] > 0 and not r.c.aborted()
+
+
 def test_vectoradd_three_arrays_write_back(bam):
     """C = A + B with all three arrays behind one cache (three ranges): the results reach the store with the flush.
     Every lane keeps a page of each array while it works, so the cache has to hold what the waves in flight can pin:
