@@ -7,5 +7,5 @@ This package is the Python host-side mirror of the reference's host objects
 CPU fallback: without the built library every call raises.
 """
 from ._lib import load, load_host, LibraryMissing  # noqa: F401
-from .host import Target, Controller, PageCache, Range, Array, Range32, Array32, sssp, vectoradd, BamError  # noqa: F401
+from .host import Target, Controller, PageCache, Range, Array, Range32, Array32, sssp, sssp_float, vectoradd, BamError  # noqa: F401
 from . import gen  # noqa: F401

@@ -61,6 +61,8 @@ SIGNATURES = {
     "bam_array32_stats": (c_int, [c_vp, P(c_u64)]),
     "bam_array32_read": (c_int, [c_vp, c_u64, c_vp, c_u64, c_u32, c_vp, c_vp]),
     "bam_sssp": (c_int, [c_vp, c_vp, c_vp, c_u64, c_u64, c_vp, P(c_u32), c_vp]),
+    "bam_sssp_float": (c_int, [c_vp, c_vp, c_vp, c_u64, c_u64, c_vp, P(c_u32), c_vp]),
+    "bam_bfs_frontier": (c_int, [c_vp, c_vp, c_u64, c_u64, c_vp, P(c_u32), c_vp]),
     "bam_gen_words": (c_int, [c_u64, c_u64, c_u64, c_vp, c_vp]),
     "bam_gen_mod": (c_int, [c_u64, c_u64, c_u64, c_u64, c_u64, c_vp, c_vp]),
     "bam_gen_rmat": (c_int, [c_u64, c_u32, c_u64, c_u64, c_vp, c_vp, c_vp]),

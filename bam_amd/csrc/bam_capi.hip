@@ -439,14 +439,47 @@ __device__ __forceinline__ void walk_packed(const uint64_t es, const uint64_t ee
 #define BAM_HEAVY_EDGES 1024u
 struct heavy_piece_t { uint64_t v, first, last; };      /* entries [first, last) of the list of vertex v */
 
-template <typename Active, typename Visit>
-__device__ __forceinline__ void walk_vertex_groups(array_d_t<uint64_t>* da, const uint64_t* vertexList, const uint64_t vertex_count, const uint64_t coarse,
-                                                   heavy_piece_t* heavy, unsigned long long* n_heavy, Active active, Visit visit)
+/*
+ * Reads with the page referenced for the one read only.  bam_ptr keeps every lane's page referenced until the lane
+ * moves on: fine where the lanes of a wave read side by side, but 64 lanes that walk lists scattered over the edge
+ * array would pin up to 64 pages per wave, and a cache with fewer free slots than that stops for good (lanes that
+ * have their page wait for those that cannot get one).  Lanes on the same page still share one pair of atomics.
+ */
+template <typename T>
+struct touch_reader {
+    array_d_t<T>* da = nullptr;
+    bam::range_view<T> view;
+    bool one_range = false;
+    __device__ __forceinline__ void init(array_d_t<T>* a)
+    {
+        da = a;
+        one_range = a->n_ranges == 1;
+        if (one_range) view.load(a->d_ranges);
+    }
+    __device__ __forceinline__ T read(const uint64_t i)
+    {
+        if (!one_range) return da->seq_read(i);
+        T ret = T();                                    /* stays T() if the wait is given up */
+        const uint64_t byte = view.byte_of(i);
+        auto use = [&](uint32_t slot) { ret = bam::ld_payload((T*)(view.slot_addr(slot) + (byte & (view.page_size - 1)))); return true; };
+        view.template acquire<true>(byte >> view.page_size_log, false, use, use);
+        return ret;
+    }
+    __device__ __forceinline__ void fini() { if (one_range) view.flush_stats(); }
+};
+
+/* the walk over `n_items` work items, each of which names a vertex and says whether it is to be walked: item(i, v).
+ * HOLD: read through bam_ptr (items whose lists lie side by side); otherwise page by page without holding any */
+template <bool HOLD, typename Item, typename Visit>
+__device__ __forceinline__ void walk_item_groups(array_d_t<uint64_t>* da, const uint64_t* vertexList, const uint64_t n_items, const uint64_t coarse,
+                                                 heavy_piece_t* heavy, unsigned long long* n_heavy, Item item, Visit visit)
 {
     const uint64_t laneIdx = threadIdx.x % BAM_WAVE_SIZE;
     unsigned long long* next_group = n_heavy + 1;
-    const uint64_t n_groups = (vertex_count + coarse - 1) / coarse;
+    const uint64_t n_groups = (n_items + coarse - 1) / coarse;
     bam_ptr<uint64_t> ptr(da);
+    touch_reader<uint64_t> touch;
+    if (!HOLD) touch.init(da);
     list_read_ahead<uint64_t> ahead;
     bool ready = false;
     for (;;) {
@@ -456,8 +489,9 @@ __device__ __forceinline__ void walk_vertex_groups(array_d_t<uint64_t>* da, cons
         if (g >= n_groups) break;
         const uint64_t first = g * coarse;
         for (uint64_t b = 0; b < coarse; b += BAM_WAVE_SIZE) {
-            const uint64_t mine = first + b + laneIdx;
-            const bool act = b + laneIdx < coarse && mine < vertex_count && active(mine);
+            const uint64_t at_item = first + b + laneIdx;
+            uint64_t mine = 0;
+            const bool act = b + laneIdx < coarse && at_item < n_items && item(at_item, mine);
             if (!bam::ballot(act)) continue;
             if (!ready) { ahead.init(da); ready = true; }
             uint64_t es = 0, ee = 0;
@@ -465,7 +499,7 @@ __device__ __forceinline__ void walk_vertex_groups(array_d_t<uint64_t>* da, cons
             /* long lists go to the queue, in pieces */
             for (uint64_t hm = bam::ballot(ee - es >= BAM_HEAVY_EDGES); hm; hm &= hm - 1) {
                 const uint32_t j = bam::first_lane(hm);
-                const uint64_t start = bam::bcast(es, j), end = bam::bcast(ee, j), v = first + b + j;
+                const uint64_t start = bam::bcast(es, j), end = bam::bcast(ee, j), v = bam::bcast(mine, j);
                 const uint64_t pieces = (end - start + BAM_HEAVY_EDGES - 1) / BAM_HEAVY_EDGES;
                 unsigned long long at = 0;
                 if (laneIdx == 0) at = atomicAdd(n_heavy, (unsigned long long)pieces);
@@ -477,9 +511,18 @@ __device__ __forceinline__ void walk_vertex_groups(array_d_t<uint64_t>* da, cons
             }
             if (ee - es >= BAM_HEAVY_EDGES) ee = es;
             ahead.group(es, ee);
-            walk_packed(es, ee, mine, [&](uint64_t i) { return ptr.read(i); }, visit);
+            walk_packed(es, ee, mine, [&](uint64_t i) { if constexpr (HOLD) return ptr.read(i); else return touch.read(i); }, visit);
         }
     }
+    if (!HOLD) touch.fini();
+}
+
+/* the items are the vertices themselves, walked where active(v) */
+template <typename Active, typename Visit>
+__device__ __forceinline__ void walk_vertex_groups(array_d_t<uint64_t>* da, const uint64_t* vertexList, const uint64_t vertex_count, const uint64_t coarse,
+                                                   heavy_piece_t* heavy, unsigned long long* n_heavy, Active active, Visit visit)
+{
+    walk_item_groups<true>(da, vertexList, vertex_count, coarse, heavy, n_heavy, [&](uint64_t i, uint64_t& v) { v = i; return active(i); }, visit);
 }
 
 /* the queued pieces, one wave at a time each: the same walk through bam_ptr, read ahead over the piece */
@@ -521,6 +564,36 @@ __global__ __launch_bounds__(128) void k_bfs_heavy_ptr_pc(array_d_t<uint64_t>* d
     bool any = false;
     walk_heavy_pieces(da, heavy, n_heavy, [&](uint64_t, uint64_t next, uint64_t) { if (label[next] == MYINFINITY) { label[next] = level + 1; any = true; } });
     if (any) *changed = 1;
+}
+
+// ---- BFS over a queue of the level's vertices (benchmarks/bfs/main.cu:409-451 kernel_frontier_coalesce_ptr_pc) ----
+/* a vertex found for the first time (the exchange on its label decides who found it) goes to the next level's queue;
+ * the lanes of a wave that found one at the same step take their places in it with one atomic */
+__device__ __forceinline__ void bfs_frontier_visit(uint32_t* label, const uint32_t level, uint32_t* next_frontier, unsigned long long* next_size, const uint64_t next)
+{
+    if (label[next] != MYINFINITY) return;
+    if (atomicExch(label + next, level + 1) != MYINFINITY) return;
+    const uint64_t mask = bam::active_mask();
+    const uint32_t leader = bam::first_lane(mask);
+    unsigned long long pos = 0;
+    if (bam::lane() == leader) pos = atomicAdd(next_size, (unsigned long long)bam::popc(mask));
+    pos = bam::bcast((uint64_t)pos, leader);
+    next_frontier[pos + bam::rank_in(mask)] = (uint32_t)next;
+}
+
+__global__ __launch_bounds__(128) void k_bfs_frontier_coalesce_ptr_pc(array_d_t<uint64_t>* da, uint32_t* label, const uint32_t level, const uint64_t* vertexList,
+                                                                     const uint32_t* curr_frontier, const uint64_t curr_size, uint32_t* next_frontier,
+                                                                     unsigned long long* next_size, uint64_t group, heavy_piece_t* heavy, unsigned long long* n_heavy)
+{
+    walk_item_groups<false>(da, vertexList, curr_size, group, heavy, n_heavy,
+                            [&](uint64_t i, uint64_t& v) { v = curr_frontier[i]; return true; },
+                            [&](uint64_t, uint64_t next, uint64_t) { bfs_frontier_visit(label, level, next_frontier, next_size, next); });
+}
+
+__global__ __launch_bounds__(128) void k_bfs_frontier_heavy_ptr_pc(array_d_t<uint64_t>* da, uint32_t* label, const uint32_t level, uint32_t* next_frontier,
+                                                                  unsigned long long* next_size, const heavy_piece_t* heavy, const unsigned long long* n_heavy)
+{
+    walk_heavy_pieces(da, heavy, n_heavy, [&](uint64_t, uint64_t next, uint64_t) { bfs_frontier_visit(label, level, next_frontier, next_size, next); });
 }
 
 // ---- CC: min-label propagation (benchmarks/cc/main.cu:123-144, 595-617) ----
@@ -814,12 +887,17 @@ __global__ void k_pr_update(bool* label, float* delta, float* residual, float* v
 // ---- SSSP (benchmarks/sssp/main.cu:174-201 kernel_coalesce_pc, :282-292 update): 32-bit costs, weights in their own array ----
 /* relaxation of the edges of the flagged vertices with the cost each has at the time (any cost a vertex holds is the cost of a
  * path to it); the group walk of the per-vertex graph kernels, the weight of entry i read through a bam_ptr of its own */
+template <bool FLOAT>
 __device__ __forceinline__ void sssp_relax(uint32_t* newCostList, const bam_ptr<uint32_t>& weights, uint64_t src, uint64_t next, uint64_t i)
 {
-    const uint32_t cost = __hip_atomic_load(&newCostList[src], __ATOMIC_RELAXED, BAM_AGENT) + weights[i];
+    const uint32_t have = __hip_atomic_load(&newCostList[src], __ATOMIC_RELAXED, BAM_AGENT), w = weights[i];
+    /* single-precision costs (benchmarks/sssp_float/main.cu:69, 91-106, 194-217) travel as their bit patterns: for floats that
+     * are not negative the order of the patterns is the order of the values, so the minimum is the integer one */
+    const uint32_t cost = FLOAT ? __float_as_uint(__uint_as_float(have) + __uint_as_float(w)) : have + w;
     if (__hip_atomic_load(&newCostList[next], __ATOMIC_RELAXED, BAM_AGENT) > cost) atomicMin(&newCostList[next], cost);
 }
 
+template <bool FLOAT>
 __global__ __launch_bounds__(128) void k_sssp_coalesce_pc(array_d_t<uint64_t>* de, array_d_t<uint32_t>* dw, const bool* label, uint32_t* newCostList,
                                                           const uint64_t vertex_count, const uint64_t* vertexList, uint64_t group,
                                                           heavy_piece_t* heavy, unsigned long long* n_heavy)
@@ -827,14 +905,15 @@ __global__ __launch_bounds__(128) void k_sssp_coalesce_pc(array_d_t<uint64_t>* d
     bam_ptr<uint32_t> wptr(dw);
     walk_vertex_groups(de, vertexList, vertex_count, group, heavy, n_heavy,
                        [&](uint64_t v) { return label[v]; },
-                       [&](uint64_t src, uint64_t next, uint64_t i) { sssp_relax(newCostList, wptr, src, next, i); });
+                       [&](uint64_t src, uint64_t next, uint64_t i) { sssp_relax<FLOAT>(newCostList, wptr, src, next, i); });
 }
 
+template <bool FLOAT>
 __global__ __launch_bounds__(128) void k_sssp_heavy_pc(array_d_t<uint64_t>* de, array_d_t<uint32_t>* dw, uint32_t* newCostList, const heavy_piece_t* heavy,
                                                        const unsigned long long* n_heavy)
 {
     bam_ptr<uint32_t> wptr(dw);
-    walk_heavy_pieces(de, heavy, n_heavy, [&](uint64_t src, uint64_t next, uint64_t i) { sssp_relax(newCostList, wptr, src, next, i); });
+    walk_heavy_pieces(de, heavy, n_heavy, [&](uint64_t src, uint64_t next, uint64_t i) { sssp_relax<FLOAT>(newCostList, wptr, src, next, i); });
 }
 
 __global__ void k_sssp_update(bool* label, uint32_t* costList, const uint32_t* newCostList, const uint64_t vertex_count, bool* changed)
@@ -1424,6 +1503,7 @@ struct heavy_queue {
     uint32_t blocks;                 /* launch of the piece walk */
     uint64_t group;                  /* vertices handed to a wave at a time */
     uint32_t group_blocks;           /* launch of the group walk: what the device holds at a time */
+    uint32_t group_blocks_max;       /* the same without regard to the number of groups */
     heavy_queue(uint64_t n_edges, uint64_t n_vertices, uint32_t coarse)
     {
         const uint64_t cap = 2 * (n_edges / BAM_HEAVY_EDGES) + 1;
@@ -1440,6 +1520,7 @@ struct heavy_queue {
         hip_err_chk(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
         const uint64_t n_groups = (n_vertices + group - 1) / group, resident = (uint64_t)cus * 16;      /* waves */
         group_blocks = (uint32_t)(((n_groups < resident ? n_groups : resident) + 1) / 2);
+        group_blocks_max = (uint32_t)((resident + 1) / 2);
     }
     void reset(hipStream_t st) { hip_err_chk(hipMemsetAsync(count, 0, 2 * sizeof(unsigned long long), st)); }
 };
@@ -1473,6 +1554,49 @@ int bam_bfs(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, 
         hip_err_chk(hipMemcpyAsync(&changed_h, changed_d, sizeof(uint64_t), hipMemcpyDeviceToHost, st));
         hip_err_chk(hipStreamSynchronize(st));
     } while (changed_h);
+    if (iterations) *iterations = iter;
+    BAM_API_END
+}
+
+int bam_bfs_frontier(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t src, uint32_t* d_labels,
+                     uint32_t* iterations, void* stream)
+{
+    if (!edges || !d_offsets || !d_labels) return fail(EINVAL, "bam_bfs_frontier: null argument");
+    if (src >= n_vertices) return fail(EINVAL, "bam_bfs_frontier: source out of range");
+    if (n_vertices > 0xFFFFFFFFull) return fail(EINVAL, "bam_bfs_frontier: the queues hold 32-bit vertex numbers");
+    BAM_API_BEGIN
+    hipStream_t st = (hipStream_t)stream;
+    /* two queues of at most every vertex once (benchmarks/bfs/main.cu:1489-1492); the size of the next one is the reference's `changed` */
+    BufferPtr queue_a = createBuffer(n_vertices * sizeof(uint32_t), 0), queue_b = createBuffer(n_vertices * sizeof(uint32_t), 0);
+    BufferPtr size_buf = createBuffer(sizeof(unsigned long long), 0);
+    uint32_t* curr = (uint32_t*)queue_a.get();
+    uint32_t* next = (uint32_t*)queue_b.get();
+    unsigned long long* next_size = (unsigned long long*)size_buf.get();
+    const uint32_t zero = 0, src32 = (uint32_t)src;
+    hip_err_chk(hipMemsetAsync(d_labels, 0xFF, n_vertices * sizeof(uint32_t), st));
+    hip_err_chk(hipMemcpyAsync(d_labels + src, &zero, sizeof(uint32_t), hipMemcpyHostToDevice, st));
+    hip_err_chk(hipMemcpyAsync(curr, &src32, sizeof(uint32_t), hipMemcpyHostToDevice, st));
+    const uint32_t threads = 128;
+    const uint64_t group = BAM_WAVE_SIZE;           /* queue entries handed to a wave at a time: one per lane */
+    heavy_queue hq(edges->a->adt.n_elems, n_vertices, 1);
+    const uint64_t resident = 2ull * hq.group_blocks_max;
+    uint32_t level = 0, iter = 0;
+    unsigned long long active = 1;
+    do {
+        hip_err_chk(hipMemsetAsync(next_size, 0, sizeof(unsigned long long), st));
+        hq.reset(st);
+        const uint64_t n_groups = (active + group - 1) / group;
+        const uint32_t blocks = (uint32_t)(((n_groups < resident ? n_groups : resident) + 1) / 2);
+        hipLaunchKernelGGL(k_bfs_frontier_coalesce_ptr_pc, dim3(blocks), dim3(threads), 0, st, edges->a->d_array_ptr, d_labels, level, d_offsets,
+                           curr, (uint64_t)active, next, next_size, group, hq.pieces, hq.count);
+        hipLaunchKernelGGL(k_bfs_frontier_heavy_ptr_pc, dim3(hq.blocks), dim3(threads), 0, st, edges->a->d_array_ptr, d_labels, level, next, next_size,
+                           hq.pieces, hq.count);
+        hip_err_chk(hipGetLastError());
+        std::swap(curr, next);
+        iter++; level++;
+        hip_err_chk(hipMemcpyAsync(&active, next_size, sizeof(unsigned long long), hipMemcpyDeviceToHost, st));
+        hip_err_chk(hipStreamSynchronize(st));
+    } while (active);
     if (iterations) *iterations = iter;
     BAM_API_END
 }
@@ -1775,22 +1899,23 @@ int bam_array32_read(bam_array32_t* a, uint64_t n_reqs, const uint64_t* d_assign
     BAM_API_END
 }
 
-int bam_sssp(bam_array_t* edges, bam_array32_t* weights, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t src, uint32_t* d_costs,
-             uint32_t* iterations, void* stream)
+namespace {
+/* the loop of benchmarks/sssp/main.cu:663-725 (and of sssp_float, :624-700): relax from the flagged vertices, adopt what got
+ * cheaper, flag it, until nothing does.  FLOAT: costs and weights are single-precision values, unreached = 1e9 (sssp_float :529) */
+void sssp_run(const bool FLOAT, bam_array_t* edges, bam_array32_t* weights, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t src, uint32_t* d_costs,
+              uint32_t* iterations, hipStream_t st)
 {
-    if (!edges || !weights || !d_offsets || !d_costs) return fail(EINVAL, "bam_sssp: null argument");
-    if (src >= n_vertices) return fail(EINVAL, "bam_sssp: source out of range");
-    if (edges->a->adt.n_elems != weights->a->adt.n_elems) return fail(EINVAL, "bam_sssp: one weight per edge");
-    BAM_API_BEGIN
-    hipStream_t st = (hipStream_t)stream;
     BufferPtr new_cost = createBuffer(n_vertices * sizeof(uint32_t), 0), label = createBuffer(n_vertices, 0), changed_buf = createBuffer(sizeof(uint64_t), 0);
     uint32_t* new_d = (uint32_t*)new_cost.get();
     bool* label_d = (bool*)label.get();
     bool* changed_d = (bool*)changed_buf.get();
-    const uint32_t zero = 0;
+    const uint32_t zero = 0;                    /* the pattern of 0.0f as well */
     const bool one = true;
-    hip_err_chk(hipMemsetAsync(d_costs, 0xFF, n_vertices * sizeof(uint32_t), st));
-    hip_err_chk(hipMemsetAsync(new_d, 0xFF, n_vertices * sizeof(uint32_t), st));
+    const float far = 1000000000.0f;
+    uint32_t unreached = 0xFFFFFFFFu;
+    if (FLOAT) memcpy(&unreached, &far, sizeof(unreached));
+    hip_err_chk(hipMemsetD32Async((hipDeviceptr_t)d_costs, (int)unreached, n_vertices, st));
+    hip_err_chk(hipMemsetD32Async((hipDeviceptr_t)new_d, (int)unreached, n_vertices, st));
     hip_err_chk(hipMemsetAsync(label_d, 0, n_vertices, st));
     hip_err_chk(hipMemcpyAsync(label_d + src, &one, sizeof(bool), hipMemcpyHostToDevice, st));
     hip_err_chk(hipMemcpyAsync(d_costs + src, &zero, sizeof(uint32_t), hipMemcpyHostToDevice, st));
@@ -1803,9 +1928,10 @@ int bam_sssp(bam_array_t* edges, bam_array32_t* weights, const uint64_t* d_offse
         changed_h = false;
         hip_err_chk(hipMemcpyAsync(changed_d, &changed_h, sizeof(bool), hipMemcpyHostToDevice, st));
         hq.reset(st);
-        hipLaunchKernelGGL(k_sssp_coalesce_pc, dim3(hq.group_blocks), dim3(threads), 0, st, edges->a->d_array_ptr, weights->a->d_array_ptr, label_d, new_d,
-                           n_vertices, d_offsets, hq.group, hq.pieces, hq.count);
-        hipLaunchKernelGGL(k_sssp_heavy_pc, dim3(hq.blocks), dim3(threads), 0, st, edges->a->d_array_ptr, weights->a->d_array_ptr, new_d, hq.pieces, hq.count);
+        hipLaunchKernelGGL(FLOAT ? k_sssp_coalesce_pc<true> : k_sssp_coalesce_pc<false>, dim3(hq.group_blocks), dim3(threads), 0, st, edges->a->d_array_ptr,
+                           weights->a->d_array_ptr, label_d, new_d, n_vertices, d_offsets, hq.group, hq.pieces, hq.count);
+        hipLaunchKernelGGL(FLOAT ? k_sssp_heavy_pc<true> : k_sssp_heavy_pc<false>, dim3(hq.blocks), dim3(threads), 0, st, edges->a->d_array_ptr,
+                           weights->a->d_array_ptr, new_d, hq.pieces, hq.count);
         hip_err_chk(hipMemsetAsync(label_d, 0, n_vertices, st));
         hipLaunchKernelGGL(k_sssp_update, dim3(blocks_for(n_vertices, 256)), dim3(256), 0, st, label_d, d_costs, new_d, n_vertices, changed_d);
         hip_err_chk(hipGetLastError());
@@ -1814,6 +1940,28 @@ int bam_sssp(bam_array_t* edges, bam_array32_t* weights, const uint64_t* d_offse
         hip_err_chk(hipStreamSynchronize(st));
     } while (changed_h);
     if (iterations) *iterations = iter;
+}
+} // namespace
+
+int bam_sssp(bam_array_t* edges, bam_array32_t* weights, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t src, uint32_t* d_costs,
+             uint32_t* iterations, void* stream)
+{
+    if (!edges || !weights || !d_offsets || !d_costs) return fail(EINVAL, "bam_sssp: null argument");
+    if (src >= n_vertices) return fail(EINVAL, "bam_sssp: source out of range");
+    if (edges->a->adt.n_elems != weights->a->adt.n_elems) return fail(EINVAL, "bam_sssp: one weight per edge");
+    BAM_API_BEGIN
+    sssp_run(false, edges, weights, d_offsets, n_vertices, src, d_costs, iterations, (hipStream_t)stream);
+    BAM_API_END
+}
+
+int bam_sssp_float(bam_array_t* edges, bam_array32_t* weights, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t src, float* d_costs,
+                   uint32_t* iterations, void* stream)
+{
+    if (!edges || !weights || !d_offsets || !d_costs) return fail(EINVAL, "bam_sssp_float: null argument");
+    if (src >= n_vertices) return fail(EINVAL, "bam_sssp_float: source out of range");
+    if (edges->a->adt.n_elems != weights->a->adt.n_elems) return fail(EINVAL, "bam_sssp_float: one weight per edge");
+    BAM_API_BEGIN
+    sssp_run(true, edges, weights, d_offsets, n_vertices, src, (uint32_t*)d_costs, iterations, (hipStream_t)stream);
     BAM_API_END
 }
 

@@ -235,12 +235,15 @@ class Array:
         self.stream_async(n_waves, n_pages_per_wave, s, assignment, mode)
         return int(s.item()) & MASK64
 
-    def bfs(self, offsets, src, coarse=1, by_page=False):
-        """Levels (uint32 bit patterns in an int32 tensor) and launch count; by_page: the edge-page kernel."""
+    def bfs(self, offsets, src, coarse=1, by_page=False, frontier=False):
+        """Levels (uint32 bit patterns in an int32 tensor) and launch count; by_page: the edge-page kernel; frontier: the
+        kernel that walks a queue of the level's vertices."""
         n_v = offsets.numel() - 1
         labels = torch.empty(n_v, dtype=torch.int32, device=offsets.device)
         it = c_u32(0)
-        if by_page:
+        if frontier:
+            _chk(self.L.bam_bfs_frontier(self.h, _ptr(offsets), n_v, int(src), _ptr(labels), ctypes.byref(it), _stream()), "bam_bfs_frontier")
+        elif by_page:
             _chk(self.L.bam_bfs_by_page(self.h, _ptr(offsets), n_v, int(src), _ptr(labels), ctypes.byref(it), _stream()), "bam_bfs_by_page")
         else:
             _chk(self.L.bam_bfs(self.h, _ptr(offsets), n_v, int(src), _ptr(labels), coarse, ctypes.byref(it), _stream()), "bam_bfs")
@@ -361,6 +364,15 @@ def sssp(edges, weights, offsets, src):
     costs = torch.empty(n_v, dtype=torch.int32, device=offsets.device)
     it = c_u32(0)
     _chk(edges.L.bam_sssp(edges.h, weights.h, _ptr(offsets), n_v, int(src), _ptr(costs), ctypes.byref(it), _stream()), "bam_sssp")
+    return costs, it.value
+
+
+def sssp_float(edges, weights, offsets, src):
+    """The same with single-precision weights (their bit patterns in the 32-bit array): float32 costs, 1e9 = unreached."""
+    n_v = offsets.numel() - 1
+    costs = torch.empty(n_v, dtype=torch.float32, device=offsets.device)
+    it = c_u32(0)
+    _chk(edges.L.bam_sssp_float(edges.h, weights.h, _ptr(offsets), n_v, int(src), _ptr(costs), ctypes.byref(it), _stream()), "bam_sssp_float")
     return costs, it.value
 
 

@@ -136,6 +136,15 @@ int bam_block_checksum(bam_page_cache_t* pc, uint64_t n_slots, uint32_t req_byte
  * bam_pagerank without by_page). */
 int bam_bfs(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t src, uint32_t* d_labels,
             uint32_t coarse, uint32_t* iterations, void* stream);
+/* ---- BFS over queues of vertices (benchmarks/bfs/main.cu:409-451 kernel_frontier_coalesce_ptr_pc, queues :1489-1492,
+ * host loop :1561-1563, 1702-1711) ----
+ * Instead of sweeping all labels, every level walks the queue of the vertices found by the level before and fills the
+ * next one: a vertex enters it when the exchange on its label finds it unreached, the lanes of a wave that found one
+ * at the same step take their places with one atomic.  64 queue entries per wave at a time, otherwise the walk of
+ * bam_bfs (lists packed 64 entries per step, long lists in pieces).  Same levels and the same *iterations as bam_bfs;
+ * the order of a queue is not defined, nothing depends on it.  n_vertices <= 2^32 - 1 (32-bit queue entries). */
+int bam_bfs_frontier(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t src, uint32_t* d_labels,
+                     uint32_t* iterations, void* stream);
 /* ---- CC (benchmarks/cc/main.cu:123-144 cc_compute, :595-617 kernel, host loop :1410-1425, 1515-1521) ----
  * Min-label propagation; d_labels[V] receives the smallest vertex id of each vertex's component. */
 int bam_cc(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t* d_labels,
@@ -204,6 +213,15 @@ int bam_array32_read(bam_array32_t* a, uint64_t n_reqs, const uint64_t* d_assign
  * unreachable).  *iterations = rounds. */
 int bam_sssp(bam_array_t* edges, bam_array32_t* weights, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t src, uint32_t* d_costs,
              uint32_t* iterations, void* stream);
+/* ---- SSSP with single-precision weights (benchmarks/sssp_float/main.cu: WeightT = float :69, AtomicMin :91-106,
+ * kernel_coalesce_pc :194-217, update :302-312, unreached = 1e9 :529) ----
+ * The elements of `weights` are the bit patterns of floats, which must not be negative (nor NaN); d_costs[V] receives
+ * the least cost, each path's weights added in single precision from the source on (1e9 = unreached, and a path is
+ * only taken while its cost stays below that).  Costs that are not negative order as their bit patterns, so the
+ * minimum is the integer atomic on the pattern.  Adding a weight keeps the order of two costs, so the result does not
+ * depend on the order of relaxation: bit-exact against a serial Dijkstra in single precision. */
+int bam_sssp_float(bam_array_t* edges, bam_array32_t* weights, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t src, float* d_costs,
+                   uint32_t* iterations, void* stream);
 
 /* ---- synthetic inputs on the device (no counterpart in the reference, which reads dataset files) ---- */
 int bam_gen_words(uint64_t seed, uint64_t first, uint64_t n, uint64_t* d_out, void* stream);                 /* out[k] = splitmix64(seed, first + k) */

@@ -1199,19 +1199,22 @@ struct bam_ptr {
             view.load(array->d_ranges + range_id);
         }
         const uint64_t pg = view.page_of(i);
-        uint32_t slot = 0;
+        uint32_t slot = BAM_NO_SLOT;
         auto keep = [&](uint32_t s_) { slot = s_; return false; };
         view.template acquire<true>(pg, false, keep, keep);
-        page = view.pages + pg;
+        page = view.pages + pg;                 /* the references of the group stay counted either way */
+        if (slot == BAM_NO_SLOT) return nullptr;        /* the wait was given up (the controller is marked aborted): no window */
         view.window(pg, start, end);
         addr = (T*)(view.slot_addr(slot) + (view.byte_of(start) & (view.page_size - 1)));
 #endif
         return addr;
     }
 
+    /* after a wait that was given up the value is T(): callers that use what they read as an index (the neighbour
+     * ids of a graph) stay inside their arrays until the host sees the abort */
     __forceinline__ __host__ __device__ T read(const size_t i)
     {
-        if (i < start || i >= end) update_page(i);
+        if (i < start || i >= end) { if (!update_page(i)) return T(); }
 #if defined(__HIP_DEVICE_COMPILE__)
         return bam::ld_payload(addr + (i - start));
 #else
@@ -1228,7 +1231,7 @@ struct bam_ptr {
 
     __forceinline__ __host__ __device__ void write(const size_t i, const T v)
     {
-        if (i < start || i >= end) update_page(i);
+        if (i < start || i >= end) { if (!update_page(i)) return; }
         mark_dirty();
         addr[i - start] = v;
     }

@@ -57,6 +57,8 @@ def lib():
         "bo_edge_weights": (None, [u64, u64, u64, _p32]),
         "bo_sssp_costs": (None, [u64, _p64, _p64, _p32, u64, _p32]),
         "bo_sssp_costs_sweep": (u32, [u64, _p64, _p64, _p32, u64, _p32]),
+        "bo_sssp_costs_float": (None, [u64, _p64, _p64, _pf32, u64, _pf32]),
+        "bo_sssp_costs_float_sweep": (u32, [u64, _p64, _p64, _pf32, u64, _pf32]),
         "bo_reduce_blocks": (None, [_p64, u64, u32, _p64]),
         "bo_scan": (None, [_p64, u64, _p64]),
         "bo_pagerank": (u32, [u64, _p64, _p64, ctypes.c_float, ctypes.c_float, u32, _pf32]),
@@ -157,6 +159,18 @@ def sssp_costs(offsets, neigh, weights, src, sweep=False):
         rounds = lib().bo_sssp_costs_sweep(len(offsets) - 1, offsets, nb, w, int(src), costs)
         return costs, rounds
     lib().bo_sssp_costs(len(offsets) - 1, offsets, nb, w, int(src), costs)
+    return costs
+
+
+def sssp_costs_float(offsets, neigh, weights, src, sweep=False):
+    """single-precision costs (unreached = 1e9) for float32 weights >= 0"""
+    costs = np.empty(len(offsets) - 1, dtype=np.float32)
+    nb = neigh if len(neigh) else np.zeros(1, dtype=np.uint64)
+    w = np.ascontiguousarray(weights, dtype=np.float32) if len(weights) else np.zeros(1, dtype=np.float32)
+    if sweep:
+        rounds = lib().bo_sssp_costs_float_sweep(len(offsets) - 1, offsets, nb, w, int(src), costs)
+        return costs, rounds
+    lib().bo_sssp_costs_float(len(offsets) - 1, offsets, nb, w, int(src), costs)
     return costs
 
 

@@ -321,6 +321,53 @@ void bo_sssp_costs(uint64_t n_vertices, const uint64_t* offsets, const uint64_t*
     free(heap);
 }
 
+/*
+ * benchmarks/sssp_float/main.cu (WeightT = float :69, unreached = 1e9 :529, relax :194-217, update :302-312): the fixed point of
+ * its rounds.  Every cost a vertex ever holds is the sum, added edge by edge in single precision from the source on, of
+ * the weights along some path; adding a weight that is not negative never lowers a cost and keeps the order of two
+ * costs, so the least such sum is what Dijkstra's order finds, whatever order the rounds relax in.  A cost that does
+ * not come out below 1e9 is never adopted.  Costs that are not negative order as their bit patterns: the heap keys.
+ */
+static uint32_t float_bits(float f) { uint32_t u; memcpy(&u, &f, sizeof(u)); return u; }
+
+void bo_sssp_costs_float(uint64_t n_vertices, const uint64_t* offsets, const uint64_t* neigh, const float* weights, uint64_t src, float* costs)
+{
+    for (uint64_t v = 0; v < n_vertices; v++) costs[v] = BO_FAR_F32;
+    heap_item* heap = (heap_item*)malloc((offsets[n_vertices] + 1) * sizeof(heap_item));
+    uint64_t n = 0;
+    costs[src] = 0.0f;
+    heap_push(heap, &n, (heap_item){0, src});
+    while (n) {
+        heap_item it = heap_pop(heap, &n);
+        if (it.cost != float_bits(costs[it.v])) continue;
+        for (uint64_t e = offsets[it.v]; e < offsets[it.v + 1]; e++) {
+            const float c = costs[it.v] + weights[e];
+            if (c < costs[neigh[e]]) {
+                costs[neigh[e]] = c;
+                heap_push(heap, &n, (heap_item){float_bits(c), neigh[e]});
+            }
+        }
+    }
+    free(heap);
+}
+
+uint32_t bo_sssp_costs_float_sweep(uint64_t n_vertices, const uint64_t* offsets, const uint64_t* neigh, const float* weights, uint64_t src, float* costs)
+{
+    for (uint64_t v = 0; v < n_vertices; v++) costs[v] = BO_FAR_F32;
+    costs[src] = 0.0f;
+    uint32_t rounds = 0;
+    for (int changed = 1; changed;) {
+        changed = 0;
+        for (uint64_t v = n_vertices; v-- > 0;)                 /* highest vertex first: not the order of the heap */
+            for (uint64_t e = offsets[v]; e < offsets[v + 1]; e++) {
+                const float c = costs[v] + weights[e];
+                if (c < costs[neigh[e]]) { costs[neigh[e]] = c; changed = 1; }
+            }
+        rounds += changed;
+    }
+    return rounds;
+}
+
 /* benchmarks/reduction/main.cu:166-195: block b of `block` threads sums elements [2 b block, 2 (b + 1) block) */
 void bo_reduce_blocks(const uint64_t* a, uint64_t n, uint32_t block, uint64_t* out)
 {

@@ -14,6 +14,8 @@
  *   bo_cc_labels             reference sample graph + scipy connected_components
  *   bo_rmat_edges/bo_uniform_edges/bo_build_csr   independent numpy restatement
  *   bo_sssp_costs            hand-computed weighted graph + scipy dijkstra + the independent sweep bo_sssp_costs_sweep
+ *   bo_sssp_costs_float      hand-computed graph whose sums round (2^24 + 1, 0.1f + 0.2f) + scipy dijkstra on weights that add exactly +
+ *                            the independent sweep bo_sssp_costs_float_sweep + a numpy float32 relaxation
  *   bo_reduce_blocks/bo_scan numpy sums and cumsum, closed form n(n+1)/2 on 0..n-1, wrap-around mod 2^64
  *   bo_pagerank              hand-computed first sweeps on a 3-vertex path; sparse solve of (I - alpha P^T) x = (1 - alpha)
  *                            (scipy, double) with the bound 0 <= x - value <= x tolerance / (1 - alpha); bo_pagerank_limit
@@ -60,6 +62,11 @@ void     bo_edge_weights(uint64_t seed, uint64_t first, uint64_t n, uint32_t* ou
  * and returns how many rounds changed something. */
 void     bo_sssp_costs(uint64_t n_vertices, const uint64_t* offsets, const uint64_t* neigh, const uint32_t* weights, uint64_t src, uint32_t* costs);
 uint32_t bo_sssp_costs_sweep(uint64_t n_vertices, const uint64_t* offsets, const uint64_t* neigh, const uint32_t* weights, uint64_t src, uint32_t* costs);
+/* the same with single-precision weights and costs (benchmarks/sssp_float/main.cu:69, 194-217, 302-312, 529): weights >= 0,
+ * unreached = BO_FAR_F32; bit-exact whatever the order of relaxation (see the .c file) */
+#define BO_FAR_F32 1000000000.0f
+void     bo_sssp_costs_float(uint64_t n_vertices, const uint64_t* offsets, const uint64_t* neigh, const float* weights, uint64_t src, float* costs);
+uint32_t bo_sssp_costs_float_sweep(uint64_t n_vertices, const uint64_t* offsets, const uint64_t* neigh, const float* weights, uint64_t src, float* costs);
 
 /* benchmarks/reduction/main.cu:166-195 and benchmarks/scan/main.cu:147-190, 89-100: per-block sums; running sums with a
  * leading zero (out holds n + 1 words) */

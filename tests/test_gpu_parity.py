@@ -598,6 +598,8 @@ def test_hub_lists_are_cut_into_pieces(bam, cache_pages, coarse):
             lv, it = a.bfs(doff, src, coarse=coarse)
             want, want_it = oracle.bfs_levels(off, nb, src)
             assert np.array_equal(lv.cpu().numpy().view(np.uint32), want) and it == want_it
+            lv, it = a.bfs(doff, src, frontier=True)
+            assert np.array_equal(lv.cpu().numpy().view(np.uint32), want) and it == want_it
         lb, _ = a.cc(doff, coarse=coarse)
         assert np.array_equal(_u64(lb), oracle.cc_labels(off, nb)[0])
         # PageRank pushes over the same lists (tolerance as in test_pagerank_values)
@@ -635,6 +637,47 @@ def test_sssp_costs_two_arrays_in_one_cache(bam, scale, cache_pages):
             assert np.array_equal(costs.cpu().numpy().view(np.uint32), oracle.sssp_costs(off, nb, w, int(src))) and rounds >= 2
         assert edges.stats()["read_io_cnt"] > 0 and weights.stats()["access_cnt"] > 0 and not r.c.aborted()
         edges.close(); weights.close(); re_.close(); rw.close(); pc.close()
+
+
+@pytest.mark.parametrize("scale,cache_pages", [(10, 2048), (13, 160)])
+def test_sssp_float_costs(bam, scale, cache_pages):
+    """benchmarks/sssp_float: single-precision weights whose sums round; costs must equal the serial Dijkstra in single
+    precision to the bit (adding a weight keeps the order of two costs, so the order of relaxation does not matter)"""
+    off, nb = oracle.rmat_csr(SEED, scale)
+    w = oracle.edge_weights(SEED, len(nb)).astype(np.float32) * np.float32(0.37) + np.float32(1e-3)
+    e_pages = (len(nb) * 8 + 4095) // 4096
+    w_pages = (len(w) * 4 + 4095) // 4096
+    with Rig(bam, (e_pages + w_pages + 1) * 4096, backing=True, n_queues=8, depth=256) as r:
+        store = r.backing((e_pages + w_pages + 1) * 512)
+        store[:len(nb)] = nb
+        store[e_pages * 512:].view(np.float32)[:len(w)] = w
+        pc = bam.PageCache(4096, cache_pages, 0, r.c)
+        re_ = bam.Range(0, len(nb), 0, e_pages, 0, 4096, pc, 0)
+        rw = bam.Range32(0, len(w), e_pages, w_pages, 0, 4096, pc, 0)
+        edges = bam.Array(len(nb), 0, [re_], 0)
+        weights = bam.Array32(len(w), e_pages * 4096, [rw], 0)
+        doff = _dev(off)
+        for src in oracle.bfs_sources(SEED, off, 3):
+            costs, rounds = bam.sssp_float(edges, weights, doff, int(src))
+            want = oracle.sssp_costs_float(off, nb, w, int(src))
+            assert np.array_equal(costs.cpu().numpy().view(np.uint32), want.view(np.uint32)) and rounds >= 2
+            assert np.any(want == np.float32(1e9)) or scale > 10        # unreached vertices are part of the case where there are any
+        assert edges.stats()["read_io_cnt"] > 0 and weights.stats()["access_cnt"] > 0 and not r.c.aborted()
+        edges.close(); weights.close(); re_.close(); rw.close(); pc.close()
+
+
+@pytest.mark.parametrize("scale,cache_pages", [(10, 4096), (14, 24), (16, 8192), (17, 700)])
+def test_bfs_levels_rmat_by_queue_of_vertices(bam, scale, cache_pages):
+    """the kernel that walks a queue of the level's vertices: same levels, same launch count"""
+    off, nb = oracle.rmat_csr(SEED, scale)
+    r, a = _graph_rig(bam, nb, cache_pages, n_queues=16, depth=256)
+    with r:
+        doff = _dev(off)
+        for src in list(oracle.bfs_sources(SEED, off, 3)) + [int(np.flatnonzero(np.diff(off) == 0)[0])]:
+            lv, it = a.bfs(doff, int(src), frontier=True)
+            ref, rit = oracle.bfs_levels(off, nb, int(src))
+            assert np.array_equal(lv.cpu().numpy().view(np.uint32), ref) and it == rit
+        assert a.stats()["read_io_cnt"] > 0 and not r.c.aborted()
 
 
 @pytest.mark.parametrize("scale,cache_pages,tol", [(10, 2048, 1e-3), (13, 96, 1e-3), (14, 512, 1e-4)])

@@ -176,6 +176,65 @@ def test_sssp_hand_computed_graph():
     assert costs.tolist() == [0, 2, 5, 6, 12, inf] and rounds >= 1
 
 
+def test_sssp_float_hand_computed_graph_whose_sums_round():
+    """0 -> 1 (2^24) -> 2 (1): 2^24 + 1 is not a float and rounds back to 2^24, which beats the direct edge of 2^24 + 2;
+    0 -> 3 (0.1) -> 4 (0.2) -> 7 (0.4): the sum added edge by edge in single precision, one unit in the last place above
+    the rounded exact sum; 5 cannot be reached; 6 only over a path whose cost does not stay below 1e9, which is never taken"""
+    f = np.float32
+    pairs = [(0, 1, f(16777216.0)), (1, 2, f(1.0)), (0, 2, f(16777218.0)), (0, 3, f(0.1)), (3, 4, f(0.2)), (4, 7, f(0.4)),
+             (4, 6, f(1e9)), (5, 0, f(1.0))]
+    n_v = 8
+    off = np.zeros(n_v + 1, dtype=np.uint64)
+    for u, _, _ in pairs:
+        off[u + 1] += 1
+    off = np.cumsum(off).astype(np.uint64)
+    order = sorted(range(len(pairs)), key=lambda k: pairs[k][0])
+    nb = np.array([pairs[k][1] for k in order], dtype=np.uint64)
+    w = np.array([pairs[k][2] for k in order], dtype=np.float32)
+    want = np.array([0.0, 16777216.0, 16777216.0, f(0.1), f(0.1) + f(0.2), 1e9, 1e9, 0.0], dtype=np.float32)
+    want.view(np.uint32)[7] = 1060320052                                    # 0.70000005: (0.1f + 0.2f) + 0.4f
+    assert np.float32(float(f(0.1)) + float(f(0.2)) + float(f(0.4))).view(np.uint32) == 1060320051      # the exact sum rounds elsewhere
+    got = oracle.sssp_costs_float(off, nb, w, 0)
+    assert got.view(np.uint32).tolist() == want.view(np.uint32).tolist()
+    swept, rounds = oracle.sssp_costs_float(off, nb, w, 0, sweep=True)
+    assert swept.view(np.uint32).tolist() == want.view(np.uint32).tolist() and rounds >= 1
+
+
+@pytest.mark.parametrize("seed,scale", [(1, 8), (42, 11)])
+def test_sssp_float_against_scipy_the_sweep_and_numpy(seed, scale):
+    from scipy.sparse import csr_matrix
+    from scipy.sparse.csgraph import dijkstra
+    off, nb = oracle.rmat_csr(seed, scale)
+    n_v = len(off) - 1
+    wi = oracle.edge_weights(seed, len(nb))
+    srcs = oracle.bfs_sources(seed, off, 2)
+    # (a) weights that add exactly in single precision (small integers and quarters): the double-precision answer is the answer
+    w_exact = (wi.astype(np.float32) * np.float32(0.25))
+    g = csr_matrix((w_exact.astype(np.float64), nb.astype(np.int64), off.astype(np.int64)), shape=(n_v, n_v))
+    for src in srcs:
+        d = dijkstra(g, directed=True, indices=int(src))
+        want = np.where(np.isinf(d), 1e9, d).astype(np.float32)
+        assert np.array_equal(oracle.sssp_costs_float(off, nb, w_exact, int(src)), want)
+    # (b) weights whose sums round: Dijkstra's order, the sweep from the highest vertex down and a numpy relaxation of
+    # all edges at once must agree to the bit
+    w = wi.astype(np.float32) * np.float32(0.37) + np.float32(1e-3)
+    u = np.repeat(np.arange(n_v, dtype=np.int64), np.diff(off).astype(np.int64))
+    v = nb.astype(np.int64)
+    for src in srcs:
+        got = oracle.sssp_costs_float(off, nb, w, int(src))
+        swept, _ = oracle.sssp_costs_float(off, nb, w, int(src), sweep=True)
+        assert np.array_equal(got.view(np.uint32), swept.view(np.uint32))
+        c = np.full(n_v, 1e9, dtype=np.float32); c[int(src)] = 0
+        while True:
+            nxt = c.copy()
+            np.minimum.at(nxt, v, c[u] + w)
+            if np.array_equal(nxt, c):
+                break
+            c = nxt
+        assert np.array_equal(got.view(np.uint32), c.view(np.uint32))
+        assert len(np.unique(got)) > 100                                    # not a degenerate case
+
+
 @pytest.mark.parametrize("seed,scale", [(42, 8), (0, 10), (7, 12)])
 def test_sssp_against_scipy_and_the_sweep(seed, scale):
     off, nb = oracle.rmat_csr(seed, scale)
