@@ -361,6 +361,44 @@ struct list_read_ahead {
         if (bam::ballot(want && pl != pf)) view.acquire_helped(pl, want && pl != pf, false, touch, touch);
         view.n_access = view.n_hit = 0;
     }
+    /*
+     * The lists of the consecutive vertices [first, last) lie side by side in the array: touch every page that holds
+     * entries of a list that is about to be walked (item(v, v) says which; lists that go to the queue of long ones are
+     * left out), `reach` pages at a time with one page per lane, so that what is not resident comes in as few, large
+     * batches of commands.  The store path moves several times more pages per second in batches of sixteen than in
+     * batches of two or three, which is what touching the lists of 64 vertices at a time gives on a graph with a few
+     * dozen edges per vertex.  False if the span is too wide for that (the caller then touches list by list).
+     */
+    template <typename Item>
+    __device__ __forceinline__ bool span(const uint64_t* vertexList, const uint64_t first, const uint64_t last, const uint64_t heavy_from, Item item)
+    {
+        if (reach < 2) return false;
+        const uint64_t e0 = vertexList[first], e1 = vertexList[last];
+        if (e1 <= e0) return true;
+        const uint64_t p0 = view.page_of(e0), p1 = view.page_of(e1 - 1);
+        if (p1 - p0 >= 4ull * reach) return false;
+        auto touch = [](uint32_t) { return true; };
+        const uint32_t lane = bam::lane();
+        for (uint64_t c = p0; c <= p1; c += reach) {
+            uint64_t m = 0;
+            for (uint64_t b = first; b < last; b += BAM_WAVE_SIZE) {
+                uint64_t v = 0;
+                if (b + lane < last && item(b + lane, v)) {
+                    const uint64_t es = vertexList[v], ee = vertexList[v + 1];
+                    if (ee > es && ee - es < heavy_from) {
+                        const uint64_t pf = view.page_of(es), pl = view.page_of(ee - 1);
+                        const uint64_t f = pf > c ? pf - c : 0, l = pl < c + reach - 1 ? pl - c : reach - 1;
+                        if (pl >= c && f <= l) m |= (~0ull >> (63 - l)) & (~0ull << f);
+                    }
+                }
+            }
+#pragma unroll
+            for (uint32_t o = BAM_WAVE_SIZE / 2; o; o >>= 1) m |= bam::shfl(m, lane ^ o);
+            if (m) view.acquire_helped(c + lane, ((m >> lane) & 1) != 0, false, touch, touch);
+        }
+        view.n_access = view.n_hit = 0;
+        return true;
+    }
     /* wave-uniform: the list is elements [start, end) */
     __device__ __forceinline__ void begin(const uint64_t start, const uint64_t end)
     {
@@ -421,23 +459,42 @@ __device__ __forceinline__ void walk_packed(const uint64_t es, const uint64_t ee
  * The traversal of the reference's coarsened per-vertex kernels (bfs/main.cu:658-689, cc/main.cu:123-144): the
  * vertices are handed out in groups of `coarse`, and the edge list of every active vertex is read through bam_ptr.
  * What differs, for the store's and the memory system's sake:
- *  - the launch has as many waves as the device holds at a time, and a wave takes the next group when it is done
- *    with its last one (one atomic per group).  One group per wave of a large grid leaves most of the device idle
+ *  - the launch has as many waves as the device holds at a time, and a wave takes the next piece of work when it is
+ *    done with its last one (one atomic each).  One group per wave of a large grid leaves most of the device idle
  *    here: groups differ in length by orders of magnitude, and workgroups are started in order;
  *  - the flags and offsets of 64 vertices are read at a time, one vertex per lane, and the lists of those vertices
  *    are walked packed (walk_packed): 64 edges per step whichever vertices they belong to;
- *  - before the walk the first and last page of every list are touched, so that what is not resident comes in as
- *    one batch of commands or two, not one trip to the store per vertex;
- *  - lists of BAM_HEAVY_EDGES entries and more are queued in pieces for a second launch (below).
+ *  - before the walk the pages that hold the lists of the group's active vertices are touched (list_read_ahead::span),
+ *    so that what is not resident comes in as one batch of commands, not one trip to the store per vertex;
+ *  - lists of BAM_HEAVY_EDGES entries and more are walked in pieces, by a wave each (below).
  */
 /*
- * A list of BAM_HEAVY_EDGES entries or more is not walked by the wave that finds it: it is cut into pieces of that
- * size, which are queued and walked by a wave each in a second launch (walk_heavy_pieces).  The hubs of a power-law
- * graph have lists of hundreds of pages; walked by one wave, a single hub takes longer than all other vertices of
- * its level together.
+ * A list of BAM_HEAVY_EDGES entries or more is not walked with its group: it is cut into pieces of BAM_PIECE_EDGES
+ * entries, each walked by a wave of its own.  The hubs of a power-law graph have lists of hundreds of pages; walked
+ * by one wave, a single hub takes longer than all other vertices of its level together.  Which lists are long does
+ * not change from sweep to sweep, so the pieces are listed once per call (k_heavy_pieces) and every sweep hands them
+ * out before the groups, longest work first: a piece whose vertex is not active costs its wave one look at the flag.
  */
 #define BAM_HEAVY_EDGES 1024u
+/* entries per piece: 16 pages of 4 KiB, which the wave that walks the piece asks for as one batch of commands.  Pieces
+ * of the threshold's size reach the store as batches of two or three commands, and the store path moves far fewer
+ * pages per second in such batches than in batches of sixteen */
+#define BAM_PIECE_EDGES 8192u
 struct heavy_piece_t { uint64_t v, first, last; };      /* entries [first, last) of the list of vertex v */
+
+__global__ void k_heavy_pieces(const uint64_t* vertexList, const uint64_t vertex_count, heavy_piece_t* pieces, unsigned long long* count)
+{
+    const uint64_t v = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (v >= vertex_count) return;
+    const uint64_t start = vertexList[v], end = vertexList[v + 1];
+    if (end - start < BAM_HEAVY_EDGES) return;
+    const uint64_t n = (end - start + BAM_PIECE_EDGES - 1) / BAM_PIECE_EDGES;
+    const unsigned long long at = atomicAdd(count, (unsigned long long)n);
+    for (uint64_t k = 0; k < n; k++) {
+        const uint64_t f = start + k * BAM_PIECE_EDGES;
+        pieces[at + k] = heavy_piece_t{v, f, f + BAM_PIECE_EDGES < end ? f + BAM_PIECE_EDGES : end};
+    }
+}
 
 /*
  * Reads with the page referenced for the one read only.  bam_ptr keeps every lane's page referenced until the lane
@@ -468,14 +525,18 @@ struct touch_reader {
     __device__ __forceinline__ void fini() { if (one_range) view.flush_stats(); }
 };
 
-/* the walk over `n_items` work items, each of which names a vertex and says whether it is to be walked: item(i, v).
- * HOLD: read through bam_ptr (items whose lists lie side by side); otherwise page by page without holding any */
-template <bool HOLD, typename Item, typename Visit>
+/*
+ * One sweep: the pieces of the long lists whose vertex is active(v), then `n_items` work items in groups of `coarse`,
+ * each of which names a vertex and says whether it is to be walked: item(i, v).  visit(src, value, i) for every entry.
+ * HOLD: the items are the vertices themselves (item i is vertex i, lists side by side), read through bam_ptr;
+ * otherwise the items' lists lie anywhere, and they are read page by page without holding any.
+ */
+template <bool HOLD, typename Item, typename Active, typename Visit>
 __device__ __forceinline__ void walk_item_groups(array_d_t<uint64_t>* da, const uint64_t* vertexList, const uint64_t n_items, const uint64_t coarse,
-                                                 heavy_piece_t* heavy, unsigned long long* n_heavy, Item item, Visit visit)
+                                                 const heavy_piece_t* heavy, const uint64_t n_heavy, unsigned long long* next_work,
+                                                 Item item, Active active, Visit visit)
 {
     const uint64_t laneIdx = threadIdx.x % BAM_WAVE_SIZE;
-    unsigned long long* next_group = n_heavy + 1;
     const uint64_t n_groups = (n_items + coarse - 1) / coarse;
     bam_ptr<uint64_t> ptr(da);
     touch_reader<uint64_t> touch;
@@ -483,11 +544,29 @@ __device__ __forceinline__ void walk_item_groups(array_d_t<uint64_t>* da, const 
     list_read_ahead<uint64_t> ahead;
     bool ready = false;
     for (;;) {
-        unsigned long long g = 0;
-        if (laneIdx == 0) g = atomicAdd(next_group, 1ull);
-        g = bam::bcast((uint64_t)g, 0);
+        unsigned long long w = 0;
+        if (laneIdx == 0) w = atomicAdd(next_work, 1ull);
+        w = bam::bcast((uint64_t)w, 0);
+        if (w < n_heavy) {
+            /* a piece of a long list, all lanes side by side through bam_ptr, read ahead over the piece */
+            const heavy_piece_t pc = heavy[w];
+            if (!active(pc.v)) continue;
+            if (!ready) { ahead.init(da); ready = true; }
+            ahead.begin(pc.first, pc.last);
+            for (uint64_t i = (pc.first & 0xFFFFFFFFFFFFFFF0ull) + laneIdx; i < pc.last; i += BAM_WAVE_SIZE) {
+                ahead.step(i - laneIdx > pc.first ? i - laneIdx : pc.first);
+                if (i >= pc.first) visit(pc.v, ptr.read(i), i);
+            }
+            continue;
+        }
+        const uint64_t g = w - n_heavy;
         if (g >= n_groups) break;
         const uint64_t first = g * coarse;
+        bool touched = false;
+        if constexpr (HOLD) {
+            if (!ready) { ahead.init(da); ready = true; }
+            touched = ahead.span(vertexList, first, first + coarse < n_items ? first + coarse : n_items, BAM_HEAVY_EDGES, item);
+        }
         for (uint64_t b = 0; b < coarse; b += BAM_WAVE_SIZE) {
             const uint64_t at_item = first + b + laneIdx;
             uint64_t mine = 0;
@@ -496,21 +575,8 @@ __device__ __forceinline__ void walk_item_groups(array_d_t<uint64_t>* da, const 
             if (!ready) { ahead.init(da); ready = true; }
             uint64_t es = 0, ee = 0;
             if (act) { es = vertexList[mine]; ee = vertexList[mine + 1]; }
-            /* long lists go to the queue, in pieces */
-            for (uint64_t hm = bam::ballot(ee - es >= BAM_HEAVY_EDGES); hm; hm &= hm - 1) {
-                const uint32_t j = bam::first_lane(hm);
-                const uint64_t start = bam::bcast(es, j), end = bam::bcast(ee, j), v = bam::bcast(mine, j);
-                const uint64_t pieces = (end - start + BAM_HEAVY_EDGES - 1) / BAM_HEAVY_EDGES;
-                unsigned long long at = 0;
-                if (laneIdx == 0) at = atomicAdd(n_heavy, (unsigned long long)pieces);
-                at = bam::bcast((uint64_t)at, 0);
-                for (uint64_t k = laneIdx; k < pieces; k += BAM_WAVE_SIZE) {
-                    const uint64_t f = start + k * BAM_HEAVY_EDGES;
-                    heavy[at + k] = heavy_piece_t{v, f, f + BAM_HEAVY_EDGES < end ? f + BAM_HEAVY_EDGES : end};
-                }
-            }
-            if (ee - es >= BAM_HEAVY_EDGES) ee = es;
-            ahead.group(es, ee);
+            if (ee - es >= BAM_HEAVY_EDGES) ee = es;            /* walked in pieces */
+            if (!touched) ahead.group(es, ee);
             walk_packed(es, ee, mine, [&](uint64_t i) { if constexpr (HOLD) return ptr.read(i); else return touch.read(i); }, visit);
         }
     }
@@ -520,49 +586,20 @@ __device__ __forceinline__ void walk_item_groups(array_d_t<uint64_t>* da, const 
 /* the items are the vertices themselves, walked where active(v) */
 template <typename Active, typename Visit>
 __device__ __forceinline__ void walk_vertex_groups(array_d_t<uint64_t>* da, const uint64_t* vertexList, const uint64_t vertex_count, const uint64_t coarse,
-                                                   heavy_piece_t* heavy, unsigned long long* n_heavy, Active active, Visit visit)
+                                                   const heavy_piece_t* heavy, const uint64_t n_heavy, unsigned long long* next_work, Active active, Visit visit)
 {
-    walk_item_groups<true>(da, vertexList, vertex_count, coarse, heavy, n_heavy, [&](uint64_t i, uint64_t& v) { v = i; return active(i); }, visit);
-}
-
-/* the queued pieces, one wave at a time each: the same walk through bam_ptr, read ahead over the piece */
-template <typename Visit>
-__device__ __forceinline__ void walk_heavy_pieces(array_d_t<uint64_t>* da, const heavy_piece_t* heavy, const unsigned long long* n_heavy, Visit visit)
-{
-    const uint64_t tid = (uint64_t)blockDim.x * blockIdx.x + threadIdx.x;
-    const uint64_t waveIdx = tid / BAM_WAVE_SIZE, laneIdx = tid % BAM_WAVE_SIZE;
-    const uint64_t n_waves = (uint64_t)gridDim.x * blockDim.x / BAM_WAVE_SIZE;
-    const uint64_t n = *n_heavy;
-    if (waveIdx >= n) return;
-    bam_ptr<uint64_t> ptr(da);
-    list_read_ahead<uint64_t> ahead;
-    ahead.init(da);
-    for (uint64_t k = waveIdx; k < n; k += n_waves) {
-        const heavy_piece_t pc = heavy[k];
-        ahead.begin(pc.first, pc.last);
-        for (uint64_t i = (pc.first & 0xFFFFFFFFFFFFFFF0ull) + laneIdx; i < pc.last; i += BAM_WAVE_SIZE) {
-            ahead.step(i - laneIdx > pc.first ? i - laneIdx : pc.first);
-            if (i >= pc.first) visit(pc.v, ptr.read(i), i);
-        }
-    }
+    walk_item_groups<true>(da, vertexList, vertex_count, coarse, heavy, n_heavy, next_work,
+                           [&](uint64_t i, uint64_t& v) { v = i; return active(i); }, active, visit);
 }
 
 __global__ __launch_bounds__(128) void k_bfs_coalesce_coarse_ptr_pc(array_d_t<uint64_t>* da, uint32_t* label, const uint32_t level, const uint64_t vertex_count,
                                                                    const uint64_t* vertexList, uint64_t* changed, uint64_t coarse,
-                                                                   heavy_piece_t* heavy, unsigned long long* n_heavy)
+                                                                   const heavy_piece_t* heavy, uint64_t n_heavy, unsigned long long* next_work)
 {
     bool any = false;
-    walk_vertex_groups(da, vertexList, vertex_count, coarse, heavy, n_heavy,
+    walk_vertex_groups(da, vertexList, vertex_count, coarse, heavy, n_heavy, next_work,
                        [&](uint64_t v) { return label[v] == level; },
                        [&](uint64_t, uint64_t next, uint64_t) { if (label[next] == MYINFINITY) { label[next] = level + 1; any = true; } });
-    if (any) *changed = 1;
-}
-
-__global__ __launch_bounds__(128) void k_bfs_heavy_ptr_pc(array_d_t<uint64_t>* da, uint32_t* label, const uint32_t level, uint64_t* changed,
-                                                         const heavy_piece_t* heavy, const unsigned long long* n_heavy)
-{
-    bool any = false;
-    walk_heavy_pieces(da, heavy, n_heavy, [&](uint64_t, uint64_t next, uint64_t) { if (label[next] == MYINFINITY) { label[next] = level + 1; any = true; } });
     if (any) *changed = 1;
 }
 
@@ -583,17 +620,13 @@ __device__ __forceinline__ void bfs_frontier_visit(uint32_t* label, const uint32
 
 __global__ __launch_bounds__(128) void k_bfs_frontier_coalesce_ptr_pc(array_d_t<uint64_t>* da, uint32_t* label, const uint32_t level, const uint64_t* vertexList,
                                                                      const uint32_t* curr_frontier, const uint64_t curr_size, uint32_t* next_frontier,
-                                                                     unsigned long long* next_size, uint64_t group, heavy_piece_t* heavy, unsigned long long* n_heavy)
+                                                                     unsigned long long* next_size, uint64_t group,
+                                                                     const heavy_piece_t* heavy, uint64_t n_heavy, unsigned long long* next_work)
 {
-    walk_item_groups<false>(da, vertexList, curr_size, group, heavy, n_heavy,
+    walk_item_groups<false>(da, vertexList, curr_size, group, heavy, n_heavy, next_work,
                             [&](uint64_t i, uint64_t& v) { v = curr_frontier[i]; return true; },
+                            [&](uint64_t v) { return label[v] == level; },
                             [&](uint64_t, uint64_t next, uint64_t) { bfs_frontier_visit(label, level, next_frontier, next_size, next); });
-}
-
-__global__ __launch_bounds__(128) void k_bfs_frontier_heavy_ptr_pc(array_d_t<uint64_t>* da, uint32_t* label, const uint32_t level, uint32_t* next_frontier,
-                                                                  unsigned long long* next_size, const heavy_piece_t* heavy, const unsigned long long* n_heavy)
-{
-    walk_heavy_pieces(da, heavy, n_heavy, [&](uint64_t, uint64_t next, uint64_t) { bfs_frontier_visit(label, level, next_frontier, next_size, next); });
 }
 
 // ---- CC: min-label propagation (benchmarks/cc/main.cu:123-144, 595-617) ----
@@ -612,17 +645,11 @@ __device__ __forceinline__ void cc_compute(uint64_t cid, unsigned long long* com
 
 __global__ __launch_bounds__(128) void k_cc_coalesce_coarse_ptr_pc(array_d_t<uint64_t>* da, bool* curr_visit, bool* next_visit, uint64_t vertex_count,
                                                                   const uint64_t* vertexList, unsigned long long* comp, bool* changed, uint64_t coarse,
-                                                                  heavy_piece_t* heavy, unsigned long long* n_heavy)
+                                                                  const heavy_piece_t* heavy, uint64_t n_heavy, unsigned long long* next_work)
 {
-    walk_vertex_groups(da, vertexList, vertex_count, coarse, heavy, n_heavy,
+    walk_vertex_groups(da, vertexList, vertex_count, coarse, heavy, n_heavy, next_work,
                        [&](uint64_t v) { return curr_visit[v]; },
                        [&](uint64_t v, uint64_t next, uint64_t) { cc_compute(v, comp, next, next_visit, changed); });
-}
-
-__global__ __launch_bounds__(128) void k_cc_heavy_ptr_pc(array_d_t<uint64_t>* da, bool* next_visit, unsigned long long* comp, bool* changed,
-                                                        const heavy_piece_t* heavy, const unsigned long long* n_heavy)
-{
-    walk_heavy_pieces(da, heavy, n_heavy, [&](uint64_t v, uint64_t next, uint64_t) { cc_compute(v, comp, next, next_visit, changed); });
 }
 
 // ---- BFS / CC by edge page (benchmarks/bfs/main.cu:1074-1140 kernel_optimized_ptr_pc, first-vertex table :122-181) ----
@@ -849,17 +876,11 @@ __global__ void k_pr_initialize(bool* label, float* delta, float* residual, floa
  * are cleared by the host loop after the sweep */
 __global__ __launch_bounds__(128) void k_pr_coalesce_pc(array_d_t<uint64_t>* da, const bool* label, const float* delta, float* residual,
                                                         const uint64_t vertex_count, const uint64_t* vertexList, uint64_t group,
-                                                        heavy_piece_t* heavy, unsigned long long* n_heavy)
+                                                        const heavy_piece_t* heavy, uint64_t n_heavy, unsigned long long* next_work)
 {
-    walk_vertex_groups(da, vertexList, vertex_count, group, heavy, n_heavy,
+    walk_vertex_groups(da, vertexList, vertex_count, group, heavy, n_heavy, next_work,
                        [&](uint64_t v) { return label[v]; },
                        [&](uint64_t src, uint64_t next, uint64_t) { unsafeAtomicAdd(&residual[next], delta[src]); });
-}
-
-__global__ __launch_bounds__(128) void k_pr_heavy_pc(array_d_t<uint64_t>* da, const float* delta, float* residual, const heavy_piece_t* heavy,
-                                                     const unsigned long long* n_heavy)
-{
-    walk_heavy_pieces(da, heavy, n_heavy, [&](uint64_t src, uint64_t next, uint64_t) { unsafeAtomicAdd(&residual[next], delta[src]); });
 }
 
 /* the same pushes taken page by page of the edge array; the flags are cleared by the host loop after the sweep */
@@ -900,20 +921,12 @@ __device__ __forceinline__ void sssp_relax(uint32_t* newCostList, const bam_ptr<
 template <bool FLOAT>
 __global__ __launch_bounds__(128) void k_sssp_coalesce_pc(array_d_t<uint64_t>* de, array_d_t<uint32_t>* dw, const bool* label, uint32_t* newCostList,
                                                           const uint64_t vertex_count, const uint64_t* vertexList, uint64_t group,
-                                                          heavy_piece_t* heavy, unsigned long long* n_heavy)
+                                                          const heavy_piece_t* heavy, uint64_t n_heavy, unsigned long long* next_work)
 {
     bam_ptr<uint32_t> wptr(dw);
-    walk_vertex_groups(de, vertexList, vertex_count, group, heavy, n_heavy,
+    walk_vertex_groups(de, vertexList, vertex_count, group, heavy, n_heavy, next_work,
                        [&](uint64_t v) { return label[v]; },
                        [&](uint64_t src, uint64_t next, uint64_t i) { sssp_relax<FLOAT>(newCostList, wptr, src, next, i); });
-}
-
-template <bool FLOAT>
-__global__ __launch_bounds__(128) void k_sssp_heavy_pc(array_d_t<uint64_t>* de, array_d_t<uint32_t>* dw, uint32_t* newCostList, const heavy_piece_t* heavy,
-                                                       const unsigned long long* n_heavy)
-{
-    bam_ptr<uint32_t> wptr(dw);
-    walk_heavy_pieces(de, heavy, n_heavy, [&](uint64_t src, uint64_t next, uint64_t i) { sssp_relax<FLOAT>(newCostList, wptr, src, next, i); });
 }
 
 __global__ void k_sssp_update(bool* label, uint32_t* costList, const uint32_t* newCostList, const uint64_t vertex_count, bool* changed)
@@ -1494,35 +1507,44 @@ int bam_block_checksum(bam_page_cache_t* pc, uint64_t n_slots, uint32_t req_byte
 }
 
 namespace {
-/* queue of the pieces of long edge lists, refilled in every sweep of the per-vertex graph kernels: a list of d >= BAM_HEAVY_EDGES
- * entries makes at most d / BAM_HEAVY_EDGES + 1 <= 2 d / BAM_HEAVY_EDGES pieces */
+/* the pieces of the long edge lists of a graph, listed once per call, and the counter that hands out the work of a sweep:
+ * a list of d >= BAM_HEAVY_EDGES entries makes at most d / BAM_PIECE_EDGES + 1 <= 2 d / BAM_HEAVY_EDGES pieces */
 struct heavy_queue {
     BufferPtr buf, cnt;
     heavy_piece_t* pieces;
-    unsigned long long* count;       /* [0] pieces queued in this sweep, [1] next group of vertices to hand out */
-    uint32_t blocks;                 /* launch of the piece walk */
+    unsigned long long* count;       /* [0] number of pieces, [1] next piece of work of the sweep */
+    uint64_t n_pieces = 0;
     uint64_t group;                  /* vertices handed to a wave at a time */
-    uint32_t group_blocks;           /* launch of the group walk: what the device holds at a time */
-    uint32_t group_blocks_max;       /* the same without regard to the number of groups */
-    heavy_queue(uint64_t n_edges, uint64_t n_vertices, uint32_t coarse)
+    uint64_t resident;               /* waves the device holds at a time */
+    heavy_queue(uint64_t n_edges, uint64_t n_vertices, uint32_t coarse, const uint64_t* d_offsets, hipStream_t st)
     {
         const uint64_t cap = 2 * (n_edges / BAM_HEAVY_EDGES) + 1;
         buf = createBuffer(cap * sizeof(heavy_piece_t), 0);
         cnt = createBuffer(2 * sizeof(unsigned long long), 0);
         pieces = (heavy_piece_t*)buf.get();
         count = (unsigned long long*)cnt.get();
-        const uint64_t waves = cap < 4096 ? cap : 4096;          /* the pieces are shared out over this many waves */
-        blocks = (uint32_t)((waves + 1) / 2);                   /* two waves per workgroup */
-        /* one atomic per group on one word: a few hundred vertices per group keep that word out of the way */
-        group = coarse > 256 ? coarse : 256;
+        /* a group's lists are asked for as one batch of commands: a few hundred vertices make that batch large enough for the
+         * store path, and keep the one word all waves take their work from out of the way */
+        group = coarse > 512 ? coarse : 512;
         int dev = 0, cus = 0;
         hip_err_chk(hipGetDevice(&dev));
         hip_err_chk(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-        const uint64_t n_groups = (n_vertices + group - 1) / group, resident = (uint64_t)cus * 16;      /* waves */
-        group_blocks = (uint32_t)(((n_groups < resident ? n_groups : resident) + 1) / 2);
-        group_blocks_max = (uint32_t)((resident + 1) / 2);
+        resident = (uint64_t)cus * 16;
+        hip_err_chk(hipMemsetAsync(count, 0, 2 * sizeof(unsigned long long), st));
+        hipLaunchKernelGGL(k_heavy_pieces, dim3(blocks_for(n_vertices, 256)), dim3(256), 0, st, d_offsets, n_vertices, pieces, count);
+        hip_err_chk(hipGetLastError());
+        unsigned long long n = 0;
+        hip_err_chk(hipMemcpyAsync(&n, count, sizeof(n), hipMemcpyDeviceToHost, st));
+        hip_err_chk(hipStreamSynchronize(st));
+        n_pieces = n;
     }
-    void reset(hipStream_t st) { hip_err_chk(hipMemsetAsync(count, 0, 2 * sizeof(unsigned long long), st)); }
+    /* workgroups of two waves for a sweep over `n_items` items in groups of `grp` */
+    uint32_t blocks(uint64_t n_items, uint64_t grp) const
+    {
+        const uint64_t work = n_pieces + (n_items + grp - 1) / grp;
+        return (uint32_t)(((work < resident ? work : resident) + 1) / 2);
+    }
+    void reset(hipStream_t st) { hip_err_chk(hipMemsetAsync(count + 1, 0, sizeof(unsigned long long), st)); }
 };
 } // namespace
 
@@ -1539,16 +1561,15 @@ int bam_bfs(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, 
     hip_err_chk(hipMemsetAsync(d_labels, 0xFF, n_vertices * sizeof(uint32_t), st));
     hip_err_chk(hipMemcpyAsync(d_labels + src, &zero, sizeof(uint32_t), hipMemcpyHostToDevice, st));
     const uint32_t threads = 128;
-    heavy_queue hq(edges->a->adt.n_elems, n_vertices, coarse);
+    heavy_queue hq(edges->a->adt.n_elems, n_vertices, coarse, d_offsets, st);
     uint32_t level = 0, iter = 0;
     uint64_t changed_h;
     do {
         changed_h = 0;
         hip_err_chk(hipMemcpyAsync(changed_d, &changed_h, sizeof(uint64_t), hipMemcpyHostToDevice, st));
         hq.reset(st);
-        hipLaunchKernelGGL(k_bfs_coalesce_coarse_ptr_pc, dim3(hq.group_blocks), dim3(threads), 0, st,
-                           edges->a->d_array_ptr, d_labels, level, n_vertices, d_offsets, changed_d, hq.group, hq.pieces, hq.count);
-        hipLaunchKernelGGL(k_bfs_heavy_ptr_pc, dim3(hq.blocks), dim3(threads), 0, st, edges->a->d_array_ptr, d_labels, level, changed_d, hq.pieces, hq.count);
+        hipLaunchKernelGGL(k_bfs_coalesce_coarse_ptr_pc, dim3(hq.blocks(n_vertices, hq.group)), dim3(threads), 0, st,
+                           edges->a->d_array_ptr, d_labels, level, n_vertices, d_offsets, changed_d, hq.group, hq.pieces, hq.n_pieces, hq.count + 1);
         hip_err_chk(hipGetLastError());
         iter++; level++;
         hip_err_chk(hipMemcpyAsync(&changed_h, changed_d, sizeof(uint64_t), hipMemcpyDeviceToHost, st));
@@ -1578,19 +1599,14 @@ int bam_bfs_frontier(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_v
     hip_err_chk(hipMemcpyAsync(curr, &src32, sizeof(uint32_t), hipMemcpyHostToDevice, st));
     const uint32_t threads = 128;
     const uint64_t group = BAM_WAVE_SIZE;           /* queue entries handed to a wave at a time: one per lane */
-    heavy_queue hq(edges->a->adt.n_elems, n_vertices, 1);
-    const uint64_t resident = 2ull * hq.group_blocks_max;
+    heavy_queue hq(edges->a->adt.n_elems, n_vertices, 1, d_offsets, st);
     uint32_t level = 0, iter = 0;
     unsigned long long active = 1;
     do {
         hip_err_chk(hipMemsetAsync(next_size, 0, sizeof(unsigned long long), st));
         hq.reset(st);
-        const uint64_t n_groups = (active + group - 1) / group;
-        const uint32_t blocks = (uint32_t)(((n_groups < resident ? n_groups : resident) + 1) / 2);
-        hipLaunchKernelGGL(k_bfs_frontier_coalesce_ptr_pc, dim3(blocks), dim3(threads), 0, st, edges->a->d_array_ptr, d_labels, level, d_offsets,
-                           curr, (uint64_t)active, next, next_size, group, hq.pieces, hq.count);
-        hipLaunchKernelGGL(k_bfs_frontier_heavy_ptr_pc, dim3(hq.blocks), dim3(threads), 0, st, edges->a->d_array_ptr, d_labels, level, next, next_size,
-                           hq.pieces, hq.count);
+        hipLaunchKernelGGL(k_bfs_frontier_coalesce_ptr_pc, dim3(hq.blocks(active, group)), dim3(threads), 0, st, edges->a->d_array_ptr, d_labels, level,
+                           d_offsets, curr, (uint64_t)active, next, next_size, group, hq.pieces, hq.n_pieces, hq.count + 1);
         hip_err_chk(hipGetLastError());
         std::swap(curr, next);
         iter++; level++;
@@ -1616,17 +1632,15 @@ int bam_cc(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, u
     hip_err_chk(hipMemsetAsync(curr, 0x01, n_vertices, st));
     hip_err_chk(hipMemsetAsync(next, 0x00, n_vertices, st));
     const uint32_t threads = 128;
-    heavy_queue hq(edges->a->adt.n_elems, n_vertices, coarse);
+    heavy_queue hq(edges->a->adt.n_elems, n_vertices, coarse, d_offsets, st);
     uint32_t iter = 0;
     bool changed_h;
     do {
         changed_h = false;
         hip_err_chk(hipMemcpyAsync(changed_d, &changed_h, sizeof(bool), hipMemcpyHostToDevice, st));
         hq.reset(st);
-        hipLaunchKernelGGL(k_cc_coalesce_coarse_ptr_pc, dim3(hq.group_blocks), dim3(threads), 0, st,
-                           edges->a->d_array_ptr, curr, next, n_vertices, d_offsets, (unsigned long long*)d_labels, changed_d, hq.group, hq.pieces, hq.count);
-        hipLaunchKernelGGL(k_cc_heavy_ptr_pc, dim3(hq.blocks), dim3(threads), 0, st, edges->a->d_array_ptr, next, (unsigned long long*)d_labels, changed_d,
-                           hq.pieces, hq.count);
+        hipLaunchKernelGGL(k_cc_coalesce_coarse_ptr_pc, dim3(hq.blocks(n_vertices, hq.group)), dim3(threads), 0, st, edges->a->d_array_ptr, curr, next,
+                           n_vertices, d_offsets, (unsigned long long*)d_labels, changed_d, hq.group, hq.pieces, hq.n_pieces, hq.count + 1);
         hip_err_chk(hipGetLastError());
         hip_err_chk(hipMemsetAsync(curr, 0x00, n_vertices, st));
         bool* t = curr; curr = next; next = t;
@@ -1805,7 +1819,7 @@ int bam_pagerank(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_verti
     if (by_page)
         if (int rc = plan_by_page(edges, d_offsets, n_vertices, st, pl)) return rc;
     const uint32_t upd_blocks = blocks_for(n_vertices, 256);
-    heavy_queue hq(edges->a->adt.n_elems, n_vertices, 1);
+    heavy_queue hq(edges->a->adt.n_elems, n_vertices, 1, d_offsets, st);
     hipLaunchKernelGGL(k_pr_initialize, dim3(upd_blocks), dim3(256), 0, st, label_d, delta_d, residual_d, d_value, n_vertices, d_offsets, alpha);
     uint32_t iter = 0;
     bool changed_h;
@@ -1819,9 +1833,8 @@ int bam_pagerank(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_verti
             hip_err_chk(hipMemsetAsync(label_d, 0, n_vertices, st));
         } else {
             hq.reset(st);
-            hipLaunchKernelGGL(k_pr_coalesce_pc, dim3(hq.group_blocks), dim3(128), 0, st, edges->a->d_array_ptr, label_d, delta_d, residual_d, n_vertices,
-                               d_offsets, hq.group, hq.pieces, hq.count);
-            hipLaunchKernelGGL(k_pr_heavy_pc, dim3(hq.blocks), dim3(128), 0, st, edges->a->d_array_ptr, delta_d, residual_d, hq.pieces, hq.count);
+            hipLaunchKernelGGL(k_pr_coalesce_pc, dim3(hq.blocks(n_vertices, hq.group)), dim3(128), 0, st, edges->a->d_array_ptr, label_d, delta_d, residual_d,
+                               n_vertices, d_offsets, hq.group, hq.pieces, hq.n_pieces, hq.count + 1);
             hip_err_chk(hipMemsetAsync(label_d, 0, n_vertices, st));
         }
         iter++;
@@ -1921,17 +1934,15 @@ void sssp_run(const bool FLOAT, bam_array_t* edges, bam_array32_t* weights, cons
     hip_err_chk(hipMemcpyAsync(d_costs + src, &zero, sizeof(uint32_t), hipMemcpyHostToDevice, st));
     hip_err_chk(hipMemcpyAsync(new_d + src, &zero, sizeof(uint32_t), hipMemcpyHostToDevice, st));
     const uint32_t threads = 128;
-    heavy_queue hq(edges->a->adt.n_elems, n_vertices, 1);
+    heavy_queue hq(edges->a->adt.n_elems, n_vertices, 1, d_offsets, st);
     uint32_t iter = 0;
     bool changed_h;
     do {
         changed_h = false;
         hip_err_chk(hipMemcpyAsync(changed_d, &changed_h, sizeof(bool), hipMemcpyHostToDevice, st));
         hq.reset(st);
-        hipLaunchKernelGGL(FLOAT ? k_sssp_coalesce_pc<true> : k_sssp_coalesce_pc<false>, dim3(hq.group_blocks), dim3(threads), 0, st, edges->a->d_array_ptr,
-                           weights->a->d_array_ptr, label_d, new_d, n_vertices, d_offsets, hq.group, hq.pieces, hq.count);
-        hipLaunchKernelGGL(FLOAT ? k_sssp_heavy_pc<true> : k_sssp_heavy_pc<false>, dim3(hq.blocks), dim3(threads), 0, st, edges->a->d_array_ptr,
-                           weights->a->d_array_ptr, new_d, hq.pieces, hq.count);
+        hipLaunchKernelGGL(FLOAT ? k_sssp_coalesce_pc<true> : k_sssp_coalesce_pc<false>, dim3(hq.blocks(n_vertices, hq.group)), dim3(threads), 0, st,
+                           edges->a->d_array_ptr, weights->a->d_array_ptr, label_d, new_d, n_vertices, d_offsets, hq.group, hq.pieces, hq.n_pieces, hq.count + 1);
         hip_err_chk(hipMemsetAsync(label_d, 0, n_vertices, st));
         hipLaunchKernelGGL(k_sssp_update, dim3(blocks_for(n_vertices, 256)), dim3(256), 0, st, label_d, d_costs, new_d, n_vertices, changed_d);
         hip_err_chk(hipGetLastError());

@@ -130,10 +130,12 @@ int bam_block_checksum(bam_page_cache_t* pc, uint64_t n_slots, uint32_t req_byte
 /* ---- BFS (benchmarks/bfs/main.cu:658-689 kernel_coalesce_coarse_ptr_pc, host loop :1557-1566, 1577-1736) ----
  * Level-synchronous BFS from src: d_offsets[V+1] in device memory, neighbour ids read through the array,
  * d_labels[V] receives the level of every vertex (0xFFFFFFFF = unreachable).  *iterations = levels swept.
- * The vertices are handed out in groups of max(coarse, 256) to as many waves as the device holds; the lists of 64
- * vertices at a time are read through bam_ptr, 64 entries per step across list ends, and lists of 1024 entries and
- * more are cut into pieces that a second launch per level walks with a wave each (the same for bam_cc, bam_sssp and
- * bam_pagerank without by_page). */
+ * The vertices are handed out in groups of max(coarse, 512) to as many waves as the device holds.  A wave first
+ * touches the pages that hold the lists of its group's active vertices (what is not resident comes in as one batch of
+ * commands), then reads the lists of 64 vertices at a time through bam_ptr, 64 entries per step across list ends.
+ * Lists of 1024 entries and more are walked in pieces of 8192 entries by a wave each; the pieces are listed once per
+ * call and handed out in every sweep before the groups (the same for bam_cc, bam_sssp and bam_pagerank without
+ * by_page). */
 int bam_bfs(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t src, uint32_t* d_labels,
             uint32_t coarse, uint32_t* iterations, void* stream);
 /* ---- BFS over queues of vertices (benchmarks/bfs/main.cu:409-451 kernel_frontier_coalesce_ptr_pc, queues :1489-1492,

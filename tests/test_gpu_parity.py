@@ -581,7 +581,7 @@ def test_cc_labels_uniform_by_edge_page(bam, n_v, n_p, cache_pages):
 @pytest.mark.parametrize("cache_pages,coarse", [(24, 1), (256, 4), (4096, 64), (4096, 200)])
 def test_hub_lists_are_cut_into_pieces(bam, cache_pages, coarse):
     """two hubs with lists of 9000 and 4096 entries (18 and 8 pages) on top of a sparse random graph: the per-vertex
-    kernels queue such lists in pieces for a second launch; levels and labels must not notice.  The hubs sit in
+    kernels walk such lists in pieces, a wave each; levels and labels must not notice.  The hubs sit in
     different components until an edge of the random part joins them."""
     n_v = 20000
     pu = np.empty(6000, dtype=np.uint64); pv = np.empty(6000, dtype=np.uint64)
