@@ -1555,7 +1555,7 @@ int bam_bfs(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, 
     if (src >= n_vertices || !coarse) return fail(EINVAL, "bam_bfs: source out of range or coarse = 0");
     BAM_API_BEGIN
     hipStream_t st = (hipStream_t)stream;
-    BufferPtr changed_buf = createBuffer(sizeof(uint64_t), edges->a->adt.n_ranges ? 0 : 0);
+    BufferPtr changed_buf = createBuffer(sizeof(uint64_t), 0);
     uint64_t* changed_d = (uint64_t*)changed_buf.get();
     const uint32_t zero = 0;
     hip_err_chk(hipMemsetAsync(d_labels, 0xFF, n_vertices * sizeof(uint32_t), st));
