@@ -576,7 +576,15 @@ __device__ __forceinline__ void walk_item_groups(array_d_t<uint64_t>* da, const 
             uint64_t es = 0, ee = 0;
             if (act) { es = vertexList[mine]; ee = vertexList[mine + 1]; }
             if (ee - es >= BAM_HEAVY_EDGES) ee = es;            /* walked in pieces */
-            if (!touched) ahead.group(es, ee);
+            if (!touched) {
+                /* a group whose lists cover too many pages for one look: the same for the 64 vertices at hand */
+                bool block_touched = false;
+                if constexpr (HOLD) {
+                    const uint64_t last = first + coarse < n_items ? first + coarse : n_items;
+                    block_touched = ahead.span(vertexList, first + b, first + b + BAM_WAVE_SIZE < last ? first + b + BAM_WAVE_SIZE : last, BAM_HEAVY_EDGES, item);
+                }
+                if (!block_touched) ahead.group(es, ee);
+            }
             walk_packed(es, ee, mine, [&](uint64_t i) { if constexpr (HOLD) return ptr.read(i); else return touch.read(i); }, visit);
         }
     }
