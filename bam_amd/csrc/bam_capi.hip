@@ -704,14 +704,25 @@ __device__ __forceinline__ void graph_by_page(array_d_t<uint64_t>* da, const uin
         /* every other sweep runs from the far end: what the last sweep left in the cache is what this one asks for first */
         const uint64_t p0 = (backwards ? n_trips - 1 - t : t) * ppw;
         const uint64_t p = p0 + lane;
-        const uint64_t pstart = p * epp;
-        bool want = false;
-        uint64_t va = 0, vb = 0;
-        if (lane < ppw && p < n_pages) {
-            va = first[p]; vb = first[p + 1];
-            const uint64_t pend = pstart + epp;
-            for (uint64_t v = va; v <= vb && !want; v++) want = active(v) && offsets[v] < pend && offsets[v + 1] > pstart;
+        /* which pages of the trip hold entries of an active vertex: the lanes go over the trip's vertices side by side
+         * (their flags and offsets are consecutive in memory) and mark the pages each active list covers */
+        const uint64_t p_end = p0 + ppw < n_pages ? p0 + ppw : n_pages;
+        const uint64_t trip_start = p0 * epp, trip_end = p_end * epp < n_edges ? p_end * epp : n_edges;
+        uint64_t marks = 0;
+        for (uint64_t vbase = first[p0], v_last = first[p_end]; vbase <= v_last; vbase += BAM_WAVE_SIZE) {
+            const uint64_t v = vbase + lane;
+            if (v <= v_last && active(v)) {
+                uint64_t es = offsets[v], ee = offsets[v + 1];
+                if (es < trip_start) es = trip_start;
+                if (ee > trip_end) ee = trip_end;
+                if (ee > es) marks |= (~0ull >> (63 - (ee - 1 - trip_start) / epp)) & (~0ull << ((es - trip_start) / epp));
+            }
         }
+#pragma unroll
+        for (uint32_t o = BAM_WAVE_SIZE / 2; o; o >>= 1) marks |= bam::shfl(marks, lane ^ o);
+        const bool want = ((marks >> lane) & 1) != 0;
+        uint64_t va = 0, vb = 0;
+        if (want) { va = first[p]; vb = first[p + 1]; }
         uint32_t slot = 0;
         if (bam::ballot(want)) {
             /* the lanes without a page of their own come along and help move what the others load */
