@@ -761,6 +761,26 @@ def test_lost_completion_ends_the_kernel_with_the_abort_flag(bam):
         assert r.c.aborted(clear=True) and not r.c.aborted()
 
 
+@pytest.mark.parametrize("kernel", [dict(coarse=4), dict(frontier=True), dict(by_page=True)])
+def test_lost_completion_during_a_graph_traversal(bam, kernel):
+    """the same while edge lists are being read, where what is read is used as an index: the sweep ends, the flag says
+    that the levels are not to be used, and neighbour ids that never arrived stay inside the label array (a read
+    through bam_ptr gives 0 after a wait that was given up; a page declared valid without its payload holds what the
+    slot or the staging page held before, which is other neighbour ids, so the padding behind the last list is zeroed
+    here as a loader would)"""
+    off, nb = oracle.rmat_csr(SEED, 13)
+    pad = (-len(nb)) % 512
+    with Rig(bam, (len(nb) + pad) * 8, backing=True, n_queues=8, depth=256, drop_every=300, limit=300_000) as r:
+        store = r.backing(len(nb) + pad)
+        store[:len(nb)] = nb
+        store[len(nb):] = 0
+        a = r.array(len(nb), 4096, 64)
+        lv, it = a.bfs(_dev(off), int(oracle.bfs_sources(SEED, off, 1)[0]), **kernel)
+        assert r.c.aborted() and r.t.stats()["dropped"] >= 1 and it >= 1
+        lv = lv.cpu().numpy().view(np.uint32)
+        assert np.all((lv == 0xFFFFFFFF) | (lv <= it))
+
+
 def test_error_completions_are_counted(bam):
     with Rig(bam, 16 << 20, fail_every=100) as r:
         a = r.array(1 << 20, 4096, 4096)
