@@ -232,9 +232,17 @@ __device__ __forceinline__ void cache_stream_body(array_d_t<uint64_t>* dr, uint6
             bam_ptr<uint64_t> ptr(dr);
             for (uint64_t p = 0; p < n_pages_per_wave; p++) {
                 const uint64_t start_idx = (start_page + p) * epp + lane;
-                for (uint64_t j = 0; j < epp; j += BAM_WAVE_SIZE) {
-                    if (MODE == 0) v += (*dr)[start_idx + j];
-                    else v += ptr[start_idx + j];
+                if (MODE == 0) {
+                    for (uint64_t j = 0; j < epp; j += BAM_WAVE_SIZE) v += (*dr)[start_idx + j];
+                } else {
+                    /* eight elements asked for before the first is used: the window test of an element needs nothing that
+                     * an earlier load brings, so the loads of a page are in flight together */
+                    for (uint64_t j = 0; j < epp; j += 8 * BAM_WAVE_SIZE) {
+                        uint64_t x[8];
+#pragma unroll
+                        for (int u = 0; u < 8; u++) x[u] = j + u * BAM_WAVE_SIZE < epp ? (uint64_t)ptr[start_idx + j + u * BAM_WAVE_SIZE] : 0;
+                        v += ((x[0] + x[1]) + (x[2] + x[3])) + ((x[4] + x[5]) + (x[6] + x[7]));
+                    }
                 }
             }
         }
