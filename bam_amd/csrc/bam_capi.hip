@@ -214,12 +214,24 @@ __device__ __forceinline__ void cache_stream_body(array_d_t<uint64_t>* dr, uint6
                     auto keep = [&](uint32_t s_) { slot = s_; return false; };
                     view.acquire<true>(page, false, keep, keep);
                 }
-                for (uint32_t k = 0; k < nb; k++) {
+                uint32_t k = 0;
+                if (n8 == 8 * BAM_WAVE_SIZE)            /* 4 KiB pages: two at a time */
+                    for (; k + 1 < nb; k += 2) {
+                        uint64_t x[16];
+                        bam::ld_payload_stream16((const uint64_t*)view.slot_addr(bam::bcast(slot, k)) + lane,
+                                                 (const uint64_t*)view.slot_addr(bam::bcast(slot, k + 1)) + lane, x);
+                        a0 += ((x[0] + x[2]) + (x[4] + x[6])) + ((x[8] + x[10]) + (x[12] + x[14]));
+                        a1 += ((x[1] + x[3]) + (x[5] + x[7])) + ((x[9] + x[11]) + (x[13] + x[15]));
+                    }
+                for (; k < nb; k++) {
                     const uint64_t* base = (const uint64_t*)view.slot_addr(bam::bcast(slot, k));
                     for (uint32_t i = (uint32_t)lane; i < n8; i += 8 * BAM_WAVE_SIZE) {
                         uint64_t x[8];
+                        if (i + 7 * BAM_WAVE_SIZE < n8) bam::ld_payload_stream8(base + i, x);
+                        else {
 #pragma unroll
-                        for (int j = 0; j < 8; j++) x[j] = i + j * BAM_WAVE_SIZE < n8 ? bam::ld_payload(base + i + j * BAM_WAVE_SIZE) : 0;
+                            for (int j = 0; j < 8; j++) x[j] = i + j * BAM_WAVE_SIZE < n8 ? bam::ld_payload(base + i + j * BAM_WAVE_SIZE) : 0;
+                        }
                         a0 += x[0] + x[2] + x[4] + x[6];
                         a1 += x[1] + x[3] + x[5] + x[7];
                     }
@@ -1022,21 +1034,24 @@ __global__ void k_copy16(const uint4* __restrict__ src, uint4* __restrict__ dst,
 {
     for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (uint64_t)gridDim.x * blockDim.x) dst[i] = src[i];
 }
-/* plain streaming read of device memory, 16 bytes per lane per load, eight loads in flight: what the memory system gives a
- * reader that does nothing else (the practical ceiling under the hit-path figure) */
-__global__ __launch_bounds__(256) void k_read16(const uint4* __restrict__ src, uint64_t n16, unsigned long long* partials)
+/* plain streaming read of device memory with the loads of the hit path (a wave reads 4 KiB pieces side by side, eight 8-byte
+ * words per lane, past the vector L1 and marked as not to be kept) and nothing else: what the memory system gives such a
+ * reader, the practical ceiling over the hit-path figure */
+__global__ __launch_bounds__(256) void k_read_stream(const uint64_t* __restrict__ src, uint64_t n8, unsigned long long* partials)
 {
     uint64_t a = 0;
-    const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
-    uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    for (; i + 7 * stride < n16; i += 8 * stride) {
-        uint4 x[8];
-#pragma unroll
-        for (int k = 0; k < 8; k++) x[k] = src[i + k * stride];
-#pragma unroll
-        for (int k = 0; k < 8; k++) a += (uint64_t)x[k].x + x[k].y + x[k].z + x[k].w;
+    const uint64_t wave = ((uint64_t)blockIdx.x * blockDim.x + threadIdx.x) / BAM_WAVE_SIZE, lane = threadIdx.x % BAM_WAVE_SIZE;
+    const uint64_t n_waves = (uint64_t)gridDim.x * blockDim.x / BAM_WAVE_SIZE;
+    const uint64_t per_wave = (n8 / n_waves) & ~511ull;             /* whole 4 KiB pieces; the rest goes to the last wave */
+    const uint64_t* p = src + wave * per_wave;
+    const uint64_t mine = wave + 1 == n_waves ? n8 - wave * per_wave : per_wave;
+    uint64_t i = 0;
+    for (; i + 512 <= mine; i += 512) {
+        uint64_t x[8];
+        bam::ld_payload_stream8(p + i + lane, x);
+        a += ((x[0] + x[1]) + (x[2] + x[3])) + ((x[4] + x[5]) + (x[6] + x[7]));
     }
-    for (; i < n16; i += stride) { const uint4 x = src[i]; a += (uint64_t)x.x + x.y + x.z + x.w; }
+    for (i += lane; i < mine; i += BAM_WAVE_SIZE) a += p[i];
     block_accumulate(partials, a);
 }
 /* plain random gather of 8-byte words from device memory: the ceiling of that access pattern without any cache protocol */
@@ -2063,7 +2078,8 @@ int bam_read_kernel(const void* d_src, uint64_t n_bytes, float* ms, void* stream
     hipStream_t st = (hipStream_t)stream;
     BufferPtr partials = createBuffer(BAM_SUM_PARTIALS * sizeof(unsigned long long), 0);
     Event a(st);
-    hipLaunchKernelGGL(k_read16, dim3(256 * 16), dim3(256), 0, st, (const uint4*)d_src, n_bytes / 16, (unsigned long long*)partials.get());
+    /* 16 KiB per wave at 1 GiB: many short waves carry more than few long ones here */
+    hipLaunchKernelGGL(k_read_stream, dim3(256 * 64), dim3(256), 0, st, (const uint64_t*)d_src, n_bytes / 8, (unsigned long long*)partials.get());
     hip_err_chk(hipGetLastError());
     Event b(st);
     if (ms) *ms = (float)((b - a) / 1e3);
