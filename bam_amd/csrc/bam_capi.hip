@@ -1551,14 +1551,14 @@ int bam_block_checksum(bam_page_cache_t* pc, uint64_t n_slots, uint32_t req_byte
 namespace {
 /* the pieces of the long edge lists of a graph, listed once per call, and the counter that hands out the work of a sweep:
  * a list of d >= BAM_HEAVY_EDGES entries makes at most d / BAM_PIECE_EDGES + 1 <= 2 d / BAM_HEAVY_EDGES pieces */
-struct heavy_queue {
+struct sweep_work {
     BufferPtr buf, cnt;
     heavy_piece_t* pieces;
     unsigned long long* count;       /* [0] number of pieces, [1] next piece of work of the sweep */
     uint64_t n_pieces = 0;
     uint64_t group;                  /* vertices handed to a wave at a time */
     uint64_t resident;               /* waves the device holds at a time */
-    heavy_queue(uint64_t n_edges, uint64_t n_vertices, uint32_t coarse, const uint64_t* d_offsets, hipStream_t st)
+    sweep_work(uint64_t n_edges, uint64_t n_vertices, uint32_t coarse, const uint64_t* d_offsets, hipStream_t st)
     {
         const uint64_t cap = 2 * (n_edges / BAM_HEAVY_EDGES) + 1;
         buf = createBuffer(cap * sizeof(heavy_piece_t), 0);
@@ -1583,8 +1583,8 @@ struct heavy_queue {
     /* workgroups of two waves for a sweep over `n_items` items in groups of `grp` */
     uint32_t blocks(uint64_t n_items, uint64_t grp) const
     {
-        const uint64_t work = n_pieces + (n_items + grp - 1) / grp;
-        return (uint32_t)(((work < resident ? work : resident) + 1) / 2);
+        const uint64_t units = n_pieces + (n_items + grp - 1) / grp;
+        return (uint32_t)(((units < resident ? units : resident) + 1) / 2);
     }
     void reset(hipStream_t st) { hip_err_chk(hipMemsetAsync(count + 1, 0, sizeof(unsigned long long), st)); }
 };
@@ -1603,15 +1603,15 @@ int bam_bfs(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, 
     hip_err_chk(hipMemsetAsync(d_labels, 0xFF, n_vertices * sizeof(uint32_t), st));
     hip_err_chk(hipMemcpyAsync(d_labels + src, &zero, sizeof(uint32_t), hipMemcpyHostToDevice, st));
     const uint32_t threads = 128;
-    heavy_queue hq(edges->a->adt.n_elems, n_vertices, coarse, d_offsets, st);
+    sweep_work work(edges->a->adt.n_elems, n_vertices, coarse, d_offsets, st);
     uint32_t level = 0, iter = 0;
     uint64_t changed_h;
     do {
         changed_h = 0;
         hip_err_chk(hipMemcpyAsync(changed_d, &changed_h, sizeof(uint64_t), hipMemcpyHostToDevice, st));
-        hq.reset(st);
-        hipLaunchKernelGGL(k_bfs_coalesce_coarse_ptr_pc, dim3(hq.blocks(n_vertices, hq.group)), dim3(threads), 0, st,
-                           edges->a->d_array_ptr, d_labels, level, n_vertices, d_offsets, changed_d, hq.group, hq.pieces, hq.n_pieces, hq.count + 1);
+        work.reset(st);
+        hipLaunchKernelGGL(k_bfs_coalesce_coarse_ptr_pc, dim3(work.blocks(n_vertices, work.group)), dim3(threads), 0, st,
+                           edges->a->d_array_ptr, d_labels, level, n_vertices, d_offsets, changed_d, work.group, work.pieces, work.n_pieces, work.count + 1);
         hip_err_chk(hipGetLastError());
         iter++; level++;
         hip_err_chk(hipMemcpyAsync(&changed_h, changed_d, sizeof(uint64_t), hipMemcpyDeviceToHost, st));
@@ -1641,14 +1641,14 @@ int bam_bfs_frontier(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_v
     hip_err_chk(hipMemcpyAsync(curr, &src32, sizeof(uint32_t), hipMemcpyHostToDevice, st));
     const uint32_t threads = 128;
     const uint64_t group = BAM_WAVE_SIZE;           /* queue entries handed to a wave at a time: one per lane */
-    heavy_queue hq(edges->a->adt.n_elems, n_vertices, 1, d_offsets, st);
+    sweep_work work(edges->a->adt.n_elems, n_vertices, 1, d_offsets, st);
     uint32_t level = 0, iter = 0;
     unsigned long long active = 1;
     do {
         hip_err_chk(hipMemsetAsync(next_size, 0, sizeof(unsigned long long), st));
-        hq.reset(st);
-        hipLaunchKernelGGL(k_bfs_frontier_coalesce_ptr_pc, dim3(hq.blocks(active, group)), dim3(threads), 0, st, edges->a->d_array_ptr, d_labels, level,
-                           d_offsets, curr, (uint64_t)active, next, next_size, group, hq.pieces, hq.n_pieces, hq.count + 1);
+        work.reset(st);
+        hipLaunchKernelGGL(k_bfs_frontier_coalesce_ptr_pc, dim3(work.blocks(active, group)), dim3(threads), 0, st, edges->a->d_array_ptr, d_labels, level,
+                           d_offsets, curr, (uint64_t)active, next, next_size, group, work.pieces, work.n_pieces, work.count + 1);
         hip_err_chk(hipGetLastError());
         std::swap(curr, next);
         iter++; level++;
@@ -1674,15 +1674,15 @@ int bam_cc(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, u
     hip_err_chk(hipMemsetAsync(curr, 0x01, n_vertices, st));
     hip_err_chk(hipMemsetAsync(next, 0x00, n_vertices, st));
     const uint32_t threads = 128;
-    heavy_queue hq(edges->a->adt.n_elems, n_vertices, coarse, d_offsets, st);
+    sweep_work work(edges->a->adt.n_elems, n_vertices, coarse, d_offsets, st);
     uint32_t iter = 0;
     bool changed_h;
     do {
         changed_h = false;
         hip_err_chk(hipMemcpyAsync(changed_d, &changed_h, sizeof(bool), hipMemcpyHostToDevice, st));
-        hq.reset(st);
-        hipLaunchKernelGGL(k_cc_coalesce_coarse_ptr_pc, dim3(hq.blocks(n_vertices, hq.group)), dim3(threads), 0, st, edges->a->d_array_ptr, curr, next,
-                           n_vertices, d_offsets, (unsigned long long*)d_labels, changed_d, hq.group, hq.pieces, hq.n_pieces, hq.count + 1);
+        work.reset(st);
+        hipLaunchKernelGGL(k_cc_coalesce_coarse_ptr_pc, dim3(work.blocks(n_vertices, work.group)), dim3(threads), 0, st, edges->a->d_array_ptr, curr, next,
+                           n_vertices, d_offsets, (unsigned long long*)d_labels, changed_d, work.group, work.pieces, work.n_pieces, work.count + 1);
         hip_err_chk(hipGetLastError());
         hip_err_chk(hipMemsetAsync(curr, 0x00, n_vertices, st));
         bool* t = curr; curr = next; next = t;
@@ -1861,7 +1861,7 @@ int bam_pagerank(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_verti
     if (by_page)
         if (int rc = plan_by_page(edges, d_offsets, n_vertices, st, pl)) return rc;
     const uint32_t upd_blocks = blocks_for(n_vertices, 256);
-    heavy_queue hq(edges->a->adt.n_elems, n_vertices, 1, d_offsets, st);
+    sweep_work work(edges->a->adt.n_elems, n_vertices, 1, d_offsets, st);
     hipLaunchKernelGGL(k_pr_initialize, dim3(upd_blocks), dim3(256), 0, st, label_d, delta_d, residual_d, d_value, n_vertices, d_offsets, alpha);
     uint32_t iter = 0;
     bool changed_h;
@@ -1874,9 +1874,9 @@ int bam_pagerank(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_verti
                                    (const uint64_t*)pl.first.get(), pl.n_edges, pl.ppw, iter);
             hip_err_chk(hipMemsetAsync(label_d, 0, n_vertices, st));
         } else {
-            hq.reset(st);
-            hipLaunchKernelGGL(k_pr_coalesce_pc, dim3(hq.blocks(n_vertices, hq.group)), dim3(128), 0, st, edges->a->d_array_ptr, label_d, delta_d, residual_d,
-                               n_vertices, d_offsets, hq.group, hq.pieces, hq.n_pieces, hq.count + 1);
+            work.reset(st);
+            hipLaunchKernelGGL(k_pr_coalesce_pc, dim3(work.blocks(n_vertices, work.group)), dim3(128), 0, st, edges->a->d_array_ptr, label_d, delta_d, residual_d,
+                               n_vertices, d_offsets, work.group, work.pieces, work.n_pieces, work.count + 1);
             hip_err_chk(hipMemsetAsync(label_d, 0, n_vertices, st));
         }
         iter++;
@@ -1976,15 +1976,15 @@ void sssp_run(const bool FLOAT, bam_array_t* edges, bam_array32_t* weights, cons
     hip_err_chk(hipMemcpyAsync(d_costs + src, &zero, sizeof(uint32_t), hipMemcpyHostToDevice, st));
     hip_err_chk(hipMemcpyAsync(new_d + src, &zero, sizeof(uint32_t), hipMemcpyHostToDevice, st));
     const uint32_t threads = 128;
-    heavy_queue hq(edges->a->adt.n_elems, n_vertices, 1, d_offsets, st);
+    sweep_work work(edges->a->adt.n_elems, n_vertices, 1, d_offsets, st);
     uint32_t iter = 0;
     bool changed_h;
     do {
         changed_h = false;
         hip_err_chk(hipMemcpyAsync(changed_d, &changed_h, sizeof(bool), hipMemcpyHostToDevice, st));
-        hq.reset(st);
-        hipLaunchKernelGGL(FLOAT ? k_sssp_coalesce_pc<true> : k_sssp_coalesce_pc<false>, dim3(hq.blocks(n_vertices, hq.group)), dim3(threads), 0, st,
-                           edges->a->d_array_ptr, weights->a->d_array_ptr, label_d, new_d, n_vertices, d_offsets, hq.group, hq.pieces, hq.n_pieces, hq.count + 1);
+        work.reset(st);
+        hipLaunchKernelGGL(FLOAT ? k_sssp_coalesce_pc<true> : k_sssp_coalesce_pc<false>, dim3(work.blocks(n_vertices, work.group)), dim3(threads), 0, st,
+                           edges->a->d_array_ptr, weights->a->d_array_ptr, label_d, new_d, n_vertices, d_offsets, work.group, work.pieces, work.n_pieces, work.count + 1);
         hip_err_chk(hipMemsetAsync(label_d, 0, n_vertices, st));
         hipLaunchKernelGGL(k_sssp_update, dim3(blocks_for(n_vertices, 256)), dim3(256), 0, st, label_d, d_costs, new_d, n_vertices, changed_d);
         hip_err_chk(hipGetLastError());
