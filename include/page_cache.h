@@ -105,7 +105,8 @@ struct page_cache_d_t {
     cache_page_t* cache_pages;
     uint32_t* page_ticket;
     uint64_t* prp1;                  /* [n_pages] bus address of each slot (direct transfers) */
-    uint32_t direct_share;           /* with staging available: of every 8 read batches, this many go direct all the same */
+    uint32_t direct_share;           /* with staging available: of every 8 read batches of the cache's miss path, this many go direct all the same */
+    uint32_t direct_share_raw;       /* the same for reads through read_data / access_data (raw block I/O into slots the caller names) */
     uint64_t* prp2;                  /* [n_pages] second page or PRP list when page_size > controller page */
     uint64_t ctrl_page_size;
     uint64_t range_cap;
@@ -202,7 +203,7 @@ __device__ __forceinline__ void copy_pages_helped(uint8_t* dst, const uint8_t* s
  * itself) and `pos` the submission-queue slot its entry went to.
  */
 __device__ __forceinline__ uint32_t io_submit_group(page_cache_d_t* pc, QueuePair* qp, uint64_t lba, uint32_t n_blocks, uint64_t pc_entry, uint8_t opcode,
-                                                    uint8_t*& stage, uint32_t& pos)
+                                                    uint8_t*& stage, uint32_t& pos, const uint32_t direct_share)
 {
     const uint64_t act = active_mask();
     const uint32_t n = popc(act), rank = rank_in(act);
@@ -225,9 +226,12 @@ __device__ __forceinline__ uint32_t io_submit_group(page_cache_d_t* pc, QueuePai
      * controller (writes into device memory): the two use opposite directions of the interconnect, so sending a
      * share of the read batches each way carries more than either alone.  Small reads stay staged: pushed in
      * pieces of a few hundred bytes they cost the controller more than they save.  Transfers larger than a staging
-     * page (cache pages above two controller pages) always go direct, through their PRP lists.
+     * page (cache pages above two controller pages) always go direct, through their PRP lists.  The share differs
+     * by caller: the cache's miss path has the waves busy with the page states as well and gains from handing three
+     * batches of eight to the controller (12.3 against 11.4 M reads/s), raw block reads do best all staged (12.8
+     * against 11.7 M).
      */
-    const bool direct = pc->prp1 && (bytes > qp->stage_stride || (opcode == NVM_IO_READ && bytes >= 2048 && ((cid >> 6) & 7u) < pc->direct_share));
+    const bool direct = pc->prp1 && (bytes > qp->stage_stride || (opcode == NVM_IO_READ && bytes >= 2048 && ((cid >> 6) & 7u) < direct_share));
     const bool staged = qp->stage && !direct;
     if (staged) {
         stage = qp->stage + (size_t)cid * qp->stage_stride;
@@ -259,12 +263,13 @@ __device__ __forceinline__ uint32_t io_submit_group(page_cache_d_t* pc, QueuePai
 }
 
 /* the whole of one batch: submit, wait for all completions, move staged payload, recycle ids */
-__device__ __forceinline__ void io_group(page_cache_d_t* pc, QueuePair* qp, uint64_t lba, uint32_t n_blocks, uint64_t pc_entry, uint8_t opcode)
+__device__ __forceinline__ void io_group(page_cache_d_t* pc, QueuePair* qp, uint64_t lba, uint32_t n_blocks, uint64_t pc_entry, uint8_t opcode,
+                                         const uint32_t direct_share)
 {
     const uint64_t act = active_mask();
     uint8_t* stage;
     uint32_t pos;
-    const uint32_t cid = io_submit_group(pc, qp, lba, n_blocks, pc_entry, opcode, stage, pos);
+    const uint32_t cid = io_submit_group(pc, qp, lba, n_blocks, pc_entry, opcode, stage, pos, direct_share);
 #ifdef BAM_PROFILE
     const uint64_t pt2 = wall_clock64();
 #endif
@@ -285,7 +290,7 @@ __device__ __forceinline__ void io_group(page_cache_d_t* pc, QueuePair* qp, uint
 inline __device__ void access_data(page_cache_d_t* pc, QueuePair* qp, const uint64_t starting_lba, const uint64_t n_blocks, const unsigned long long pc_entry, const uint8_t opcode)
 {
     bam::for_each_group((uint64_t)qp, (uint64_t)pc, [&](uint64_t q, uint64_t c) {
-        bam::io_group((page_cache_d_t*)c, (QueuePair*)q, starting_lba, (uint32_t)n_blocks, pc_entry, opcode);
+        bam::io_group((page_cache_d_t*)c, (QueuePair*)q, starting_lba, (uint32_t)n_blocks, pc_entry, opcode, ((page_cache_d_t*)c)->direct_share_raw);
     });
 }
 
@@ -306,14 +311,14 @@ inline __device__ void read_begin(page_cache_d_t* pc, QueuePair* qp, const uint6
     cid = 0;
     if (!one_group) {
         bam::for_each_group((uint64_t)qp, (uint64_t)pc, [&](uint64_t q, uint64_t c) {
-            bam::io_group((page_cache_d_t*)c, (QueuePair*)q, starting_lba, (uint32_t)n_blocks, pc_entry, NVM_IO_READ);
+            bam::io_group((page_cache_d_t*)c, (QueuePair*)q, starting_lba, (uint32_t)n_blocks, pc_entry, NVM_IO_READ, ((page_cache_d_t*)c)->direct_share);
         });
         return;
     }
     QueuePair* cur = (QueuePair*)bam::first((uint64_t)qp);
     page_cache_d_t* cpc = (page_cache_d_t*)bam::first((uint64_t)pc);
     uint32_t pos;
-    cid = bam::io_submit_group(cpc, cur, starting_lba, (uint32_t)n_blocks, pc_entry, NVM_IO_READ, stage, pos);
+    cid = bam::io_submit_group(cpc, cur, starting_lba, (uint32_t)n_blocks, pc_entry, NVM_IO_READ, stage, pos, cpc->direct_share);
 #ifdef BAM_PROFILE
     const uint64_t pt2 = wall_clock64();
 #endif
@@ -352,7 +357,7 @@ inline __device__ void access_data_async(page_cache_d_t* pc, QueuePair* qp, cons
         page_cache_d_t* cpc = (page_cache_d_t*)c;
         uint8_t* stage;
         uint32_t pos;
-        const uint32_t id = bam::io_submit_group(cpc, cur, starting_lba, (uint32_t)n_blocks, pc_entry, opcode, stage, pos);
+        const uint32_t id = bam::io_submit_group(cpc, cur, starting_lba, (uint32_t)n_blocks, pc_entry, opcode, stage, pos, cpc->direct_share_raw);
         if (stage) {
             cur->async_dst[id] = opcode == NVM_IO_READ ? (uint64_t)(cpc->base_addr + pc_entry * cpc->page_size) : 0;
             cur->async_len[id] = (uint32_t)n_blocks << cur->block_size_log;
@@ -1554,8 +1559,10 @@ struct page_cache_t {
         const uint64_t cache_size = ps * np;
         pdt.direct_share = 3;        /* measured best on the random-gather workload: 12.1M 4 KiB reads/s against 11.4M all staged, 10.4M all direct */
         if (const char* e = getenv("BAM_DIRECT_SHARE")) pdt.direct_share = (uint32_t)atoi(e);
-        if (!staged) pdt.direct_share = 0;
-        if (staged && ps > ctrl.h_qps[0]->stage_stride) pdt.direct_share = 8;      /* pages that do not fit a staging page: all direct */
+        pdt.direct_share_raw = 0;    /* raw 4 KiB block reads: 12.8 M/s all staged, 11.7 M with three of eight direct, 10.4 M all direct */
+        if (const char* e = getenv("BAM_DIRECT_SHARE_RAW")) pdt.direct_share_raw = (uint32_t)atoi(e);
+        if (!staged) pdt.direct_share = pdt.direct_share_raw = 0;
+        if (staged && ps > ctrl.h_qps[0]->stage_stride) pdt.direct_share = pdt.direct_share_raw = 8;      /* pages that do not fit a staging page: all direct */
         if (staged && pdt.direct_share == 0) {
             /* the controller never addresses the cache: plain device memory, no PRP tables */
             pages_buf = createBuffer(cache_size, hipDevice);

@@ -340,9 +340,13 @@ def test_wave_memcpy_out_of_the_cache(bam):
 
 # ---------------------------------------------------------------- raw block
 
-@pytest.mark.parametrize("req,lba,order", [(4096, 512, 0), (512, 512, 2), (4096, 4096, 1)])
-def test_block_reads_payload_checksums(bam, req, lba, order):
+@pytest.mark.parametrize("req,lba,order,raw_share", [(4096, 512, 0, None), (4096, 512, 0, "3"), (4096, 512, 0, "8"), (512, 512, 2, None), (4096, 4096, 1, None)])
+def test_block_reads_payload_checksums(bam, req, lba, order, raw_share, monkeypatch):
+    """raw reads into slots the caller names; by default all of them staged, with BAM_DIRECT_SHARE_RAW three of eight
+    batches or all of them placed by the target"""
     from bam_amd import gen
+    if raw_share is not None:
+        monkeypatch.setenv("BAM_DIRECT_SHARE_RAW", raw_share)
     n, ns = 1 << 16, 64 << 30
     with Rig(bam, ns, lba=lba, n_queues=16, depth=256, order=order) as r:
         pc = bam.PageCache(4096, n, 0, r.c)
