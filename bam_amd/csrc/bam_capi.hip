@@ -390,15 +390,18 @@ struct list_read_ahead {
      * dozen edges per vertex.  False if the span is too wide for that (the caller then touches list by list).
      */
     template <typename Item>
-    __device__ __forceinline__ bool span(const uint64_t* vertexList, const uint64_t first, const uint64_t last, const uint64_t heavy_from, Item item)
+    __device__ __forceinline__ bool span(const uint64_t* vertexList, const uint64_t first, const uint64_t last, const uint64_t heavy_from, Item item,
+                                         bool& nothing)
     {
+        nothing = false;
         if (reach < 2) return false;
         const uint64_t e0 = vertexList[first], e1 = vertexList[last];
-        if (e1 <= e0) return true;
+        if (e1 <= e0) { nothing = true; return true; }
         const uint64_t p0 = view.page_of(e0), p1 = view.page_of(e1 - 1);
         if (p1 - p0 >= 4ull * reach) return false;
         auto touch = [](uint32_t) { return true; };
         const uint32_t lane = bam::lane();
+        uint64_t seen = 0;
         for (uint64_t c = p0; c <= p1; c += reach) {
             uint64_t m = 0;
             for (uint64_t b = first; b < last; b += BAM_WAVE_SIZE) {
@@ -415,8 +418,10 @@ struct list_read_ahead {
 #pragma unroll
             for (uint32_t o = BAM_WAVE_SIZE / 2; o; o >>= 1) m |= bam::shfl(m, lane ^ o);
             if (m) view.acquire_helped(c + lane, ((m >> lane) & 1) != 0, false, touch, touch);
+            seen |= m;
         }
         view.n_access = view.n_hit = 0;
+        nothing = seen == 0;            /* no list to walk in [first, last): the caller need not look again */
         return true;
     }
     /* wave-uniform: the list is elements [start, end) */
@@ -500,6 +505,7 @@ __device__ __forceinline__ void walk_packed(const uint64_t es, const uint64_t ee
  * of the threshold's size reach the store as batches of two or three commands, and the store path moves far fewer
  * pages per second in such batches than in batches of sixteen */
 #define BAM_PIECE_EDGES 8192u
+#define BAM_PIECE_BUNDLE 4u             /* pieces handed to a wave at a time */
 struct heavy_piece_t { uint64_t v, first, last; };      /* entries [first, last) of the list of vertex v */
 
 __global__ void k_heavy_pieces(const uint64_t* vertexList, const uint64_t vertex_count, heavy_piece_t* pieces, unsigned long long* count)
@@ -558,6 +564,7 @@ __device__ __forceinline__ void walk_item_groups(array_d_t<uint64_t>* da, const 
 {
     const uint64_t laneIdx = threadIdx.x % BAM_WAVE_SIZE;
     const uint64_t n_groups = (n_items + coarse - 1) / coarse;
+    const uint64_t n_bundles = (n_heavy + BAM_PIECE_BUNDLE - 1) / BAM_PIECE_BUNDLE;
     bam_ptr<uint64_t> ptr(da);
     touch_reader<uint64_t> touch;
     if (!HOLD) touch.init(da);
@@ -567,25 +574,30 @@ __device__ __forceinline__ void walk_item_groups(array_d_t<uint64_t>* da, const 
         unsigned long long w = 0;
         if (laneIdx == 0) w = atomicAdd(next_work, 1ull);
         w = bam::bcast((uint64_t)w, 0);
-        if (w < n_heavy) {
-            /* a piece of a long list, all lanes side by side through bam_ptr, read ahead over the piece */
-            const heavy_piece_t pc = heavy[w];
-            if (!active(pc.v)) continue;
-            if (!ready) { ahead.init(da); ready = true; }
-            ahead.begin(pc.first, pc.last);
-            for (uint64_t i = (pc.first & 0xFFFFFFFFFFFFFFF0ull) + laneIdx; i < pc.last; i += BAM_WAVE_SIZE) {
-                ahead.step(i - laneIdx > pc.first ? i - laneIdx : pc.first);
-                if (i >= pc.first) visit(pc.v, ptr.read(i), i);
+        if (w < n_bundles) {
+            /* pieces of long lists, BAM_PIECE_BUNDLE per turn at the counter (every turn costs one atomic on one word, and on
+             * a sweep with little to do those atomics are what the sweep takes): all lanes side by side through bam_ptr,
+             * read ahead over the piece */
+            for (uint64_t k = w * BAM_PIECE_BUNDLE; k < (w + 1) * BAM_PIECE_BUNDLE && k < n_heavy; k++) {
+                const heavy_piece_t pc = heavy[k];
+                if (!active(pc.v)) continue;
+                if (!ready) { ahead.init(da); ready = true; }
+                ahead.begin(pc.first, pc.last);
+                for (uint64_t i = (pc.first & 0xFFFFFFFFFFFFFFF0ull) + laneIdx; i < pc.last; i += BAM_WAVE_SIZE) {
+                    ahead.step(i - laneIdx > pc.first ? i - laneIdx : pc.first);
+                    if (i >= pc.first) visit(pc.v, ptr.read(i), i);
+                }
             }
             continue;
         }
-        const uint64_t g = w - n_heavy;
+        const uint64_t g = w - n_bundles;
         if (g >= n_groups) break;
         const uint64_t first = g * coarse;
-        bool touched = false;
+        bool touched = false, nothing = false;
         if constexpr (HOLD) {
             if (!ready) { ahead.init(da); ready = true; }
-            touched = ahead.span(vertexList, first, first + coarse < n_items ? first + coarse : n_items, BAM_HEAVY_EDGES, item);
+            touched = ahead.span(vertexList, first, first + coarse < n_items ? first + coarse : n_items, BAM_HEAVY_EDGES, item, nothing);
+            if (nothing) continue;
         }
         for (uint64_t b = 0; b < coarse; b += BAM_WAVE_SIZE) {
             const uint64_t at_item = first + b + laneIdx;
@@ -601,7 +613,8 @@ __device__ __forceinline__ void walk_item_groups(array_d_t<uint64_t>* da, const 
                 bool block_touched = false;
                 if constexpr (HOLD) {
                     const uint64_t last = first + coarse < n_items ? first + coarse : n_items;
-                    block_touched = ahead.span(vertexList, first + b, first + b + BAM_WAVE_SIZE < last ? first + b + BAM_WAVE_SIZE : last, BAM_HEAVY_EDGES, item);
+                    bool none;
+                    block_touched = ahead.span(vertexList, first + b, first + b + BAM_WAVE_SIZE < last ? first + b + BAM_WAVE_SIZE : last, BAM_HEAVY_EDGES, item, none);
                 }
                 if (!block_touched) ahead.group(es, ee);
             }
@@ -1583,7 +1596,7 @@ struct sweep_work {
     /* workgroups of two waves for a sweep over `n_items` items in groups of `grp` */
     uint32_t blocks(uint64_t n_items, uint64_t grp) const
     {
-        const uint64_t units = n_pieces + (n_items + grp - 1) / grp;
+        const uint64_t units = (n_pieces + BAM_PIECE_BUNDLE - 1) / BAM_PIECE_BUNDLE + (n_items + grp - 1) / grp;
         return (uint32_t)(((units < resident ? units : resident) + 1) / 2);
     }
     void reset(hipStream_t st) { hip_err_chk(hipMemsetAsync(count + 1, 0, sizeof(unsigned long long), st)); }
