@@ -424,14 +424,27 @@ struct list_read_ahead {
         nothing = seen == 0;            /* no list to walk in [first, last): the caller need not look again */
         return true;
     }
-    /* wave-uniform: the list is elements [start, end) */
-    __device__ __forceinline__ void begin(const uint64_t start, const uint64_t end)
+    /* wave-uniform: the list is elements [start, end); its first `asked` pages have been touched already */
+    __device__ __forceinline__ void begin(const uint64_t start, const uint64_t end, const uint32_t asked = 0)
     {
         long_list = false;
         if (reach < 2 || end <= start) return;
         last_page = view.page_of(end - 1);
         long_list = last_page > view.page_of(start);
-        asked_to = 0;
+        asked_to = asked ? view.page_of(start) + asked : 0;
+    }
+    /* lane l brings page (l mod 16) of a run of elements [start, end) of its own (four runs per wave, `want` says whether
+     * the lane's run is to be read at all): one batch of commands for what is not resident of the first sixteen pages of
+     * each.  False if the cache is too small for a wave to ask for that much at a time. */
+    __device__ __forceinline__ bool quads(const uint64_t start, const uint64_t end, const bool want)
+    {
+        if (reach < BAM_WAVE_SIZE) return false;
+        auto touch = [](uint32_t) { return true; };
+        const uint64_t page = want ? view.page_of(start) + (bam::lane() & 15u) : 0;
+        const bool take = want && end > start && page <= view.page_of(end - 1);
+        if (bam::ballot(take)) view.acquire_helped(page, take, false, touch, touch);
+        view.n_access = view.n_hit = 0;
+        return true;
     }
     /* wave-uniform: the walk is about to read from element `at` on */
     __device__ __forceinline__ void step(const uint64_t at)
@@ -505,7 +518,8 @@ __device__ __forceinline__ void walk_packed(const uint64_t es, const uint64_t ee
  * of the threshold's size reach the store as batches of two or three commands, and the store path moves far fewer
  * pages per second in such batches than in batches of sixteen */
 #define BAM_PIECE_EDGES 8192u
-#define BAM_PIECE_BUNDLE 4u             /* pieces handed to a wave at a time */
+#define BAM_PIECE_BUNDLE 4u             /* pieces handed to a wave at a time: sixteen lanes look after the sixteen pages of each */
+static_assert(BAM_PIECE_BUNDLE * 16u == BAM_WAVE_SIZE && BAM_PIECE_EDGES * 8u == 16u * 4096u, "a bundle's pages are shared out one per lane");
 struct heavy_piece_t { uint64_t v, first, last; };      /* entries [first, last) of the list of vertex v */
 
 __global__ void k_heavy_pieces(const uint64_t* vertexList, const uint64_t vertex_count, heavy_piece_t* pieces, unsigned long long* count)
@@ -578,11 +592,24 @@ __device__ __forceinline__ void walk_item_groups(array_d_t<uint64_t>* da, const 
             /* pieces of long lists, BAM_PIECE_BUNDLE per turn at the counter (every turn costs one atomic on one word, and on
              * a sweep with little to do those atomics are what the sweep takes): all lanes side by side through bam_ptr,
              * read ahead over the piece */
+            /* what the active pieces of the bundle need comes in as one batch: a piece by itself asks for six pages on
+             * average on a power-law graph, where most long lists are just over the threshold */
+            bool asked = false;
+            {
+                const uint64_t k = w * BAM_PIECE_BUNDLE + laneIdx / 16;
+                heavy_piece_t mine = {0, 0, 0};
+                bool want = false;
+                if (k < n_heavy) { mine = heavy[k]; want = active(mine.v); }
+                if (bam::ballot(want)) {
+                    if (!ready) { ahead.init(da); ready = true; }
+                    asked = ahead.quads(mine.first, mine.last, want);
+                }
+            }
             for (uint64_t k = w * BAM_PIECE_BUNDLE; k < (w + 1) * BAM_PIECE_BUNDLE && k < n_heavy; k++) {
                 const heavy_piece_t pc = heavy[k];
                 if (!active(pc.v)) continue;
                 if (!ready) { ahead.init(da); ready = true; }
-                ahead.begin(pc.first, pc.last);
+                ahead.begin(pc.first, pc.last, asked ? 16u : 0u);
                 for (uint64_t i = (pc.first & 0xFFFFFFFFFFFFFFF0ull) + laneIdx; i < pc.last; i += BAM_WAVE_SIZE) {
                     ahead.step(i - laneIdx > pc.first ? i - laneIdx : pc.first);
                     if (i >= pc.first) visit(pc.v, ptr.read(i), i);
