@@ -134,8 +134,8 @@ int bam_block_checksum(bam_page_cache_t* pc, uint64_t n_slots, uint32_t req_byte
  * touches the pages that hold the lists of its group's active vertices (what is not resident comes in as one batch of
  * commands), then reads the lists of 64 vertices at a time through bam_ptr, 64 entries per step across list ends.
  * Lists of 1024 entries and more are walked in pieces of 8192 entries by a wave each; the pieces are listed once per
- * call and handed out in every sweep before the groups (the same for bam_cc, bam_sssp and bam_pagerank without
- * by_page). */
+ * call and handed out in every sweep before the groups, four per turn, their pages asked for as one batch (the same
+ * for bam_cc, bam_sssp and bam_pagerank without by_page). */
 int bam_bfs(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t src, uint32_t* d_labels,
             uint32_t coarse, uint32_t* iterations, void* stream);
 /* ---- BFS over queues of vertices (benchmarks/bfs/main.cu:409-451 kernel_frontier_coalesce_ptr_pc, queues :1489-1492,
