@@ -829,6 +829,39 @@ __global__ __launch_bounds__(64) void k_cc_by_page(array_d_t<uint64_t>* da, bool
                   [&](uint64_t src, uint64_t next, uint64_t) { cc_compute(src, comp, next, next_visit, changed); });
 }
 
+/*
+ * Read-ahead for kernels in which consecutive threads read consecutive elements (one element or two per thread, as in
+ * benchmarks/vectoradd, reduction and scan).  Left to themselves such kernels ask the store for one page per wave
+ * and trip, and the store path takes about a million such batches per second whatever their size: 1 GiB comes in
+ * at 5 GB/s.  Here the wave that reads the first element of a window of W pages (W = a 64th of the cache, at most
+ * 64) touches the W pages that lie up to 32 windows further on, one page per lane, taken and dropped again: they come
+ * in as one batch of W commands, before the waves that read them are started (workgroups start in order, and the
+ * device holds a few thousand waves, that is up to a thousand pages, at a time).  The first windows are touched by
+ * their own first waves.  `first` is the index of the wave's first element (wave-uniform).
+ */
+template <typename T>
+__device__ __forceinline__ void touch_ahead(array_d_t<T>* da, const uint64_t first, const uint64_t n_elems)
+{
+    if (da->n_ranges != 1) return;
+    const page_cache_d_t& cache = da->d_ranges[0].cache;
+    const uint64_t w_pages = cache.n_pages >> 6 > BAM_WAVE_SIZE ? BAM_WAVE_SIZE : cache.n_pages >> 6;
+    if (w_pages < 2) return;
+    const uint64_t epp = cache.page_size / sizeof(T), w_elems = w_pages * epp;
+    if (first % w_elems) return;
+    /* how far ahead: beyond what the waves in flight cover (a few thousand waves at one page per four to eight waves), within a
+     * quarter of the cache */
+    uint64_t dist = (cache.n_pages / 4) / w_pages;
+    dist = (dist > 32 ? 32 : dist < 1 ? 1 : dist) * w_elems;
+    bam::range_view<T> view;
+    view.load(da->d_ranges);
+    auto touch = [](uint32_t) { return true; };
+    const uint64_t mine = first + bam::lane() * epp;
+    if (first < dist) view.acquire_helped(view.page_of(mine < n_elems ? mine : first), bam::lane() < w_pages && mine < n_elems, false, touch, touch);
+    const uint64_t ahead = mine + dist;
+    if (first + dist < n_elems) view.acquire_helped(view.page_of(ahead < n_elems ? ahead : first), bam::lane() < w_pages && ahead < n_elems, false, touch, touch);
+    view.n_access = view.n_hit = 0;
+}
+
 // ---- vectoradd (benchmarks/vectoradd/main.cu:102-117 kernel_baseline_ptr_pc): C[i] = A[i] + B[i], all three behind the cache ----
 __global__ __launch_bounds__(64) void k_vectoradd_ptr_pc(array_d_t<uint64_t>* da, array_d_t<uint64_t>* db, uint64_t n_elems, array_d_t<uint64_t>* dc)
 {
@@ -838,6 +871,12 @@ __global__ __launch_bounds__(64) void k_vectoradd_ptr_pc(array_d_t<uint64_t>* da
     bam_ptr<uint64_t> Cptr(dc);
     const bam_ptr<uint64_t>& A = Aptr;
     const bam_ptr<uint64_t>& B = Bptr;
+    const uint64_t first = tid - threadIdx.x % BAM_WAVE_SIZE;
+    if (first < n_elems) {
+        touch_ahead(da, first, n_elems);
+        touch_ahead(db, first, n_elems);
+        touch_ahead(dc, first, n_elems);
+    }
     if (tid < n_elems) Cptr[tid] = A[tid] + B[tid];
 }
 
@@ -850,6 +889,10 @@ __global__ void k_reduce_ptr_pc(array_d_t<uint64_t>* da, unsigned long long* out
     {
         bam_ptr<uint64_t> in_ptr(da);
         const bam_ptr<uint64_t>& input = in_ptr;
+        /* a workgroup reads 2 x blockDim consecutive elements: its waves' first elements */
+        const uint64_t first = start + tid - tid % BAM_WAVE_SIZE;
+        if (first < len) touch_ahead(da, first, len);
+        if (first + blockDim.x < len) touch_ahead(da, first + blockDim.x, len);
         if (start + tid < len) v = input[start + tid];
         if (blockDim.x + start + tid < len) v += input[blockDim.x + start + tid];
     }
@@ -890,6 +933,9 @@ __global__ void k_scan_ptr_pc(array_d_t<uint64_t>* da, unsigned long long* outpu
     {
         bam_ptr<uint64_t> in_ptr(da);
         const bam_ptr<uint64_t>& ptr = in_ptr;
+        const uint64_t first = idx - t % BAM_WAVE_SIZE;
+        if (first < len) touch_ahead(da, first, len);
+        if (first + B < len) touch_ahead(da, first + B, len);
         scan_mem[t] = idx < len ? ptr[idx] : 0;
         scan_mem[t + B] = idx + B < len ? ptr[idx + B] : 0;
     }
