@@ -848,9 +848,9 @@ __device__ __forceinline__ void touch_ahead(array_d_t<T>* da, const uint64_t fir
     if (w_pages < 2) return;
     const uint64_t epp = cache.page_size / sizeof(T), w_elems = w_pages * epp;
     if (first % w_elems) return;
-    /* how far ahead: beyond what the waves in flight cover (a few thousand waves at one page per four to eight waves), within a
-     * quarter of the cache */
-    uint64_t dist = (cache.n_pages / 4) / w_pages;
+    /* how far ahead: beyond what the waves in flight cover (a few thousand waves at one page per four to eight waves), within an
+     * eighth of the cache (a kernel may walk several arrays behind one cache at a time) */
+    uint64_t dist = (cache.n_pages / 8) / w_pages;
     dist = (dist > 32 ? 32 : dist < 1 ? 1 : dist) * w_elems;
     bam::range_view<T> view;
     view.load(da->d_ranges);
