@@ -478,6 +478,9 @@ def test_reduction_and_scan_through_bam_ptr(bam, n, block, cache_pages):
         r.backing(n + pad)[:n] = vals
         a = r.array(n, 4096, cache_pages)
         assert np.array_equal(_u64(a.reduce(n, block)), oracle.reduce_blocks(vals, block))
+        if cache_pages >= (n + pad) // 512:
+            # the read-ahead of these kernels touches pages before their readers come: every page still comes in once
+            assert a.stats(reset=False)["read_io_cnt"] == (n + pad) // 512
         assert np.array_equal(_u64(a.scan(n, block)), oracle.scan(vals))
         # a prefix of the array only: the tail must not leak in
         m = n - n // 3
