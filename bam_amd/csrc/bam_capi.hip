@@ -574,7 +574,7 @@ struct touch_reader {
 template <bool HOLD, typename Item, typename Active, typename Visit>
 __device__ __forceinline__ void walk_item_groups(array_d_t<uint64_t>* da, const uint64_t* vertexList, const uint64_t n_items, const uint64_t coarse,
                                                  const heavy_piece_t* heavy, const uint64_t n_heavy, unsigned long long* next_work,
-                                                 Item item, Active active, Visit visit)
+                                                 const bool backwards, Item item, Active active, Visit visit)
 {
     const uint64_t laneIdx = threadIdx.x % BAM_WAVE_SIZE;
     const uint64_t n_groups = (n_items + coarse - 1) / coarse;
@@ -588,6 +588,9 @@ __device__ __forceinline__ void walk_item_groups(array_d_t<uint64_t>* da, const 
         unsigned long long w = 0;
         if (laneIdx == 0) w = atomicAdd(next_work, 1ull);
         w = bam::bcast((uint64_t)w, 0);
+        /* every other sweep runs from the far end of both lists of work: what the last sweep left in the cache is what
+         * this one asks for first */
+        const uint64_t wb = backwards ? n_bundles - 1 - w : w;
         if (w < n_bundles) {
             /* pieces of long lists, BAM_PIECE_BUNDLE per turn at the counter (every turn costs one atomic on one word, and on
              * a sweep with little to do those atomics are what the sweep takes): all lanes side by side through bam_ptr,
@@ -596,7 +599,7 @@ __device__ __forceinline__ void walk_item_groups(array_d_t<uint64_t>* da, const 
              * average on a power-law graph, where most long lists are just over the threshold */
             bool asked = false;
             {
-                const uint64_t k = w * BAM_PIECE_BUNDLE + laneIdx / 16;
+                const uint64_t k = wb * BAM_PIECE_BUNDLE + laneIdx / 16;
                 heavy_piece_t mine = {0, 0, 0};
                 bool want = false;
                 if (k < n_heavy) { mine = heavy[k]; want = active(mine.v); }
@@ -605,7 +608,7 @@ __device__ __forceinline__ void walk_item_groups(array_d_t<uint64_t>* da, const 
                     asked = ahead.quads(mine.first, mine.last, want);
                 }
             }
-            for (uint64_t k = w * BAM_PIECE_BUNDLE; k < (w + 1) * BAM_PIECE_BUNDLE && k < n_heavy; k++) {
+            for (uint64_t k = wb * BAM_PIECE_BUNDLE; k < (wb + 1) * BAM_PIECE_BUNDLE && k < n_heavy; k++) {
                 const heavy_piece_t pc = heavy[k];
                 if (!active(pc.v)) continue;
                 if (!ready) { ahead.init(da); ready = true; }
@@ -617,8 +620,8 @@ __device__ __forceinline__ void walk_item_groups(array_d_t<uint64_t>* da, const 
             }
             continue;
         }
-        const uint64_t g = w - n_bundles;
-        if (g >= n_groups) break;
+        if (w - n_bundles >= n_groups) break;
+        const uint64_t g = backwards ? n_groups - 1 - (w - n_bundles) : w - n_bundles;
         const uint64_t first = g * coarse;
         bool touched = false, nothing = false;
         if constexpr (HOLD) {
@@ -654,9 +657,10 @@ __device__ __forceinline__ void walk_item_groups(array_d_t<uint64_t>* da, const 
 /* the items are the vertices themselves, walked where active(v) */
 template <typename Active, typename Visit>
 __device__ __forceinline__ void walk_vertex_groups(array_d_t<uint64_t>* da, const uint64_t* vertexList, const uint64_t vertex_count, const uint64_t coarse,
-                                                   const heavy_piece_t* heavy, const uint64_t n_heavy, unsigned long long* next_work, Active active, Visit visit)
+                                                   const heavy_piece_t* heavy, const uint64_t n_heavy, unsigned long long* next_work, const bool backwards,
+                                                   Active active, Visit visit)
 {
-    walk_item_groups<true>(da, vertexList, vertex_count, coarse, heavy, n_heavy, next_work,
+    walk_item_groups<true>(da, vertexList, vertex_count, coarse, heavy, n_heavy, next_work, backwards,
                            [&](uint64_t i, uint64_t& v) { v = i; return active(i); }, active, visit);
 }
 
@@ -665,7 +669,7 @@ __global__ __launch_bounds__(128) void k_bfs_coalesce_coarse_ptr_pc(array_d_t<ui
                                                                    const heavy_piece_t* heavy, uint64_t n_heavy, unsigned long long* next_work)
 {
     bool any = false;
-    walk_vertex_groups(da, vertexList, vertex_count, coarse, heavy, n_heavy, next_work,
+    walk_vertex_groups(da, vertexList, vertex_count, coarse, heavy, n_heavy, next_work, (level & 1u) != 0,
                        [&](uint64_t v) { return label[v] == level; },
                        [&](uint64_t, uint64_t next, uint64_t) { if (label[next] == MYINFINITY) { label[next] = level + 1; any = true; } });
     if (any) *changed = 1;
@@ -691,7 +695,7 @@ __global__ __launch_bounds__(128) void k_bfs_frontier_coalesce_ptr_pc(array_d_t<
                                                                      unsigned long long* next_size, uint64_t group,
                                                                      const heavy_piece_t* heavy, uint64_t n_heavy, unsigned long long* next_work)
 {
-    walk_item_groups<false>(da, vertexList, curr_size, group, heavy, n_heavy, next_work,
+    walk_item_groups<false>(da, vertexList, curr_size, group, heavy, n_heavy, next_work, false,
                             [&](uint64_t i, uint64_t& v) { v = curr_frontier[i]; return true; },
                             [&](uint64_t v) { return label[v] == level; },
                             [&](uint64_t, uint64_t next, uint64_t) { bfs_frontier_visit(label, level, next_frontier, next_size, next); });
@@ -713,9 +717,9 @@ __device__ __forceinline__ void cc_compute(uint64_t cid, unsigned long long* com
 
 __global__ __launch_bounds__(128) void k_cc_coalesce_coarse_ptr_pc(array_d_t<uint64_t>* da, bool* curr_visit, bool* next_visit, uint64_t vertex_count,
                                                                   const uint64_t* vertexList, unsigned long long* comp, bool* changed, uint64_t coarse,
-                                                                  const heavy_piece_t* heavy, uint64_t n_heavy, unsigned long long* next_work)
+                                                                  const heavy_piece_t* heavy, uint64_t n_heavy, unsigned long long* next_work, uint32_t sweep)
 {
-    walk_vertex_groups(da, vertexList, vertex_count, coarse, heavy, n_heavy, next_work,
+    walk_vertex_groups(da, vertexList, vertex_count, coarse, heavy, n_heavy, next_work, (sweep & 1u) != 0,
                        [&](uint64_t v) { return curr_visit[v]; },
                        [&](uint64_t v, uint64_t next, uint64_t) { cc_compute(v, comp, next, next_visit, changed); });
 }
@@ -1001,9 +1005,9 @@ __global__ void k_pr_initialize(bool* label, float* delta, float* residual, floa
  * are cleared by the host loop after the sweep */
 __global__ __launch_bounds__(128) void k_pr_coalesce_pc(array_d_t<uint64_t>* da, const bool* label, const float* delta, float* residual,
                                                         const uint64_t vertex_count, const uint64_t* vertexList, uint64_t group,
-                                                        const heavy_piece_t* heavy, uint64_t n_heavy, unsigned long long* next_work)
+                                                        const heavy_piece_t* heavy, uint64_t n_heavy, unsigned long long* next_work, uint32_t sweep)
 {
-    walk_vertex_groups(da, vertexList, vertex_count, group, heavy, n_heavy, next_work,
+    walk_vertex_groups(da, vertexList, vertex_count, group, heavy, n_heavy, next_work, (sweep & 1u) != 0,
                        [&](uint64_t v) { return label[v]; },
                        [&](uint64_t src, uint64_t next, uint64_t) { unsafeAtomicAdd(&residual[next], delta[src]); });
 }
@@ -1046,10 +1050,10 @@ __device__ __forceinline__ void sssp_relax(uint32_t* newCostList, const bam_ptr<
 template <bool FLOAT>
 __global__ __launch_bounds__(128) void k_sssp_coalesce_pc(array_d_t<uint64_t>* de, array_d_t<uint32_t>* dw, const bool* label, uint32_t* newCostList,
                                                           const uint64_t vertex_count, const uint64_t* vertexList, uint64_t group,
-                                                          const heavy_piece_t* heavy, uint64_t n_heavy, unsigned long long* next_work)
+                                                          const heavy_piece_t* heavy, uint64_t n_heavy, unsigned long long* next_work, uint32_t sweep)
 {
     bam_ptr<uint32_t> wptr(dw);
-    walk_vertex_groups(de, vertexList, vertex_count, group, heavy, n_heavy, next_work,
+    walk_vertex_groups(de, vertexList, vertex_count, group, heavy, n_heavy, next_work, (sweep & 1u) != 0,
                        [&](uint64_t v) { return label[v]; },
                        [&](uint64_t src, uint64_t next, uint64_t i) { sssp_relax<FLOAT>(newCostList, wptr, src, next, i); });
 }
@@ -1768,7 +1772,7 @@ int bam_cc(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, u
         hip_err_chk(hipMemcpyAsync(changed_d, &changed_h, sizeof(bool), hipMemcpyHostToDevice, st));
         work.reset(st);
         hipLaunchKernelGGL(k_cc_coalesce_coarse_ptr_pc, dim3(work.blocks(n_vertices, work.group)), dim3(threads), 0, st, edges->a->d_array_ptr, curr, next,
-                           n_vertices, d_offsets, (unsigned long long*)d_labels, changed_d, work.group, work.pieces, work.n_pieces, work.count + 1);
+                           n_vertices, d_offsets, (unsigned long long*)d_labels, changed_d, work.group, work.pieces, work.n_pieces, work.count + 1, iter);
         hip_err_chk(hipGetLastError());
         hip_err_chk(hipMemsetAsync(curr, 0x00, n_vertices, st));
         bool* t = curr; curr = next; next = t;
@@ -1962,7 +1966,7 @@ int bam_pagerank(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_verti
         } else {
             work.reset(st);
             hipLaunchKernelGGL(k_pr_coalesce_pc, dim3(work.blocks(n_vertices, work.group)), dim3(128), 0, st, edges->a->d_array_ptr, label_d, delta_d, residual_d,
-                               n_vertices, d_offsets, work.group, work.pieces, work.n_pieces, work.count + 1);
+                               n_vertices, d_offsets, work.group, work.pieces, work.n_pieces, work.count + 1, iter);
             hip_err_chk(hipMemsetAsync(label_d, 0, n_vertices, st));
         }
         iter++;
@@ -2070,7 +2074,7 @@ void sssp_run(const bool FLOAT, bam_array_t* edges, bam_array32_t* weights, cons
         hip_err_chk(hipMemcpyAsync(changed_d, &changed_h, sizeof(bool), hipMemcpyHostToDevice, st));
         work.reset(st);
         hipLaunchKernelGGL(FLOAT ? k_sssp_coalesce_pc<true> : k_sssp_coalesce_pc<false>, dim3(work.blocks(n_vertices, work.group)), dim3(threads), 0, st,
-                           edges->a->d_array_ptr, weights->a->d_array_ptr, label_d, new_d, n_vertices, d_offsets, work.group, work.pieces, work.n_pieces, work.count + 1);
+                           edges->a->d_array_ptr, weights->a->d_array_ptr, label_d, new_d, n_vertices, d_offsets, work.group, work.pieces, work.n_pieces, work.count + 1, iter);
         hip_err_chk(hipMemsetAsync(label_d, 0, n_vertices, st));
         hipLaunchKernelGGL(k_sssp_update, dim3(blocks_for(n_vertices, 256)), dim3(256), 0, st, label_d, d_costs, new_d, n_vertices, changed_d);
         hip_err_chk(hipGetLastError());
