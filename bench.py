@@ -341,11 +341,21 @@ def main():
                 break
             ref = new
         assert torch.equal(ref, lb) and not ctrl.aborted(), "CC labels differ from the fixed point"
+        # the reference's per-vertex kernel (edge lists through bam_ptr) on the same graph, starting on what the sweeps above left in the cache
+        a2, b2 = event(), event()
+        L.bam_event_record(a2, stream)
+        lb2, it2 = ac.cc(off, coarse=64)
+        L.bam_event_record(b2, stream)
+        ms2 = elapsed_ms(a2, b2)
+        st2 = ac.stats()
+        assert torch.equal(ref, lb2) and not ctrl.aborted(), "CC labels of the per-vertex kernel differ from the fixed point"
         cc = {"log2_vertices": args.cc_logv, "edges": n_e, "cache_pages": cache_pages, "ms": ms, "iterations": it,
               "GTEPS": it * n_e / ms / 1e6, "read_ios": st["read_io_cnt"], "MIOPS": st["read_io_cnt"] / ms / 1e3,
-              "components": int(torch.unique(lb).numel()), "kernel": "by_page"}
+              "components": int(torch.unique(lb).numel()), "kernel": "by_page",
+              "per_vertex_bam_ptr": {"coarse": 64, "ms": ms2, "iterations": it2, "GTEPS": it2 * n_e / ms2 / 1e6,
+                                     "read_ios": st2["read_io_cnt"], "MIOPS": st2["read_io_cnt"] / ms2 / 1e3}}
         log("[bench] cc: %s" % cc)
-        del src, ref, new, nb, off, lb, store_words
+        del src, ref, new, nb, off, lb, lb2, store_words
         ac.close(); rc_.close(); pcc.close()
 
     ctrl.close(); target.close()
