@@ -574,7 +574,8 @@ struct touch_reader {
 template <bool HOLD, typename Item, typename Active, typename Visit>
 __device__ __forceinline__ void walk_item_groups(array_d_t<uint64_t>* da, const uint64_t* vertexList, const uint64_t n_items, const uint64_t coarse,
                                                  const heavy_piece_t* heavy, const uint64_t n_heavy, unsigned long long* next_work,
-                                                 const bool backwards, Item item, Active active, Visit visit)
+                                                 const bool backwards, Item item, Active active, Visit visit,
+                                                 list_read_ahead<uint32_t>* with = nullptr)
 {
     const uint64_t laneIdx = threadIdx.x % BAM_WAVE_SIZE;
     const uint64_t n_groups = (n_items + coarse - 1) / coarse;
@@ -606,6 +607,7 @@ __device__ __forceinline__ void walk_item_groups(array_d_t<uint64_t>* da, const 
                 if (bam::ballot(want)) {
                     if (!ready) { ahead.init(da); ready = true; }
                     asked = ahead.quads(mine.first, mine.last, want);
+                    if (with) with->quads(mine.first, mine.last, want);
                 }
             }
             for (uint64_t k = wb * BAM_PIECE_BUNDLE; k < (wb + 1) * BAM_PIECE_BUNDLE && k < n_heavy; k++) {
@@ -613,8 +615,10 @@ __device__ __forceinline__ void walk_item_groups(array_d_t<uint64_t>* da, const 
                 if (!active(pc.v)) continue;
                 if (!ready) { ahead.init(da); ready = true; }
                 ahead.begin(pc.first, pc.last, asked ? 16u : 0u);
+                if (with) with->begin(pc.first, pc.last, asked ? 16u : 0u);
                 for (uint64_t i = (pc.first & 0xFFFFFFFFFFFFFFF0ull) + laneIdx; i < pc.last; i += BAM_WAVE_SIZE) {
                     ahead.step(i - laneIdx > pc.first ? i - laneIdx : pc.first);
+                    if (with) with->step(i - laneIdx > pc.first ? i - laneIdx : pc.first);
                     if (i >= pc.first) visit(pc.v, ptr.read(i), i);
                 }
             }
@@ -627,6 +631,7 @@ __device__ __forceinline__ void walk_item_groups(array_d_t<uint64_t>* da, const 
         if constexpr (HOLD) {
             if (!ready) { ahead.init(da); ready = true; }
             touched = ahead.span(vertexList, first, first + coarse < n_items ? first + coarse : n_items, BAM_HEAVY_EDGES, item, nothing);
+            if (with && touched && !nothing) { bool none; with->span(vertexList, first, first + coarse < n_items ? first + coarse : n_items, BAM_HEAVY_EDGES, item, none); }
             if (nothing) continue;
         }
         for (uint64_t b = 0; b < coarse; b += BAM_WAVE_SIZE) {
@@ -645,8 +650,9 @@ __device__ __forceinline__ void walk_item_groups(array_d_t<uint64_t>* da, const 
                     const uint64_t last = first + coarse < n_items ? first + coarse : n_items;
                     bool none;
                     block_touched = ahead.span(vertexList, first + b, first + b + BAM_WAVE_SIZE < last ? first + b + BAM_WAVE_SIZE : last, BAM_HEAVY_EDGES, item, none);
+                    if (with && block_touched) with->span(vertexList, first + b, first + b + BAM_WAVE_SIZE < last ? first + b + BAM_WAVE_SIZE : last, BAM_HEAVY_EDGES, item, none);
                 }
-                if (!block_touched) ahead.group(es, ee);
+                if (!block_touched) { ahead.group(es, ee); if (with) with->group(es, ee); }
             }
             walk_packed(es, ee, mine, [&](uint64_t i) { if constexpr (HOLD) return ptr.read(i); else return touch.read(i); }, visit);
         }
@@ -658,10 +664,10 @@ __device__ __forceinline__ void walk_item_groups(array_d_t<uint64_t>* da, const 
 template <typename Active, typename Visit>
 __device__ __forceinline__ void walk_vertex_groups(array_d_t<uint64_t>* da, const uint64_t* vertexList, const uint64_t vertex_count, const uint64_t coarse,
                                                    const heavy_piece_t* heavy, const uint64_t n_heavy, unsigned long long* next_work, const bool backwards,
-                                                   Active active, Visit visit)
+                                                   Active active, Visit visit, list_read_ahead<uint32_t>* with = nullptr)
 {
     walk_item_groups<true>(da, vertexList, vertex_count, coarse, heavy, n_heavy, next_work, backwards,
-                           [&](uint64_t i, uint64_t& v) { v = i; return active(i); }, active, visit);
+                           [&](uint64_t i, uint64_t& v) { v = i; return active(i); }, active, visit, with);
 }
 
 __global__ __launch_bounds__(128) void k_bfs_coalesce_coarse_ptr_pc(array_d_t<uint64_t>* da, uint32_t* label, const uint32_t level, const uint64_t vertex_count,
@@ -1053,9 +1059,12 @@ __global__ __launch_bounds__(128) void k_sssp_coalesce_pc(array_d_t<uint64_t>* d
                                                           const heavy_piece_t* heavy, uint64_t n_heavy, unsigned long long* next_work, uint32_t sweep)
 {
     bam_ptr<uint32_t> wptr(dw);
+    /* entry i of the weight array belongs to entry i of the edge array: what is touched ahead for the one is touched for the other */
+    list_read_ahead<uint32_t> wahead;
+    wahead.init(dw);
     walk_vertex_groups(de, vertexList, vertex_count, group, heavy, n_heavy, next_work, (sweep & 1u) != 0,
                        [&](uint64_t v) { return label[v]; },
-                       [&](uint64_t src, uint64_t next, uint64_t i) { sssp_relax<FLOAT>(newCostList, wptr, src, next, i); });
+                       [&](uint64_t src, uint64_t next, uint64_t i) { sssp_relax<FLOAT>(newCostList, wptr, src, next, i); }, &wahead);
 }
 
 __global__ void k_sssp_update(bool* label, uint32_t* costList, const uint32_t* newCostList, const uint64_t vertex_count, bool* changed)
