@@ -93,11 +93,50 @@ __global__ void k_fold_partials(unsigned long long* partials, unsigned long long
     if (bam::lane() == 0 && v) atomicAdd(sum, (unsigned long long)v);
 }
 
+/*
+ * Read-ahead for kernels in which consecutive threads read consecutive elements (one element or two per thread, as in
+ * benchmarks/vectoradd, reduction and scan).  Left to themselves such kernels ask the store for one page per wave
+ * and trip, and the store path takes about a million such batches per second whatever their size: 1 GiB comes in
+ * at 5 GB/s.  Here the wave that reads the first element of a window of W pages (W = a 64th of the cache, at most
+ * 64) touches the W pages that lie up to 32 windows further on, one page per lane, taken and dropped again: they come
+ * in as one batch of W commands, before the waves that read them are started (workgroups start in order, and the
+ * device holds a few thousand waves, that is up to a thousand pages, at a time).  The first windows are touched by
+ * their own first waves.  `first` is the index of the wave's first element (wave-uniform), `wave_span` the elements
+ * from one wave's first to the next one's (more than 64 where the threads read with a stride).
+ */
+template <typename T>
+__device__ __forceinline__ void touch_ahead(array_d_t<T>* da, const uint64_t first, const uint64_t n_elems, const uint64_t wave_span = BAM_WAVE_SIZE)
+{
+    if (da->n_ranges != 1) return;
+    const page_cache_d_t& cache = da->d_ranges[0].cache;
+    const uint64_t w_pages = cache.n_pages >> 6 > BAM_WAVE_SIZE ? BAM_WAVE_SIZE : cache.n_pages >> 6;
+    if (w_pages < 2) return;
+    const uint64_t epp = cache.page_size / sizeof(T), w_elems = w_pages * epp;
+    if (first % w_elems >= wave_span) return;           /* not the first wave that begins in its window (`wave_span` elements per wave) */
+    /* how far ahead: beyond what the waves in flight cover (a few thousand waves at one page per four to eight waves), within an
+     * eighth of the cache (a kernel may walk several arrays behind one cache at a time) */
+    uint64_t dist = (cache.n_pages / 8) / w_pages;
+    dist = (dist > 32 ? 32 : dist < 1 ? 1 : dist) * w_elems;
+    bam::range_view<T> view;
+    view.load(da->d_ranges);
+    auto touch = [](uint32_t) { return true; };
+    const uint64_t mine = first - first % w_elems + bam::lane() * epp;
+    if (first < dist) view.acquire_helped(view.page_of(mine < n_elems ? mine : first), bam::lane() < w_pages && mine < n_elems, false, touch, touch);
+    const uint64_t ahead = mine + dist;
+    if (first + dist < n_elems) view.acquire_helped(view.page_of(ahead < n_elems ? ahead : first), bam::lane() < w_pages && ahead < n_elems, false, touch, touch);
+    view.n_access = view.n_hit = 0;
+}
+
 // ---- array benchmark (benchmarks/array/main.cu:43-65), with a checksum ----
 __global__ void k_array_read(array_d_t<uint64_t>* dr, uint64_t n_reqs, const uint64_t* assignment, uint64_t stride, uint64_t reqs_per_thread, unsigned long long* sum)
 {
     const uint64_t tid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
     uint64_t v = 0;
+    /* thread t reads element t * stride: where a wave covers only a few pages (less than 32 KiB) they are touched ahead in
+     * windows, or every wave would ask the store for its one page or its few by itself */
+    const uint64_t first_tid = tid - threadIdx.x % BAM_WAVE_SIZE;
+    if (!assignment && stride && first_tid < n_reqs && BAM_WAVE_SIZE * stride * sizeof(uint64_t) < 32768)
+        touch_ahead(dr, first_tid * stride, (n_reqs - 1) * stride + 1, BAM_WAVE_SIZE * stride);
     if (tid < n_reqs) {
         const uint64_t idx = assignment ? assignment[tid] : tid * stride;
         for (uint64_t i = 0; i < reqs_per_thread; i++) v += (*dr)[idx];
@@ -837,39 +876,6 @@ __global__ __launch_bounds__(64) void k_cc_by_page(array_d_t<uint64_t>* da, bool
     graph_by_page(da, offsets, first, n_edges, ppw, (sweep & 1u) != 0,
                   [&](uint64_t v) { return curr_visit[v]; },
                   [&](uint64_t src, uint64_t next, uint64_t) { cc_compute(src, comp, next, next_visit, changed); });
-}
-
-/*
- * Read-ahead for kernels in which consecutive threads read consecutive elements (one element or two per thread, as in
- * benchmarks/vectoradd, reduction and scan).  Left to themselves such kernels ask the store for one page per wave
- * and trip, and the store path takes about a million such batches per second whatever their size: 1 GiB comes in
- * at 5 GB/s.  Here the wave that reads the first element of a window of W pages (W = a 64th of the cache, at most
- * 64) touches the W pages that lie up to 32 windows further on, one page per lane, taken and dropped again: they come
- * in as one batch of W commands, before the waves that read them are started (workgroups start in order, and the
- * device holds a few thousand waves, that is up to a thousand pages, at a time).  The first windows are touched by
- * their own first waves.  `first` is the index of the wave's first element (wave-uniform).
- */
-template <typename T>
-__device__ __forceinline__ void touch_ahead(array_d_t<T>* da, const uint64_t first, const uint64_t n_elems)
-{
-    if (da->n_ranges != 1) return;
-    const page_cache_d_t& cache = da->d_ranges[0].cache;
-    const uint64_t w_pages = cache.n_pages >> 6 > BAM_WAVE_SIZE ? BAM_WAVE_SIZE : cache.n_pages >> 6;
-    if (w_pages < 2) return;
-    const uint64_t epp = cache.page_size / sizeof(T), w_elems = w_pages * epp;
-    if (first % w_elems) return;
-    /* how far ahead: beyond what the waves in flight cover (a few thousand waves at one page per four to eight waves), within an
-     * eighth of the cache (a kernel may walk several arrays behind one cache at a time) */
-    uint64_t dist = (cache.n_pages / 8) / w_pages;
-    dist = (dist > 32 ? 32 : dist < 1 ? 1 : dist) * w_elems;
-    bam::range_view<T> view;
-    view.load(da->d_ranges);
-    auto touch = [](uint32_t) { return true; };
-    const uint64_t mine = first + bam::lane() * epp;
-    if (first < dist) view.acquire_helped(view.page_of(mine < n_elems ? mine : first), bam::lane() < w_pages && mine < n_elems, false, touch, touch);
-    const uint64_t ahead = mine + dist;
-    if (first + dist < n_elems) view.acquire_helped(view.page_of(ahead < n_elems ? ahead : first), bam::lane() < w_pages && ahead < n_elems, false, touch, touch);
-    view.n_access = view.n_hit = 0;
 }
 
 // ---- vectoradd (benchmarks/vectoradd/main.cu:102-117 kernel_baseline_ptr_pc): C[i] = A[i] + B[i], all three behind the cache ----
