@@ -105,14 +105,17 @@ __global__ void k_fold_partials(unsigned long long* partials, unsigned long long
  * from one wave's first to the next one's (more than 64 where the threads read with a stride).
  */
 template <typename T>
-__device__ __forceinline__ void touch_ahead(array_d_t<T>* da, const uint64_t first, const uint64_t n_elems, const uint64_t wave_span = BAM_WAVE_SIZE)
+__device__ __forceinline__ void touch_ahead(array_d_t<T>* da, const uint64_t first, const uint64_t n_elems, const uint64_t wave_span = BAM_WAVE_SIZE,
+                                            const uint32_t which = 0)
 {
     if (da->n_ranges != 1) return;
     const page_cache_d_t& cache = da->d_ranges[0].cache;
     const uint64_t w_pages = cache.n_pages >> 6 > BAM_WAVE_SIZE ? BAM_WAVE_SIZE : cache.n_pages >> 6;
     if (w_pages < 2) return;
     const uint64_t epp = cache.page_size / sizeof(T), w_elems = w_pages * epp;
-    if (first % w_elems >= wave_span) return;           /* not the first wave that begins in its window (`wave_span` elements per wave) */
+    /* the wave that does it is the `which`-th of those that begin in the window (`wave_span` elements per wave): a kernel
+     * that walks several arrays gives each array's windows to a different wave, and their batches are in flight together */
+    if ((first % w_elems) / wave_span != which) return;
     /* how far ahead: beyond what the waves in flight cover (a few thousand waves at one page per four to eight waves), within an
      * eighth of the cache (a kernel may walk several arrays behind one cache at a time) */
     uint64_t dist = (cache.n_pages / 8) / w_pages;
@@ -889,9 +892,9 @@ __global__ __launch_bounds__(64) void k_vectoradd_ptr_pc(array_d_t<uint64_t>* da
     const bam_ptr<uint64_t>& B = Bptr;
     const uint64_t first = tid - threadIdx.x % BAM_WAVE_SIZE;
     if (first < n_elems) {
-        touch_ahead(da, first, n_elems);
-        touch_ahead(db, first, n_elems);
-        touch_ahead(dc, first, n_elems);
+        touch_ahead(da, first, n_elems, BAM_WAVE_SIZE, 0);
+        touch_ahead(db, first, n_elems, BAM_WAVE_SIZE, 1);
+        touch_ahead(dc, first, n_elems, BAM_WAVE_SIZE, 2);
     }
     if (tid < n_elems) Cptr[tid] = A[tid] + B[tid];
 }
