@@ -166,7 +166,11 @@ int bam_cc_by_page(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_ver
 
 /* ---- vectoradd (benchmarks/vectoradd/main.cu:102-117 kernel_baseline_ptr_pc) ----
  * c[i] = a[i] + b[i] for i < n_elems, one thread per element, all three arrays read and written through bam_ptr; the
- * results reach the store when their pages are evicted or the cache is flushed (bam_page_cache_flush). */
+ * results reach the store when their pages are evicted or the cache is flushed (bam_page_cache_flush).
+ * In this kernel, in bam_reduce, bam_scan and in bam_array_read without an assignment, consecutive threads read
+ * consecutive (or evenly spaced) elements: the first wave of every window of up to 64 pages touches a window further
+ * on, one page per lane, so that the store is asked for pages in batches of a window and not one page per wave
+ * (arrays of one range; off for caches under 128 pages).  Results and counters of accesses are not affected. */
 int bam_vectoradd(bam_array_t* a, bam_array_t* b, bam_array_t* c, uint64_t n_elems, void* stream);
 
 /* ---- reduction (benchmarks/reduction/main.cu:166-195 kernel_reduce_baseline_ptr_pc, launch :476) ----
