@@ -105,10 +105,11 @@ __global__ void k_fold_partials(unsigned long long* partials, unsigned long long
  * from one wave's first to the next one's (more than 64 where the threads read with a stride).
  */
 template <typename T>
-__device__ __forceinline__ void touch_ahead(array_d_t<T>* da, const uint64_t first, const uint64_t n_elems, const uint64_t wave_span = BAM_WAVE_SIZE,
+__device__ __forceinline__ void touch_ahead(array_d_t<T>* da, const uint64_t first, const uint64_t n_read, const uint64_t wave_span = BAM_WAVE_SIZE,
                                             const uint32_t which = 0)
 {
     if (da->n_ranges != 1) return;
+    const uint64_t n_elems = n_read < da->n_elems ? n_read : da->n_elems;         /* nothing is touched that the array does not hold */
     const page_cache_d_t& cache = da->d_ranges[0].cache;
     const uint64_t w_pages = cache.n_pages >> 6 > BAM_WAVE_SIZE ? BAM_WAVE_SIZE : cache.n_pages >> 6;
     if (w_pages < 2) return;
