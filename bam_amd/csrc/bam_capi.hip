@@ -93,6 +93,14 @@ __global__ void k_fold_partials(unsigned long long* partials, unsigned long long
     if (bam::lane() == 0 && v) atomicAdd(sum, (unsigned long long)v);
 }
 
+/* a page that is not resident as far as one look at its state tells: what the read-ahead asks for (a page that is resident is
+ * left alone, which spares its state word two atomics per touch; if it goes before it is read, it is read on demand) */
+template <typename T>
+__device__ __forceinline__ bool page_absent(const bam::range_view<T>& view, const uint64_t page)
+{
+    return (bam::ld_relaxed(&view.pages[page].state) & VALID) == 0;
+}
+
 /*
  * Read-ahead for kernels in which consecutive threads read consecutive elements (one element or two per thread, as in
  * benchmarks/vectoradd, reduction and scan).  Left to themselves such kernels ask the store for one page per wave
@@ -125,9 +133,17 @@ __device__ __forceinline__ void touch_ahead(array_d_t<T>* da, const uint64_t fir
     view.load(da->d_ranges);
     auto touch = [](uint32_t) { return true; };
     const uint64_t mine = first - first % w_elems + bam::lane() * epp;
-    if (first < dist) view.acquire_helped(view.page_of(mine < n_elems ? mine : first), bam::lane() < w_pages && mine < n_elems, false, touch, touch);
+    if (first < dist) {
+        const uint64_t page = view.page_of(mine < n_elems ? mine : first);
+        const bool take = bam::lane() < w_pages && mine < n_elems && page_absent(view, page);
+        if (bam::ballot(take)) view.acquire_helped(page, take, false, touch, touch);
+    }
     const uint64_t ahead = mine + dist;
-    if (first + dist < n_elems) view.acquire_helped(view.page_of(ahead < n_elems ? ahead : first), bam::lane() < w_pages && ahead < n_elems, false, touch, touch);
+    if (first + dist < n_elems) {
+        const uint64_t page = view.page_of(ahead < n_elems ? ahead : first);
+        const bool take = bam::lane() < w_pages && ahead < n_elems && page_absent(view, page);
+        if (bam::ballot(take)) view.acquire_helped(page, take, false, touch, touch);
+    }
     view.n_access = view.n_hit = 0;
 }
 
@@ -228,6 +244,20 @@ __global__ void k_array_write(array_d_t<uint64_t>* dr, uint64_t n_reqs, const ui
     if (tid < n_reqs) (*dr)(assignment ? assignment[tid] : tid * stride, values[tid]);
 }
 
+/* the pages [first, first + n) of a range (n <= 64), one per lane: those that are not resident are taken and dropped again as
+ * one batch.  A function of its own: the view of the range it works on lives in registers only while it runs. */
+__device__ __attribute__((noinline)) void stream_touch(range_d_t<uint64_t>* r, const uint64_t first, const uint64_t n)
+{
+    bam::range_view<uint64_t> view;
+    view.load(r);
+    auto touch = [](uint32_t) { return true; };
+    const uint64_t lane = bam::lane(), epp = r->n_elems_per_page;
+    const uint64_t page = view.page_of((first + (lane < n ? lane : 0)) * epp);
+    const bool take = lane < n && page_absent(view, page);
+    if (bam::ballot(take)) view.template acquire_helped<true>(page, take, false, touch, touch);
+    view.n_access = view.n_hit = 0;
+}
+
 // ---- cache / pattern benchmark (benchmarks/cache/main.cu:44-114): a wave streams whole pages ----
 template <int MODE>
 __device__ __forceinline__ void cache_stream_body(array_d_t<uint64_t>* dr, uint64_t n_waves, uint64_t n_pages_per_wave, const uint64_t* assignment, unsigned long long* sum)
@@ -285,9 +315,16 @@ __device__ __forceinline__ void cache_stream_body(array_d_t<uint64_t>* dr, uint6
             view.flush_stats();
         } else {
             bam_ptr<uint64_t> ptr(dr);
+            /* a wave reads its pages one after the other: those of the next stretch that are not resident are touched
+             * together, one page per lane, so that a cold run asks the store for a batch per stretch and not for a page
+             * per trip (1.5 M pages/s otherwise); on a resident cache this costs one look at a state word per page */
+            /* (modes 3 and 4: the helper needs more registers than the kernels themselves, which costs them a third of the
+             * waves they run with on a resident cache, hence modes 0 and 1 without) */
+            const uint32_t reach = MODE < 3 || dr->n_ranges != 1 ? 0 : (uint32_t)(r0->cache.n_pages >> 6 > BAM_WAVE_SIZE ? BAM_WAVE_SIZE : r0->cache.n_pages >> 6);
             for (uint64_t p = 0; p < n_pages_per_wave; p++) {
+                if (MODE >= 3 && reach >= 2 && p % reach == 0) stream_touch(r0, start_page + p, n_pages_per_wave - p < reach ? n_pages_per_wave - p : reach);
                 const uint64_t start_idx = (start_page + p) * epp + lane;
-                if (MODE == 0) {
+                if (MODE == 0 || MODE == 4) {
                     for (uint64_t j = 0; j < epp; j += BAM_WAVE_SIZE) v += (*dr)[start_idx + j];
                 } else {
                     /* eight elements asked for before the first is used: the window test of an element needs nothing that
@@ -420,8 +457,9 @@ struct list_read_ahead {
         auto touch = [](uint32_t) { return true; };
         const uint64_t pf = want ? view.page_of(es) : 0, pl = want ? view.page_of(ee - 1) : 0;
         /* all lanes go in: those without a page of their own help move what the others load */
-        view.acquire_helped(pf, want, false, touch, touch);
-        if (bam::ballot(want && pl != pf)) view.acquire_helped(pl, want && pl != pf, false, touch, touch);
+        const bool take_f = want && page_absent(view, pf), take_l = want && pl != pf && page_absent(view, pl);
+        if (bam::ballot(take_f)) view.acquire_helped(pf, take_f, false, touch, touch);
+        if (bam::ballot(take_l)) view.acquire_helped(pl, take_l, false, touch, touch);
         view.n_access = view.n_hit = 0;
     }
     /*
@@ -460,7 +498,8 @@ struct list_read_ahead {
             }
 #pragma unroll
             for (uint32_t o = BAM_WAVE_SIZE / 2; o; o >>= 1) m |= bam::shfl(m, lane ^ o);
-            if (m) view.acquire_helped(c + lane, ((m >> lane) & 1) != 0, false, touch, touch);
+            const bool take = ((m >> lane) & 1) != 0 && page_absent(view, c + lane);
+            if (bam::ballot(take)) view.acquire_helped(c + lane, take, false, touch, touch);
             seen |= m;
         }
         view.n_access = view.n_hit = 0;
@@ -484,7 +523,7 @@ struct list_read_ahead {
         if (reach < BAM_WAVE_SIZE) return false;
         auto touch = [](uint32_t) { return true; };
         const uint64_t page = want ? view.page_of(start) + (bam::lane() & 15u) : 0;
-        const bool take = want && end > start && page <= view.page_of(end - 1);
+        const bool take = want && end > start && page <= view.page_of(end - 1) && page_absent(view, page);
         if (bam::ballot(take)) view.acquire_helped(page, take, false, touch, touch);
         view.n_access = view.n_hit = 0;
         return true;
@@ -497,7 +536,8 @@ struct list_read_ahead {
         if (pg < asked_to) return;
         const uint64_t p = pg + bam::lane();
         auto touch = [](uint32_t) { return true; };
-        view.acquire_helped(p, bam::lane() < reach && p <= last_page, false, touch, touch);
+        const bool take = bam::lane() < reach && p <= last_page && page_absent(view, p);
+        if (bam::ballot(take)) view.acquire_helped(p, take, false, touch, touch);
         asked_to = pg + reach;
         view.n_access = view.n_hit = 0;         /* not accesses of the kernel's own: kept out of the counters */
     }
@@ -1493,7 +1533,7 @@ int bam_cache_stream(bam_array_t* a, uint64_t n_waves, uint64_t n_pages_per_wave
                      uint64_t* d_sum, void* stream)
 {
     if (!a || !d_sum) return fail(EINVAL, "bam_cache_stream: null argument");
-    if (mode < 0 || mode > 2) return fail(EINVAL, "bam_cache_stream: mode must be 0, 1 or 2");
+    if (mode < 0 || mode > 4) return fail(EINVAL, "bam_cache_stream: mode must be 0 to 4");
     if (!n_waves || !n_pages_per_wave) return 0;
     BAM_API_BEGIN
     const uint32_t bs = 256;
@@ -1502,6 +1542,8 @@ int bam_cache_stream(bam_array_t* a, uint64_t n_waves, uint64_t n_pages_per_wave
     unsigned long long* s = (unsigned long long*)a->partials.get();
     if (mode == 0) hipLaunchKernelGGL(k_cache_stream<0>, grid, block, 0, (hipStream_t)stream, d, n_waves, n_pages_per_wave, d_assignment, s);
     else if (mode == 1) hipLaunchKernelGGL(k_cache_stream<1>, grid, block, 0, (hipStream_t)stream, d, n_waves, n_pages_per_wave, d_assignment, s);
+    else if (mode == 3) hipLaunchKernelGGL(k_cache_stream<3>, grid, block, 0, (hipStream_t)stream, d, n_waves, n_pages_per_wave, d_assignment, s);
+    else if (mode == 4) hipLaunchKernelGGL(k_cache_stream<4>, grid, block, 0, (hipStream_t)stream, d, n_waves, n_pages_per_wave, d_assignment, s);
     else hipLaunchKernelGGL(k_cache_stream_pages, grid, block, 0, (hipStream_t)stream, d, n_waves, n_pages_per_wave, d_assignment, s);
     hipLaunchKernelGGL(k_fold_partials, dim3(1), dim3(1024), 0, (hipStream_t)stream, s, (unsigned long long*)d_sum);
     hip_err_chk(hipGetLastError());
