@@ -458,8 +458,20 @@ struct list_read_ahead {
         const uint64_t pf = want ? view.page_of(es) : 0, pl = want ? view.page_of(ee - 1) : 0;
         /* all lanes go in: those without a page of their own help move what the others load */
         const bool take_f = want && page_absent(view, pf), take_l = want && pl != pf && page_absent(view, pl);
-        if (bam::ballot(take_f)) view.acquire_helped(pf, take_f, false, touch, touch);
-        if (bam::ballot(take_l)) view.acquire_helped(pl, take_l, false, touch, touch);
+        /* the last pages go along with the first ones as far as there are lanes without a first page to ask for (the k-th such
+         * lane takes the last page of the k-th lane that has one): one batch of commands instead of two, of which the second
+         * would be small (few lists cross a page boundary) */
+        const uint64_t need_l = bam::ballot(take_l), idle = ~bam::ballot(take_f);
+        const uint32_t k = bam::popc(idle & bam::lanes_below(bam::lane()));
+        const bool adopt = !take_f && k < bam::popc(need_l);
+        uint64_t m = need_l;
+        if (adopt) for (uint32_t i = 0; i < k; i++) m &= m - 1;
+        const uint64_t adopted = bam::shfl(pl, adopt ? bam::first_lane(m) : 0u);
+        const bool take_1 = take_f || adopt;
+        if (bam::ballot(take_1)) view.acquire_helped(take_f ? pf : adopted, take_1, false, touch, touch);
+        /* last pages nobody had a lane for */
+        const bool take_2 = take_l && bam::popc(need_l & bam::lanes_below(bam::lane())) >= bam::popc(idle);
+        if (bam::ballot(take_2)) view.acquire_helped(pl, take_2, false, touch, touch);
         view.n_access = view.n_hit = 0;
     }
     /*
