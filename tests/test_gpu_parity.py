@@ -618,6 +618,31 @@ def test_hub_lists_are_cut_into_pieces(bam, cache_pages, coarse):
         assert not r.c.aborted()
 
 
+@pytest.mark.parametrize("empty_every", [0, 4, 2])
+def test_lists_that_all_cross_a_page_boundary(bam, empty_every):
+    """every list has 600 entries (a page holds 512), so each one ends on another page than it starts on, and every
+    `empty_every`-th vertex has none: the read-ahead of a group asks for the last pages on the lanes that have no first
+    page to ask for, and for the rest in a second batch (none empty: all in the second batch; every second one empty:
+    all in the first).  Neighbours are the next 600 vertices, so the levels step through the graph."""
+    n_v, d = 4096, 600
+    deg = np.full(n_v, d, dtype=np.uint64)
+    if empty_every:
+        deg[empty_every - 1::empty_every] = 0
+    off = np.concatenate([[0], np.cumsum(deg)]).astype(np.uint64)
+    owner = np.repeat(np.arange(n_v, dtype=np.uint64), deg.astype(np.int64))
+    nb = (owner + 1 + (np.arange(len(owner), dtype=np.uint64) - off[owner])) % np.uint64(n_v)
+    r, a = _graph_rig(bam, nb, 256, n_queues=8, depth=256)
+    with r:
+        doff = _dev(off)
+        for src in (0, 1000, 4092):
+            want, want_it = oracle.bfs_levels(off, nb, src)
+            assert want_it >= 6
+            for kw in (dict(coarse=1), dict(coarse=64), dict(frontier=True)):
+                lv, it = a.bfs(doff, src, **kw)
+                assert np.array_equal(lv.cpu().numpy().view(np.uint32), want) and it == want_it
+        assert a.stats()["read_io_cnt"] > len(nb) // 512 and not r.c.aborted()
+
+
 @pytest.mark.parametrize("scale,cache_pages", [(10, 2048), (13, 160)])
 def test_sssp_costs_two_arrays_in_one_cache(bam, scale, cache_pages):
     """neighbour ids (64-bit) and weights (32-bit) as two arrays behind one page cache; costs against Dijkstra"""
