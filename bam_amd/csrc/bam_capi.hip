@@ -5,6 +5,7 @@
 #include "bam_amd.h"
 
 #include <hip/hip_runtime.h>
+#include <hipcub/hipcub.hpp>
 #include <fcntl.h>
 #include <sys/mman.h>
 #include <sys/stat.h>
@@ -475,7 +476,8 @@ struct list_read_ahead {
         view.n_access = view.n_hit = 0;
     }
     /*
-     * The lists of the consecutive vertices [first, last) lie side by side in the array: touch every page that holds
+     * The lists of the items [first, last) lie in the array in the order of the items (consecutive vertices, or a sorted
+     * queue of them): touch every page that holds
      * entries of a list that is about to be walked (item(v, v) says which; lists that go to the queue of long ones are
      * left out), `reach` pages at a time with one page per lane, so that what is not resident comes in as few, large
      * batches of commands.  The store path moves several times more pages per second in batches of sixteen than in
@@ -488,7 +490,9 @@ struct list_read_ahead {
     {
         nothing = false;
         if (reach < 2) return false;
-        const uint64_t e0 = vertexList[first], e1 = vertexList[last];
+        uint64_t v_first = 0, v_last = 0;
+        item(first, v_first); item(last - 1, v_last);
+        const uint64_t e0 = vertexList[v_first], e1 = vertexList[v_last + 1];
         if (e1 <= e0) { nothing = true; return true; }
         const uint64_t p0 = view.page_of(e0), p1 = view.page_of(e1 - 1);
         if (p1 - p0 >= 4ull * reach) return false;
@@ -670,7 +674,7 @@ template <bool HOLD, typename Item, typename Active, typename Visit>
 __device__ __forceinline__ void walk_item_groups(array_d_t<uint64_t>* da, const uint64_t* vertexList, const uint64_t n_items, const uint64_t coarse,
                                                  const heavy_piece_t* heavy, const uint64_t n_heavy, unsigned long long* next_work,
                                                  const bool backwards, Item item, Active active, Visit visit,
-                                                 list_read_ahead<uint32_t>* with = nullptr)
+                                                 list_read_ahead<uint32_t>* with = nullptr, const bool in_order = HOLD)
 {
     const uint64_t laneIdx = threadIdx.x % BAM_WAVE_SIZE;
     const uint64_t n_groups = (n_items + coarse - 1) / coarse;
@@ -723,7 +727,7 @@ __device__ __forceinline__ void walk_item_groups(array_d_t<uint64_t>* da, const 
         const uint64_t g = backwards ? n_groups - 1 - (w - n_bundles) : w - n_bundles;
         const uint64_t first = g * coarse;
         bool touched = false, nothing = false;
-        if constexpr (HOLD) {
+        if (in_order) {
             if (!ready) { ahead.init(da); ready = true; }
             touched = ahead.span(vertexList, first, first + coarse < n_items ? first + coarse : n_items, BAM_HEAVY_EDGES, item, nothing);
             if (with && touched && !nothing) { bool none; with->span(vertexList, first, first + coarse < n_items ? first + coarse : n_items, BAM_HEAVY_EDGES, item, none); }
@@ -741,7 +745,7 @@ __device__ __forceinline__ void walk_item_groups(array_d_t<uint64_t>* da, const 
             if (!touched) {
                 /* a group whose lists cover too many pages for one look: the same for the 64 vertices at hand */
                 bool block_touched = false;
-                if constexpr (HOLD) {
+                if (in_order) {
                     const uint64_t last = first + coarse < n_items ? first + coarse : n_items;
                     bool none;
                     block_touched = ahead.span(vertexList, first + b, first + b + BAM_WAVE_SIZE < last ? first + b + BAM_WAVE_SIZE : last, BAM_HEAVY_EDGES, item, none);
@@ -794,12 +798,13 @@ __device__ __forceinline__ void bfs_frontier_visit(uint32_t* label, const uint32
 __global__ __launch_bounds__(128) void k_bfs_frontier_coalesce_ptr_pc(array_d_t<uint64_t>* da, uint32_t* label, const uint32_t level, const uint64_t* vertexList,
                                                                      const uint32_t* curr_frontier, const uint64_t curr_size, uint32_t* next_frontier,
                                                                      unsigned long long* next_size, uint64_t group,
-                                                                     const heavy_piece_t* heavy, uint64_t n_heavy, unsigned long long* next_work)
+                                                                     const heavy_piece_t* heavy, uint64_t n_heavy, unsigned long long* next_work, bool sorted)
 {
     walk_item_groups<false>(da, vertexList, curr_size, group, heavy, n_heavy, next_work, false,
                             [&](uint64_t i, uint64_t& v) { v = curr_frontier[i]; return true; },
                             [&](uint64_t v) { return label[v] == level; },
-                            [&](uint64_t, uint64_t next, uint64_t) { bfs_frontier_visit(label, level, next_frontier, next_size, next); });
+                            [&](uint64_t, uint64_t next, uint64_t) { bfs_frontier_visit(label, level, next_frontier, next_size, next); },
+                            nullptr, sorted);
 }
 
 // ---- CC: min-label propagation (benchmarks/cc/main.cu:123-144, 595-617) ----
@@ -1803,20 +1808,38 @@ int bam_bfs_frontier(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_v
     hip_err_chk(hipMemcpyAsync(d_labels + src, &zero, sizeof(uint32_t), hipMemcpyHostToDevice, st));
     hip_err_chk(hipMemcpyAsync(curr, &src32, sizeof(uint32_t), hipMemcpyHostToDevice, st));
     const uint32_t threads = 128;
-    const uint64_t group = BAM_WAVE_SIZE;           /* queue entries handed to a wave at a time: one per lane */
+    uint64_t group = BAM_WAVE_SIZE;                 /* queue entries handed to a wave at a time: one per lane, more of a sorted queue */
+    bool sorted = true;                             /* the first queue holds the source alone */
     sweep_work work(edges->a->adt.n_elems, n_vertices, 1, d_offsets, st);
     uint32_t level = 0, iter = 0;
     unsigned long long active = 1;
+    const char* e = getenv("BAM_FRONTIER_SORT");
+    const bool sort_queue = !e || atoi(e) != 0;
+    int vertex_bits = 1;
+    while (vertex_bits < 32 && (1ull << vertex_bits) < n_vertices) vertex_bits++;
+    size_t sort_bytes = 0;
+    if (sort_queue) hip_err_chk(hipcub::DeviceRadixSort::SortKeys(nullptr, sort_bytes, curr, next, (int)std::min<uint64_t>(n_vertices, 0x7FFFFFFFull), 0, vertex_bits, st));
+    BufferPtr sort_tmp = createBuffer(sort_bytes ? sort_bytes : 8, 0);
     do {
         hip_err_chk(hipMemsetAsync(next_size, 0, sizeof(unsigned long long), st));
         work.reset(st);
         hipLaunchKernelGGL(k_bfs_frontier_coalesce_ptr_pc, dim3(work.blocks(active, group)), dim3(threads), 0, st, edges->a->d_array_ptr, d_labels, level,
-                           d_offsets, curr, (uint64_t)active, next, next_size, group, work.pieces, work.n_pieces, work.count + 1);
+                           d_offsets, curr, (uint64_t)active, next, next_size, group, work.pieces, work.n_pieces, work.count + 1, sorted);
         hip_err_chk(hipGetLastError());
-        std::swap(curr, next);
         iter++; level++;
         hip_err_chk(hipMemcpyAsync(&active, next_size, sizeof(unsigned long long), hipMemcpyDeviceToHost, st));
         hip_err_chk(hipStreamSynchronize(st));
+        sorted = sort_queue && active <= 0x7FFFFFFFull;
+        group = sorted ? work.group : BAM_WAVE_SIZE;
+        if (sorted && active > 1) {
+            /* the queue comes out in the order of discovery; sorted by vertex, the level reads the edge array front to back
+             * (neighbouring lists share pages, a page is not evicted between two of its lists, and the pages under the
+             * lists of a group of entries can be asked for together as in the sweep over all vertices).  The sorted queue
+             * goes into the buffer the level just walked, so the two do not change places. */
+            size_t need = sort_bytes;
+            hip_err_chk(hipcub::DeviceRadixSort::SortKeys(sort_tmp.get(), need, next, curr, (int)active, 0, vertex_bits, st));
+        } else
+            std::swap(curr, next);
     } while (active);
     if (iterations) *iterations = iter;
     BAM_API_END

@@ -273,13 +273,15 @@ def main():
         legs = {}
         # the edge-page kernel on every source; the reference-shaped kernel (a wave per vertex, bam_ptr per element) on the first two
         # (64 vertices per wave: consecutive vertices share pages, so the more vertices a wave has, the more distinct pages are asked for at a time)
-        for name, by_page, n_src, coarse in (("by_page", True, len(srcs), 1), ("per_vertex_bam_ptr", False, min(4, len(srcs)), 64)):
+        # and the kernel that walks a queue of the level's vertices, sorted between levels
+        for name, by_page, n_src, coarse in (("by_page", True, len(srcs), 1), ("per_vertex_bam_ptr", False, min(4, len(srcs)), 64),
+                                             ("queue_of_vertices", False, min(4, len(srcs)), 0)):
             tot_ms, tot_edges, levels_ok, iters = 0.0, 0, True, []
             ag.stats()
             for k, src in enumerate(srcs[:n_src]):
                 a, b = event(), event()
                 L.bam_event_record(a, stream)
-                lv, it = ag.bfs(off, int(src), coarse=coarse, by_page=by_page)
+                lv, it = ag.bfs(off, int(src), frontier=True) if not coarse else ag.bfs(off, int(src), coarse=coarse, by_page=by_page)
                 L.bam_event_record(b, stream)
                 ms = elapsed_ms(a, b)
                 lv_h = lv.cpu().numpy().view(np.uint32)

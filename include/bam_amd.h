@@ -145,9 +145,13 @@ int bam_bfs(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, 
  * host loop :1561-1563, 1702-1711) ----
  * Instead of sweeping all labels, every level walks the queue of the vertices found by the level before and fills the
  * next one: a vertex enters it when the exchange on its label finds it unreached, the lanes of a wave that found one
- * at the same step take their places with one atomic.  64 queue entries per wave at a time, otherwise the walk of
- * bam_bfs (lists packed 64 entries per step, long lists in pieces).  Same levels and the same *iterations as bam_bfs;
- * the order of a queue is not defined, nothing depends on it.  n_vertices <= 2^32 - 1 (32-bit queue entries). */
+ * at the same step take their places with one atomic.  Otherwise the walk of bam_bfs (lists packed 64 entries per
+ * step, long lists in pieces).  Same levels and the same *iterations as bam_bfs; no result depends on the order of a
+ * queue, which is that of discovery when a level ends.  Between levels the queue is sorted by vertex (radix sort on
+ * the device), so that a level reads the edge array front to back and a wave can take 512 entries at a time and ask
+ * for the pages under their lists as one batch, as bam_bfs does for 512 vertices; environment BAM_FRONTIER_SORT=0
+ * leaves the queue as it comes (64 entries per wave at a time, first and last page of each list asked for).
+ * n_vertices <= 2^32 - 1 (32-bit queue entries). */
 int bam_bfs_frontier(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t src, uint32_t* d_labels,
                      uint32_t* iterations, void* stream);
 /* ---- CC (benchmarks/cc/main.cu:123-144 cc_compute, :595-617 kernel, host loop :1410-1425, 1515-1521) ----

@@ -700,8 +700,11 @@ def test_sssp_float_costs(bam, scale, cache_pages):
 
 
 @pytest.mark.parametrize("scale,cache_pages", [(10, 4096), (14, 24), (16, 8192), (17, 700)])
-def test_bfs_levels_rmat_by_queue_of_vertices(bam, scale, cache_pages):
-    """the kernel that walks a queue of the level's vertices: same levels, same launch count"""
+@pytest.mark.parametrize("sort", ["1", "0"])
+def test_bfs_levels_rmat_by_queue_of_vertices(bam, scale, cache_pages, sort, monkeypatch):
+    """the kernel that walks a queue of the level's vertices: same levels, same launch count, whether the queue is
+    sorted between levels (the default) or walked in the order of discovery"""
+    monkeypatch.setenv("BAM_FRONTIER_SORT", sort)
     off, nb = oracle.rmat_csr(SEED, scale)
     r, a = _graph_rig(bam, nb, cache_pages, n_queues=16, depth=256)
     with r:
