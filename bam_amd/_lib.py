@@ -39,6 +39,8 @@ SIGNATURES = {
     "bam_array_stats": (c_int, [c_vp, P(c_u64), c_int]),
     "bam_array_read": (c_int, [c_vp, c_u64, c_vp, c_u64, c_u64, c_u32, c_vp, c_vp]),
     "bam_array_write": (c_int, [c_vp, c_u64, c_vp, c_u64, c_vp, c_u32, c_vp]),
+    "bam_array_update": (c_int, [c_vp, c_int, c_u64, c_vp, c_vp, c_vp, c_u32, c_vp]),
+    "bam_sqe_image": (c_int, [ctypes.c_uint16, ctypes.c_uint8, c_u32, c_u64, c_u64, c_u64, ctypes.c_uint16, c_int, c_u32, P(c_u32), c_vp, c_vp]),
     "bam_cache_stream": (c_int, [c_vp, c_u64, c_u64, c_vp, c_int, c_vp, c_vp]),
     "bam_block_io": (c_int, [c_vp, c_vp, c_u64, c_u32, c_vp, c_int, c_int, c_u32, c_vp]),
     "bam_block_checksum": (c_int, [c_vp, c_u64, c_u32, c_vp, c_vp]),
@@ -80,7 +82,8 @@ SIGNATURES = {
 
 
 def lib_path():
-    return os.path.join(_HERE, "libbam_amd.so")
+    """The built library; BAM_AMD_LIB names another build of it (the one with the phase timers, `make prof`)."""
+    return os.environ.get("BAM_AMD_LIB") or os.path.join(_HERE, "libbam_amd.so")
 
 
 def host_lib_path():

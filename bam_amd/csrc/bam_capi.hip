@@ -14,6 +14,7 @@
 #include <cerrno>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <string>
 #include <thread>
 #include <vector>
@@ -245,6 +246,50 @@ __global__ void k_array_write(array_d_t<uint64_t>* dr, uint64_t n_reqs, const ui
     if (tid < n_reqs) (*dr)(assignment ? assignment[tid] : tid * stride, values[tid]);
 }
 
+/*
+ * Read-modify-write through the three routes the reference offers for it (include/page_cache.h:1647 AtomicAdd, :467 memref,
+ * :478 non-const operator[] used as an lvalue): element assignment[t] += values[t], old[t] = what the element held before.
+ *   0  array_d_t::AtomicAdd                      (any indices, colliding ones included)
+ *   1  atomicAdd on the address bam_ptr::memref hands out   (any indices)
+ *   2  ptr[i] += v through a non-const bam_ptr   (a plain read and write: the indices of one launch must differ)
+ */
+template <int API>
+__global__ void k_array_update(array_d_t<uint64_t>* dr, uint64_t n_reqs, const uint64_t* assignment, const uint64_t* values, uint64_t* old)
+{
+    const uint64_t tid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (tid >= n_reqs) return;
+    const uint64_t idx = assignment[tid], val = values[tid];
+    uint64_t before = 0;
+    if (API == 0) before = dr->AtomicAdd(idx, val);
+    else {
+        bam_ptr<uint64_t> ptr(dr);
+        if (API == 1) {
+            unsigned long long* p = (unsigned long long*)ptr.memref(idx);
+            if (p) before = atomicAdd(p, (unsigned long long)val);
+        } else {
+            before = ptr[idx];
+            ptr[idx] += val;
+        }
+    }
+    if (old) old[tid] = before;
+}
+
+/* lane l encodes the submission entry of command (cid + l) for block (lba + l) the way the miss path does (nvm_cmd_header,
+ * nvm_cmd_data_ptr, nvm_cmd_rw_blks, and nvm_cmd_seal with ticket + l on top when asked): 64 entries of 16 dwords */
+__global__ void k_sqe_image(uint16_t cid, uint8_t opcode, uint32_t nsid, uint64_t prp1, uint64_t prp2, uint64_t lba, uint16_t n_blocks, int seal, uint32_t ticket,
+                            uint32_t* out)
+{
+    const uint32_t l = bam::lane();
+    nvm_cmd_t cmd;
+#pragma unroll
+    for (int i = 0; i < 16; i++) cmd.dword[i] = 0;
+    nvm_cmd_header(&cmd, (uint16_t)(cid + l), opcode, nsid);
+    nvm_cmd_data_ptr(&cmd, prp1, prp2);
+    nvm_cmd_rw_blks(&cmd, lba + l, n_blocks);
+    if (seal) nvm_cmd_seal(&cmd, ticket + l);
+    for (int i = 0; i < 16; i++) out[l * 16 + i] = cmd.dword[i];
+}
+
 /* the pages [first, first + n) of a range (n <= 64), one per lane: those that are not resident are taken and dropped again as
  * one batch.  A function of its own: the view of the range it works on lives in registers only while it runs. */
 __device__ __attribute__((noinline)) void stream_touch(range_d_t<uint64_t>* r, const uint64_t first, const uint64_t n)
@@ -282,13 +327,15 @@ __device__ __forceinline__ void cache_stream_body(array_d_t<uint64_t>* dr, uint6
             uint64_t a0 = 0, a1 = 0;
             for (uint64_t p0 = 0; p0 < n_pages_per_wave; p0 += 16) {
                 const uint32_t nb = (uint32_t)(n_pages_per_wave - p0 < 16 ? n_pages_per_wave - p0 : 16);
-                uint32_t slot = 0;
+                uint32_t slot = BAM_NO_SLOT;
                 const uint64_t page = view.page_of((start_page + p0 + (lane < nb ? lane : 0)) * epp);
                 if (lane < nb) {
                     auto keep = [&](uint32_t s_) { slot = s_; return false; };
                     view.acquire<true>(page, false, keep, keep);
                 }
-                uint32_t k = 0;
+                /* a page whose wait was given up (the controller is marked aborted) has no slot: nothing of the batch is read */
+                const bool all_in = bam::ballot(lane < nb && slot == BAM_NO_SLOT) == 0;
+                uint32_t k = all_in ? 0 : nb;
                 if (n8 == 8 * BAM_WAVE_SIZE)            /* 4 KiB pages: two at a time */
                     for (; k + 1 < nb; k += 2) {
                         uint64_t x[16];
@@ -645,18 +692,23 @@ template <typename T>
 struct touch_reader {
     array_d_t<T>* da = nullptr;
     bam::range_view<T> view;
-    bool one_range = false;
+    bool one_range = false, fast = false;
     __device__ __forceinline__ void init(array_d_t<T>* a)
     {
         da = a;
         one_range = a->n_ranges == 1;
-        if (one_range) view.load(a->d_ranges);
+        if (one_range) { view.load(a->d_ranges); fast = a->d_ranges[0].cache.fast_reads != 0; }
     }
     __device__ __forceinline__ T read(const uint64_t i)
     {
         if (!one_range) return da->seq_read(i);
         T ret = T();                                    /* stays T() if the wait is given up */
         const uint64_t byte = view.byte_of(i);
+        /* resident pages without a reference at all, as array_d_t::seq_read does */
+        if (fast && bam_read_unpinned(view.pages + (byte >> view.page_size_log), view.base_addr, view.page_size_log, byte & (view.page_size - 1), ret)) {
+            view.account(true);
+            return ret;
+        }
         auto use = [&](uint32_t slot) { ret = bam::ld_payload((T*)(view.slot_addr(slot) + (byte & (view.page_size - 1)))); return true; };
         view.template acquire<true>(byte >> view.page_size_log, false, use, use);
         return ret;
@@ -893,13 +945,14 @@ __device__ __forceinline__ void graph_by_page(array_d_t<uint64_t>* da, const uin
         const bool want = ((marks >> lane) & 1) != 0;
         uint64_t va = 0, vb = 0;
         if (want) { va = first[p]; vb = first[p + 1]; }
-        uint32_t slot = 0;
+        uint32_t slot = BAM_NO_SLOT;
         if (bam::ballot(want)) {
             /* the lanes without a page of their own come along and help move what the others load */
             auto keep = [&](uint32_t s_) { slot = s_; return false; };
             view.acquire_helped(p + pso_pages, want, false, keep, keep);
         }
-        for (uint64_t m = bam::ballot(want); m; m &= m - 1) {
+        /* a page whose wait was given up (the controller is marked aborted) has no slot and is not walked */
+        for (uint64_t m = bam::ballot(want && slot != BAM_NO_SLOT); m; m &= m - 1) {
             const uint32_t j = bam::first_lane(m);
             const uint64_t va_j = bam::bcast(va, j), vb_j = bam::bcast(vb, j);
             const uint64_t ps = (p0 + j) * epp, pe = ps + epp < n_edges ? ps + epp : n_edges;
@@ -1407,13 +1460,13 @@ int bam_page_cache_info(bam_page_cache_t* pc, uint64_t* out)
     return 0;
 }
 
-int bam_page_cache_profile(bam_page_cache_t* pc, uint64_t* out16, int reset)
+int bam_page_cache_profile(bam_page_cache_t* pc, uint64_t* out32, int reset)
 {
-    if (!pc || !out16) return fail(EINVAL, "bam_page_cache_profile: null argument");
+    if (!pc || !out32) return fail(EINVAL, "bam_page_cache_profile: null argument");
     BAM_API_BEGIN
     hip_err_chk(hipDeviceSynchronize());
-    hip_err_chk(hipMemcpy(out16, pc->pc->pdt.prof, 16 * sizeof(uint64_t), hipMemcpyDeviceToHost));
-    if (reset) hip_err_chk(hipMemset(pc->pc->pdt.prof, 0, 16 * sizeof(uint64_t)));
+    hip_err_chk(hipMemcpy(out32, pc->pc->pdt.prof, 32 * sizeof(uint64_t), hipMemcpyDeviceToHost));
+    if (reset) hip_err_chk(hipMemset(pc->pc->pdt.prof, 0, 32 * sizeof(uint64_t)));
     BAM_API_END
 }
 
@@ -1543,6 +1596,45 @@ int bam_array_write(bam_array_t* a, uint64_t n_reqs, const uint64_t* d_assignmen
     hipLaunchKernelGGL(k_array_write, dim3(blocks_for(n_reqs, block_size)), dim3(block_size), 0, (hipStream_t)stream,
                        a->a->d_array_ptr, n_reqs, d_assignment, stride, d_values);
     hip_err_chk(hipGetLastError());
+    BAM_API_END
+}
+
+int bam_array_update(bam_array_t* a, int api, uint64_t n_reqs, const uint64_t* d_assignment, const uint64_t* d_values, uint64_t* d_old,
+                     uint32_t block_size, void* stream)
+{
+    if (!a || !d_assignment || !d_values) return fail(EINVAL, "bam_array_update: null argument");
+    if (api < 0 || api > 2) return fail(EINVAL, "bam_array_update: api must be 0, 1 or 2");
+    if (!block_size || block_size % BAM_WAVE_SIZE || block_size > 1024) return fail(EINVAL, "bam_array_update: block size must be a multiple of 64, at most 1024");
+    if (!n_reqs) return 0;
+    BAM_API_BEGIN
+    const dim3 grid(blocks_for(n_reqs, block_size)), block(block_size);
+    hipStream_t st = (hipStream_t)stream;
+    array_d_t<uint64_t>* d = a->a->d_array_ptr;
+    if (api == 0) hipLaunchKernelGGL(k_array_update<0>, grid, block, 0, st, d, n_reqs, d_assignment, d_values, d_old);
+    else if (api == 1) hipLaunchKernelGGL(k_array_update<1>, grid, block, 0, st, d, n_reqs, d_assignment, d_values, d_old);
+    else hipLaunchKernelGGL(k_array_update<2>, grid, block, 0, st, d, n_reqs, d_assignment, d_values, d_old);
+    hip_err_chk(hipGetLastError());
+    BAM_API_END
+}
+
+int bam_sqe_image(uint16_t cid, uint8_t opcode, uint32_t nsid, uint64_t prp1, uint64_t prp2, uint64_t lba, uint16_t n_blocks, int seal, uint32_t ticket,
+                  uint32_t* host_out16, uint32_t* d_out64x16, void* stream)
+{
+    if (!host_out16 && !d_out64x16) return fail(EINVAL, "bam_sqe_image: null argument");
+    BAM_API_BEGIN
+    if (host_out16) {
+        nvm_cmd_t cmd;
+        memset(&cmd, 0, sizeof(cmd));
+        nvm_cmd_header(&cmd, cid, opcode, nsid);
+        nvm_cmd_data_ptr(&cmd, prp1, prp2);
+        nvm_cmd_rw_blks(&cmd, lba, n_blocks);
+        if (seal) nvm_cmd_seal(&cmd, ticket);
+        memcpy(host_out16, cmd.dword, sizeof(cmd.dword));
+    }
+    if (d_out64x16) {
+        hipLaunchKernelGGL(k_sqe_image, dim3(1), dim3(BAM_WAVE_SIZE), 0, (hipStream_t)stream, cid, opcode, nsid, prp1, prp2, lba, n_blocks, seal, ticket, d_out64x16);
+        hip_err_chk(hipGetLastError());
+    }
     BAM_API_END
 }
 

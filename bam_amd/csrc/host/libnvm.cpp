@@ -21,6 +21,8 @@
 #include <cstring>
 #include <mutex>
 #include <thread>
+#include <fcntl.h>
+#include <sys/mman.h>
 #include <unistd.h>
 
 namespace {
@@ -31,6 +33,8 @@ struct CtrlBox {
     nvm_ctrl_t handle;      // first member: the public handle is the box address
     std::mutex mu;
     int refs = 1;
+    void* mapped = nullptr;     // register window this layer mapped itself (nvm_ctrl_init): unmapped with the last reference
+    size_t mapped_size = 0;
 };
 
 struct DmaBox {
@@ -47,7 +51,10 @@ void ctrl_put(CtrlBox* b)
 {
     bool last;
     { std::lock_guard<std::mutex> g(b->mu); last = --b->refs == 0; }
-    if (last) delete b;
+    if (last) {
+        if (b->mapped) munmap(b->mapped, b->mapped_size);
+        delete b;
+    }
 }
 
 inline uint32_t rd32(volatile void* base, uint32_t off) { return __atomic_load_n((uint32_t*)((char*)base + off), __ATOMIC_ACQUIRE); }
@@ -94,6 +101,23 @@ int nvm_raw_ctrl_init(nvm_ctrl_t** ctrl, volatile void* mm_ptr, size_t mm_size)
     b->handle.mm_size = mm_size;
     b->handle.mm_ptr = mm_ptr;
     *ctrl = &b->handle;
+    return 0;
+}
+
+// The reference maps BAR0 of the device behind `fd` (a /dev/libnvmN node of its kernel module, or a sysfs resource
+// file) and reads the handle from it (src/ctrl.cpp:147-199, src/linux/device.cpp:137-160).  The same here for any
+// descriptor that can be mapped shared and read-write: errno of the failing call otherwise (EBADF, ENODEV, EACCES ...).
+int nvm_ctrl_init(nvm_ctrl_t** ctrl, int fd)
+{
+    if (!ctrl) return EINVAL;
+    *ctrl = nullptr;
+    if (fcntl(fd, F_GETFL) == -1) return errno;
+    void* mm = mmap(nullptr, NVM_CTRL_MEM_MINSIZE, PROT_READ | PROT_WRITE, MAP_SHARED, fd, 0);
+    if (mm == MAP_FAILED) return errno ? errno : ENODEV;
+    int err = nvm_raw_ctrl_init(ctrl, mm, NVM_CTRL_MEM_MINSIZE);
+    if (err) { munmap(mm, NVM_CTRL_MEM_MINSIZE); return err; }
+    box_of(*ctrl)->mapped = mm;
+    box_of(*ctrl)->mapped_size = NVM_CTRL_MEM_MINSIZE;
     return 0;
 }
 

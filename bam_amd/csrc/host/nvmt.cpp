@@ -254,11 +254,21 @@ bool post_cpl(nvmt* t, Stats& st_, Cq& cq, uint16_t sqid, uint16_t sqhd, uint16_
         cpu_relax();
     }
     nvm_cpl_t* e = cq.mem + cq.tail;
+    const uint32_t dw2 = (uint32_t)sqhd | ((uint32_t)sqid << 16);
+    const uint32_t dw3 = (uint32_t)cid | (cq.phase << 16) | ((uint32_t)status << 17);
+#if defined(__x86_64__)
+    // The whole entry as one aligned 16-byte store.  The ring may be device memory reached through a write-combining
+    // window, where separate stores to one entry can leave in pieces and in any order; a 16-byte store leaves in one
+    // piece or in aligned halves, and SQHD shares its half with the phase tag, which is what the consumer reads together.
+    std::atomic_thread_fence(std::memory_order_release);
+    _mm_store_si128((__m128i*)e, _mm_set_epi32((int)dw3, (int)dw2, 0, (int)dw0));
+#else
     e->dword[0] = dw0;
     e->dword[1] = 0;
-    e->dword[2] = (uint32_t)sqhd | ((uint32_t)sqid << 16);
+    e->dword[2] = dw2;
     // DW3 carries the phase tag: it must become visible last
-    st<uint32_t>(&e->dword[3], (uint32_t)cid | (cq.phase << 16) | ((uint32_t)status << 17));
+    st<uint32_t>(&e->dword[3], dw3);
+#endif
     cq.tail = next;
     if (next == 0) cq.phase ^= 1;
     if (status) st_.bump(st_.error_cpls);
@@ -338,6 +348,8 @@ void serve_sq(nvmt* t, IoThread* me, Sq& sq)
             const uint16_t cid = batch[order[k]].dword[0] >> 16;
             if (!post_cpl(t, st_, cq, sq.id, (uint16_t)sq.head, cid, statuses[k], 0)) return;
         }
+        copy_out_fence();       // completions written through a write-combining window (a ring in device memory) leave now
+
     }
 }
 

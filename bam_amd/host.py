@@ -131,9 +131,12 @@ class PageCache:
 
     def profile(self, reset=True):
         """Miss-path phase timers (only a library built with -DBAM_PROFILE fills them)."""
-        out = (c_u64 * 16)()
+        out = (c_u64 * 32)()
         _chk(self.L.bam_page_cache_profile(self.h, out, int(reset)), "bam_page_cache_profile")
-        keys = ("batches", "commands", "t_cid", "t_submit", "t_wait", "t_copy", "t_find_slot", "find_slot_calls", "find_slot_lanes")
+        keys = ("batches", "commands", "t_cid", "t_submit", "t_wait", "t_copy", "t_find_slot", "find_slot_calls", "find_slot_lanes",
+                "t_sq_ticket", "t_sq_write", "t_sq_cover", "sq_cover_trips", "sq_sweeps", "sq_swept", "sq_doorbells",
+                "cq_wait_trips", "cq_drains", "cq_drained", "t_cq_drain", "cq_empty_looks", "t_cq_notice",
+                "n_ld_dev", "t_ld_dev", "n_sqe_store", "t_sqe_store", "t_doorbell", "n_ld_cqe", "t_ld_cqe")
         return dict(zip(keys, list(out)))
 
     def block_io(self, n_reqs, req_bytes, lbas=None, write=False, queue_policy=1, block_size=64):
@@ -271,6 +274,14 @@ class Array:
         out = torch.empty(n_elems + 1, dtype=torch.int64, device=f"cuda:{self.device}")
         _chk(self.L.bam_scan(self.h, n_elems, block_size, _ptr(out), _stream()), "bam_scan")
         return out
+
+    def update(self, api, assignment, values, block_size=64):
+        """element assignment[t] += values[t] through AtomicAdd (api 0), an atomic on bam_ptr::memref (1) or ptr[i] += v (2);
+        returns what each element held before (int64 tensor of bit patterns)."""
+        n = assignment.numel()
+        old = torch.zeros(n, dtype=torch.int64, device=f"cuda:{self.device}")
+        _chk(self.L.bam_array_update(self.h, api, n, _ptr(assignment), _ptr(values), _ptr(old), block_size, _stream()), "bam_array_update")
+        return old
 
     def pagerank(self, offsets, alpha=0.85, tolerance=0.001, max_iterations=100, by_page=False):
         """PageRank values (float32) by residual pushes over the CSR whose neighbour ids this array holds, and the sweeps taken."""

@@ -67,10 +67,14 @@ void bam_page_cache_destroy(bam_page_cache_t* pc);
 /* out[5]: n_pages, page_size, wave_batch, staged(0/1), of every 8 read batches how many bypass the staging pages */
 int bam_page_cache_info(bam_page_cache_t* pc, uint64_t* out);
 int bam_page_cache_flush(bam_page_cache_t* pc);
-/* phase timers of the miss path (100 MHz ticks), non-zero only in a library built with -DBAM_PROFILE; out16[0..8]:
- * I/O batches, commands, ticks waiting for command ids, submitting, waiting for completions, moving payload,
- * ticks in the victim search, victim searches, lanes searching */
-int bam_page_cache_profile(bam_page_cache_t* pc, uint64_t* out16, int reset);
+/* phase timers of the miss path (100 MHz ticks, summed over the batches of the cache's first controller), non-zero only in
+ * a library built with -DBAM_PROFILE (make prof); out32[0..8]: I/O batches, commands, ticks waiting for command ids,
+ * submitting, waiting for completions, moving payload, ticks in the victim search, victim searches, lanes searching;
+ * [9..15] inside the submission: ticks for the slot tickets, until the entries are written and marked, until they are
+ * covered by a doorbell, trips of that wait, tail sweeps done, entries swept, doorbells; [16..21] inside the wait for
+ * completions: trips, ring drains done by the waiting wave, entries drained, ticks draining, looks at an empty ring,
+ * ticks between the last drain that flagged this wave's commands and the wave noticing */
+int bam_page_cache_profile(bam_page_cache_t* pc, uint64_t* out32, int reset);
 int bam_range_create(bam_range_t** out, uint64_t index_start, uint64_t count, uint64_t page_start, uint64_t page_count,
                      uint64_t page_start_offset, uint64_t page_size, bam_page_cache_t* pc, uint32_t device, int dist);
 void bam_range_destroy(bam_range_t* r);
@@ -95,6 +99,20 @@ int bam_array_read_via(bam_array_t* a, int api, uint64_t n_reqs, const uint64_t*
 /* same request pattern through array_d_t::operator() (seq_write): element <- d_values[t] */
 int bam_array_write(bam_array_t* a, uint64_t n_reqs, const uint64_t* d_assignment, uint64_t stride, const uint64_t* d_values,
                     uint32_t block_size, void* stream);
+
+/* read-modify-write through the three routes the reference's kernels have for it: element d_assignment[t] += d_values[t],
+ * d_old[t] (may be NULL) = what the element held before.  api 0: array_d_t::AtomicAdd (include/page_cache.h:1647), api 1:
+ * an atomic add on the address bam_ptr::memref returns (:467), api 2: ptr[i] += v on a non-const bam_ptr (:478; a plain read
+ * and write, so the indices of one launch must be distinct).  The pages touched are dirty afterwards and reach the store
+ * on eviction or bam_page_cache_flush. */
+int bam_array_update(bam_array_t* a, int api, uint64_t n_reqs, const uint64_t* d_assignment, const uint64_t* d_values, uint64_t* d_old,
+                     uint32_t block_size, void* stream);
+/* The submission entry the device path builds for one read or write (nvm_cmd_header / nvm_cmd_data_ptr / nvm_cmd_rw_blks,
+ * include/nvm_cmd.h:54-88 of the reference; with seal != 0 also nvm_cmd_seal for slot ticket `ticket`): host_out16 (may be
+ * NULL) receives the 16 dwords as the host compiler encodes them, d_out64x16 (device memory, may be NULL) 64 entries
+ * encoded by the 64 lanes of one wave, lane l for command id cid + l, block lba + l and ticket + l. */
+int bam_sqe_image(uint16_t cid, uint8_t opcode, uint32_t nsid, uint64_t prp1, uint64_t prp2, uint64_t lba, uint16_t n_blocks, int seal, uint32_t ticket,
+                  uint32_t* host_out16, uint32_t* d_out64x16, void* stream);
 
 /* ---- cache / pattern benchmark kernels (benchmarks/cache/main.cu:44-114, benchmarks/pattern/main.cu:105-170) ----
  * One wave per run of n_pages_per_wave whole pages starting at page d_assignment[w] (or w * n_pages_per_wave),

@@ -120,6 +120,9 @@ __device__ __forceinline__ void for_each_group(const uint64_t key, F&& body)
 /* compute-unit identity across the whole device: XCC, shader engine and CU bits */
 __device__ __forceinline__ uint32_t cu_id() { return __smid(); }
 
+/* which of the device's clusters of compute units (XCDs) this wave runs on */
+__device__ __forceinline__ uint32_t xcc_id() { return __builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20) & 7u; }
+
 /*
  * A number that differs between the waves resident on the device at one time
  * and is spread evenly: hash of the hardware wave slot (XCC, SE, CU, SIMD,

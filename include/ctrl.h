@@ -50,9 +50,15 @@ struct Controller
     uint32_t                blk_size;
     uint32_t                blk_size_log;
     bam_guard_t*            guard;          /* host-pinned; shared by every queue of this controller */
+    bam_dma_place           cq_place;       /* completion rings in host-pinned or in device memory */
+    int                     sq_seal;        /* submission entries sealed (nvm_cmd_seal) */
+    uint32_t                sq_flush;       /* unsealed queues: nvm_queue_t::flush */
+    uint32_t                pull_limit;     /* waves per compute-unit cluster that pull staged payload at a time (0 = no limit) */
     void*                   d_ctrl_ptr;
 
-    struct Owners { DmaPtr aq_mem; BufferPtr d_ctrl_buff, guard_buff; };
+    unsigned long long*     prof;           /* [32] phase timers of the miss path in device memory (100 MHz ticks; builds with BAM_PROFILE fill them) */
+
+    struct Owners { DmaPtr aq_mem; BufferPtr d_ctrl_buff, guard_buff, prof_buff, pull_buff; };
     Owners*                 own;
 
     Controller(const char* path, uint32_t nvmNamespace, uint32_t hipDevice, uint64_t queueDepth, uint64_t numQueues,
@@ -158,10 +164,26 @@ private:
         guard->abort = 0;
         guard->spin_limit = spin_limit;
 
+        own->prof_buff = createBuffer(32 * sizeof(unsigned long long), deviceId);
+        prof = (unsigned long long*)own->prof_buff.get();
         h_qps = (QueuePair**)calloc(n_qps, sizeof(QueuePair*));
         hip_err_chk(hipMalloc((void**)&d_qps, sizeof(QueuePair) * n_qps));
+        /* runtime policy of the queue pairs: where the completion rings live, whether submission entries are sealed, and
+         * what an unsealed queue does to know its entries have arrived (see QueuePair and nvm_parallel_queue.h) */
+        cq_place = BAM_DMA_DEVICE; sq_seal = 1; sq_flush = 2;
+        if (const char* e = getenv("BAM_CQ_PLACE")) cq_place = (e[0] == 'd' || e[0] == '1') ? BAM_DMA_DEVICE : BAM_DMA_HOST;
+        if (const char* e = getenv("BAM_SQ_SEAL")) sq_seal = atoi(e) != 0;
+        if (const char* e = getenv("BAM_SQ_FLUSH")) sq_flush = (uint32_t)atoi(e);
+        /* staged payload is pulled from host memory by the waves themselves, and a compute unit returns the loads of
+         * all its waves in order: while one wave waits for host memory, every other load of that unit waits with it.
+         * With more pulls in flight than the interconnect needs to stay busy, each waits longer and so does everybody
+         * else; the number of waves pulling at a time is therefore bounded (per cluster of compute units). */
+        pull_limit = 8;
+        if (const char* e = getenv("BAM_PULL_LIMIT")) pull_limit = (uint32_t)atoi(e);
+        own->pull_buff = createBuffer(8 * 64, deviceId);
         for (size_t i = 0; i < n_qps; i++) {
-            h_qps[i] = new QueuePair(ctrl, deviceId, ns, info, aq_ref, (uint16_t)(i + 1), queueDepth, guard, stage_bytes);
+            h_qps[i] = new QueuePair(ctrl, deviceId, ns, info, aq_ref, (uint16_t)(i + 1), queueDepth, guard, stage_bytes, BAM_DMA_HOST, cq_place, sq_seal, sq_flush, prof,
+                                     (uint32_t*)own->pull_buff.get(), pull_limit);
             h_qps[i]->bind_device(d_qps + i);
             hip_err_chk(hipMemcpy((void*)(d_qps + i), (const void*)h_qps[i], sizeof(QueuePair), hipMemcpyHostToDevice));
         }

@@ -1,9 +1,9 @@
 /*
  * Controller handle.  Replaces include/nvm_ctrl.h of the reference
- * (nvm_raw_ctrl_init :53, nvm_ctrl_free :60, nvm_raw_ctrl_reset :76).  The
- * fd/ioctl variant nvm_ctrl_init(ctrl, fd) :41 needs the reference's kernel
- * module and is not provided; the register window comes from the software
- * NVMe target (nvmt.h) or from a caller that has mapped a real BAR0.
+ * (nvm_ctrl_init :36, nvm_raw_ctrl_init :53, nvm_ctrl_free :60,
+ * nvm_raw_ctrl_reset :76).  The register window comes from the software NVMe
+ * target (nvmt.h), from a caller that has mapped a real BAR0, or from a
+ * descriptor that nvm_ctrl_init maps itself.
  */
 #ifndef __NVM_CTRL_H__
 #define __NVM_CTRL_H__
@@ -16,6 +16,10 @@
 #ifdef __cplusplus
 extern "C" {
 #endif
+/* Map the first NVM_CTRL_MEM_MINSIZE bytes behind `fd` shared and read-write (BAR0 of a device node or sysfs resource
+ * file) and build a handle from the registers found there; the mapping goes with the handle's last reference.  0 or
+ * errno (EBADF not a descriptor, ENODEV/EACCES it cannot be mapped, EINVAL/ERANGE as nvm_raw_ctrl_init). */
+int nvm_ctrl_init(nvm_ctrl_t** ctrl, int fd);
 /* Read CAP from a mapped register window and build a handle.  0 or errno
  * (EINVAL window too small, ERANGE host page size outside MPSMIN..MPSMAX). */
 int nvm_raw_ctrl_init(nvm_ctrl_t** ctrl, volatile void* mm_ptr, size_t mm_size);

@@ -33,14 +33,29 @@
 #define LOCKED   1
 #define UNLOCKED 0
 #define BAM_CID_DONE 2u
+#define BAM_CID_ERR  4u          /* completed with a non-zero status: the transfer did not happen */
 
 namespace bam {
 
-#ifndef BAM_CQ_IDLE_TICKS
-#define BAM_CQ_IDLE_TICKS 200u          /* 100 MHz ticks between looks at an idle completion ring */
-#endif
-
 struct spin_t { uint32_t n = 0, slp = 1; uint64_t t0 = 0; };
+
+/* phase timers: compiled in with -DBAM_PROFILE only */
+#ifdef BAM_PROFILE
+/* the clock, read once everything the wave has in flight has come back (the clock is a scalar read that the hardware
+ * would otherwise let overtake vector memory operations it does not depend on) */
+__device__ __forceinline__ uint64_t prof_clock()
+{
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    const uint64_t t = wall_clock64();
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    return t;
+}
+#define BAM_PROF_NOW() bam::prof_clock()
+#define BAM_PROF_ADD(q, i, v) do { if ((q)->prof) atomicAdd(&(q)->prof[i], (unsigned long long)(v)); } while (0)
+#else
+#define BAM_PROF_NOW() 0ull
+#define BAM_PROF_ADD(q, i, v) do { } while (0)
+#endif
 
 /*
  * One back-off step of a wait loop; true = give up.  Every 256 steps the loop
@@ -131,8 +146,10 @@ __device__ __forceinline__ void cq_drain_group(nvm_queue_t* cq, nvm_queue_t* sq,
  * waiting wave comes through here, so an idle ring must cost next to nothing:
  * the holder of head_lock first reads the one entry at the head (a single
  * small read), and only when that entry is new does the group read a window
- * of 64; after an empty look the queue is left alone for two microseconds
- * (the time is kept in the otherwise unused `tail` word of the CQ descriptor).
+ * of 64; after an empty look a ring in host memory is left alone for
+ * cq->idle_ticks (two microseconds; the time is kept in the otherwise unused
+ * `tail` word of the CQ descriptor).  A ring in device memory has no such
+ * pause: a look at it stays on the device.
  */
 __device__ __forceinline__ bool try_drain_group(nvm_queue_t* cq, nvm_queue_t* sq)
 {
@@ -141,24 +158,29 @@ __device__ __forceinline__ bool try_drain_group(nvm_queue_t* cq, nvm_queue_t* sq
     uint32_t got = 0;
     if (lane() == leader) {
         /* the word holds the time of the next look (low 32 bits of the clock): wait only while that lies within
-         * the next two microseconds, so that a stale or never-written value can never hold anybody up */
-        const uint32_t ahead = ld_relaxed(&cq->tail) - (uint32_t)wall_clock64();
-        if (ahead - 1u >= BAM_CQ_IDLE_TICKS && ld_relaxed(&cq->head_lock) == UNLOCKED &&
+         * the next idle_ticks, so that a stale or never-written value can never hold anybody up */
+        const uint32_t idle = cq->idle_ticks;
+        const uint32_t ahead = idle ? ld_relaxed(&cq->tail) - (uint32_t)wall_clock64() : 0u;
+        if (ahead - 1u >= idle && ld_relaxed(&cq->head_lock) == UNLOCKED &&
             __hip_atomic_exchange(&cq->head_lock, (uint32_t)LOCKED, __ATOMIC_RELAXED, BAM_AGENT) == UNLOCKED) {
             fence_meta();
             const uint32_t h = ld_relaxed(&cq->head);
+            [[maybe_unused]] const uint64_t po5 = BAM_PROF_NOW();
             const uint32_t dw3 = ld_relaxed_sys(&((nvm_cpl_t*)cq->vaddr)[h & cq->qs_minus_1].dword[3]);
+            BAM_PROF_ADD(cq, 27, 1); BAM_PROF_ADD(cq, 28, BAM_PROF_NOW() - po5);
             if (((dw3 >> 16) & 1u) == ((~(h >> cq->qs_log2)) & 1u)) got = 1;
             else {
-                st_relaxed(&cq->tail, (uint32_t)wall_clock64() + BAM_CQ_IDLE_TICKS);      /* nothing new: leave the ring alone for a while */
+                if (idle) st_relaxed(&cq->tail, (uint32_t)wall_clock64() + idle);      /* nothing new: leave the ring alone for a while */
                 st_publish(&cq->head_lock, (uint32_t)UNLOCKED);
+                BAM_PROF_ADD(cq, 20, 1);
             }
         }
     }
     got = bcast(got, leader);
     if (got) {
+        [[maybe_unused]] const uint64_t pd0 = BAM_PROF_NOW();
         cq_drain_group(cq, sq, act);
-        if (lane() == leader) st_publish(&cq->head_lock, (uint32_t)UNLOCKED);
+        if (lane() == leader) { st_publish(&cq->head_lock, (uint32_t)UNLOCKED); BAM_PROF_ADD(cq, 17, 1); BAM_PROF_ADD(cq, 19, BAM_PROF_NOW() - pd0); }
     }
     return got != 0;
 }
@@ -174,25 +196,57 @@ __device__ __forceinline__ uint32_t sq_enqueue_group(nvm_queue_t* sq, nvm_cmd_t*
     const uint32_t n = popc(act), rank = rank_in(act), leader = first_lane(act);
     const uint32_t mask = sq->qs_minus_1;
     uint32_t t0 = 0;
+    [[maybe_unused]] const uint64_t pq0 = BAM_PROF_NOW();
+    [[maybe_unused]] uint64_t pq2 = 0;
+    [[maybe_unused]] uint32_t p_trips = 0;
     if (lane() == leader) t0 = __hip_atomic_fetch_add(&sq->in_ticket, n, __ATOMIC_RELAXED, BAM_AGENT);
     t0 = bcast(t0, leader);
+    [[maybe_unused]] const uint64_t pq1 = BAM_PROF_NOW();
     const uint32_t ticket = t0 + rank, pos = ticket & mask;
-    const uint32_t want = (ticket >> sq->qs_log2) * 2u;      /* slot is free for my lap when tickets[pos] == want */
     if (sq->sealed) nvm_cmd_seal(cmd, ticket);
     bool written = false;
     spin_t sp;
     for (;;) {
-        if (!written && ld_relaxed(&sq->tickets[pos].val) == want) {
+#ifdef BAM_PROFILE
+        const uint64_t po0 = BAM_PROF_NOW();
+        const uint32_t slot_word = ld_relaxed(&sq->tickets[pos].val);
+        const uint64_t po1 = BAM_PROF_NOW();
+        if (lane() == leader && !written) { BAM_PROF_ADD(sq, 22, 1); BAM_PROF_ADD(sq, 23, po1 - po0); }
+#else
+        const uint32_t slot_word = ld_relaxed(&sq->tickets[pos].val);
+#endif
+        if (!written && nvm_sq_slot_free(slot_word, ticket, sq->qs_log2)) {
             fence_meta();
+            [[maybe_unused]] const uint64_t po2 = BAM_PROF_NOW();
             /* written through to the ring, which may be host memory the L2 would otherwise hold on to */
             uint64_t* dst = (uint64_t*)(((nvm_cmd_t*)sq->vaddr) + pos);
             const uint64_t* src = (const uint64_t*)cmd->dword;
 #pragma unroll
             for (int i = 0; i < 8; i++) __hip_atomic_store(dst + i, src[i], __ATOMIC_RELAXED, BAM_SYSTEM);
-            /* the entry must have left for the controller before the mark can be swept into a doorbell */
+            /*
+             * The entry must be in the ring before its mark can be swept into a doorbell.  A sealed queue leaves that
+             * to the controller (it takes an entry only once the seal verifies).  An unsealed one (a controller that
+             * follows the NVMe specification to the letter) has to know: the wait on the wave's own store counters
+             * says that the stores have been handed on, not that they have arrived, and the doorbell, written later by
+             * another wave, may travel another way.  Reading the entry back does say so: the reply to a read does not
+             * pass writes posted before it.
+             */
+#ifdef BAM_PROFILE
+            { const uint64_t po3 = BAM_PROF_NOW(); if (lane() == leader) { BAM_PROF_ADD(sq, 24, 1); BAM_PROF_ADD(sq, 25, po3 - po2); } }
+#endif
+            if (!sq->sealed) {
+                if (sq->flush == 1u) fence_release_sys();
+                else if (sq->flush == 2u) {
+                    fence_meta();
+                    const uint64_t back = __hip_atomic_load(dst + 7, __ATOMIC_RELAXED, BAM_SYSTEM);
+                    asm volatile("" :: "v"(back));
+                }
+            }
             st_publish(&sq->tail_mark[pos].val, 1u);
             written = true;
         }
+        if (!pq2 && !ballot(!written)) pq2 = BAM_PROF_NOW();
+        p_trips++;
         const uint32_t tl = ld_relaxed(&sq->tail);
         const bool covered = written && (int32_t)(tl - ticket) > 0;
         if (!ballot(!covered)) break;
@@ -221,10 +275,14 @@ __device__ __forceinline__ uint32_t sq_enqueue_group(nvm_queue_t* sq, nvm_cmd_t*
                 fence_meta();                /* the marks read and cleared above: before the doorbell and the unlock */
                 if (lane() == leader) {
                     if (total) {
+                        [[maybe_unused]] const uint64_t po4 = BAM_PROF_NOW();
                         st_relaxed_sys(sq->db, (cur + total) & mask);     /* one doorbell for the whole run */
+                        BAM_PROF_ADD(sq, 26, BAM_PROF_NOW() - po4);
                         st_relaxed(&sq->tail, cur + total);
+                        BAM_PROF_ADD(sq, 15, 1); BAM_PROF_ADD(sq, 14, total);
                     }
                     st_publish(&sq->tail_lock, (uint32_t)UNLOCKED);
+                    BAM_PROF_ADD(sq, 13, 1);
                 }
                 progressed = total != 0;
             }
@@ -236,6 +294,13 @@ __device__ __forceinline__ uint32_t sq_enqueue_group(nvm_queue_t* sq, nvm_cmd_t*
             if (spin_giveup(sq, sp)) break;
         }
     }
+#ifdef BAM_PROFILE
+    if (lane() == leader) {
+        const uint64_t pq3 = BAM_PROF_NOW();
+        if (!pq2) pq2 = pq3;
+        BAM_PROF_ADD(sq, 9, pq1 - pq0); BAM_PROF_ADD(sq, 10, pq2 - pq1); BAM_PROF_ADD(sq, 11, pq3 - pq2); BAM_PROF_ADD(sq, 12, p_trips);
+    }
+#endif
     return pos;
 }
 
@@ -254,20 +319,21 @@ __device__ __forceinline__ void cq_drain_group(nvm_queue_t* cq, nvm_queue_t* sq,
     for (;;) {
         const uint32_t idx = h + moved + rank, loc = idx & mask;
         const uint32_t phase = (~(idx >> cq->qs_log2)) & 1u;          /* first lap carries phase 1 */
-        const uint32_t dw3 = ld_relaxed_sys(&ring[loc].dword[3]);
+        /* SQHD and the phase tag in one access: the controller may write an entry in pieces of eight bytes */
+        const uint64_t dw23 = __hip_atomic_load((uint64_t*)&ring[loc].dword[2], __ATOMIC_RELAXED, BAM_SYSTEM);
+        const uint32_t dw3 = (uint32_t)(dw23 >> 32);
         fence_meta();
         const bool valid = ((dw3 >> 16) & 1u) == phase && moved + rank < mask;
         const uint32_t run = leading_run(act, ballot(valid));
         if (rank < run) {
-            if (dw3 >> 17) __hip_atomic_fetch_add(&cq->n_errors, 1u, __ATOMIC_RELAXED, BAM_AGENT);
-            st_relaxed(&sq->cid[dw3 & sq->cid_mask].val, (uint32_t)LOCKED | BAM_CID_DONE);
+            const bool err = (dw3 >> 17) != 0;
+            if (err) __hip_atomic_fetch_add(&cq->n_errors, 1u, __ATOMIC_RELAXED, BAM_AGENT);
+            st_relaxed(&sq->cid[dw3 & sq->cid_mask].val, (uint32_t)LOCKED | BAM_CID_DONE | (err ? BAM_CID_ERR : 0u));
         }
         if (run) {
-            uint32_t v = 0;
-            if (rank == run - 1) v = ld_relaxed_sys(&ring[loc].dword[2]) & 0xffffu;
             /* lane holding the newest entry of the run */
-            uint64_t holder = ballot(rank == run - 1);
-            sqhd = bcast(v, first_lane(holder));
+            const uint64_t holder = ballot(rank == run - 1);
+            sqhd = bcast((uint32_t)dw23 & 0xffffu, first_lane(holder));
         }
         moved += run;
         if (run < n) break;
@@ -283,22 +349,32 @@ __device__ __forceinline__ void cq_drain_group(nvm_queue_t* cq, nvm_queue_t* sq,
             if (freed) st_relaxed(&sq->head, sh + freed);
             st_relaxed_sys(cq->db, (h + moved) & mask);                /* one doorbell for the whole run */
             st_relaxed(&cq->head, h + moved);
+            BAM_PROF_ADD(cq, 18, moved);
         }
     }
 }
 
-/* Wait until the command `cid` of every active lane has completed on (sq, cq) (wave-uniform). */
-__device__ __forceinline__ void cq_wait_group(nvm_queue_t* cq, nvm_queue_t* sq, uint32_t cid)
+/*
+ * Wait until the command `cid` of every active lane has completed on (sq, cq) (wave-uniform).  True for the lanes
+ * whose command completed without an error status; false where the transfer did not happen (error completion) or
+ * nobody knows (the wait was given up).
+ */
+__device__ __forceinline__ bool cq_wait_group(nvm_queue_t* cq, nvm_queue_t* sq, uint32_t cid)
 {
     spin_t sp;
+    uint32_t w;
+    [[maybe_unused]] uint32_t p_trips = 0;
     for (;;) {
-        const bool done = (ld_relaxed(&sq->cid[cid].val) & BAM_CID_DONE) != 0;
-        if (!ballot(!done)) break;
+        w = ld_relaxed(&sq->cid[cid].val);
+        if (!ballot((w & BAM_CID_DONE) == 0)) break;
+        p_trips++;
         try_drain_group(cq, sq);
         if (spin_giveup(cq, sp)) break;
     }
+    if (lane() == first_lane(active_mask())) BAM_PROF_ADD(cq, 16, p_trips);
     /* what the controller wrote before posting the completion is visible from here on */
     fence_acquire_sys();
+    return (w & (BAM_CID_DONE | BAM_CID_ERR)) == BAM_CID_DONE;
 }
 
 } // namespace bam

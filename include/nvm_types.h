@@ -86,6 +86,10 @@ typedef struct
     padded_struct*          pos_locks;      /* SQ [n_cids / 64]: command ids are handed out to a wave in blocks of 64; turn counter of each block */
     uint32_t                cid_mask;       /* n_cids - 1 */
     uint32_t                sealed;         /* SQ: entries carry a sequence number and checksum (nvm_cmd_seal) */
+    uint32_t                flush;          /* SQ, unsealed: how a written entry is known to have reached the ring before its mark is set
+                                               (0 nothing beyond the wave's own store counters, 1 system-scope release, 2 read the entry back) */
+    uint32_t                idle_ticks;     /* CQ: 100 MHz ticks an empty ring is left alone after a look (0: ring in device memory, a look costs nothing) */
+    unsigned long long*     prof;           /* device path: [32] phase timers, filled only by builds with BAM_PROFILE (may be NULL) */
     struct bam_guard*       guard;          /* device path: bounded-wait control (may be NULL) */
     uint32_t                spin_limit;     /* device path: copy of guard->spin_limit */
     void*                   pair;           /* device path: the CQ of an SQ / the SQ of a CQ (device address) */
@@ -101,6 +105,20 @@ typedef struct
     volatile void*          vaddr;          /* Queue memory */
     uint64_t                ioaddr;         /* Bus address of queue memory */
 } nvm_queue_t;
+
+/*
+ * Is SQ slot `ticket & (qs - 1)` free for the submitter holding `ticket`?  tickets[slot] counts 2 per lap (the
+ * drainer adds 2 when the controller has consumed the slot's entry), the lap of a ticket is ticket >> qs_log2.
+ * The 32-bit ticket counter wraps after 2^(32 - qs_log2) laps while the slot word keeps counting to twice that,
+ * so the two are compared modulo the lap range.
+ */
+__host__ __device__ static inline
+int nvm_sq_slot_free(uint32_t slot_word, uint32_t ticket, uint32_t qs_log2)
+{
+    const uint32_t want = (ticket >> qs_log2) * 2u;
+    const uint32_t lap_mask = (uint32_t)((2ull << (32u - qs_log2)) - 1ull);
+    return ((slot_word - want) & lap_mask) == 0;
+}
 
 typedef struct __attribute__((aligned(32)))
 {

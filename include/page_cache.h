@@ -66,6 +66,14 @@ enum data_dist_t { REPLICATE = 0, STRIPE = 1 };
 #define V_NB  0x02U
 #define V_B   0x03U
 
+/*
+ * data_page_t::offset: the cache slot in the low BAM_SLOT_BITS bits, above them a count of how many times the page has
+ * been loaded (mod 32).  Readers that take no reference (bam_read_unpinned) look at the descriptor before and after
+ * their load and need the second look to tell them that the page has not left the slot and come back in between.
+ */
+#define BAM_SLOT_BITS 27u
+#define BAM_SLOT_MASK ((1u << BAM_SLOT_BITS) - 1u)
+
 #define BAM_TOKEN_SLOTS 4096u
 #define BAM_STAT_SHARDS 4096
 
@@ -123,9 +131,10 @@ struct page_cache_d_t {
     bool prps;
     uint64_t n_blocks_per_page;
     uint32_t wave_batch;             /* distinct pages one wave loads side by side (64: a whole wave) */
+    uint32_t fast_reads;             /* element reads (seq_read, operator[]) of resident pages take no reference: bam_read_unpinned */
     uint32_t* miss_tokens;           /* number of waves inside the miss path right now */
     uint32_t miss_waves;             /* at most this many at a time per compute unit (0 = no limit) */
-    unsigned long long* prof;        /* [16] phase timers in 100 MHz ticks, filled only by builds with BAM_PROFILE */
+    unsigned long long* prof;        /* [32] phase timers in 100 MHz ticks (the first controller's), filled only by builds with BAM_PROFILE */
     bam_guard_t* guard;
     uint32_t spin_limit;
 
@@ -182,6 +191,35 @@ __device__ __forceinline__ void copy_pages(uint8_t* dst, const uint8_t* src, uin
         for (; i < nb; i += movers) d[i] = s[i];
     }
 }
+/*
+ * Permission to pull staged payload from host memory, taken by the wave (all active lanes call, one lane acts) before
+ * it loads from a staging page and given back when the loads are in: see Controller::pull_limit.  The holder waits for
+ * nothing but its own loads, so the permission always comes back; a wait that is given up goes ahead without one.
+ */
+__device__ __forceinline__ uint32_t* pull_begin(QueuePair* qp)
+{
+    const uint32_t limit = qp->pull_limit;
+    if (!limit) return nullptr;
+    uint32_t* word = qp->pull_tokens + xcc_id() * 16u;
+    if (lane() == first_lane(active_mask())) {
+        spin_t sp;
+        for (;;) {
+            if (ld_relaxed(word) < limit) {
+                if (__hip_atomic_fetch_add(word, 1u, __ATOMIC_RELAXED, BAM_AGENT) < limit) break;
+                __hip_atomic_fetch_add(word, 0u - 1u, __ATOMIC_RELAXED, BAM_AGENT);
+            }
+            if (spin_giveup(&qp->cq, sp)) { __hip_atomic_fetch_add(word, 1u, __ATOMIC_RELAXED, BAM_AGENT); break; }
+        }
+    }
+    return word;
+}
+__device__ __forceinline__ void pull_end(uint32_t* word)
+{
+    if (!word) return;
+    fence_meta();                    /* the loads from host memory have come back */
+    if (lane() == first_lane(active_mask())) __hip_atomic_fetch_add(word, 0u - 1u, __ATOMIC_RELAXED, BAM_AGENT);
+}
+
 /*
  * The same with helpers: called by all active lanes, of which those with `mine` have payload to move; the others
  * lend their load slots.  A wave that loads one page for all of its lanes (a bam_ptr walking an edge list) moves it
@@ -262,8 +300,9 @@ __device__ __forceinline__ uint32_t io_submit_group(page_cache_d_t* pc, QueuePai
     return cid;
 }
 
-/* the whole of one batch: submit, wait for all completions, move staged payload, recycle ids */
-__device__ __forceinline__ void io_group(page_cache_d_t* pc, QueuePair* qp, uint64_t lba, uint32_t n_blocks, uint64_t pc_entry, uint8_t opcode,
+/* the whole of one batch: submit, wait for all completions, move staged payload, recycle ids; true for the lanes whose
+ * transfer happened (completed, without an error status) */
+__device__ __forceinline__ bool io_group(page_cache_d_t* pc, QueuePair* qp, uint64_t lba, uint32_t n_blocks, uint64_t pc_entry, uint8_t opcode,
                                          const uint32_t direct_share)
 {
     const uint64_t act = active_mask();
@@ -273,16 +312,21 @@ __device__ __forceinline__ void io_group(page_cache_d_t* pc, QueuePair* qp, uint
 #ifdef BAM_PROFILE
     const uint64_t pt2 = wall_clock64();
 #endif
-    cq_wait_group(&qp->cq, &qp->sq, cid);
+    const bool ok = cq_wait_group(&qp->cq, &qp->sq, cid);
 #ifdef BAM_PROFILE
     const uint64_t pt3 = wall_clock64();
 #endif
-    if (stage && opcode == NVM_IO_READ)
-        copy_pages(pc->base_addr + pc_entry * pc->page_size, stage, n_blocks << qp->block_size_log, act, popc(act), rank_in(act));
+    /* a read that failed leaves its destination alone: the staging page holds what the last command of this id brought */
+    if (ballot(stage && opcode == NVM_IO_READ && ok)) {
+        uint32_t* pull = pull_begin(qp);
+        copy_pages(pc->base_addr + pc_entry * pc->page_size, stage, stage && opcode == NVM_IO_READ && ok ? n_blocks << qp->block_size_log : 0u, act, popc(act), rank_in(act));
+        pull_end(pull);
+    }
     put_cid_group(&qp->sq, cid);
 #ifdef BAM_PROFILE
     if (pc->prof && lane() == first_lane(act)) { atomicAdd(&pc->prof[4], pt3 - pt2); atomicAdd(&pc->prof[5], wall_clock64() - pt3); }
 #endif
+    return ok;
 }
 
 } // namespace bam
@@ -302,16 +346,17 @@ inline __device__ void access_data(page_cache_d_t* pc, QueuePair* qp, const uint
  * with several groups each one runs its whole transfer before the next starts, and `held` comes back false.
  */
 inline __device__ void read_begin(page_cache_d_t* pc, QueuePair* qp, const uint64_t starting_lba, const uint64_t n_blocks, const unsigned long long pc_entry,
-                                  uint32_t& cid, uint8_t*& stage, bool& held)
+                                  uint32_t& cid, uint8_t*& stage, bool& held, bool& ok)
 {
     const uint64_t all = bam::active_mask();
     const bool one_group = bam::ballot(qp == (QueuePair*)bam::first((uint64_t)qp) && pc == (page_cache_d_t*)bam::first((uint64_t)pc)) == all;
     held = one_group;
     stage = nullptr;
     cid = 0;
+    ok = false;
     if (!one_group) {
         bam::for_each_group((uint64_t)qp, (uint64_t)pc, [&](uint64_t q, uint64_t c) {
-            bam::io_group((page_cache_d_t*)c, (QueuePair*)q, starting_lba, (uint32_t)n_blocks, pc_entry, NVM_IO_READ, ((page_cache_d_t*)c)->direct_share);
+            ok = bam::io_group((page_cache_d_t*)c, (QueuePair*)q, starting_lba, (uint32_t)n_blocks, pc_entry, NVM_IO_READ, ((page_cache_d_t*)c)->direct_share);
         });
         return;
     }
@@ -322,7 +367,7 @@ inline __device__ void read_begin(page_cache_d_t* pc, QueuePair* qp, const uint6
 #ifdef BAM_PROFILE
     const uint64_t pt2 = wall_clock64();
 #endif
-    bam::cq_wait_group(&cur->cq, &cur->sq, cid);
+    ok = bam::cq_wait_group(&cur->cq, &cur->sq, cid);
 #ifdef BAM_PROFILE
     if (cpc->prof && bam::lane() == bam::first_lane(all)) atomicAdd(&cpc->prof[4], wall_clock64() - pt2);
 #endif
@@ -358,8 +403,10 @@ inline __device__ void access_data_async(page_cache_d_t* pc, QueuePair* qp, cons
         uint8_t* stage;
         uint32_t pos;
         const uint32_t id = bam::io_submit_group(cpc, cur, starting_lba, (uint32_t)n_blocks, pc_entry, opcode, stage, pos, cpc->direct_share_raw);
-        if (stage) {
-            cur->async_dst[id] = opcode == NVM_IO_READ ? (uint64_t)(cpc->base_addr + pc_entry * cpc->page_size) : 0;
+        /* written for every command of a queue pair that has staging pages, staged or not: the id may have been used
+         * by a staged read before, and poll_async must not find that command's destination */
+        if (cur->stage) {
+            cur->async_dst[id] = stage && opcode == NVM_IO_READ ? (uint64_t)(cpc->base_addr + pc_entry * cpc->page_size) : 0;
             cur->async_len[id] = (uint32_t)n_blocks << cur->block_size_log;
         }
         *cid = (uint16_t)id;
@@ -373,12 +420,15 @@ inline __device__ void poll_async(QueuePair* qp, uint16_t cid, uint16_t sq_pos)
     bam::for_each_group((uint64_t)qp, [&](uint64_t q) {
         QueuePair* cur = (QueuePair*)q;
         const uint64_t act = bam::active_mask();
-        bam::cq_wait_group(&cur->cq, &cur->sq, cid);
+        const bool ok = bam::cq_wait_group(&cur->cq, &cur->sq, cid);
         uint8_t* dst = nullptr;
         uint32_t len = 0;
-        if (cur->stage) { dst = (uint8_t*)cur->async_dst[cid]; len = cur->async_len[cid]; }
-        if (bam::ballot(dst != nullptr))
+        if (cur->stage && ok) { dst = (uint8_t*)cur->async_dst[cid]; len = cur->async_len[cid]; }
+        if (bam::ballot(dst != nullptr)) {
+            uint32_t* pull = bam::pull_begin(cur);
             bam::copy_pages(dst, cur->stage + (size_t)cid * cur->stage_stride, dst ? len : 0, act, bam::popc(act), bam::rank_in(act));
+            bam::pull_end(pull);
+        }
         bam::put_cid_group(&cur->sq, cid);
     });
 }
@@ -498,7 +548,7 @@ struct range_d_t {
     __forceinline__ __device__ void release_page(const size_t pg, const uint32_t count, const bool wrote) const { bam_release_refs(&pages[pg], count, wrote); }
     __forceinline__ __device__ void release_page(const size_t pg) const { release_page(pg, 1, true); }
     __forceinline__ __device__ void release_page(const size_t pg, const uint32_t count) const { release_page(pg, count, true); }
-    __forceinline__ __device__ cache_page_t* get_cache_page(const size_t pg) const { return cache.get_cache_page(pages[pg].offset); }
+    __forceinline__ __device__ cache_page_t* get_cache_page(const size_t pg) const { return cache.get_cache_page(pages[pg].offset & BAM_SLOT_MASK); }
     __forceinline__ __device__ uint64_t get_cache_page_addr(const uint32_t page_trans) const { return (uint64_t)(cache.base_addr + (uint64_t)page_trans * cache.page_size); }
     __forceinline__ __device__ void mark_page_dirty(const size_t index) { __hip_atomic_fetch_or(&pages[index].state, DIRTY, __ATOMIC_RELAXED, BAM_AGENT); }
     __forceinline__ __device__ uint64_t acquire_page(const size_t pg, const uint32_t count, const bool write, const uint32_t ctrl, const uint32_t queue);
@@ -541,8 +591,28 @@ __forceinline__ __device__ bool bam_try_hit(data_page_t* dp, const uint32_t coun
     const uint32_t s = (uint32_t)sv;
     if ((s >> (CNT_SHIFT + 1)) != V_NB) return false;
     if (write && (s & DIRTY) == 0) __hip_atomic_fetch_or(&dp->state, DIRTY, __ATOMIC_RELAXED, BAM_AGENT);
-    slot = (uint32_t)(sv >> 32);
+    slot = (uint32_t)(sv >> 32) & BAM_SLOT_MASK;
     return true;
+}
+
+/*
+ * Read one element of a resident page without taking a reference: look at the descriptor, load the element, and once it
+ * has arrived look at the descriptor again.  If both looks show the page valid, not busy, in the same slot and loaded
+ * the same number of times, the slot held the page for the whole of the load: an evictor sets BUSY before it touches
+ * anything, and a page that comes back carries a new load count.  False if the page is not resident or the looks
+ * differ; the caller then goes the counted way (bam_try_hit).  This takes both read-modify-write operations out of a
+ * hit: scattered over the descriptor table, the device does some ten thousand million such pairs per second, and five
+ * times as many plain loads.  Reads only: a writer needs the page to stay until it has marked it dirty.
+ */
+template <typename T>
+__forceinline__ __device__ bool bam_read_unpinned(const data_page_t* dp, const uint8_t* base_addr, const uint32_t page_size_log, const uint64_t in_page, T& out)
+{
+    const uint64_t s1 = __hip_atomic_load((const uint64_t*)dp, __ATOMIC_RELAXED, BAM_AGENT);
+    const bool resident = ((uint32_t)s1 >> (CNT_SHIFT + 1)) == V_NB;
+    if (resident) out = bam::ld_payload((const T*)(base_addr + ((uint64_t)((uint32_t)(s1 >> 32) & BAM_SLOT_MASK) << page_size_log) + in_page));
+    bam::fence_meta();                               /* the element is here before the second look goes out */
+    const uint64_t s2 = __hip_atomic_load((const uint64_t*)dp, __ATOMIC_RELAXED, BAM_AGENT);
+    return resident && ((s1 ^ s2) & 0xFFFFFFFFC0000000ull) == 0;
 }
 
 namespace bam {
@@ -594,7 +664,7 @@ bool range_d_t<T>::slow_step(const size_t pg, const bool write, const uint32_t q
         /* here only to help move payload */
     } else if (st == V_NB) {
         if (write && (s & DIRTY) == 0) __hip_atomic_fetch_or(&dp->state, DIRTY, __ATOMIC_RELAXED, BAM_AGENT);
-        slot = (uint32_t)(sv >> 32);
+        slot = (uint32_t)(sv >> 32) & BAM_SLOT_MASK;
         was_hit = true;
         resolved = true;
     } else if (st == NV_NB) {
@@ -611,7 +681,7 @@ bool range_d_t<T>::slow_step(const size_t pg, const bool write, const uint32_t q
     uint32_t found = BAM_NO_SLOT, cid = 0;
     uint8_t* stage = nullptr;
     QueuePair* qp = nullptr;
-    bool held = false;
+    bool held = false, io_ok = false;
     if (load_me) {
 #ifdef BAM_PROFILE
         const uint64_t pf0 = wall_clock64();
@@ -631,25 +701,56 @@ bool range_d_t<T>::slow_step(const size_t pg, const bool write, const uint32_t q
             stat_add((unsigned long long*)&ctl->access_counter, 1);
             stat_add(&shard()->read_io_cnt, 1);
             qp = ctl->d_qps + (queue % ctl->n_qps);
-            read_begin(&cache, qp, get_backing_page(pg) * cache.n_blocks_per_page, cache.n_blocks_per_page, found, cid, stage, held);
+            read_begin(&cache, qp, get_backing_page(pg) * cache.n_blocks_per_page, cache.n_blocks_per_page, found, cid, stage, held, io_ok);
         }
     }
     /* staged payload is moved by every lane that came in, whether it loaded a page itself or not */
 #ifdef BAM_PROFILE
     const uint64_t pc0 = wall_clock64();
 #endif
-    copy_pages_helped(cache.base_addr + (uint64_t)found * cache.page_size, stage, (uint32_t)cache.page_size, load_me && stage != nullptr);
+    if (bam::ballot(load_me && io_ok && stage != nullptr)) {
+        /* all lanes that came in are here: the queue pair of any lane that has payload to move will do for the permission */
+        QueuePair* pq = (QueuePair*)bam::bcast((uint64_t)qp, bam::first_lane(bam::ballot(load_me && io_ok && stage != nullptr)));
+        uint32_t* pull = bam::pull_begin(pq);
+        copy_pages_helped(cache.base_addr + (uint64_t)found * cache.page_size, stage, (uint32_t)cache.page_size, load_me && io_ok && stage != nullptr);
+        bam::pull_end(pull);
+    }
 #ifdef BAM_PROFILE
     if (cache.prof && bam::ballot(load_me) && bam::lane() == bam::first_lane(bam::active_mask())) atomicAdd(&cache.prof[5], wall_clock64() - pc0);
 #endif
     if (load_me) {
         if (held) read_end(qp, cid);
-        st_relaxed(&dp->offset, found);
-        if (write) __hip_atomic_fetch_or(&dp->state, DIRTY, __ATOMIC_RELAXED, BAM_AGENT);
-        /* payload this wave (helpers included) moved in with plain stores has to be written back for the other
-         * compute units before the page shows as valid; payload the controller placed is in memory already */
-        if (bam::ballot(stage != nullptr || !held)) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+        if (!io_ok) {
+            /*
+             * The read did not happen (error completion) or nobody knows whether it did (the wait was given up): the
+             * page must not show as valid with whatever the slot or the staging page held before.  The slot goes back
+             * to the free ones and the page stays invalid; the caller's next pass finds it so and tries again, or, after
+             * a wait that was given up, finds the abort flag.  While this lane holds BUSY nobody else takes the slot
+             * (an evictor that lands on it finds its page busy and moves on), so its lock is free within a few steps.
+             */
+            cache_page_t* cp = &cache.cache_pages[found];
+            bam::spin_t lk;
+            bool locked = false;
+            while (!locked) {
+                locked = __hip_atomic_exchange(&cp->page_take_lock, (uint32_t)LOCKED, __ATOMIC_RELAXED, BAM_AGENT) == UNLOCKED;
+                if (!locked && cache.spin_giveup(lk)) break;
+            }
+            if (locked) st_publish(&cp->page_take_lock, (uint32_t)FREE);
+            fence_meta();
+            __hip_atomic_fetch_and(&dp->state, DISABLE_BUSY_MASK, __ATOMIC_RELAXED, BAM_AGENT);
+        } else {
+            /* the slot, and one more load of this page on the count above it (this lane owns the descriptor while BUSY is set) */
+            st_relaxed(&dp->offset, found | (((ld_relaxed(&dp->offset) >> BAM_SLOT_BITS) + 1u) << BAM_SLOT_BITS));
+            if (write) __hip_atomic_fetch_or(&dp->state, DIRTY, __ATOMIC_RELAXED, BAM_AGENT);
+        }
+    }
+    /* payload this wave (helpers included) moved in with plain stores has to be written back for the other
+     * compute units before the page shows as valid; payload the controller placed is in memory already */
+    if (bam::ballot(load_me && io_ok)) {
+        if (bam::ballot(load_me && io_ok && (stage != nullptr || !held))) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
         else fence_meta();
+    }
+    if (load_me && io_ok) {
         /* BUSY -> 0 and VALID -> 1 in one step; publishes the payload and the offset */
         __hip_atomic_fetch_xor(&dp->state, DISABLE_BUSY_ENABLE_VALID, __ATOMIC_RELAXED, BAM_AGENT);
         slot = found;
@@ -700,7 +801,8 @@ __forceinline__ __device__ bam_pass_t bam_slow_pass(range_d_t<T>* r, const uint6
     else return bam_slow_pass_inline(r, pg, queue, sv, slot, in);
 }
 
-/* the reference's entry point: references + slot, and the access is accounted in the range's counters */
+/* the reference's entry point: references + slot, and the access is accounted in the range's counters; BAM_NO_SLOT
+ * (with the references taken all the same) when the wait for the page was given up */
 template <typename T>
 __forceinline__ __device__
 uint64_t range_d_t<T>::acquire_page(const size_t pg, const uint32_t count, const bool write, const uint32_t ctrl_, const uint32_t queue)
@@ -719,7 +821,7 @@ uint64_t range_d_t<T>::acquire_page(const size_t pg, const uint32_t count, const
             const bool progressed = (ps.flags & BAM_PASS_PROGRESSED) != 0;
             if (!resolved) { sv = ps.sv; slot = ps.slot; hit = (ps.flags & BAM_PASS_HIT) != 0; resolved = (ps.flags & BAM_PASS_RESOLVED) != 0; }
             if (!bam::ballot(!resolved)) break;
-            if (!bam::ballot(progressed) && cache.spin_giveup(sp)) { if (!resolved) slot = 0; break; }
+            if (!bam::ballot(progressed) && cache.spin_giveup(sp)) { if (!resolved) slot = BAM_NO_SLOT; break; }
         }
     }
     bam_stat_shard_t* sh = shard();
@@ -972,11 +1074,11 @@ struct array_d_t {
         eq_mask = bam::match_any(page, (uint64_t)v.r);
         master = (int)bam::first_lane(eq_mask);
         count = bam::popc(eq_mask);
-        uint32_t slot = 0;
+        uint32_t slot = BAM_NO_SLOT;
         auto keep = [&](uint32_t s_) { slot = s_; return false; };
         v.acquire(page, write, keep, keep);
         v.template flush_stats<false>();
-        base_master = slot;
+        base_master = slot;                     /* BAM_NO_SLOT if the wait for the page was given up */
     }
 
     /* run fn(address of element i in the cache) with the page referenced, for every active lane */
@@ -994,7 +1096,21 @@ struct array_d_t {
     __forceinline__ __device__ T seq_read(const size_t i) const
     {
         T ret = T();
-        with_element(i, false, [&](T* p) { ret = bam::ld_payload(p); });
+        bam::range_view<T> v;
+        if (!view_of(i, v)) return ret;
+        const uint64_t byte = v.byte_of(i);
+        /* resident pages are read without a reference (each lane for itself: lanes on one page load the same descriptor
+         * word, which costs the memory system one access); what is left goes the counted way, coalesced */
+        bool got = false;
+        if (v.r->cache.fast_reads) {
+            got = bam_read_unpinned(v.pages + (byte >> v.page_size_log), v.base_addr, v.page_size_log, byte & (v.page_size - 1), ret);
+            if (got) v.account(true);
+        }
+        if (!got) {
+            auto use = [&](uint32_t slot) { ret = bam::ld_payload((T*)(v.slot_addr(slot) + (byte & (v.page_size - 1)))); return true; };
+            v.template acquire<true>(byte >> v.page_size_log, false, use, use);
+        }
+        v.template flush_stats<false>();
         return ret;
     }
 
@@ -1026,12 +1142,13 @@ struct array_d_t {
         bam::range_view<T> v;
         v.load(d_ranges + r);
         const uint64_t page = v.page_of(i);
-        uint32_t slot = 0;
+        uint32_t slot = BAM_NO_SLOT;
         auto keep = [&](uint32_t s_) { slot = s_; return false; };
         v.acquire(page, false, keep, keep);
         v.template flush_stats<false>();
         page_ = v.pages + page;
         v.window(page, start, end);
+        if (slot == BAM_NO_SLOT) { start = end = 0; return nullptr; }        /* wait given up; the references stay counted: release_page as usual */
         return (void*)(v.slot_addr(slot) + (v.byte_of(start) & (v.page_size - 1)));
     }
 
@@ -1071,6 +1188,7 @@ struct array_d_t {
         bam::range_view<T> v;
         v.load(r_);
         v.window(page, start, end);
+        if (slot == BAM_NO_SLOT) { start = end = 0; return nullptr; }        /* the reference is held all the same: release_page as usual */
         return (void*)(v.slot_addr(slot) + (v.byte_of(start) & (v.page_size - 1)));
     }
 
@@ -1086,10 +1204,11 @@ struct array_d_t {
         bam::range_view<T> v;
         if (!view_of(i, v)) return ret;
         const uint64_t byte = v.byte_of(i);
-        uint32_t slot = 0;
+        uint32_t slot = BAM_NO_SLOT;
         auto keep = [&](uint32_t s_) { slot = s_; return false; };
         v.acquire(byte >> v.page_size_log, false, keep, keep);
         v.template flush_stats<false>();
+        if (slot == BAM_NO_SLOT) return ret;         /* wait given up: addr NULL, size 0; release_raw as usual */
         ret.addr = (T*)v.slot_addr(slot);
         ret.size = v.page_size / sizeof(T);
         ret.offset = (uint32_t)((byte & (v.page_size - 1)) / sizeof(T));
@@ -1146,6 +1265,7 @@ struct bam_ref {
     __forceinline__ __host__ __device__ bam_ref& operator=(T v) { p->write(i, v); return *this; }
     __forceinline__ __host__ __device__ bam_ref& operator=(const bam_ref& o) { p->write(i, (T)o); return *this; }
     __forceinline__ __host__ __device__ bam_ref& operator+=(T v) { p->write(i, p->read(i) + v); return *this; }
+    __forceinline__ __host__ __device__ bam_ref& operator-=(T v) { p->write(i, p->read(i) - v); return *this; }
 };
 
 /*
@@ -1244,10 +1364,11 @@ struct bam_ptr {
     __forceinline__ __host__ __device__ T operator[](const size_t i) const { return const_cast<bam_ptr*>(this)->read(i); }
     __forceinline__ __host__ __device__ bam_ref<T> operator[](const size_t i) { return bam_ref<T>{this, i}; }
 
-    /* address of element i for the caller to read or write: counts as a write */
+    /* address of element i for the caller to read or write: counts as a write.  NULL when no range holds i or the wait
+     * for the page was given up (the reference returns an address computed from a null window there) */
     __forceinline__ __host__ __device__ T* memref(size_t i)
     {
-        if (i < start || i >= end) update_page(i);
+        if (i < start || i >= end) { if (!update_page(i)) return nullptr; }
         mark_dirty();
         return addr + (i - start);
     }
@@ -1330,20 +1451,29 @@ struct tlb {
             for (uint32_t tries = 0; !settled && !go_direct; tries++) {
                 const uint32_t st = __hip_atomic_fetch_or(&entry->state, TLB_LOCK_, __ATOMIC_ACQUIRE, BAM_AGENT);
                 if ((st & TLB_LOCK_) == 0) {
+                    /* the lock goes, and the users come, with one add: users that leave meanwhile (tlb_entry::release,
+                     * an add of its own) are not written over */
                     if (entry->page != nullptr && entry->global_id == gid) {
                         slot = entry->slot;
-                        __hip_atomic_store(&entry->state, st + count, __ATOMIC_RELEASE, BAM_AGENT);
+                        __hip_atomic_fetch_add(&entry->state, count - TLB_LOCK_, __ATOMIC_RELEASE, BAM_AGENT);
                         settled = true;
                     } else if (entry->page == nullptr || (st & TLB_COUNT_) == 0) {
                         entry->release();
                         slot = (uint32_t)range->acquire_page(page_, 1, false, 0, wave_slot_hash());
-                        entry->page = &range->pages[page_];
-                        entry->slot = slot;
-                        entry->global_id = gid;
-                        __hip_atomic_store(&entry->state, st + count, __ATOMIC_RELEASE, BAM_AGENT);
-                        settled = true;
+                        if (slot == BAM_NO_SLOT) {
+                            /* the wait for the page was given up: the entry stays empty */
+                            range->release_page(page_, 1, false);
+                            __hip_atomic_fetch_add(&entry->state, 0u - TLB_LOCK_, __ATOMIC_RELEASE, BAM_AGENT);
+                            go_direct = true;
+                        } else {
+                            entry->page = &range->pages[page_];
+                            entry->slot = slot;
+                            entry->global_id = gid;
+                            __hip_atomic_fetch_add(&entry->state, count - TLB_LOCK_, __ATOMIC_RELEASE, BAM_AGENT);
+                            settled = true;
+                        }
                     } else {
-                        __hip_atomic_store(&entry->state, st, __ATOMIC_RELEASE, BAM_AGENT);     /* in use for another page */
+                        __hip_atomic_fetch_add(&entry->state, 0u - TLB_LOCK_, __ATOMIC_RELEASE, BAM_AGENT);     /* in use for another page */
                         go_direct = true;
                     }
                 } else if (tries >= 8) go_direct = true;
@@ -1356,6 +1486,7 @@ struct tlb {
         range_view<T> v;
         v.load(range);
         v.window(page_, start, end);
+        if ((uint32_t)pack == BAM_NO_SLOT) { start = end = 0; return nullptr; }      /* wait given up (direct, references counted): release as usual */
         return (T*)(v.slot_addr((uint32_t)pack) + (v.byte_of(start) & (v.page_size - 1)));
     }
 
@@ -1385,10 +1516,13 @@ struct bam_ptr_tlb {
     __forceinline__ __device__ ~bam_ptr_tlb() { fini(); }
     __forceinline__ __device__ void init(array_d_t<T>* a, tlb<T, n, _scope, loc>* t) { array = a; tlb_ = t; }
 
+    bool held = false;               /* a reference (on the table's entry or on the page) is out */
+
     __forceinline__ __device__ void fini(void)
     {
-        if (addr) {
+        if (held) {
             tlb_->release(gid, direct, range, page);
+            held = false;
             addr = nullptr;
             start = end = 0;
         }
@@ -1398,20 +1532,24 @@ struct bam_ptr_tlb {
     {
         fini();
         array->get_page_gid(i, range, page, gid);
-        if (range) addr = tlb_->acquire(i, gid, start, end, range, page, direct);
+        if (range) { addr = tlb_->acquire(i, gid, start, end, range, page, direct); held = true; }
     }
 
+    /* T() when no range holds i or the wait for the page was given up */
     __forceinline__ __device__ T operator[](const size_t i) const
     {
         bam_ptr_tlb* self = const_cast<bam_ptr_tlb*>(this);
         if (i < start || i >= end) self->update_page(i);
+        if (!self->addr || i < self->start || i >= self->end) return T();
         return bam::ld_payload(self->addr + (i - start));
     }
 
-    /* address of element i for the caller to write through: the page is marked dirty */
+    /* address of element i for the caller to write through: the page is marked dirty; NULL when no range holds i or
+     * the wait for the page was given up */
     __forceinline__ __device__ T* memref(const size_t i)
     {
         if (i < start || i >= end) update_page(i);
+        if (!addr || i < start || i >= end) return nullptr;
         range->mark_page_dirty(page);
         return addr + (i - start);
     }
@@ -1431,7 +1569,7 @@ static __global__ void __flush(page_cache_d_t* pc)
     const uint64_t range = g & pc->n_ranges_mask, addr = g >> pc->n_ranges_bits;
     data_page_t* dp = &pc->ranges[range][addr];
     const uint32_t s = bam::ld_relaxed(&dp->state);
-    if ((s & DIRTY) == 0 || (s & VALID) == 0 || bam::ld_relaxed(&dp->offset) != page) return;
+    if ((s & DIRTY) == 0 || (s & VALID) == 0 || (bam::ld_relaxed(&dp->offset) & BAM_SLOT_MASK) != page) return;
     const data_dist_t dist = pc->ranges_dists[range];
     const uint64_t index = get_backing_page_(pc->ranges_page_starts[range], addr, pc->n_ctrls, dist);
     uint64_t c = get_backing_ctrl_(addr, pc->n_ctrls, dist);
@@ -1464,7 +1602,6 @@ struct page_cache_t {
     BufferPtr page_ticket_buf;
     BufferPtr ctrl_counter_buf;
     BufferPtr extra_reads_buf;
-    BufferPtr prof_buf;
     BufferPtr tokens_buf;
 
     uint64_t reset_stats()
@@ -1547,13 +1684,15 @@ struct page_cache_t {
         page_ticket_buf = createBuffer(sizeof(uint32_t), hipDevice);
         pdt.page_ticket = (uint32_t*)page_ticket_buf.get();
 
+        if (np > BAM_SLOT_MASK) throw error(string("page_cache_t: more cache pages than a page descriptor can name"));
         pdt.wave_batch = BAM_WAVE_SIZE;
+        pdt.fast_reads = 1;
+        if (const char* e = getenv("BAM_FAST_READS")) pdt.fast_reads = atoi(e) != 0;
         tokens_buf = createBuffer(BAM_TOKEN_SLOTS * 64, hipDevice);
         pdt.miss_tokens = (uint32_t*)tokens_buf.get();
         pdt.miss_waves = 4;
         if (const char* e = getenv("BAM_MISS_WAVES")) pdt.miss_waves = (uint32_t)atoi(e);
-        prof_buf = createBuffer(16 * sizeof(unsigned long long), hipDevice);
-        pdt.prof = (unsigned long long*)prof_buf.get();
+        pdt.prof = ctrl.prof;
 
         const bool staged = ctrl.n_qps && ctrl.h_qps[0]->stage != nullptr;
         const uint64_t cache_size = ps * np;

@@ -27,6 +27,8 @@
 #include "nvm_types.h"
 #include "util.h"
 
+#define BAM_CQ_IDLE_TICKS_DEFAULT 200u       /* 2 us at 100 MHz: an empty completion ring in host memory is left alone that long after a look */
+
 struct QueuePair
 {
     uint32_t            pageSize;
@@ -40,6 +42,8 @@ struct QueuePair
     uint8_t*            stage;          /* staging window (NULL: PRPs address device memory directly) */
     uint64_t            stage_ioaddr;
     uint32_t            stage_stride;   /* bytes per command id */
+    uint32_t*           pull_tokens;    /* [8 x 16] waves pulling staged payload from host memory right now, one word per compute-unit cluster, 64 bytes apart */
+    uint32_t            pull_limit;     /* at most this many per cluster at a time (0 = no limit) */
     uint64_t*           async_dst;      /* [n_cids] staged asynchronous reads: destination address, 0 = none */
     uint32_t*           async_len;      /* [n_cids] and length in bytes */
 
@@ -53,7 +57,9 @@ struct QueuePair
 
     QueuePair(const nvm_ctrl_t* ctrl, const uint32_t hipDevice, const struct nvm_ns_info ns, const struct nvm_ctrl_info info,
               nvm_aq_ref& aq_ref, const uint16_t qp_id, const uint64_t queueDepth,
-              bam_guard_t* guard = nullptr, uint32_t stage_bytes = 4096, bam_dma_place ring_place = BAM_DMA_HOST)
+              bam_guard_t* guard = nullptr, uint32_t stage_bytes = 4096, bam_dma_place ring_place = BAM_DMA_HOST,
+              bam_dma_place cq_place = BAM_DMA_HOST, int seal = 1, uint32_t flush = 2, unsigned long long* prof = nullptr,
+              uint32_t* pull_tokens_ = nullptr, uint32_t pull_limit_ = 0)
     {
         own = new Owners();
         aq = aq_ref;
@@ -63,7 +69,10 @@ struct QueuePair
         while ((uint64_t)qs * 2 <= depth) qs *= 2;
 
         own->sq_mem = createDma(ctrl, NVM_PAGE_ALIGN(qs * sizeof(nvm_cmd_t), 1UL << 16), hipDevice, ring_place);
-        own->cq_mem = createDma(ctrl, NVM_PAGE_ALIGN(qs * sizeof(nvm_cpl_t), 1UL << 16), hipDevice, ring_place);
+        /* the completion ring may sit in device memory: the controller then posts completions across the interconnect
+         * (16-byte writes behind the payload) and the waves look for them in local memory, which costs them nothing
+         * and keeps those looks out of the way of the payload they pull from host memory */
+        own->cq_mem = createDma(ctrl, NVM_PAGE_ALIGN(qs * sizeof(nvm_cpl_t), 1UL << 16), hipDevice, cq_place);
 
         pageSize = info.page_size;
         block_size = ns.lba_data_size;
@@ -79,10 +88,13 @@ struct QueuePair
 
         /* the ring is filled by the GPU across the interconnect and fetched by the controller from the other side:
          * have entries sealed so that one that has not fully arrived is never taken (see nvm_cmd_seal) */
-        status = nvm_admin_sq_set_sealed(aq_ref, &sq);
+        status = seal ? nvm_admin_sq_set_sealed(aq_ref, &sq) : 0;
         /* a controller that does not know the vendor command (a real device) answers with an NVMe status: the queue
          * then runs unsealed, as the NVMe specification has it; anything else is a failed admin round trip */
         if (!nvm_ok(status) && status > 0) { nvm_admin_sq_delete(aq_ref, &sq, &cq); nvm_admin_cq_delete(aq_ref, &cq); delete own; throw std::runtime_error(std::string("Failed to seal submission queue: ") + nvm_strerror(status)); }
+        /* unsealed: a submitter makes sure its entry is in the ring before the entry can be covered by a doorbell */
+        sq.flush = flush;
+        cq.idle_ticks = cq_place == BAM_DMA_HOST ? BAM_CQ_IDLE_TICKS_DEFAULT : 0;
 
         /* device-side protocol state */
         const uint32_t n_cids = qs < 64 ? 64 : qs;      /* handed out in blocks of 64, one block per wave */
@@ -99,10 +111,12 @@ struct QueuePair
         sq.head_mark = (padded_struct*)own->sq_cid_left.get();
         cq.cid = sq.cid;
         cq.cid_mask = sq.cid_mask;
+        sq.prof = cq.prof = prof;
         sq.guard = cq.guard = guard;
         sq.spin_limit = cq.spin_limit = guard ? guard->spin_limit : 0;
 
         stage = nullptr; stage_ioaddr = 0; stage_stride = 0; async_dst = nullptr; async_len = nullptr;
+        pull_tokens = pull_tokens_; pull_limit = pull_tokens_ ? pull_limit_ : 0;
         if (stage_bytes > 2 * ctrl->page_size || (stage_bytes & (stage_bytes - 1)))
             throw std::runtime_error("QueuePair: the staging page must be a power of two of at most two controller pages (PRP1 + PRP2)");
         if (stage_bytes) {

@@ -6,6 +6,8 @@
 #include <cstring>
 #include <ctime>
 #include <vector>
+#include <fcntl.h>
+#include <unistd.h>
 #include <time.h>
 #include "nvm_admin.h"
 #include "nvm_aq.h"
@@ -275,6 +277,85 @@ int main()
         double iops = nvmt_selftest_iops(&cfg, 2, 32, 20000, 4096);
         CHECK("selftest_iops_positive", iops > 1000.0);
         CHECK("selftest_rejects_bad_args", nvmt_selftest_iops(&cfg, 0, 32, 10, 4096) < 0 && nvmt_selftest_iops(&cfg, 1, 1024, 10, 4096) < 0);
+    }
+    // ---- nvm_ctrl_init(fd): maps the register window behind a descriptor (reference include/nvm_ctrl.h:36) ----
+    {
+        nvm_ctrl_t* c = nullptr;
+        CHECK("ctrl_init_fd_bad_descriptor", nvm_ctrl_init(&c, -1) == EBADF && !c);
+        char path[] = "/tmp/bam_bar0_XXXXXX";
+        int fd = mkstemp(path);
+        std::vector<uint8_t> img(NVM_CTRL_MEM_MINSIZE, 0);
+        // CAP: MQES = 255, TO = 3 (1500 ms), DSTRD = 2, MPSMIN = 0 (4 KiB), MPSMAX = 4
+        uint64_t cap = 255ull | (3ull << 24) | (2ull << 32) | (0ull << 48) | (4ull << 52);
+        memcpy(img.data(), &cap, 8);
+        bool wrote = write(fd, img.data(), img.size()) == (ssize_t)img.size();
+        int s = nvm_ctrl_init(&c, fd);
+        CHECK("ctrl_init_fd_maps_and_reads_cap", wrote && s == 0 && c && c->max_qs == 256 && c->timeout == 1500 && c->dstrd == 2 && c->page_size == 4096 && c->mm_size == NVM_CTRL_MEM_MINSIZE);
+        if (c) { *(volatile uint32_t*)((volatile char*)c->mm_ptr + 0x14) = 0x00460001u; }
+        uint32_t cc = 0;
+        bool through = c && pread(fd, &cc, 4, 0x14) == 4 && cc == 0x00460001u;       // a shared mapping: register writes reach the file
+        CHECK("ctrl_init_fd_mapping_is_shared", through);
+        nvm_ctrl_free(c);
+        close(fd); unlink(path);
+        int pfd[2];
+        if (pipe(pfd) == 0) {
+            c = nullptr;
+            int e = nvm_ctrl_init(&c, pfd[0]);
+            CHECK("ctrl_init_fd_unmappable", e != 0 && e > 0 && !c);
+            close(pfd[0]); close(pfd[1]);
+        }
+    }
+    // ---- SQ slot laps across the wrap of the 32-bit ticket counter ----
+    {
+        bool ok = true;
+        for (uint32_t qs_log2 : {1u, 4u, 10u, 16u}) {
+            const uint32_t qs = 1u << qs_log2;
+            uint32_t word = 0;                                    // the slot word of slot 5 % qs, freed once per lap
+            const uint32_t pos = 5u % qs;
+            // walk the laps up to and across the wrap of the ticket counter: start a few laps before 2^32
+            const uint64_t laps_total = 1ull << (32 - qs_log2);
+            const uint64_t first_lap = laps_total - 3;
+            word = (uint32_t)(first_lap * 2);                     // freed first_lap times so far
+            for (uint64_t lap = first_lap; lap < laps_total + 4; lap++) {
+                const uint32_t ticket = (uint32_t)(lap * qs + pos);   // wraps with the counter
+                ok &= nvm_sq_slot_free(word, ticket, qs_log2) == 1;                       // my lap: free
+                ok &= nvm_sq_slot_free(word, ticket + qs, qs_log2) == 0;                  // the next lap's holder must wait
+                ok &= nvm_sq_slot_free(word - 2, ticket, qs_log2) == 0;                   // not yet freed for my lap
+                word += 2;                                                                // the drainer frees the slot
+            }
+        }
+        CHECK("sq_slot_laps_across_ticket_wrap", ok);
+    }
+    // ---- submission entry image against the NVMe layout, byte for byte (reference include/nvm_cmd.h:54-88) ----
+    {
+        nvm_cmd_t c; memset(&c, 0, sizeof(c));
+        nvm_cmd_header(&c, 0xBEEF, NVM_IO_READ, 1);
+        nvm_cmd_data_ptr(&c, 0x1122334455667000ull, 0xAABBCCDD00112000ull);
+        nvm_cmd_rw_blks(&c, 0x0123456789ABCDEFull, 8);
+        const uint8_t want[64] = {
+            0x02, 0x00, 0xEF, 0xBE,  0x01, 0x00, 0x00, 0x00,                               // opcode, FUSE/PSDT, CID | NSID
+            0, 0, 0, 0, 0, 0, 0, 0,  0, 0, 0, 0, 0, 0, 0, 0,                               // CDW2-3, MPTR
+            0x00, 0x70, 0x66, 0x55, 0x44, 0x33, 0x22, 0x11,                                // PRP1
+            0x00, 0x20, 0x11, 0x00, 0xDD, 0xCC, 0xBB, 0xAA,                                // PRP2
+            0xEF, 0xCD, 0xAB, 0x89, 0x67, 0x45, 0x23, 0x01,                                // SLBA
+            0x07, 0x00, 0x00, 0x00,  0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0 };                 // NLB (zero based), CDW13-15
+        CHECK("sqe_read_image_matches_spec_bytes", memcmp(c.dword, want, 64) == 0);
+        nvm_cmd_t w; memset(&w, 0xff, sizeof(w));               // the encoders must not depend on what the entry held, except DW12's upper half
+        for (int i = 0; i < 16; i++) w.dword[i] = 0;
+        nvm_cmd_header(&w, 0x0001, NVM_IO_WRITE, 0xffffffffu);
+        nvm_cmd_data_ptr(&w, 0x1000, 0);
+        nvm_cmd_rw_blks(&w, 0, 1);
+        const uint8_t* wb = (const uint8_t*)w.dword;
+        CHECK("sqe_write_image", wb[0] == 0x01 && wb[2] == 0x01 && wb[3] == 0x00 && w.dword[1] == 0xffffffffu && w.dword[6] == 0x1000 && w.dword[12] == 0);
+        // the seal only touches CDW2 and CDW3, verifies, and breaks on any change of the entry or of the ticket
+        nvm_cmd_t sld = c;
+        nvm_cmd_seal(&sld, 0x12345678u);
+        bool only23 = true;
+        for (int i = 0; i < 16; i++) if (i != 2 && i != 3) only23 &= sld.dword[i] == c.dword[i];
+        bool breaks = nvm_cmd_seal_ok(&sld, 0x12345678u) && !nvm_cmd_seal_ok(&sld, 0x12345679u) && !nvm_cmd_seal_ok(&c, 0);
+        for (int i = 0; i < 16 && breaks; i++)
+            for (int b = 0; b < 32; b += 7) { nvm_cmd_t x = sld; x.dword[i] ^= 1u << b; breaks &= !nvm_cmd_seal_ok(&x, 0x12345678u); }
+        CHECK("sqe_seal_touches_cdw2_cdw3_only_and_verifies", only23 && sld.dword[2] == 0x12345678u && breaks);
     }
     printf("%s (%d failures)\n", failures ? "FAILED" : "PASSED", failures);
     return failures ? 1 : 0;

@@ -786,6 +786,169 @@ def test_graph_file_to_store_then_traverse(bam, tmp_path):
         assert r.t.stats()["write_cmds"] == (n_e * 8 + 4095) // 4096 and not r.c.aborted()
 
 
+
+# ---------------------------------------------------------------- read-modify-write routes
+
+def _check_add_chains(x0, idx, vals, olds, final):
+    """Every element that received adds v_1..v_k (in whatever order the device applied them) must show that order in what
+    the adds returned: sorted by (old - x0), the returned values are x0, x0 + v_a, x0 + v_a + v_b, ... and the element
+    ends at x0 + sum(v).  The steps between consecutive returned values (and from the last one to the final value) are
+    therefore a permutation of the values added."""
+    order = np.argsort(idx, kind="stable")
+    idx_s, vals_s, olds_s = idx[order], vals[order], olds[order]
+    starts = np.flatnonzero(np.r_[True, idx_s[1:] != idx_s[:-1]])
+    ends = np.r_[starts[1:], len(idx_s)]
+    for a, b in zip(starts, ends):
+        e = int(idx_s[a])
+        d = np.sort((olds_s[a:b] - x0[e]).astype(np.uint64))           # mod 2^64
+        steps = np.diff(np.r_[d, (final[e] - x0[e]).astype(np.uint64)])
+        assert d[0] == 0, "element %d: no add saw the initial value" % e
+        assert np.array_equal(np.sort(steps), np.sort(vals_s[a:b])), "element %d: returned values do not chain" % e
+
+
+@pytest.mark.parametrize("api,cache_pages,block", [(0, 24, 64), (0, 300, 256), (1, 4096, 64)])
+def test_atomic_add_on_scattered_and_colliding_elements(bam, api, cache_pages, block):
+    """array_d_t::AtomicAdd (reference include/page_cache.h:1647) and atomics on the address bam_ptr::memref hands out (:467):
+    several launches of adds to elements drawn from a small hot set (many lanes of a launch on one element) and from all
+    over the array, through a cache smaller than what is touched, so dirty pages are evicted, written back and read again
+    between the adds.  A numpy array plays the store; the values returned must chain (see above)."""
+    n_elems, n = 1 << 23, 2048                                       # 16384 pages of data; 2048 adds per launch
+    rng = np.random.default_rng(SEED + api)
+    with Rig(bam, n_elems * 8, backing=True, n_queues=8, depth=256) as r:
+        x0 = r.backing(n_elems).copy()
+        model = x0.copy()
+        a = r.array(n_elems, 4096, cache_pages)
+        hot = rng.integers(0, n_elems, 64).astype(np.uint64)
+        all_idx, all_val, all_old = [], [], []
+        for launch in range(5):
+            idx = np.where(rng.random(n) < 0.5, hot[rng.integers(0, len(hot), n)], rng.integers(0, n_elems, n).astype(np.uint64)).astype(np.uint64)
+            vals = rng.integers(1, 1 << 20, n).astype(np.uint64)
+            old = _u64(a.update(api, _dev(idx), _dev(vals), block_size=block))
+            np.add.at(model, idx.astype(np.int64), vals)
+            all_idx.append(idx); all_val.append(vals); all_old.append(old)
+        r.objs[0][2].flush()
+        final = r.backing(n_elems)
+        assert np.array_equal(final, model)
+        _check_add_chains(x0, np.concatenate(all_idx), np.concatenate(all_val), np.concatenate(all_old), final)
+        idx = np.concatenate(all_idx)
+        assert a.read(len(idx), _dev(idx), block_size=64) == int(np.sum(model[idx.astype(np.int64)], dtype=np.uint64))
+        ts = r.t.stats()
+        assert ts["write_cmds"] > 0 and not r.c.aborted() and r.c.info()["error_completions"] == 0
+
+
+def test_add_assign_through_a_bam_ptr_lvalue(bam):
+    """ptr[i] += v on a non-const bam_ptr (reference include/page_cache.h:478: operator[] as an lvalue marks the page
+    dirty): distinct elements per launch, several launches over the same elements, a cache smaller than what they touch"""
+    n_elems, n = 1 << 23, 2048
+    rng = np.random.default_rng(SEED)
+    with Rig(bam, n_elems * 8, backing=True, n_queues=8, depth=256) as r:
+        model = r.backing(n_elems).copy()
+        a = r.array(n_elems, 4096, 4096)
+        for launch in range(6):
+            idx = rng.permutation(n_elems)[:n].astype(np.uint64)
+            if launch % 2:
+                idx[: n // 2] = prev[: n // 2]                         # half of them again: read back what the last launch wrote
+                idx = np.unique(idx)
+            vals = rng.integers(0, 1 << 63, len(idx)).astype(np.uint64)
+            old = _u64(a.update(2, _dev(idx), _dev(vals), block_size=64))
+            assert np.array_equal(old, model[idx.astype(np.int64)]), "launch %d" % launch
+            model[idx.astype(np.int64)] += vals
+            prev = idx
+        r.objs[0][2].flush()
+        assert np.array_equal(r.backing(n_elems), model)
+        assert r.t.stats()["write_cmds"] > 0 and not r.c.aborted()
+
+
+def _seal_value(dw, ticket):
+    """nvm_cmd_seal_value restated: a multiplicative hash over the dwords of the entry except CDW3, keyed by the ticket"""
+    M = 0xFFFFFFFF
+    h = (ticket * 0x9E3779B1 + 0x7F4A7C15) & M
+    for i in range(16):
+        if i == 3:
+            continue
+        h = ((h ^ int(dw[i])) * 0x85EBCA6B) & M
+        h ^= h >> 13
+    return h | 1
+
+
+@pytest.mark.parametrize("opcode", [0x02, 0x01])
+def test_submission_entries_built_on_the_device_match_the_nvme_layout(bam, opcode):
+    """the product's encoders (include/nvm_cmd.h; reference include/nvm_cmd.h:54-88), compiled for the host and for gfx950,
+    against the oracle's independent encoder and the NVMe byte layout; then sealed, against a restatement of the seal"""
+    import torch
+    L = bam.load()
+    cid, nsid, prp1, prp2, lba, nblk, ticket = 0xBE00, 1, 0x1122334455667000, 0xAABBCCDD00112000, 0x0123456789ABCD00, 8, 0xFFFFFFF0
+    for seal in (0, 1):
+        host = (ctypes.c_uint32 * 16)()
+        dev = torch.zeros(64 * 16, dtype=torch.int32, device="cuda")
+        assert L.bam_sqe_image(cid, opcode, nsid, prp1, prp2, lba, nblk, seal, ticket, host, ctypes.c_void_p(dev.data_ptr()), None) == 0
+        torch.cuda.synchronize()
+        d = dev.cpu().numpy().view(np.uint32).reshape(64, 16)
+        for lane in range(64):
+            want = np.zeros(16, dtype=np.uint32)
+            oracle.lib().bo_cmd_rw(want, cid + lane, opcode, nsid, prp1, prp2, lba + lane, nblk)
+            if seal:
+                want[2] = (ticket + lane) & 0xFFFFFFFF               # the ticket wraps within the wave
+                want[3] = _seal_value(want, int(want[2]))
+            assert np.array_equal(d[lane], want), "lane %d seal %d" % (lane, seal)
+        assert np.array_equal(np.frombuffer(host, dtype=np.uint32), d[0])
+        if not seal:
+            b = d[0].tobytes()
+            assert b[0] == opcode and b[1] == 0 and b[2:4] == bytes([0x00, 0xBE]) and b[4:8] == (1).to_bytes(4, "little")
+            assert b[8:24] == bytes(16) and b[24:32] == prp1.to_bytes(8, "little") and b[32:40] == prp2.to_bytes(8, "little")
+            assert b[40:48] == lba.to_bytes(8, "little") and b[48:50] == (7).to_bytes(2, "little") and b[50:64] == bytes(14)
+
+
+# ---------------------------------------------------------------- queue policies: ring placement, unsealed entries
+
+@pytest.mark.parametrize("place", ["host", "device"])
+@pytest.mark.parametrize("order,depth", [(0, 256), (2, 16), (1, 64)])
+def test_completion_ring_placement(bam, place, order, depth, monkeypatch):
+    """completion rings in host-pinned memory or in device memory (written by the controller across the interconnect):
+    in-order, shuffled and reversed completions, queues so shallow that the completion ring fills up"""
+    from bam_amd import gen
+    monkeypatch.setenv("BAM_CQ_PLACE", place)
+    n_elems, n = 1 << 22, 1 << 18
+    with Rig(bam, 64 << 20, n_queues=4, depth=depth, order=order) as r:
+        a = r.array(n_elems, 4096, 1024)
+        idx = gen.gather_indices(SEED, n, n_elems)
+        assert a.read(n, idx, block_size=128) == oracle.lib().bo_gather_sum(SEED, SEED, 0, n, n_elems)
+        st, ts = a.stats(), r.t.stats()
+        assert st["access_cnt"] == n and st["read_io_cnt"] == ts["read_cmds"] > 0
+        assert not r.c.aborted() and r.c.info()["error_completions"] == 0 and ts["error_cpls"] == 0
+    ns = 1 << 30
+    with Rig(bam, ns, n_queues=2, depth=depth, order=order) as r:                 # raw block reads, far more commands than ring entries
+        nb = 1 << 14
+        pc = bam.PageCache(4096, nb, 0, r.c)
+        lbas = gen.block_lbas(SEED, nb, ns, 4096, 512)
+        pc.block_io(nb, 4096, lbas)
+        ref = np.array([oracle.lib().bo_block_checksum(SEED, int(x), 512, 4096) for x in _u64(lbas)], dtype=np.uint64)
+        assert np.array_equal(_u64(pc.block_checksums(nb, 4096)), ref) and not r.c.aborted()
+        pc.close()
+
+
+@pytest.mark.parametrize("flush", ["2", "1"])
+def test_unsealed_submission_entries(bam, flush, monkeypatch):
+    """submission queues as the NVMe specification has them, no seal in the entries (what a real controller needs): a
+    submitter makes sure its entry has arrived before the entry can be covered by a doorbell.  Checksum, no error
+    completions, no wait given up; the target's counters say what it saw."""
+    from bam_amd import gen
+    monkeypatch.setenv("BAM_SQ_SEAL", "0")
+    monkeypatch.setenv("BAM_SQ_FLUSH", flush)
+    n_elems, n = 1 << 24, 1 << 20
+    with Rig(bam, n_elems * 8, n_queues=32, depth=256, io_threads=8) as r:
+        a = r.array(n_elems, 4096, 8192)
+        for rep in range(3):
+            idx = gen.gather_indices(SEED + rep, n, n_elems)
+            got = a.read(n, idx, block_size=256)
+            if flush == "2":
+                assert got == oracle.lib().bo_gather_sum(SEED, SEED + rep, 0, n, n_elems)
+        ts = r.t.stats()
+        print("unsealed, flush %s: %d commands, %d doorbells, %d stale doorbells, %d entry retries" % (flush, ts["read_cmds"], ts["sq_doorbells"], ts["stale_doorbells"], ts["sqe_retries"]))
+        assert ts["sqe_retries"] == 0                                     # nothing is verified on an unsealed queue
+        if flush == "2":
+            assert not r.c.aborted() and r.c.info()["error_completions"] == 0 and ts["error_cpls"] == 0
+
 # ---------------------------------------------------------------- failure handling
 
 def test_lost_completion_ends_the_kernel_with_the_abort_flag(bam):
@@ -818,11 +981,16 @@ def test_lost_completion_during_a_graph_traversal(bam, kernel):
 
 
 def test_error_completions_are_counted(bam):
+    """one command in 100 completes with an error status: its page is not shown as valid with whatever the slot held,
+    the read is issued again, and the sum comes out right"""
+    n = 1 << 18
     with Rig(bam, 16 << 20, fail_every=100) as r:
         a = r.array(1 << 20, 4096, 4096)
-        a.read(1 << 18, block_size=64)
+        assert a.read(n, block_size=64) == oracle.lib().bo_store_sum(SEED, 0, 1, n)
         assert not r.c.aborted()
-        assert r.c.info()["error_completions"] == r.t.stats()["error_cpls"] > 0
+        ts = r.t.stats()
+        assert r.c.info()["error_completions"] == ts["error_cpls"] > 0
+        assert a.stats()["read_io_cnt"] == ts["read_cmds"] + ts["error_cpls"] == n // 512 + ts["error_cpls"]
 
 
 # ---------------------------------------------------------------- full size (config 2)
