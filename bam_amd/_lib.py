@@ -55,6 +55,7 @@ SIGNATURES = {
     "bam_vectoradd": (c_int, [c_vp, c_vp, c_vp, c_u64, c_vp]),
     "bam_reduce": (c_int, [c_vp, c_u64, c_u32, c_vp, c_vp]),
     "bam_scan": (c_int, [c_vp, c_u64, c_u32, c_vp, c_vp]),
+    "bam_scan_noalloc": (c_int, [c_vp, c_u64, c_u32, c_vp, c_vp]),
     "bam_pagerank": (c_int, [c_vp, c_vp, c_u64, ctypes.c_float, ctypes.c_float, c_u32, c_int, c_vp, P(c_u32), c_vp]),
     "bam_range32_create": (c_int, [P(c_vp), c_u64, c_u64, c_u64, c_u64, c_u64, c_u64, c_vp, c_u32, c_int]),
     "bam_range32_destroy": (None, [c_vp]),

@@ -2121,6 +2121,70 @@ int bam_scan(bam_array_t* a, uint64_t n_elems, uint32_t block_size, uint64_t* d_
     BAM_API_END
 }
 
+} // extern "C"
+
+/*
+ * bam_scan for callers that cannot allocate (code under stream capture, serving loops, harnesses that forbid it): the block
+ * totals, which bam_scan keeps in a buffer it allocates and frees per call, live in a file-scope device array of fixed size.
+ * Every device the library runs on holds its own copy of the array at its own address until the process ends; the address is
+ * looked up once per device (the array's name means nothing to the host) and handed to the kernels like any other buffer.
+ */
+/* BAM_SCAN_NOALLOC_MAX_BLOCKS (bam_amd.h): 65536 block totals, 512 KiB */
+#define BAM_SCAN_NOALLOC_MAX_DEVICES 64
+static __device__ __align__(256) unsigned long long scratch[BAM_SCAN_NOALLOC_MAX_BLOCKS];
+
+namespace {
+std::mutex g_scratch_mu;
+unsigned long long* g_scratch_ptr[BAM_SCAN_NOALLOC_MAX_DEVICES];      /* per device: where its copy of `scratch` lives */
+
+/* the current device's copy of the array; NULL (and the error recorded) if it cannot be found */
+unsigned long long* scan_scratch_of_current_device()
+{
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= BAM_SCAN_NOALLOC_MAX_DEVICES) { g_err = "bam_scan_noalloc: no current device"; return nullptr; }
+    std::lock_guard<std::mutex> g(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) { g_err = std::string("bam_scan_noalloc: hipGetSymbolAddress: ") + hipGetErrorString(e); return nullptr; }
+        g_scratch_ptr[dev] = (unsigned long long*)p;
+    }
+    return g_scratch_ptr[dev];
+}
+
+__global__ void k_store_zero64(unsigned long long* p) { *p = 0; }
+} // namespace
+
+extern "C" {
+
+int bam_scan_noalloc(bam_array_t* a, uint64_t n_elems, uint32_t block_size, uint64_t* d_result, void* stream)
+{
+    if (!a || !d_result) return fail(EINVAL, "bam_scan_noalloc: null argument");
+    if (!block_size || block_size % BAM_WAVE_SIZE || block_size > 1024) return fail(EINVAL, "bam_scan_noalloc: block size must be a multiple of 64, at most 1024");
+    if (n_elems > a->a->adt.n_elems) return fail(EINVAL, "bam_scan_noalloc: more elements than the array holds");
+    const uint64_t n_blocks = (n_elems + 2ull * block_size - 1) / (2ull * block_size);
+    if (n_blocks > BAM_SCAN_NOALLOC_MAX_BLOCKS)
+        return fail(E2BIG, "bam_scan_noalloc: " + std::to_string(n_elems) + " elements in blocks of " + std::to_string(2ull * block_size) + " need " + std::to_string(n_blocks) +
+                           " block totals, the fixed scratch array holds " + std::to_string(BAM_SCAN_NOALLOC_MAX_BLOCKS) + " (use bam_scan, or a larger block size)");
+    unsigned long long* totals = scan_scratch_of_current_device();
+    if (!totals) return EIO;
+    hipStream_t st = (hipStream_t)stream;
+    unsigned long long* out = (unsigned long long*)d_result + 1;
+    /* no memset node: a fill kernel clears the first word (a caller may be capturing this stream) */
+    hipLaunchKernelGGL(k_store_zero64, dim3(1), dim3(1), 0, st, (unsigned long long*)d_result);
+    if (n_elems) {
+        /* totals[0 .. n_blocks) are written by the first kernel before the second reads them; what an earlier, longer call
+         * left behind them is never read, so nothing has to be cleared */
+        const size_t lds = (2 * block_size + 1024 / BAM_WAVE_SIZE) * sizeof(uint64_t);
+        hipLaunchKernelGGL(k_scan_ptr_pc, dim3((uint32_t)n_blocks), dim3(block_size), lds, st, a->a->d_array_ptr, out, totals, n_elems);
+        hipLaunchKernelGGL(k_scan_block_totals, dim3(1), dim3(1024), 0, st, totals, n_blocks);
+        hipLaunchKernelGGL(k_scan_finalsum, dim3((uint32_t)n_blocks), dim3(block_size), 0, st, (const unsigned long long*)totals, out, n_elems);
+    }
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(EIO, std::string("bam_scan_noalloc: ") + hipGetErrorString(e));
+    return 0;
+}
+
 int bam_pagerank(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, float alpha, float tolerance, uint32_t max_iterations,
                  int by_page, float* d_value, uint32_t* iterations, void* stream)
 {

@@ -275,6 +275,10 @@ class Array:
         _chk(self.L.bam_scan(self.h, n_elems, block_size, _ptr(out), _stream()), "bam_scan")
         return out
 
+    def scan_noalloc(self, n_elems, out, block_size=64):
+        """bam_scan into `out` (n_elems + 1 words) without any allocation by the library; does not synchronise."""
+        _chk(self.L.bam_scan_noalloc(self.h, n_elems, block_size, _ptr(out), _stream()), "bam_scan_noalloc")
+
     def update(self, api, assignment, values, block_size=64):
         """element assignment[t] += values[t] through AtomicAdd (api 0), an atomic on bam_ptr::memref (1) or ptr[i] += v (2);
         returns what each element held before (int64 tensor of bit patterns)."""

@@ -211,6 +211,17 @@ int bam_reduce(bam_array_t* a, uint64_t n_elems, uint32_t block_size, uint64_t* 
  * a scan of the block totals, and the pass that adds them back. */
 int bam_scan(bam_array_t* a, uint64_t n_elems, uint32_t block_size, uint64_t* d_result, void* stream);
 
+/* ---- bam_scan without allocation ----
+ * No counterpart in the reference.  For callers that cannot allocate device memory: code under stream capture, tight
+ * serving loops, harnesses that forbid it.  Same arguments and same result as bam_scan; the block totals, which bam_scan
+ * keeps in a buffer it allocates and frees per call, live in a device array of fixed size inside the library (512 KiB,
+ * held by every device the library runs on until the process ends), so n_elems may need at most
+ * BAM_SCAN_NOALLOC_MAX_BLOCKS blocks of 2 * block_size elements (E2BIG beyond that, nothing launched).  Calls no
+ * hipMalloc / hipFree and does not synchronise; the first call on a device looks the array's address up (make that call
+ * outside a capture).  All calls on one device share the array: calls that overlap on a device race. */
+#define BAM_SCAN_NOALLOC_MAX_BLOCKS 65536u
+int bam_scan_noalloc(bam_array_t* a, uint64_t n_elems, uint32_t block_size, uint64_t* d_result, void* stream);
+
 /* ---- PageRank (benchmarks/pagerank/main.cu: initialize :107-115, kernel_coalesce_pc :252-273, update :412-421,
  * host loop :704-768; the reference runs alpha = 0.85, tolerance = 0.001, at most 100 iterations, :476-477) ----
  * Residual pushes in single precision: every flagged vertex adds its delta to the residual of each neighbour (atomic
