@@ -25,6 +25,8 @@ SIGNATURES = {
     "bam_ctrl_create": (c_int, [P(c_vp), ctypes.c_char_p, c_u32, c_u32, c_u64, c_u64, c_u32, c_u32]),
     "bam_ctrl_destroy": (None, [c_vp]),
     "bam_ctrl_info": (c_int, [c_vp, P(c_u64), c_int]),
+    "bam_ctrl_queue_state": (c_int, [c_vp, c_u32, P(c_u64), P(c_u32), c_u32]),
+    "bam_target_queue_state": (c_int, [c_vp, c_u32, P(c_u64)]),
     "bam_ctrl_aborted": (c_int, [c_vp, c_int]),
     "bam_page_cache_create": (c_int, [P(c_vp), c_u64, c_u64, c_u32, c_vp, c_u64]),
     "bam_page_cache_create_multi": (c_int, [P(c_vp), c_u64, c_u64, c_u32, P(c_vp), c_u32, c_u64]),

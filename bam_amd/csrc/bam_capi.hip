@@ -1,90 +1,17 @@
 // C-ABI of the GPU-side storage-access path: handle management over the C++
-// host objects (ctrl.h, page_cache.h) and the gfx950 kernels that drive them.
-// Kernel shapes follow the reference's benchmark kernels (cited per kernel);
-// lane arithmetic is for 64-wide waves.
-#include "bam_amd.h"
+// host objects (ctrl.h, page_cache.h) and the gfx950 kernels of the array, cache,
+// pattern and block benchmarks.  Kernel shapes follow the reference's benchmark
+// kernels (cited per kernel); lane arithmetic is for 64-wide waves.  The graph
+// kernels are in bam_graph.hip, vectoradd / reduction / scan in bam_apps.hip.
+#include "bam_capi_internal.h"
 
-#include <hip/hip_runtime.h>
-#include <hipcub/hipcub.hpp>
-#include <fcntl.h>
-#include <sys/mman.h>
-#include <sys/stat.h>
-#include <unistd.h>
-#include <algorithm>
-#include <cerrno>
-#include <cstdlib>
-#include <cstring>
-#include <mutex>
-#include <string>
-#include <thread>
-#include <vector>
+std::string& bam_err()
+{
+    static thread_local std::string err;
+    return err;
+}
 
-#include "ctrl.h"
-#include "event.h"
-#include "nvmt.h"
-#include "page_cache.h"
-#include "bafs_ptr.h"
-
-// ---------------------------------------------------------------------------
-// error plumbing
-// ---------------------------------------------------------------------------
-static thread_local std::string g_err;
-
-#define BAM_API_BEGIN try {
-#define BAM_API_END                                                        \
-    return 0;                                                              \
-    } catch (const std::exception& e) { g_err = e.what(); return EIO; }    \
-      catch (...) { g_err = "unknown error"; return EIO; }
-
-static int fail(int code, const char* msg) { g_err = msg; return code; }
-static int fail(int code, const std::string& msg) { g_err = msg; return code; }
-
-struct bam_target {
-    nvmt_t* t = nullptr;
-    void* bar = nullptr;
-    void* backing = nullptr;
-    size_t backing_bytes = 0;
-    nvmt_config_t cfg{};
-};
-struct bam_ctrl { Controller* c; };
-struct bam_page_cache { page_cache_t* pc; Controller* ctrl; };      /* ctrl: the first controller of the cache */
-struct bam_range { range_t<uint64_t>* r; };
-#define BAM_SUM_PARTIALS 4096
-struct bam_array { array_t<uint64_t>* a; BufferPtr partials; };
-struct bam_range32 { range_t<uint32_t>* r; };
-struct bam_array32 { array_t<uint32_t>* a; BufferPtr partials; };      /* partials: [BAM_SUM_PARTIALS] checksum shards, zero between launches */
-
-// ---------------------------------------------------------------------------
-// device helpers
-// ---------------------------------------------------------------------------
 namespace {
-
-__device__ __forceinline__ uint64_t mix64(uint64_t z)
-{
-    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
-    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
-    return z ^ (z >> 31);
-}
-__device__ __forceinline__ uint64_t splitmix64(uint64_t seed, uint64_t i) { return mix64(seed + (i + 1) * 0x9E3779B97F4A7C15ull); }
-
-/* sum over the 64 lanes of a wave (all lanes active); result valid in every lane */
-__device__ __forceinline__ uint64_t wave_sum(uint64_t v)
-{
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += bam::shfl(v, bam::lane() ^ o);
-    return v;
-}
-
-/*
- * Add the wave's values into the launch's checksum.  A single word would take one atomic per wave of the
- * whole grid, all serialised on one address (about 12 ns each: a million waves cost more than the reads they
- * sum), so the sum is kept in BAM_SUM_PARTIALS shards picked by workgroup and folded by k_fold_partials.
- */
-__device__ __forceinline__ void block_accumulate(unsigned long long* partials, uint64_t v)
-{
-    v = wave_sum(v);
-    if (bam::lane() == 0 && v) atomicAdd(&partials[(blockIdx.x * 0x9E3779B1u) >> 20], (unsigned long long)v);
-}
 
 /* one block of 1024 threads: *sum += all shards; shards are left zero for the next launch */
 __global__ void k_fold_partials(unsigned long long* partials, unsigned long long* sum)
@@ -93,60 +20,6 @@ __global__ void k_fold_partials(unsigned long long* partials, unsigned long long
     for (uint32_t i = threadIdx.x; i < BAM_SUM_PARTIALS; i += blockDim.x) { v += partials[i]; partials[i] = 0; }
     v = wave_sum(v);
     if (bam::lane() == 0 && v) atomicAdd(sum, (unsigned long long)v);
-}
-
-/* a page that is not resident as far as one look at its state tells: what the read-ahead asks for (a page that is resident is
- * left alone, which spares its state word two atomics per touch; if it goes before it is read, it is read on demand) */
-template <typename T>
-__device__ __forceinline__ bool page_absent(const bam::range_view<T>& view, const uint64_t page)
-{
-    return (bam::ld_relaxed(&view.pages[page].state) & VALID) == 0;
-}
-
-/*
- * Read-ahead for kernels in which consecutive threads read consecutive elements (one element or two per thread, as in
- * benchmarks/vectoradd, reduction and scan).  Left to themselves such kernels ask the store for one page per wave
- * and trip, and the store path takes about a million such batches per second whatever their size: 1 GiB comes in
- * at 5 GB/s.  Here the wave that reads the first element of a window of W pages (W = a 64th of the cache, at most
- * 64) touches the W pages that lie up to 32 windows further on, one page per lane, taken and dropped again: they come
- * in as one batch of W commands, before the waves that read them are started (workgroups start in order, and the
- * device holds a few thousand waves, that is up to a thousand pages, at a time).  The first windows are touched by
- * their own first waves.  `first` is the index of the wave's first element (wave-uniform), `wave_span` the elements
- * from one wave's first to the next one's (more than 64 where the threads read with a stride).
- */
-template <typename T>
-__device__ __forceinline__ void touch_ahead(array_d_t<T>* da, const uint64_t first, const uint64_t n_read, const uint64_t wave_span = BAM_WAVE_SIZE,
-                                            const uint32_t which = 0)
-{
-    if (da->n_ranges != 1) return;
-    const uint64_t n_elems = n_read < da->n_elems ? n_read : da->n_elems;         /* nothing is touched that the array does not hold */
-    const page_cache_d_t& cache = da->d_ranges[0].cache;
-    const uint64_t w_pages = cache.n_pages >> 6 > BAM_WAVE_SIZE ? BAM_WAVE_SIZE : cache.n_pages >> 6;
-    if (w_pages < 2) return;
-    const uint64_t epp = cache.page_size / sizeof(T), w_elems = w_pages * epp;
-    /* the wave that does it is the `which`-th of those that begin in the window (`wave_span` elements per wave): a kernel
-     * that walks several arrays gives each array's windows to a different wave, and their batches are in flight together */
-    if ((first % w_elems) / wave_span != which) return;
-    /* how far ahead: beyond what the waves in flight cover (a few thousand waves at one page per four to eight waves), within an
-     * eighth of the cache (a kernel may walk several arrays behind one cache at a time) */
-    uint64_t dist = (cache.n_pages / 8) / w_pages;
-    dist = (dist > 32 ? 32 : dist < 1 ? 1 : dist) * w_elems;
-    bam::range_view<T> view;
-    view.load(da->d_ranges);
-    auto touch = [](uint32_t) { return true; };
-    const uint64_t mine = first - first % w_elems + bam::lane() * epp;
-    if (first < dist) {
-        const uint64_t page = view.page_of(mine < n_elems ? mine : first);
-        const bool take = bam::lane() < w_pages && mine < n_elems && page_absent(view, page);
-        if (bam::ballot(take)) view.acquire_helped(page, take, false, touch, touch);
-    }
-    const uint64_t ahead = mine + dist;
-    if (first + dist < n_elems) {
-        const uint64_t page = view.page_of(ahead < n_elems ? ahead : first);
-        const bool take = bam::lane() < w_pages && ahead < n_elems && page_absent(view, page);
-        if (bam::ballot(take)) view.acquire_helped(page, take, false, touch, touch);
-    }
-    view.n_access = view.n_hit = 0;
 }
 
 // ---- array benchmark (benchmarks/array/main.cu:43-65), with a checksum ----
@@ -470,733 +343,6 @@ __global__ void k_block_checksum(page_cache_d_t* pc, uint64_t n_slots, uint32_t 
     if (wave < n_slots && bam::lane() == 0) out[wave] = v;
 }
 
-// ---- BFS: wave per `coarse` vertices, edges through bam_ptr (benchmarks/bfs/main.cu:658-689) ----
-#define MYINFINITY 0xFFFFFFFFu
-/*
- * Read-ahead for a wave that walks one vertex's edge list through bam_ptr.  Left to itself the walk meets the
- * pages of the list one after the other and pays one full trip to the store for each; the list of a hub of a
- * power-law graph covers hundreds of pages, and the one wave that has it then decides how long the whole level
- * takes.  Whenever the walk is about to enter pages it has not asked for yet, the lanes touch the next pages of
- * the list (one each, taken and dropped again): those that are not resident are loaded as one batch of commands,
- * and the walk that follows finds them there.  Nothing is held, so a page that is evicted again before the walk
- * gets to it is simply read once more; results do not depend on it.  Arrays of one range only, and the reach
- * scales with the cache (a 64th of its pages, at most one page per lane).
- */
-template <typename T>
-struct list_read_ahead {
-    bam::range_view<T> view;
-    uint64_t asked_to = 0, last_page = 0;
-    uint32_t reach = 0;
-    bool long_list = false;
-    __device__ __forceinline__ void init(array_d_t<T>* da)
-    {
-        if (da->n_ranges != 1) return;
-        view.load(da->d_ranges);
-        const uint64_t r = da->d_ranges[0].cache.n_pages >> 6;
-        reach = r > BAM_WAVE_SIZE ? BAM_WAVE_SIZE : (uint32_t)r;
-    }
-    /* every lane's elements [es, ee) (empty for lanes without any) are about to be read: touch the first and the last page
-     * of each run, so that what is not resident comes in as one batch or two, not one trip to the store per run */
-    __device__ __forceinline__ void group(const uint64_t es, const uint64_t ee)
-    {
-        if (reach < 2) return;
-        const bool want = ee > es;
-        if (!bam::ballot(want)) return;
-        auto touch = [](uint32_t) { return true; };
-        const uint64_t pf = want ? view.page_of(es) : 0, pl = want ? view.page_of(ee - 1) : 0;
-        /* all lanes go in: those without a page of their own help move what the others load */
-        const bool take_f = want && page_absent(view, pf), take_l = want && pl != pf && page_absent(view, pl);
-        /* the last pages go along with the first ones as far as there are lanes without a first page to ask for (the k-th such
-         * lane takes the last page of the k-th lane that has one): one batch of commands instead of two, of which the second
-         * would be small (few lists cross a page boundary) */
-        const uint64_t need_l = bam::ballot(take_l), idle = ~bam::ballot(take_f);
-        const uint32_t k = bam::popc(idle & bam::lanes_below(bam::lane()));
-        const bool adopt = !take_f && k < bam::popc(need_l);
-        uint64_t m = need_l;
-        if (adopt) for (uint32_t i = 0; i < k; i++) m &= m - 1;
-        const uint64_t adopted = bam::shfl(pl, adopt ? bam::first_lane(m) : 0u);
-        const bool take_1 = take_f || adopt;
-        if (bam::ballot(take_1)) view.acquire_helped(take_f ? pf : adopted, take_1, false, touch, touch);
-        /* last pages nobody had a lane for */
-        const bool take_2 = take_l && bam::popc(need_l & bam::lanes_below(bam::lane())) >= bam::popc(idle);
-        if (bam::ballot(take_2)) view.acquire_helped(pl, take_2, false, touch, touch);
-        view.n_access = view.n_hit = 0;
-    }
-    /*
-     * The lists of the items [first, last) lie in the array in the order of the items (consecutive vertices, or a sorted
-     * queue of them): touch every page that holds
-     * entries of a list that is about to be walked (item(v, v) says which; lists that go to the queue of long ones are
-     * left out), `reach` pages at a time with one page per lane, so that what is not resident comes in as few, large
-     * batches of commands.  The store path moves several times more pages per second in batches of sixteen than in
-     * batches of two or three, which is what touching the lists of 64 vertices at a time gives on a graph with a few
-     * dozen edges per vertex.  False if the span is too wide for that (the caller then touches list by list).
-     */
-    template <typename Item>
-    __device__ __forceinline__ bool span(const uint64_t* vertexList, const uint64_t first, const uint64_t last, const uint64_t heavy_from, Item item,
-                                         bool& nothing)
-    {
-        nothing = false;
-        if (reach < 2) return false;
-        uint64_t v_first = 0, v_last = 0;
-        item(first, v_first); item(last - 1, v_last);
-        const uint64_t e0 = vertexList[v_first], e1 = vertexList[v_last + 1];
-        if (e1 <= e0) { nothing = true; return true; }
-        const uint64_t p0 = view.page_of(e0), p1 = view.page_of(e1 - 1);
-        if (p1 - p0 >= 4ull * reach) return false;
-        auto touch = [](uint32_t) { return true; };
-        const uint32_t lane = bam::lane();
-        uint64_t seen = 0;
-        for (uint64_t c = p0; c <= p1; c += reach) {
-            uint64_t m = 0;
-            for (uint64_t b = first; b < last; b += BAM_WAVE_SIZE) {
-                uint64_t v = 0;
-                if (b + lane < last && item(b + lane, v)) {
-                    const uint64_t es = vertexList[v], ee = vertexList[v + 1];
-                    if (ee > es && ee - es < heavy_from) {
-                        const uint64_t pf = view.page_of(es), pl = view.page_of(ee - 1);
-                        const uint64_t f = pf > c ? pf - c : 0, l = pl < c + reach - 1 ? pl - c : reach - 1;
-                        if (pl >= c && f <= l) m |= (~0ull >> (63 - l)) & (~0ull << f);
-                    }
-                }
-            }
-#pragma unroll
-            for (uint32_t o = BAM_WAVE_SIZE / 2; o; o >>= 1) m |= bam::shfl(m, lane ^ o);
-            const bool take = ((m >> lane) & 1) != 0 && page_absent(view, c + lane);
-            if (bam::ballot(take)) view.acquire_helped(c + lane, take, false, touch, touch);
-            seen |= m;
-        }
-        view.n_access = view.n_hit = 0;
-        nothing = seen == 0;            /* no list to walk in [first, last): the caller need not look again */
-        return true;
-    }
-    /* wave-uniform: the list is elements [start, end); its first `asked` pages have been touched already */
-    __device__ __forceinline__ void begin(const uint64_t start, const uint64_t end, const uint32_t asked = 0)
-    {
-        long_list = false;
-        if (reach < 2 || end <= start) return;
-        last_page = view.page_of(end - 1);
-        long_list = last_page > view.page_of(start);
-        asked_to = asked ? view.page_of(start) + asked : 0;
-    }
-    /* lane l brings page (l mod 16) of a run of elements [start, end) of its own (four runs per wave, `want` says whether
-     * the lane's run is to be read at all): one batch of commands for what is not resident of the first sixteen pages of
-     * each.  False if the cache is too small for a wave to ask for that much at a time. */
-    __device__ __forceinline__ bool quads(const uint64_t start, const uint64_t end, const bool want)
-    {
-        if (reach < BAM_WAVE_SIZE) return false;
-        auto touch = [](uint32_t) { return true; };
-        const uint64_t page = want ? view.page_of(start) + (bam::lane() & 15u) : 0;
-        const bool take = want && end > start && page <= view.page_of(end - 1) && page_absent(view, page);
-        if (bam::ballot(take)) view.acquire_helped(page, take, false, touch, touch);
-        view.n_access = view.n_hit = 0;
-        return true;
-    }
-    /* wave-uniform: the walk is about to read from element `at` on */
-    __device__ __forceinline__ void step(const uint64_t at)
-    {
-        if (!long_list) return;
-        const uint64_t pg = view.page_of(at);
-        if (pg < asked_to) return;
-        const uint64_t p = pg + bam::lane();
-        auto touch = [](uint32_t) { return true; };
-        const bool take = bam::lane() < reach && p <= last_page && page_absent(view, p);
-        if (bam::ballot(take)) view.acquire_helped(p, take, false, touch, touch);
-        asked_to = pg + reach;
-        view.n_access = view.n_hit = 0;         /* not accesses of the kernel's own: kept out of the counters */
-    }
-};
-
-/*
- * Every lane brings a run of elements [es, ee) (possibly empty, each shorter than 2^20) and the vertex `src` the run
- * belongs to; the wave visits all elements of all runs, 64 per step, consecutive lanes taking consecutive elements
- * across the ends of the runs.  With lists of a dozen edges, walking one list per step leaves most lanes idle and
- * pays the whole chain of dependent loads (offsets, payload, label) once per vertex; packed, it is paid once per 64
- * edges.  A lane finds the run its element belongs to by binary search in the running sums of the run lengths
- * (six shuffles).  `read(i)` fetches element i, `visit(src, value, i)` consumes it.
- */
-template <typename Read, typename Visit>
-__device__ __forceinline__ void walk_packed(const uint64_t es, const uint64_t ee, const uint64_t src, Read read, Visit visit)
-{
-    const uint32_t lane = bam::lane();
-    const uint32_t len = (uint32_t)(ee - es);
-    uint32_t incl = len;
-#pragma unroll
-    for (uint32_t o = 1; o < BAM_WAVE_SIZE; o <<= 1) {
-        const uint32_t u = bam::shfl(incl, lane >= o ? lane - o : lane);
-        if (lane >= o) incl += u;
-    }
-    const uint32_t total = bam::shfl(incl, BAM_WAVE_SIZE - 1), excl = incl - len;
-    for (uint32_t base = 0; base < total; base += BAM_WAVE_SIZE) {
-        const uint32_t k = base + lane;
-        uint32_t j = 0;                                          /* number of runs that end at or before k */
-#pragma unroll
-        for (uint32_t step = BAM_WAVE_SIZE / 2; step; step >>= 1)
-            if (bam::shfl(incl, j + step - 1) <= k) j += step;
-        j &= BAM_WAVE_SIZE - 1;                                  /* lanes past the end: any valid lane, they do not visit */
-        const uint64_t i = bam::shfl(es, j) + (k - bam::shfl(excl, j));
-        const uint64_t s = bam::shfl(src, j);
-        if (k < total) visit(s, read(i), i);
-    }
-}
-
-/*
- * The traversal of the reference's coarsened per-vertex kernels (bfs/main.cu:658-689, cc/main.cu:123-144): the
- * vertices are handed out in groups of `coarse`, and the edge list of every active vertex is read through bam_ptr.
- * What differs, for the store's and the memory system's sake:
- *  - the launch has as many waves as the device holds at a time, and a wave takes the next piece of work when it is
- *    done with its last one (one atomic each).  One group per wave of a large grid leaves most of the device idle
- *    here: groups differ in length by orders of magnitude, and workgroups are started in order;
- *  - the flags and offsets of 64 vertices are read at a time, one vertex per lane, and the lists of those vertices
- *    are walked packed (walk_packed): 64 edges per step whichever vertices they belong to;
- *  - before the walk the pages that hold the lists of the group's active vertices are touched (list_read_ahead::span),
- *    so that what is not resident comes in as one batch of commands, not one trip to the store per vertex;
- *  - lists of BAM_HEAVY_EDGES entries and more are walked in pieces, by a wave each (below).
- */
-/*
- * A list of BAM_HEAVY_EDGES entries or more is not walked with its group: it is cut into pieces of BAM_PIECE_EDGES
- * entries, each walked by a wave of its own.  The hubs of a power-law graph have lists of hundreds of pages; walked
- * by one wave, a single hub takes longer than all other vertices of its level together.  Which lists are long does
- * not change from sweep to sweep, so the pieces are listed once per call (k_heavy_pieces) and every sweep hands them
- * out before the groups, longest work first: a piece whose vertex is not active costs its wave one look at the flag.
- */
-#define BAM_HEAVY_EDGES 1024u
-/* entries per piece: 16 pages of 4 KiB, which the wave that walks the piece asks for as one batch of commands.  Pieces
- * of the threshold's size reach the store as batches of two or three commands, and the store path moves far fewer
- * pages per second in such batches than in batches of sixteen */
-#define BAM_PIECE_EDGES 8192u
-#define BAM_PIECE_BUNDLE 4u             /* pieces handed to a wave at a time: sixteen lanes look after the sixteen pages of each */
-static_assert(BAM_PIECE_BUNDLE * 16u == BAM_WAVE_SIZE && BAM_PIECE_EDGES * 8u == 16u * 4096u, "a bundle's pages are shared out one per lane");
-struct heavy_piece_t { uint64_t v, first, last; };      /* entries [first, last) of the list of vertex v */
-
-__global__ void k_heavy_pieces(const uint64_t* vertexList, const uint64_t vertex_count, heavy_piece_t* pieces, unsigned long long* count)
-{
-    const uint64_t v = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (v >= vertex_count) return;
-    const uint64_t start = vertexList[v], end = vertexList[v + 1];
-    if (end - start < BAM_HEAVY_EDGES) return;
-    const uint64_t n = (end - start + BAM_PIECE_EDGES - 1) / BAM_PIECE_EDGES;
-    const unsigned long long at = atomicAdd(count, (unsigned long long)n);
-    for (uint64_t k = 0; k < n; k++) {
-        const uint64_t f = start + k * BAM_PIECE_EDGES;
-        pieces[at + k] = heavy_piece_t{v, f, f + BAM_PIECE_EDGES < end ? f + BAM_PIECE_EDGES : end};
-    }
-}
-
-/*
- * Reads with the page referenced for the one read only.  bam_ptr keeps every lane's page referenced until the lane
- * moves on: fine where the lanes of a wave read side by side, but 64 lanes that walk lists scattered over the edge
- * array would pin up to 64 pages per wave, and a cache with fewer free slots than that stops for good (lanes that
- * have their page wait for those that cannot get one).  Lanes on the same page still share one pair of atomics.
- */
-template <typename T>
-struct touch_reader {
-    array_d_t<T>* da = nullptr;
-    bam::range_view<T> view;
-    bool one_range = false, fast = false;
-    __device__ __forceinline__ void init(array_d_t<T>* a)
-    {
-        da = a;
-        one_range = a->n_ranges == 1;
-        if (one_range) { view.load(a->d_ranges); fast = a->d_ranges[0].cache.fast_reads != 0; }
-    }
-    __device__ __forceinline__ T read(const uint64_t i)
-    {
-        if (!one_range) return da->seq_read(i);
-        T ret = T();                                    /* stays T() if the wait is given up */
-        const uint64_t byte = view.byte_of(i);
-        /* resident pages without a reference at all, as array_d_t::seq_read does */
-        if (fast && bam_read_unpinned(view.pages + (byte >> view.page_size_log), view.base_addr, view.page_size_log, byte & (view.page_size - 1), ret)) {
-            view.account(true);
-            return ret;
-        }
-        auto use = [&](uint32_t slot) { ret = bam::ld_payload((T*)(view.slot_addr(slot) + (byte & (view.page_size - 1)))); return true; };
-        view.template acquire<true>(byte >> view.page_size_log, false, use, use);
-        return ret;
-    }
-    __device__ __forceinline__ void fini() { if (one_range) view.flush_stats(); }
-};
-
-/*
- * One sweep: the pieces of the long lists whose vertex is active(v), then `n_items` work items in groups of `coarse`,
- * each of which names a vertex and says whether it is to be walked: item(i, v).  visit(src, value, i) for every entry.
- * HOLD: the items are the vertices themselves (item i is vertex i, lists side by side), read through bam_ptr;
- * otherwise the items' lists lie anywhere, and they are read page by page without holding any.
- */
-template <bool HOLD, typename Item, typename Active, typename Visit>
-__device__ __forceinline__ void walk_item_groups(array_d_t<uint64_t>* da, const uint64_t* vertexList, const uint64_t n_items, const uint64_t coarse,
-                                                 const heavy_piece_t* heavy, const uint64_t n_heavy, unsigned long long* next_work,
-                                                 const bool backwards, Item item, Active active, Visit visit,
-                                                 list_read_ahead<uint32_t>* with = nullptr, const bool in_order = HOLD)
-{
-    const uint64_t laneIdx = threadIdx.x % BAM_WAVE_SIZE;
-    const uint64_t n_groups = (n_items + coarse - 1) / coarse;
-    const uint64_t n_bundles = (n_heavy + BAM_PIECE_BUNDLE - 1) / BAM_PIECE_BUNDLE;
-    bam_ptr<uint64_t> ptr(da);
-    touch_reader<uint64_t> touch;
-    if (!HOLD) touch.init(da);
-    list_read_ahead<uint64_t> ahead;
-    bool ready = false;
-    for (;;) {
-        unsigned long long w = 0;
-        if (laneIdx == 0) w = atomicAdd(next_work, 1ull);
-        w = bam::bcast((uint64_t)w, 0);
-        /* every other sweep runs from the far end of both lists of work: what the last sweep left in the cache is what
-         * this one asks for first */
-        const uint64_t wb = backwards ? n_bundles - 1 - w : w;
-        if (w < n_bundles) {
-            /* pieces of long lists, BAM_PIECE_BUNDLE per turn at the counter (every turn costs one atomic on one word, and on
-             * a sweep with little to do those atomics are what the sweep takes): all lanes side by side through bam_ptr,
-             * read ahead over the piece */
-            /* what the active pieces of the bundle need comes in as one batch: a piece by itself asks for six pages on
-             * average on a power-law graph, where most long lists are just over the threshold */
-            bool asked = false;
-            {
-                const uint64_t k = wb * BAM_PIECE_BUNDLE + laneIdx / 16;
-                heavy_piece_t mine = {0, 0, 0};
-                bool want = false;
-                if (k < n_heavy) { mine = heavy[k]; want = active(mine.v); }
-                if (bam::ballot(want)) {
-                    if (!ready) { ahead.init(da); ready = true; }
-                    asked = ahead.quads(mine.first, mine.last, want);
-                    if (with) with->quads(mine.first, mine.last, want);
-                }
-            }
-            for (uint64_t k = wb * BAM_PIECE_BUNDLE; k < (wb + 1) * BAM_PIECE_BUNDLE && k < n_heavy; k++) {
-                const heavy_piece_t pc = heavy[k];
-                if (!active(pc.v)) continue;
-                if (!ready) { ahead.init(da); ready = true; }
-                ahead.begin(pc.first, pc.last, asked ? 16u : 0u);
-                if (with) with->begin(pc.first, pc.last, asked ? 16u : 0u);
-                for (uint64_t i = (pc.first & 0xFFFFFFFFFFFFFFF0ull) + laneIdx; i < pc.last; i += BAM_WAVE_SIZE) {
-                    ahead.step(i - laneIdx > pc.first ? i - laneIdx : pc.first);
-                    if (with) with->step(i - laneIdx > pc.first ? i - laneIdx : pc.first);
-                    if (i >= pc.first) visit(pc.v, ptr.read(i), i);
-                }
-            }
-            continue;
-        }
-        if (w - n_bundles >= n_groups) break;
-        const uint64_t g = backwards ? n_groups - 1 - (w - n_bundles) : w - n_bundles;
-        const uint64_t first = g * coarse;
-        bool touched = false, nothing = false;
-        if (in_order) {
-            if (!ready) { ahead.init(da); ready = true; }
-            touched = ahead.span(vertexList, first, first + coarse < n_items ? first + coarse : n_items, BAM_HEAVY_EDGES, item, nothing);
-            if (with && touched && !nothing) { bool none; with->span(vertexList, first, first + coarse < n_items ? first + coarse : n_items, BAM_HEAVY_EDGES, item, none); }
-            if (nothing) continue;
-        }
-        for (uint64_t b = 0; b < coarse; b += BAM_WAVE_SIZE) {
-            const uint64_t at_item = first + b + laneIdx;
-            uint64_t mine = 0;
-            const bool act = b + laneIdx < coarse && at_item < n_items && item(at_item, mine);
-            if (!bam::ballot(act)) continue;
-            if (!ready) { ahead.init(da); ready = true; }
-            uint64_t es = 0, ee = 0;
-            if (act) { es = vertexList[mine]; ee = vertexList[mine + 1]; }
-            if (ee - es >= BAM_HEAVY_EDGES) ee = es;            /* walked in pieces */
-            if (!touched) {
-                /* a group whose lists cover too many pages for one look: the same for the 64 vertices at hand */
-                bool block_touched = false;
-                if (in_order) {
-                    const uint64_t last = first + coarse < n_items ? first + coarse : n_items;
-                    bool none;
-                    block_touched = ahead.span(vertexList, first + b, first + b + BAM_WAVE_SIZE < last ? first + b + BAM_WAVE_SIZE : last, BAM_HEAVY_EDGES, item, none);
-                    if (with && block_touched) with->span(vertexList, first + b, first + b + BAM_WAVE_SIZE < last ? first + b + BAM_WAVE_SIZE : last, BAM_HEAVY_EDGES, item, none);
-                }
-                if (!block_touched) { ahead.group(es, ee); if (with) with->group(es, ee); }
-            }
-            walk_packed(es, ee, mine, [&](uint64_t i) { if constexpr (HOLD) return ptr.read(i); else return touch.read(i); }, visit);
-        }
-    }
-    if (!HOLD) touch.fini();
-}
-
-/* the items are the vertices themselves, walked where active(v) */
-template <typename Active, typename Visit>
-__device__ __forceinline__ void walk_vertex_groups(array_d_t<uint64_t>* da, const uint64_t* vertexList, const uint64_t vertex_count, const uint64_t coarse,
-                                                   const heavy_piece_t* heavy, const uint64_t n_heavy, unsigned long long* next_work, const bool backwards,
-                                                   Active active, Visit visit, list_read_ahead<uint32_t>* with = nullptr)
-{
-    walk_item_groups<true>(da, vertexList, vertex_count, coarse, heavy, n_heavy, next_work, backwards,
-                           [&](uint64_t i, uint64_t& v) { v = i; return active(i); }, active, visit, with);
-}
-
-__global__ __launch_bounds__(128) void k_bfs_coalesce_coarse_ptr_pc(array_d_t<uint64_t>* da, uint32_t* label, const uint32_t level, const uint64_t vertex_count,
-                                                                   const uint64_t* vertexList, uint64_t* changed, uint64_t coarse,
-                                                                   const heavy_piece_t* heavy, uint64_t n_heavy, unsigned long long* next_work)
-{
-    bool any = false;
-    walk_vertex_groups(da, vertexList, vertex_count, coarse, heavy, n_heavy, next_work, (level & 1u) != 0,
-                       [&](uint64_t v) { return label[v] == level; },
-                       [&](uint64_t, uint64_t next, uint64_t) { if (label[next] == MYINFINITY) { label[next] = level + 1; any = true; } });
-    if (any) *changed = 1;
-}
-
-// ---- BFS over a queue of the level's vertices (benchmarks/bfs/main.cu:409-451 kernel_frontier_coalesce_ptr_pc) ----
-/* a vertex found for the first time (the exchange on its label decides who found it) goes to the next level's queue;
- * the lanes of a wave that found one at the same step take their places in it with one atomic */
-__device__ __forceinline__ void bfs_frontier_visit(uint32_t* label, const uint32_t level, uint32_t* next_frontier, unsigned long long* next_size, const uint64_t next)
-{
-    if (label[next] != MYINFINITY) return;
-    if (atomicExch(label + next, level + 1) != MYINFINITY) return;
-    const uint64_t mask = bam::active_mask();
-    const uint32_t leader = bam::first_lane(mask);
-    unsigned long long pos = 0;
-    if (bam::lane() == leader) pos = atomicAdd(next_size, (unsigned long long)bam::popc(mask));
-    pos = bam::bcast((uint64_t)pos, leader);
-    next_frontier[pos + bam::rank_in(mask)] = (uint32_t)next;
-}
-
-__global__ __launch_bounds__(128) void k_bfs_frontier_coalesce_ptr_pc(array_d_t<uint64_t>* da, uint32_t* label, const uint32_t level, const uint64_t* vertexList,
-                                                                     const uint32_t* curr_frontier, const uint64_t curr_size, uint32_t* next_frontier,
-                                                                     unsigned long long* next_size, uint64_t group,
-                                                                     const heavy_piece_t* heavy, uint64_t n_heavy, unsigned long long* next_work, bool sorted)
-{
-    walk_item_groups<false>(da, vertexList, curr_size, group, heavy, n_heavy, next_work, false,
-                            [&](uint64_t i, uint64_t& v) { v = curr_frontier[i]; return true; },
-                            [&](uint64_t v) { return label[v] == level; },
-                            [&](uint64_t, uint64_t next, uint64_t) { bfs_frontier_visit(label, level, next_frontier, next_size, next); },
-                            nullptr, sorted);
-}
-
-// ---- CC: min-label propagation (benchmarks/cc/main.cu:123-144, 595-617) ----
-__device__ __forceinline__ void cc_compute(uint64_t cid, unsigned long long* comp, uint64_t next, bool* next_visit, bool* changed)
-{
-    const unsigned long long comp_src = comp[cid], comp_next = comp[next];
-    if (comp_next == comp_src) return;
-    uint64_t next_target;
-    unsigned long long comp_target;
-    if (comp_src < comp_next) { next_target = next; comp_target = comp_src; }
-    else { next_target = cid; comp_target = comp_next; }
-    atomicMin(&comp[next_target], comp_target);
-    next_visit[next_target] = true;
-    *changed = true;
-}
-
-__global__ __launch_bounds__(128) void k_cc_coalesce_coarse_ptr_pc(array_d_t<uint64_t>* da, bool* curr_visit, bool* next_visit, uint64_t vertex_count,
-                                                                  const uint64_t* vertexList, unsigned long long* comp, bool* changed, uint64_t coarse,
-                                                                  const heavy_piece_t* heavy, uint64_t n_heavy, unsigned long long* next_work, uint32_t sweep)
-{
-    walk_vertex_groups(da, vertexList, vertex_count, coarse, heavy, n_heavy, next_work, (sweep & 1u) != 0,
-                       [&](uint64_t v) { return curr_visit[v]; },
-                       [&](uint64_t v, uint64_t next, uint64_t) { cc_compute(v, comp, next, next_visit, changed); });
-}
-
-// ---- BFS / CC by edge page (benchmarks/bfs/main.cu:1074-1140 kernel_optimized_ptr_pc, first-vertex table :122-181) ----
-/*
- * first[p], p = 0 .. n_pages: the vertex whose edge list holds edge p * epp (the last vertex with
- * offsets[v] <= p * epp); first[n_pages] = V - 1.  The vertices with edges on page p are first[p] .. first[p + 1].
- */
-__global__ void k_page_first_vertex(const uint64_t* offsets, uint64_t n_vertices, uint64_t epp, uint64_t n_pages, uint64_t* first)
-{
-    const uint64_t p = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (p > n_pages) return;
-    const uint64_t e = p * epp;
-    uint64_t lo = 0, hi = n_vertices + 1;            /* first index with offsets[idx] > e */
-    while (lo < hi) {
-        const uint64_t mid = (lo + hi) >> 1;
-        if (offsets[mid] > e) hi = mid; else lo = mid + 1;
-    }
-    uint64_t v = lo ? lo - 1 : 0;
-    if (v >= n_vertices) v = n_vertices - 1;
-    first[p] = v;
-}
-
-/*
- * One wave, `ppw` consecutive pages of the edge array per trip (lane l looks after page l of the trip), trips
- * handed out wave by wave along the array.  A page is wanted when one of its vertices is active; the wanted pages
- * of a trip are taken with one acquire, so their misses go to the store as one batch of commands, and the whole
- * wave then walks the active vertices of each page, 64 edges at a time, before the references are dropped.
- * A wave holds at most `ppw` pages at a time; the launch keeps waves x ppw under half the cache.
- */
-template <typename Active, typename Visit>
-__device__ __forceinline__ void graph_by_page(array_d_t<uint64_t>* da, const uint64_t* offsets, const uint64_t* first, const uint64_t n_edges,
-                                              const uint32_t ppw, const bool backwards, Active active, Visit visit)
-{
-    const uint32_t lane = bam::lane();
-    const uint64_t wave = ((uint64_t)blockIdx.x * blockDim.x + threadIdx.x) / BAM_WAVE_SIZE;
-    const uint64_t n_waves = (uint64_t)gridDim.x * blockDim.x / BAM_WAVE_SIZE;
-    bam::range_view<uint64_t> view;
-    view.load(da->d_ranges);
-    const uint32_t epp = view.page_size / 8;
-    const uint64_t n_pages = (n_edges + epp - 1) / epp;
-    const uint64_t pso_pages = view.pso >> view.page_size_log;
-    const uint64_t n_trips = (n_pages + ppw - 1) / ppw;
-    for (uint64_t t = wave; t < n_trips; t += n_waves) {
-        /* every other sweep runs from the far end: what the last sweep left in the cache is what this one asks for first */
-        const uint64_t p0 = (backwards ? n_trips - 1 - t : t) * ppw;
-        const uint64_t p = p0 + lane;
-        /* which pages of the trip hold entries of an active vertex: the lanes go over the trip's vertices side by side
-         * (their flags and offsets are consecutive in memory) and mark the pages each active list covers */
-        const uint64_t p_end = p0 + ppw < n_pages ? p0 + ppw : n_pages;
-        const uint64_t trip_start = p0 * epp, trip_end = p_end * epp < n_edges ? p_end * epp : n_edges;
-        uint64_t marks = 0;
-        for (uint64_t vbase = first[p0], v_last = first[p_end]; vbase <= v_last; vbase += BAM_WAVE_SIZE) {
-            const uint64_t v = vbase + lane;
-            if (v <= v_last && active(v)) {
-                uint64_t es = offsets[v], ee = offsets[v + 1];
-                if (es < trip_start) es = trip_start;
-                if (ee > trip_end) ee = trip_end;
-                if (ee > es) marks |= (~0ull >> (63 - (ee - 1 - trip_start) / epp)) & (~0ull << ((es - trip_start) / epp));
-            }
-        }
-#pragma unroll
-        for (uint32_t o = BAM_WAVE_SIZE / 2; o; o >>= 1) marks |= bam::shfl(marks, lane ^ o);
-        const bool want = ((marks >> lane) & 1) != 0;
-        uint64_t va = 0, vb = 0;
-        if (want) { va = first[p]; vb = first[p + 1]; }
-        uint32_t slot = BAM_NO_SLOT;
-        if (bam::ballot(want)) {
-            /* the lanes without a page of their own come along and help move what the others load */
-            auto keep = [&](uint32_t s_) { slot = s_; return false; };
-            view.acquire_helped(p + pso_pages, want, false, keep, keep);
-        }
-        /* a page whose wait was given up (the controller is marked aborted) has no slot and is not walked */
-        for (uint64_t m = bam::ballot(want && slot != BAM_NO_SLOT); m; m &= m - 1) {
-            const uint32_t j = bam::first_lane(m);
-            const uint64_t va_j = bam::bcast(va, j), vb_j = bam::bcast(vb, j);
-            const uint64_t ps = (p0 + j) * epp, pe = ps + epp < n_edges ? ps + epp : n_edges;
-            const uint64_t* payload = (const uint64_t*)view.slot_addr(bam::bcast(slot, j));
-            for (uint64_t vbase = va_j; vbase <= vb_j; vbase += BAM_WAVE_SIZE) {
-                const uint64_t v = vbase + lane;
-                uint64_t es = 0, ee = 0;
-                if (v <= vb_j && active(v)) {
-                    es = offsets[v]; ee = offsets[v + 1];
-                    if (es < ps) es = ps;
-                    if (ee > pe) ee = pe;
-                }
-                if (ee < es) ee = es;
-                walk_packed(es, ee, v, [&](uint64_t i) { return bam::ld_payload(payload + (i - ps)); }, visit);
-            }
-        }
-        if (want) view.release(p + pso_pages, false);
-    }
-    view.flush_stats();
-}
-
-__global__ __launch_bounds__(64) void k_bfs_by_page(array_d_t<uint64_t>* da, uint32_t* label, const uint32_t level, const uint64_t* offsets,
-                                                     const uint64_t* first, uint64_t n_edges, uint32_t ppw, uint64_t* changed)
-{
-    bool any = false;
-    graph_by_page(da, offsets, first, n_edges, ppw, (level & 1u) != 0,
-                  [&](uint64_t v) { return label[v] == level; },
-                  [&](uint64_t, uint64_t next, uint64_t) { if (label[next] == MYINFINITY) { label[next] = level + 1; any = true; } });
-    if (any) *changed = 1;
-}
-
-__global__ __launch_bounds__(64) void k_cc_by_page(array_d_t<uint64_t>* da, bool* curr_visit, bool* next_visit, const uint64_t* offsets,
-                                                    const uint64_t* first, uint64_t n_edges, uint32_t ppw, uint32_t sweep, unsigned long long* comp, bool* changed)
-{
-    graph_by_page(da, offsets, first, n_edges, ppw, (sweep & 1u) != 0,
-                  [&](uint64_t v) { return curr_visit[v]; },
-                  [&](uint64_t src, uint64_t next, uint64_t) { cc_compute(src, comp, next, next_visit, changed); });
-}
-
-// ---- vectoradd (benchmarks/vectoradd/main.cu:102-117 kernel_baseline_ptr_pc): C[i] = A[i] + B[i], all three behind the cache ----
-__global__ __launch_bounds__(64) void k_vectoradd_ptr_pc(array_d_t<uint64_t>* da, array_d_t<uint64_t>* db, uint64_t n_elems, array_d_t<uint64_t>* dc)
-{
-    const uint64_t tid = (uint64_t)blockDim.x * blockIdx.x + threadIdx.x;
-    bam_ptr<uint64_t> Aptr(da);
-    bam_ptr<uint64_t> Bptr(db);
-    bam_ptr<uint64_t> Cptr(dc);
-    const bam_ptr<uint64_t>& A = Aptr;
-    const bam_ptr<uint64_t>& B = Bptr;
-    const uint64_t first = tid - threadIdx.x % BAM_WAVE_SIZE;
-    if (first < n_elems) {
-        touch_ahead(da, first, n_elems, BAM_WAVE_SIZE, 0);
-        touch_ahead(db, first, n_elems, BAM_WAVE_SIZE, 1);
-        touch_ahead(dc, first, n_elems, BAM_WAVE_SIZE, 2);
-    }
-    if (tid < n_elems) Cptr[tid] = A[tid] + B[tid];
-}
-
-// ---- reduction (benchmarks/reduction/main.cu:166-195 kernel_reduce_baseline_ptr_pc): output[b] = sum of the 2 x blockDim elements of block b ----
-__global__ void k_reduce_ptr_pc(array_d_t<uint64_t>* da, unsigned long long* output, uint64_t len)
-{
-    __shared__ uint64_t wave_total[1024 / BAM_WAVE_SIZE];
-    const uint64_t tid = threadIdx.x, start = 2ull * blockDim.x * blockIdx.x;
-    uint64_t v = 0;
-    {
-        bam_ptr<uint64_t> in_ptr(da);
-        const bam_ptr<uint64_t>& input = in_ptr;
-        /* a workgroup reads 2 x blockDim consecutive elements: its waves' first elements */
-        const uint64_t first = start + tid - tid % BAM_WAVE_SIZE;
-        if (first < len) touch_ahead(da, first, len);
-        if (first + blockDim.x < len) touch_ahead(da, first + blockDim.x, len);
-        if (start + tid < len) v = input[start + tid];
-        if (blockDim.x + start + tid < len) v += input[blockDim.x + start + tid];
-    }
-    v = wave_sum(v);
-    if (bam::lane() == 0) wave_total[tid / BAM_WAVE_SIZE] = v;
-    __syncthreads();
-    if (tid < BAM_WAVE_SIZE) {
-        v = wave_sum(tid < blockDim.x / BAM_WAVE_SIZE ? wave_total[tid] : 0);
-        if (tid == 0) output[blockIdx.x] = v;
-    }
-}
-
-// ---- scan (benchmarks/scan/main.cu:147-190 kernel_scan_baseline_ptr_pc, :89-100 finalsum) ----
-/* inclusive sums over the 64 lanes of a wave (all lanes active) */
-__device__ __forceinline__ uint64_t wave_inclusive_sum(uint64_t v)
-{
-    const uint32_t lane = bam::lane();
-#pragma unroll
-    for (uint32_t o = 1; o < BAM_WAVE_SIZE; o <<= 1) {
-        const uint64_t u = bam::shfl(v, lane >= o ? lane - o : lane);
-        if (lane >= o) v += u;
-    }
-    return v;
-}
-
-/*
- * Block b scans its 2 x blockDim elements: output[i] = sum of the block's elements up to and including i,
- * intermediate[b] = the block's total.  The elements are read as the reference reads them (thread t takes t and
- * t + blockDim, so a wave reads consecutive elements through one page reference); the scan itself runs over wave
- * shuffles on pairs of neighbours rather than the two tree passes over shared memory.
- */
-__global__ void k_scan_ptr_pc(array_d_t<uint64_t>* da, unsigned long long* output, unsigned long long* intermediate, uint64_t len)
-{
-    extern __shared__ uint64_t scan_mem[];                      /* 2 x blockDim elements, then one total per wave */
-    const uint32_t B = blockDim.x, t = threadIdx.x;
-    uint64_t* wave_total = scan_mem + 2 * B;
-    const uint64_t idx = 2ull * blockIdx.x * B + t;
-    {
-        bam_ptr<uint64_t> in_ptr(da);
-        const bam_ptr<uint64_t>& ptr = in_ptr;
-        const uint64_t first = idx - t % BAM_WAVE_SIZE;
-        if (first < len) touch_ahead(da, first, len);
-        if (first + B < len) touch_ahead(da, first + B, len);
-        scan_mem[t] = idx < len ? ptr[idx] : 0;
-        scan_mem[t + B] = idx + B < len ? ptr[idx + B] : 0;
-    }
-    __syncthreads();
-    const uint64_t a = scan_mem[2 * t], b = a + scan_mem[2 * t + 1];
-    const uint64_t s = wave_inclusive_sum(b);
-    if (bam::lane() == BAM_WAVE_SIZE - 1) wave_total[t / BAM_WAVE_SIZE] = s;
-    __syncthreads();
-    uint64_t before = s - b;
-    for (uint32_t w = 0; w < t / BAM_WAVE_SIZE; w++) before += wave_total[w];
-    scan_mem[2 * t] = before + a;
-    scan_mem[2 * t + 1] = before + b;
-    __syncthreads();
-    if (idx < len) output[idx] = scan_mem[t];
-    if (idx + B < len) output[idx + B] = scan_mem[t + B];
-    if (intermediate && t == B - 1) intermediate[blockIdx.x] = before + b;
-}
-
-/* one block: v[i] = v[0] + ... + v[i] in place (the reference calls cub::DeviceScan::InclusiveSum here, scan/main.cu:416-418) */
-__global__ void k_scan_block_totals(unsigned long long* v, uint64_t n)
-{
-    __shared__ uint64_t wave_total[1024 / BAM_WAVE_SIZE];
-    __shared__ uint64_t carry_s;
-    const uint32_t t = threadIdx.x;
-    if (t == 0) carry_s = 0;
-    __syncthreads();
-    for (uint64_t base = 0; base < n; base += blockDim.x) {
-        const uint64_t x = base + t < n ? v[base + t] : 0;
-        const uint64_t s = wave_inclusive_sum(x);
-        if (bam::lane() == BAM_WAVE_SIZE - 1) wave_total[t / BAM_WAVE_SIZE] = s;
-        __syncthreads();
-        uint64_t r = carry_s + s;
-        for (uint32_t w = 0; w < t / BAM_WAVE_SIZE; w++) r += wave_total[w];
-        if (base + t < n) v[base + t] = r;
-        __syncthreads();
-        if (t == blockDim.x - 1) carry_s = r;
-        __syncthreads();
-    }
-}
-
-__global__ void k_scan_finalsum(const unsigned long long* scanned_totals, unsigned long long* output, uint64_t len)
-{
-    if (blockIdx.x == 0) return;
-    const uint64_t B = blockDim.x, idx = 2ull * blockIdx.x * B + threadIdx.x;
-    const uint64_t add = scanned_totals[blockIdx.x - 1];
-    if (idx < len) output[idx] += add;
-    if (idx + B < len) output[idx + B] += add;
-}
-
-// ---- PageRank by residual pushes (benchmarks/pagerank/main.cu:107-115 initialize, :252-273 kernel_coalesce_pc, :412-421 update) ----
-__global__ void k_pr_initialize(bool* label, float* delta, float* residual, float* value, const uint64_t vertex_count, const uint64_t* vertexList, float alpha)
-{
-    const uint64_t tid = (uint64_t)blockDim.x * blockIdx.x + threadIdx.x;
-    if (tid < vertex_count) {
-        value[tid] = 1.0f - alpha;
-        delta[tid] = (1.0f - alpha) * alpha / (vertexList[tid + 1] - vertexList[tid]);
-        residual[tid] = 0.0f;
-        label[tid] = true;
-    }
-}
-
-/* every neighbour of a flagged vertex receives the vertex's delta: the group walk of the per-vertex graph kernels; the flags
- * are cleared by the host loop after the sweep */
-__global__ __launch_bounds__(128) void k_pr_coalesce_pc(array_d_t<uint64_t>* da, const bool* label, const float* delta, float* residual,
-                                                        const uint64_t vertex_count, const uint64_t* vertexList, uint64_t group,
-                                                        const heavy_piece_t* heavy, uint64_t n_heavy, unsigned long long* next_work, uint32_t sweep)
-{
-    walk_vertex_groups(da, vertexList, vertex_count, group, heavy, n_heavy, next_work, (sweep & 1u) != 0,
-                       [&](uint64_t v) { return label[v]; },
-                       [&](uint64_t src, uint64_t next, uint64_t) { unsafeAtomicAdd(&residual[next], delta[src]); });
-}
-
-/* the same pushes taken page by page of the edge array; the flags are cleared by the host loop after the sweep */
-__global__ __launch_bounds__(64) void k_pr_by_page(array_d_t<uint64_t>* da, const bool* label, const float* delta, float* residual, const uint64_t* offsets,
-                                                    const uint64_t* first, uint64_t n_edges, uint32_t ppw, uint32_t sweep)
-{
-    graph_by_page(da, offsets, first, n_edges, ppw, (sweep & 1u) != 0,
-                  [&](uint64_t v) { return label[v]; },
-                  [&](uint64_t src, uint64_t next, uint64_t) { unsafeAtomicAdd(&residual[next], delta[src]); });
-}
-
-__global__ void k_pr_update(bool* label, float* delta, float* residual, float* value, const uint64_t vertex_count, const uint64_t* vertexList,
-                            float tolerance, float alpha, bool* changed)
-{
-    const uint64_t tid = (uint64_t)blockDim.x * blockIdx.x + threadIdx.x;
-    if (tid < vertex_count && residual[tid] > tolerance) {
-        value[tid] += residual[tid];
-        delta[tid] = residual[tid] * alpha / (vertexList[tid + 1] - vertexList[tid]);
-        residual[tid] = 0.0f;
-        label[tid] = true;
-        *changed = true;
-    }
-}
-
-// ---- SSSP (benchmarks/sssp/main.cu:174-201 kernel_coalesce_pc, :282-292 update): 32-bit costs, weights in their own array ----
-/* relaxation of the edges of the flagged vertices with the cost each has at the time (any cost a vertex holds is the cost of a
- * path to it); the group walk of the per-vertex graph kernels, the weight of entry i read through a bam_ptr of its own */
-template <bool FLOAT>
-__device__ __forceinline__ void sssp_relax(uint32_t* newCostList, const bam_ptr<uint32_t>& weights, uint64_t src, uint64_t next, uint64_t i)
-{
-    const uint32_t have = __hip_atomic_load(&newCostList[src], __ATOMIC_RELAXED, BAM_AGENT), w = weights[i];
-    /* single-precision costs (benchmarks/sssp_float/main.cu:69, 91-106, 194-217) travel as their bit patterns: for floats that
-     * are not negative the order of the patterns is the order of the values, so the minimum is the integer one */
-    const uint32_t cost = FLOAT ? __float_as_uint(__uint_as_float(have) + __uint_as_float(w)) : have + w;
-    if (__hip_atomic_load(&newCostList[next], __ATOMIC_RELAXED, BAM_AGENT) > cost) atomicMin(&newCostList[next], cost);
-}
-
-template <bool FLOAT>
-__global__ __launch_bounds__(128) void k_sssp_coalesce_pc(array_d_t<uint64_t>* de, array_d_t<uint32_t>* dw, const bool* label, uint32_t* newCostList,
-                                                          const uint64_t vertex_count, const uint64_t* vertexList, uint64_t group,
-                                                          const heavy_piece_t* heavy, uint64_t n_heavy, unsigned long long* next_work, uint32_t sweep)
-{
-    bam_ptr<uint32_t> wptr(dw);
-    /* entry i of the weight array belongs to entry i of the edge array: what is touched ahead for the one is touched for the other */
-    list_read_ahead<uint32_t> wahead;
-    wahead.init(dw);
-    walk_vertex_groups(de, vertexList, vertex_count, group, heavy, n_heavy, next_work, (sweep & 1u) != 0,
-                       [&](uint64_t v) { return label[v]; },
-                       [&](uint64_t src, uint64_t next, uint64_t i) { sssp_relax<FLOAT>(newCostList, wptr, src, next, i); }, &wahead);
-}
-
-__global__ void k_sssp_update(bool* label, uint32_t* costList, const uint32_t* newCostList, const uint64_t vertex_count, bool* changed)
-{
-    const uint64_t tid = (uint64_t)blockDim.x * blockIdx.x + threadIdx.x;
-    if (tid < vertex_count && newCostList[tid] < costList[tid]) {
-        costList[tid] = newCostList[tid];
-        label[tid] = true;
-        *changed = true;
-    }
-}
-
 /* one thread per request over an array of 32-bit elements: sum of the values read */
 __global__ void k_array32_read(array_d_t<uint32_t>* dr, uint64_t n_reqs, const uint64_t* assignment, uint64_t stride, unsigned long long* sum)
 {
@@ -1204,12 +350,6 @@ __global__ void k_array32_read(array_d_t<uint32_t>* dr, uint64_t n_reqs, const u
     uint64_t v = 0;
     if (tid < n_reqs) v = (*dr)[assignment ? assignment[tid] : tid * stride];
     block_accumulate(sum, v);
-}
-
-__global__ void k_iota(unsigned long long* p, uint64_t n)
-{
-    const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) p[i] = i;
 }
 
 // ---- synthetic inputs ----
@@ -1290,8 +430,6 @@ __global__ void k_host_pull(const uint4* __restrict__ host, uint4* __restrict__ 
         for (uint32_t i = bam::lane(); i < chunk16; i += BAM_WAVE_SIZE) d[i] = s[i];
     }
 }
-
-inline uint32_t blocks_for(uint64_t n, uint32_t bs) { return (uint32_t)((n + bs - 1) / bs); }
 
 void fill_backing(uint64_t seed, uint64_t* p, uint64_t n_words)
 {
@@ -1405,6 +543,35 @@ int bam_ctrl_info(bam_ctrl_t* c, uint64_t* out, int reset)
     else hip_err_chk(hipMemcpy(&out[4], c->c->d_ctrl_ptr, sizeof(uint64_t), hipMemcpyDeviceToHost));
     out[5] = c->c->completion_errors();
     BAM_API_END
+}
+
+int bam_ctrl_queue_state(bam_ctrl_t* c, uint32_t qp, uint64_t* out16, uint32_t* slots, uint32_t n_slots)
+{
+    if (!c || !out16) return fail(EINVAL, "bam_ctrl_queue_state: null argument");
+    if (qp >= c->c->n_qps) return fail(EINVAL, "bam_ctrl_queue_state: no such queue pair");
+    BAM_API_BEGIN
+    nvm_queue_t sq, cq;
+    hip_err_chk(hipMemcpy(&sq, &c->c->d_qps[qp].sq, sizeof(sq), hipMemcpyDeviceToHost));
+    hip_err_chk(hipMemcpy(&cq, &c->c->d_qps[qp].cq, sizeof(cq), hipMemcpyDeviceToHost));
+    out16[0] = sq.qs; out16[1] = sq.in_ticket; out16[2] = sq.tail_lock >> 1; out16[3] = sq.tail_lock & 1u; out16[4] = sq.head;
+    out16[5] = cq.head_lock >> 1; out16[6] = cq.head_lock & 1u; out16[7] = cq.n_errors;
+    for (uint32_t k = 0; k < 8; k++) out16[8 + k] = 0;
+    if (slots && n_slots) {
+        const uint32_t n = n_slots < sq.qs ? n_slots : sq.qs;
+        std::vector<uint32_t> a(sq.qs), b(sq.qs), d(sq.qs);
+        hip_err_chk(hipMemcpy(a.data(), sq.tickets, sq.qs * 4, hipMemcpyDeviceToHost));
+        hip_err_chk(hipMemcpy(b.data(), sq.tail_mark, sq.qs * 4, hipMemcpyDeviceToHost));
+        hip_err_chk(hipMemcpy(d.data(), sq.cid, sq.qs * 4, hipMemcpyDeviceToHost));
+        for (uint32_t i = 0; i < n; i++) { slots[3 * i] = a[i]; slots[3 * i + 1] = b[i]; slots[3 * i + 2] = d[i]; }
+    }
+    BAM_API_END
+}
+
+int bam_target_queue_state(bam_target_t* t, uint32_t qid, uint64_t* out8)
+{
+    if (!t || !out8) return fail(EINVAL, "bam_target_queue_state: null argument");
+    const int rc = nvmt_queue_state(t->t, (uint16_t)qid, out8);
+    return rc ? fail(rc, "bam_target_queue_state: no such queue") : 0;
 }
 
 int bam_ctrl_aborted(bam_ctrl_t* c, int clear)
@@ -1808,429 +975,6 @@ int bam_block_checksum(bam_page_cache_t* pc, uint64_t n_slots, uint32_t req_byte
     BAM_API_END
 }
 
-namespace {
-/* the pieces of the long edge lists of a graph, listed once per call, and the counter that hands out the work of a sweep:
- * a list of d >= BAM_HEAVY_EDGES entries makes at most d / BAM_PIECE_EDGES + 1 <= 2 d / BAM_HEAVY_EDGES pieces */
-struct sweep_work {
-    BufferPtr buf, cnt;
-    heavy_piece_t* pieces;
-    unsigned long long* count;       /* [0] number of pieces, [1] next piece of work of the sweep */
-    uint64_t n_pieces = 0;
-    uint64_t group;                  /* vertices handed to a wave at a time */
-    uint64_t resident;               /* waves the device holds at a time */
-    sweep_work(uint64_t n_edges, uint64_t n_vertices, uint32_t coarse, const uint64_t* d_offsets, hipStream_t st)
-    {
-        const uint64_t cap = 2 * (n_edges / BAM_HEAVY_EDGES) + 1;
-        buf = createBuffer(cap * sizeof(heavy_piece_t), 0);
-        cnt = createBuffer(2 * sizeof(unsigned long long), 0);
-        pieces = (heavy_piece_t*)buf.get();
-        count = (unsigned long long*)cnt.get();
-        /* a group's lists are asked for as one batch of commands: a few hundred vertices make that batch large enough for the
-         * store path, and keep the one word all waves take their work from out of the way */
-        group = coarse > 512 ? coarse : 512;
-        int dev = 0, cus = 0;
-        hip_err_chk(hipGetDevice(&dev));
-        hip_err_chk(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-        resident = (uint64_t)cus * 16;
-        hip_err_chk(hipMemsetAsync(count, 0, 2 * sizeof(unsigned long long), st));
-        hipLaunchKernelGGL(k_heavy_pieces, dim3(blocks_for(n_vertices, 256)), dim3(256), 0, st, d_offsets, n_vertices, pieces, count);
-        hip_err_chk(hipGetLastError());
-        unsigned long long n = 0;
-        hip_err_chk(hipMemcpyAsync(&n, count, sizeof(n), hipMemcpyDeviceToHost, st));
-        hip_err_chk(hipStreamSynchronize(st));
-        n_pieces = n;
-    }
-    /* workgroups of two waves for a sweep over `n_items` items in groups of `grp` */
-    uint32_t blocks(uint64_t n_items, uint64_t grp) const
-    {
-        const uint64_t units = (n_pieces + BAM_PIECE_BUNDLE - 1) / BAM_PIECE_BUNDLE + (n_items + grp - 1) / grp;
-        return (uint32_t)(((units < resident ? units : resident) + 1) / 2);
-    }
-    void reset(hipStream_t st) { hip_err_chk(hipMemsetAsync(count + 1, 0, sizeof(unsigned long long), st)); }
-};
-} // namespace
-
-int bam_bfs(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t src, uint32_t* d_labels,
-            uint32_t coarse, uint32_t* iterations, void* stream)
-{
-    if (!edges || !d_offsets || !d_labels) return fail(EINVAL, "bam_bfs: null argument");
-    if (src >= n_vertices || !coarse) return fail(EINVAL, "bam_bfs: source out of range or coarse = 0");
-    BAM_API_BEGIN
-    hipStream_t st = (hipStream_t)stream;
-    BufferPtr changed_buf = createBuffer(sizeof(uint64_t), 0);
-    uint64_t* changed_d = (uint64_t*)changed_buf.get();
-    const uint32_t zero = 0;
-    hip_err_chk(hipMemsetAsync(d_labels, 0xFF, n_vertices * sizeof(uint32_t), st));
-    hip_err_chk(hipMemcpyAsync(d_labels + src, &zero, sizeof(uint32_t), hipMemcpyHostToDevice, st));
-    const uint32_t threads = 128;
-    sweep_work work(edges->a->adt.n_elems, n_vertices, coarse, d_offsets, st);
-    uint32_t level = 0, iter = 0;
-    uint64_t changed_h;
-    do {
-        changed_h = 0;
-        hip_err_chk(hipMemcpyAsync(changed_d, &changed_h, sizeof(uint64_t), hipMemcpyHostToDevice, st));
-        work.reset(st);
-        hipLaunchKernelGGL(k_bfs_coalesce_coarse_ptr_pc, dim3(work.blocks(n_vertices, work.group)), dim3(threads), 0, st,
-                           edges->a->d_array_ptr, d_labels, level, n_vertices, d_offsets, changed_d, work.group, work.pieces, work.n_pieces, work.count + 1);
-        hip_err_chk(hipGetLastError());
-        iter++; level++;
-        hip_err_chk(hipMemcpyAsync(&changed_h, changed_d, sizeof(uint64_t), hipMemcpyDeviceToHost, st));
-        hip_err_chk(hipStreamSynchronize(st));
-    } while (changed_h);
-    if (iterations) *iterations = iter;
-    BAM_API_END
-}
-
-int bam_bfs_frontier(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t src, uint32_t* d_labels,
-                     uint32_t* iterations, void* stream)
-{
-    if (!edges || !d_offsets || !d_labels) return fail(EINVAL, "bam_bfs_frontier: null argument");
-    if (src >= n_vertices) return fail(EINVAL, "bam_bfs_frontier: source out of range");
-    if (n_vertices > 0xFFFFFFFFull) return fail(EINVAL, "bam_bfs_frontier: the queues hold 32-bit vertex numbers");
-    BAM_API_BEGIN
-    hipStream_t st = (hipStream_t)stream;
-    /* two queues of at most every vertex once (benchmarks/bfs/main.cu:1489-1492); the size of the next one is the reference's `changed` */
-    BufferPtr queue_a = createBuffer(n_vertices * sizeof(uint32_t), 0), queue_b = createBuffer(n_vertices * sizeof(uint32_t), 0);
-    BufferPtr size_buf = createBuffer(sizeof(unsigned long long), 0);
-    uint32_t* curr = (uint32_t*)queue_a.get();
-    uint32_t* next = (uint32_t*)queue_b.get();
-    unsigned long long* next_size = (unsigned long long*)size_buf.get();
-    const uint32_t zero = 0, src32 = (uint32_t)src;
-    hip_err_chk(hipMemsetAsync(d_labels, 0xFF, n_vertices * sizeof(uint32_t), st));
-    hip_err_chk(hipMemcpyAsync(d_labels + src, &zero, sizeof(uint32_t), hipMemcpyHostToDevice, st));
-    hip_err_chk(hipMemcpyAsync(curr, &src32, sizeof(uint32_t), hipMemcpyHostToDevice, st));
-    const uint32_t threads = 128;
-    uint64_t group = BAM_WAVE_SIZE;                 /* queue entries handed to a wave at a time: one per lane, more of a sorted queue */
-    bool sorted = true;                             /* the first queue holds the source alone */
-    sweep_work work(edges->a->adt.n_elems, n_vertices, 1, d_offsets, st);
-    uint32_t level = 0, iter = 0;
-    unsigned long long active = 1;
-    const char* e = getenv("BAM_FRONTIER_SORT");
-    const bool sort_queue = !e || atoi(e) != 0;
-    int vertex_bits = 1;
-    while (vertex_bits < 32 && (1ull << vertex_bits) < n_vertices) vertex_bits++;
-    size_t sort_bytes = 0;
-    if (sort_queue) hip_err_chk(hipcub::DeviceRadixSort::SortKeys(nullptr, sort_bytes, curr, next, (int)std::min<uint64_t>(n_vertices, 0x7FFFFFFFull), 0, vertex_bits, st));
-    BufferPtr sort_tmp = createBuffer(sort_bytes ? sort_bytes : 8, 0);
-    do {
-        hip_err_chk(hipMemsetAsync(next_size, 0, sizeof(unsigned long long), st));
-        work.reset(st);
-        hipLaunchKernelGGL(k_bfs_frontier_coalesce_ptr_pc, dim3(work.blocks(active, group)), dim3(threads), 0, st, edges->a->d_array_ptr, d_labels, level,
-                           d_offsets, curr, (uint64_t)active, next, next_size, group, work.pieces, work.n_pieces, work.count + 1, sorted);
-        hip_err_chk(hipGetLastError());
-        iter++; level++;
-        hip_err_chk(hipMemcpyAsync(&active, next_size, sizeof(unsigned long long), hipMemcpyDeviceToHost, st));
-        hip_err_chk(hipStreamSynchronize(st));
-        sorted = sort_queue && active <= 0x7FFFFFFFull;
-        group = sorted ? work.group : BAM_WAVE_SIZE;
-        if (sorted && active > 1) {
-            /* the queue comes out in the order of discovery; sorted by vertex, the level reads the edge array front to back
-             * (neighbouring lists share pages, a page is not evicted between two of its lists, and the pages under the
-             * lists of a group of entries can be asked for together as in the sweep over all vertices).  The sorted queue
-             * goes into the buffer the level just walked, so the two do not change places. */
-            size_t need = sort_bytes;
-            hip_err_chk(hipcub::DeviceRadixSort::SortKeys(sort_tmp.get(), need, next, curr, (int)active, 0, vertex_bits, st));
-        } else
-            std::swap(curr, next);
-    } while (active);
-    if (iterations) *iterations = iter;
-    BAM_API_END
-}
-
-int bam_cc(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t* d_labels,
-           uint32_t coarse, uint32_t* iterations, void* stream)
-{
-    if (!edges || !d_offsets || !d_labels) return fail(EINVAL, "bam_cc: null argument");
-    if (!coarse || !n_vertices) return fail(EINVAL, "bam_cc: empty graph or coarse = 0");
-    BAM_API_BEGIN
-    hipStream_t st = (hipStream_t)stream;
-    BufferPtr visit_a = createBuffer(n_vertices, 0), visit_b = createBuffer(n_vertices, 0), changed_buf = createBuffer(sizeof(uint64_t), 0);
-    bool* curr = (bool*)visit_a.get();
-    bool* next = (bool*)visit_b.get();
-    bool* changed_d = (bool*)changed_buf.get();
-    hipLaunchKernelGGL(k_iota, dim3(blocks_for(n_vertices, 256)), dim3(256), 0, st, (unsigned long long*)d_labels, n_vertices);
-    hip_err_chk(hipMemsetAsync(curr, 0x01, n_vertices, st));
-    hip_err_chk(hipMemsetAsync(next, 0x00, n_vertices, st));
-    const uint32_t threads = 128;
-    sweep_work work(edges->a->adt.n_elems, n_vertices, coarse, d_offsets, st);
-    uint32_t iter = 0;
-    bool changed_h;
-    do {
-        changed_h = false;
-        hip_err_chk(hipMemcpyAsync(changed_d, &changed_h, sizeof(bool), hipMemcpyHostToDevice, st));
-        work.reset(st);
-        hipLaunchKernelGGL(k_cc_coalesce_coarse_ptr_pc, dim3(work.blocks(n_vertices, work.group)), dim3(threads), 0, st, edges->a->d_array_ptr, curr, next,
-                           n_vertices, d_offsets, (unsigned long long*)d_labels, changed_d, work.group, work.pieces, work.n_pieces, work.count + 1, iter);
-        hip_err_chk(hipGetLastError());
-        hip_err_chk(hipMemsetAsync(curr, 0x00, n_vertices, st));
-        bool* t = curr; curr = next; next = t;
-        iter++;
-        hip_err_chk(hipMemcpyAsync(&changed_h, changed_d, sizeof(bool), hipMemcpyDeviceToHost, st));
-        hip_err_chk(hipStreamSynchronize(st));
-    } while (changed_h);
-    if (iterations) *iterations = iter;
-    BAM_API_END
-}
-
-namespace {
-/* launch shape of the by-page graph kernels: pages per wave trip and number of waves, so that what the waves hold
- * at any time stays under half of the cache */
-struct by_page_plan { uint64_t n_edges, n_pages; uint32_t epp, ppw, blocks; BufferPtr first; };
-
-int plan_by_page(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, hipStream_t st, by_page_plan& pl)
-{
-    array_t<uint64_t>* a = edges->a;
-    if (a->adt.n_ranges != 1) return fail(EINVAL, "by-page graph kernels take an array of one range");
-    const range_d_t<uint64_t>& r = a->h_ranges[0];
-    if (r.index_start != 0 || r.page_start_offset % r.cache.page_size) return fail(EINVAL, "by-page graph kernels need a range that starts on a page boundary");
-    pl.n_edges = a->adt.n_elems;
-    pl.epp = (uint32_t)(r.cache.page_size / 8);
-    pl.n_pages = (pl.n_edges + pl.epp - 1) / pl.epp;
-    const uint64_t budget = r.cache.n_pages / 2;               /* pages all waves together may hold */
-    if (!budget) return fail(EINVAL, "by-page graph kernels need a cache of at least two pages");
-    int dev = 0, cus = 0;
-    hip_err_chk(hipGetDevice(&dev));
-    hip_err_chk(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-    const uint64_t max_waves = (uint64_t)cus * 8;              /* eight waves per compute unit */
-    uint64_t ppw = budget / max_waves;
-    if (ppw > BAM_WAVE_SIZE) ppw = BAM_WAVE_SIZE;
-    if (ppw < 1) ppw = 1;
-    uint64_t waves = budget / ppw;
-    if (waves > max_waves) waves = max_waves;
-    const uint64_t trips = (pl.n_pages + ppw - 1) / ppw;
-    if (waves > trips) waves = trips;
-    pl.ppw = (uint32_t)ppw;
-    pl.blocks = (uint32_t)waves;                               /* one wave per workgroup */
-    pl.first = createBuffer((pl.n_pages + 1) * sizeof(uint64_t), dev);
-    hipLaunchKernelGGL(k_page_first_vertex, dim3(blocks_for(pl.n_pages + 1, 256)), dim3(256), 0, st, d_offsets, n_vertices, (uint64_t)pl.epp, pl.n_pages,
-                       (uint64_t*)pl.first.get());
-    hip_err_chk(hipGetLastError());
-    return 0;
-}
-} // namespace
-
-int bam_bfs_by_page(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t src, uint32_t* d_labels,
-                    uint32_t* iterations, void* stream)
-{
-    if (!edges || !d_offsets || !d_labels) return fail(EINVAL, "bam_bfs_by_page: null argument");
-    if (src >= n_vertices) return fail(EINVAL, "bam_bfs_by_page: source out of range");
-    BAM_API_BEGIN
-    hipStream_t st = (hipStream_t)stream;
-    by_page_plan pl;
-    if (int rc = plan_by_page(edges, d_offsets, n_vertices, st, pl)) return rc;
-    BufferPtr changed_buf = createBuffer(sizeof(uint64_t), 0);
-    uint64_t* changed_d = (uint64_t*)changed_buf.get();
-    const uint32_t zero = 0;
-    hip_err_chk(hipMemsetAsync(d_labels, 0xFF, n_vertices * sizeof(uint32_t), st));
-    hip_err_chk(hipMemcpyAsync(d_labels + src, &zero, sizeof(uint32_t), hipMemcpyHostToDevice, st));
-    uint32_t level = 0, iter = 0;
-    uint64_t changed_h;
-    do {
-        changed_h = 0;
-        hip_err_chk(hipMemcpyAsync(changed_d, &changed_h, sizeof(uint64_t), hipMemcpyHostToDevice, st));
-        if (pl.n_pages)
-            hipLaunchKernelGGL(k_bfs_by_page, dim3(pl.blocks), dim3(BAM_WAVE_SIZE), 0, st, edges->a->d_array_ptr, d_labels, level, d_offsets,
-                               (const uint64_t*)pl.first.get(), pl.n_edges, pl.ppw, changed_d);
-        hip_err_chk(hipGetLastError());
-        iter++; level++;
-        hip_err_chk(hipMemcpyAsync(&changed_h, changed_d, sizeof(uint64_t), hipMemcpyDeviceToHost, st));
-        hip_err_chk(hipStreamSynchronize(st));
-    } while (changed_h);
-    if (iterations) *iterations = iter;
-    BAM_API_END
-}
-
-int bam_cc_by_page(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t* d_labels, uint32_t* iterations, void* stream)
-{
-    if (!edges || !d_offsets || !d_labels) return fail(EINVAL, "bam_cc_by_page: null argument");
-    if (!n_vertices) return fail(EINVAL, "bam_cc_by_page: empty graph");
-    BAM_API_BEGIN
-    hipStream_t st = (hipStream_t)stream;
-    by_page_plan pl;
-    if (int rc = plan_by_page(edges, d_offsets, n_vertices, st, pl)) return rc;
-    BufferPtr visit_a = createBuffer(n_vertices, 0), visit_b = createBuffer(n_vertices, 0), changed_buf = createBuffer(sizeof(uint64_t), 0);
-    bool* curr = (bool*)visit_a.get();
-    bool* next = (bool*)visit_b.get();
-    bool* changed_d = (bool*)changed_buf.get();
-    hipLaunchKernelGGL(k_iota, dim3(blocks_for(n_vertices, 256)), dim3(256), 0, st, (unsigned long long*)d_labels, n_vertices);
-    hip_err_chk(hipMemsetAsync(curr, 0x01, n_vertices, st));
-    hip_err_chk(hipMemsetAsync(next, 0x00, n_vertices, st));
-    uint32_t iter = 0;
-    bool changed_h;
-    do {
-        changed_h = false;
-        hip_err_chk(hipMemcpyAsync(changed_d, &changed_h, sizeof(bool), hipMemcpyHostToDevice, st));
-        if (pl.n_pages)
-            hipLaunchKernelGGL(k_cc_by_page, dim3(pl.blocks), dim3(BAM_WAVE_SIZE), 0, st, edges->a->d_array_ptr, curr, next, d_offsets,
-                               (const uint64_t*)pl.first.get(), pl.n_edges, pl.ppw, iter, (unsigned long long*)d_labels, changed_d);
-        hip_err_chk(hipGetLastError());
-        hip_err_chk(hipMemsetAsync(curr, 0x00, n_vertices, st));
-        bool* t = curr; curr = next; next = t;
-        iter++;
-        hip_err_chk(hipMemcpyAsync(&changed_h, changed_d, sizeof(bool), hipMemcpyDeviceToHost, st));
-        hip_err_chk(hipStreamSynchronize(st));
-    } while (changed_h);
-    if (iterations) *iterations = iter;
-    BAM_API_END
-}
-
-int bam_vectoradd(bam_array_t* a, bam_array_t* b, bam_array_t* c, uint64_t n_elems, void* stream)
-{
-    if (!a || !b || !c) return fail(EINVAL, "bam_vectoradd: null argument");
-    if (n_elems > a->a->adt.n_elems || n_elems > b->a->adt.n_elems || n_elems > c->a->adt.n_elems) return fail(EINVAL, "bam_vectoradd: more elements than the arrays hold");
-    if (!n_elems) return 0;
-    BAM_API_BEGIN
-    hipLaunchKernelGGL(k_vectoradd_ptr_pc, dim3(blocks_for(n_elems, 64)), dim3(64), 0, (hipStream_t)stream,
-                       a->a->d_array_ptr, b->a->d_array_ptr, n_elems, c->a->d_array_ptr);
-    hip_err_chk(hipGetLastError());
-    BAM_API_END
-}
-
-int bam_reduce(bam_array_t* a, uint64_t n_elems, uint32_t block_size, uint64_t* d_partials, void* stream)
-{
-    if (!a || !d_partials) return fail(EINVAL, "bam_reduce: null argument");
-    if (!block_size || block_size % BAM_WAVE_SIZE || block_size > 1024) return fail(EINVAL, "bam_reduce: block size must be a multiple of 64, at most 1024");
-    if (n_elems > a->a->adt.n_elems) return fail(EINVAL, "bam_reduce: more elements than the array holds");
-    if (!n_elems) return 0;
-    BAM_API_BEGIN
-    hipLaunchKernelGGL(k_reduce_ptr_pc, dim3(blocks_for(n_elems, 2ull * block_size)), dim3(block_size), 0, (hipStream_t)stream,
-                       a->a->d_array_ptr, (unsigned long long*)d_partials, n_elems);
-    hip_err_chk(hipGetLastError());
-    BAM_API_END
-}
-
-int bam_scan(bam_array_t* a, uint64_t n_elems, uint32_t block_size, uint64_t* d_result, void* stream)
-{
-    if (!a || !d_result) return fail(EINVAL, "bam_scan: null argument");
-    if (!block_size || block_size % BAM_WAVE_SIZE || block_size > 1024) return fail(EINVAL, "bam_scan: block size must be a multiple of 64, at most 1024");
-    if (n_elems > a->a->adt.n_elems) return fail(EINVAL, "bam_scan: more elements than the array holds");
-    BAM_API_BEGIN
-    hipStream_t st = (hipStream_t)stream;
-    hip_err_chk(hipMemsetAsync(d_result, 0, sizeof(uint64_t), st));
-    if (n_elems) {
-        const uint64_t n_blocks = blocks_for(n_elems, 2ull * block_size);
-        BufferPtr totals = createBuffer(n_blocks * sizeof(uint64_t), 0);
-        unsigned long long* out = (unsigned long long*)d_result + 1;
-        const size_t lds = (2 * block_size + 1024 / BAM_WAVE_SIZE) * sizeof(uint64_t);
-        hipLaunchKernelGGL(k_scan_ptr_pc, dim3(n_blocks), dim3(block_size), lds, st, a->a->d_array_ptr, out, (unsigned long long*)totals.get(), n_elems);
-        hipLaunchKernelGGL(k_scan_block_totals, dim3(1), dim3(1024), 0, st, (unsigned long long*)totals.get(), n_blocks);
-        hipLaunchKernelGGL(k_scan_finalsum, dim3(n_blocks), dim3(block_size), 0, st, (const unsigned long long*)totals.get(), out, n_elems);
-        hip_err_chk(hipGetLastError());
-        hip_err_chk(hipStreamSynchronize(st));         /* `totals` is released on return */
-    }
-    BAM_API_END
-}
-
-} // extern "C"
-
-/*
- * bam_scan for callers that cannot allocate (code under stream capture, serving loops, harnesses that forbid it): the block
- * totals, which bam_scan keeps in a buffer it allocates and frees per call, live in a file-scope device array of fixed size.
- * Every device the library runs on holds its own copy of the array at its own address until the process ends; the address is
- * looked up once per device (the array's name means nothing to the host) and handed to the kernels like any other buffer.
- */
-/* BAM_SCAN_NOALLOC_MAX_BLOCKS (bam_amd.h): 65536 block totals, 512 KiB */
-#define BAM_SCAN_NOALLOC_MAX_DEVICES 64
-static __device__ __align__(256) unsigned long long scratch[BAM_SCAN_NOALLOC_MAX_BLOCKS];
-
-namespace {
-std::mutex g_scratch_mu;
-unsigned long long* g_scratch_ptr[BAM_SCAN_NOALLOC_MAX_DEVICES];      /* per device: where its copy of `scratch` lives */
-
-/* the current device's copy of the array; NULL (and the error recorded) if it cannot be found */
-unsigned long long* scan_scratch_of_current_device()
-{
-    int dev = -1;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= BAM_SCAN_NOALLOC_MAX_DEVICES) { g_err = "bam_scan_noalloc: no current device"; return nullptr; }
-    std::lock_guard<std::mutex> g(g_scratch_mu);
-    if (!g_scratch_ptr[dev]) {
-        void* p = nullptr;
-        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
-        if (e != hipSuccess || !p) { g_err = std::string("bam_scan_noalloc: hipGetSymbolAddress: ") + hipGetErrorString(e); return nullptr; }
-        g_scratch_ptr[dev] = (unsigned long long*)p;
-    }
-    return g_scratch_ptr[dev];
-}
-
-__global__ void k_store_zero64(unsigned long long* p) { *p = 0; }
-} // namespace
-
-extern "C" {
-
-int bam_scan_noalloc(bam_array_t* a, uint64_t n_elems, uint32_t block_size, uint64_t* d_result, void* stream)
-{
-    if (!a || !d_result) return fail(EINVAL, "bam_scan_noalloc: null argument");
-    if (!block_size || block_size % BAM_WAVE_SIZE || block_size > 1024) return fail(EINVAL, "bam_scan_noalloc: block size must be a multiple of 64, at most 1024");
-    if (n_elems > a->a->adt.n_elems) return fail(EINVAL, "bam_scan_noalloc: more elements than the array holds");
-    const uint64_t n_blocks = (n_elems + 2ull * block_size - 1) / (2ull * block_size);
-    if (n_blocks > BAM_SCAN_NOALLOC_MAX_BLOCKS)
-        return fail(E2BIG, "bam_scan_noalloc: " + std::to_string(n_elems) + " elements in blocks of " + std::to_string(2ull * block_size) + " need " + std::to_string(n_blocks) +
-                           " block totals, the fixed scratch array holds " + std::to_string(BAM_SCAN_NOALLOC_MAX_BLOCKS) + " (use bam_scan, or a larger block size)");
-    unsigned long long* totals = scan_scratch_of_current_device();
-    if (!totals) return EIO;
-    hipStream_t st = (hipStream_t)stream;
-    unsigned long long* out = (unsigned long long*)d_result + 1;
-    /* no memset node: a fill kernel clears the first word (a caller may be capturing this stream) */
-    hipLaunchKernelGGL(k_store_zero64, dim3(1), dim3(1), 0, st, (unsigned long long*)d_result);
-    if (n_elems) {
-        /* totals[0 .. n_blocks) are written by the first kernel before the second reads them; what an earlier, longer call
-         * left behind them is never read, so nothing has to be cleared */
-        const size_t lds = (2 * block_size + 1024 / BAM_WAVE_SIZE) * sizeof(uint64_t);
-        hipLaunchKernelGGL(k_scan_ptr_pc, dim3((uint32_t)n_blocks), dim3(block_size), lds, st, a->a->d_array_ptr, out, totals, n_elems);
-        hipLaunchKernelGGL(k_scan_block_totals, dim3(1), dim3(1024), 0, st, totals, n_blocks);
-        hipLaunchKernelGGL(k_scan_finalsum, dim3((uint32_t)n_blocks), dim3(block_size), 0, st, (const unsigned long long*)totals, out, n_elems);
-    }
-    const hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return fail(EIO, std::string("bam_scan_noalloc: ") + hipGetErrorString(e));
-    return 0;
-}
-
-int bam_pagerank(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, float alpha, float tolerance, uint32_t max_iterations,
-                 int by_page, float* d_value, uint32_t* iterations, void* stream)
-{
-    if (!edges || !d_offsets || !d_value) return fail(EINVAL, "bam_pagerank: null argument");
-    if (iterations) *iterations = 0;
-    if (!n_vertices) return 0;
-    BAM_API_BEGIN
-    hipStream_t st = (hipStream_t)stream;
-    BufferPtr delta = createBuffer(n_vertices * sizeof(float), 0), residual = createBuffer(n_vertices * sizeof(float), 0),
-              label = createBuffer(n_vertices, 0), changed_buf = createBuffer(sizeof(uint64_t), 0);
-    float* delta_d = (float*)delta.get();
-    float* residual_d = (float*)residual.get();
-    bool* label_d = (bool*)label.get();
-    bool* changed_d = (bool*)changed_buf.get();
-    by_page_plan pl{};
-    if (by_page)
-        if (int rc = plan_by_page(edges, d_offsets, n_vertices, st, pl)) return rc;
-    const uint32_t upd_blocks = blocks_for(n_vertices, 256);
-    sweep_work work(edges->a->adt.n_elems, n_vertices, 1, d_offsets, st);
-    hipLaunchKernelGGL(k_pr_initialize, dim3(upd_blocks), dim3(256), 0, st, label_d, delta_d, residual_d, d_value, n_vertices, d_offsets, alpha);
-    uint32_t iter = 0;
-    bool changed_h;
-    do {
-        changed_h = false;
-        hip_err_chk(hipMemcpyAsync(changed_d, &changed_h, sizeof(bool), hipMemcpyHostToDevice, st));
-        if (by_page) {
-            if (pl.n_pages)
-                hipLaunchKernelGGL(k_pr_by_page, dim3(pl.blocks), dim3(BAM_WAVE_SIZE), 0, st, edges->a->d_array_ptr, label_d, delta_d, residual_d, d_offsets,
-                                   (const uint64_t*)pl.first.get(), pl.n_edges, pl.ppw, iter);
-            hip_err_chk(hipMemsetAsync(label_d, 0, n_vertices, st));
-        } else {
-            work.reset(st);
-            hipLaunchKernelGGL(k_pr_coalesce_pc, dim3(work.blocks(n_vertices, work.group)), dim3(128), 0, st, edges->a->d_array_ptr, label_d, delta_d, residual_d,
-                               n_vertices, d_offsets, work.group, work.pieces, work.n_pieces, work.count + 1, iter);
-            hip_err_chk(hipMemsetAsync(label_d, 0, n_vertices, st));
-        }
-        iter++;
-        hipLaunchKernelGGL(k_pr_update, dim3(upd_blocks), dim3(256), 0, st, label_d, delta_d, residual_d, d_value, n_vertices, d_offsets, tolerance, alpha, changed_d);
-        hip_err_chk(hipGetLastError());
-        hip_err_chk(hipMemcpyAsync(&changed_h, changed_d, sizeof(bool), hipMemcpyDeviceToHost, st));
-        hip_err_chk(hipStreamSynchronize(st));
-    } while (changed_h && iter < max_iterations);
-    if (iterations) *iterations = iter;
-    BAM_API_END
-}
-
 // ---- arrays of 32-bit elements and SSSP ----
 int bam_range32_create(bam_range32_t** out, uint64_t index_start, uint64_t count, uint64_t page_start, uint64_t page_count,
                        uint64_t page_start_offset, uint64_t page_size, bam_page_cache_t* pc, uint32_t device, int dist)
@@ -2293,70 +1037,6 @@ int bam_array32_read(bam_array32_t* a, uint64_t n_reqs, const uint64_t* d_assign
                        a->a->d_array_ptr, n_reqs, d_assignment, stride, (unsigned long long*)a->partials.get());
     hipLaunchKernelGGL(k_fold_partials, dim3(1), dim3(1024), 0, (hipStream_t)stream, (unsigned long long*)a->partials.get(), (unsigned long long*)d_sum);
     hip_err_chk(hipGetLastError());
-    BAM_API_END
-}
-
-namespace {
-/* the loop of benchmarks/sssp/main.cu:663-725 (and of sssp_float, :624-700): relax from the flagged vertices, adopt what got
- * cheaper, flag it, until nothing does.  FLOAT: costs and weights are single-precision values, unreached = 1e9 (sssp_float :529) */
-void sssp_run(const bool FLOAT, bam_array_t* edges, bam_array32_t* weights, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t src, uint32_t* d_costs,
-              uint32_t* iterations, hipStream_t st)
-{
-    BufferPtr new_cost = createBuffer(n_vertices * sizeof(uint32_t), 0), label = createBuffer(n_vertices, 0), changed_buf = createBuffer(sizeof(uint64_t), 0);
-    uint32_t* new_d = (uint32_t*)new_cost.get();
-    bool* label_d = (bool*)label.get();
-    bool* changed_d = (bool*)changed_buf.get();
-    const uint32_t zero = 0;                    /* the pattern of 0.0f as well */
-    const bool one = true;
-    const float far = 1000000000.0f;
-    uint32_t unreached = 0xFFFFFFFFu;
-    if (FLOAT) memcpy(&unreached, &far, sizeof(unreached));
-    hip_err_chk(hipMemsetD32Async((hipDeviceptr_t)d_costs, (int)unreached, n_vertices, st));
-    hip_err_chk(hipMemsetD32Async((hipDeviceptr_t)new_d, (int)unreached, n_vertices, st));
-    hip_err_chk(hipMemsetAsync(label_d, 0, n_vertices, st));
-    hip_err_chk(hipMemcpyAsync(label_d + src, &one, sizeof(bool), hipMemcpyHostToDevice, st));
-    hip_err_chk(hipMemcpyAsync(d_costs + src, &zero, sizeof(uint32_t), hipMemcpyHostToDevice, st));
-    hip_err_chk(hipMemcpyAsync(new_d + src, &zero, sizeof(uint32_t), hipMemcpyHostToDevice, st));
-    const uint32_t threads = 128;
-    sweep_work work(edges->a->adt.n_elems, n_vertices, 1, d_offsets, st);
-    uint32_t iter = 0;
-    bool changed_h;
-    do {
-        changed_h = false;
-        hip_err_chk(hipMemcpyAsync(changed_d, &changed_h, sizeof(bool), hipMemcpyHostToDevice, st));
-        work.reset(st);
-        hipLaunchKernelGGL(FLOAT ? k_sssp_coalesce_pc<true> : k_sssp_coalesce_pc<false>, dim3(work.blocks(n_vertices, work.group)), dim3(threads), 0, st,
-                           edges->a->d_array_ptr, weights->a->d_array_ptr, label_d, new_d, n_vertices, d_offsets, work.group, work.pieces, work.n_pieces, work.count + 1, iter);
-        hip_err_chk(hipMemsetAsync(label_d, 0, n_vertices, st));
-        hipLaunchKernelGGL(k_sssp_update, dim3(blocks_for(n_vertices, 256)), dim3(256), 0, st, label_d, d_costs, new_d, n_vertices, changed_d);
-        hip_err_chk(hipGetLastError());
-        iter++;
-        hip_err_chk(hipMemcpyAsync(&changed_h, changed_d, sizeof(bool), hipMemcpyDeviceToHost, st));
-        hip_err_chk(hipStreamSynchronize(st));
-    } while (changed_h);
-    if (iterations) *iterations = iter;
-}
-} // namespace
-
-int bam_sssp(bam_array_t* edges, bam_array32_t* weights, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t src, uint32_t* d_costs,
-             uint32_t* iterations, void* stream)
-{
-    if (!edges || !weights || !d_offsets || !d_costs) return fail(EINVAL, "bam_sssp: null argument");
-    if (src >= n_vertices) return fail(EINVAL, "bam_sssp: source out of range");
-    if (edges->a->adt.n_elems != weights->a->adt.n_elems) return fail(EINVAL, "bam_sssp: one weight per edge");
-    BAM_API_BEGIN
-    sssp_run(false, edges, weights, d_offsets, n_vertices, src, d_costs, iterations, (hipStream_t)stream);
-    BAM_API_END
-}
-
-int bam_sssp_float(bam_array_t* edges, bam_array32_t* weights, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t src, float* d_costs,
-                   uint32_t* iterations, void* stream)
-{
-    if (!edges || !weights || !d_offsets || !d_costs) return fail(EINVAL, "bam_sssp_float: null argument");
-    if (src >= n_vertices) return fail(EINVAL, "bam_sssp_float: source out of range");
-    if (edges->a->adt.n_elems != weights->a->adt.n_elems) return fail(EINVAL, "bam_sssp_float: one weight per edge");
-    BAM_API_BEGIN
-    sssp_run(true, edges, weights, d_offsets, n_vertices, src, (uint32_t*)d_costs, iterations, (hipStream_t)stream);
     BAM_API_END
 }
 

@@ -1,0 +1,146 @@
+// Shared by the translation units of the C-ABI library (bam_capi.hip, bam_graph.hip, bam_apps.hip): error plumbing, the
+// handle types behind the opaque pointers of include/bam_amd.h, and the device helpers the kernels of every unit use.
+#ifndef __BAM_CAPI_INTERNAL_H__
+#define __BAM_CAPI_INTERNAL_H__
+#include "bam_amd.h"
+
+#include <hip/hip_runtime.h>
+#include <fcntl.h>
+#include <sys/mman.h>
+#include <sys/stat.h>
+#include <unistd.h>
+#include <algorithm>
+#include <cerrno>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <thread>
+#include <vector>
+
+#include "ctrl.h"
+#include "event.h"
+#include "nvmt.h"
+#include "page_cache.h"
+#include "bafs_ptr.h"
+
+// ---------------------------------------------------------------------------
+// error plumbing
+// ---------------------------------------------------------------------------
+std::string& bam_err();            /* message of the last failure on the calling thread (defined in bam_capi.hip) */
+#define g_err bam_err()
+
+#define BAM_API_BEGIN try {
+#define BAM_API_END                                                        \
+    return 0;                                                              \
+    } catch (const std::exception& e) { g_err = e.what(); return EIO; }    \
+      catch (...) { g_err = "unknown error"; return EIO; }
+
+static inline int fail(int code, const char* msg) { g_err = msg; return code; }
+static inline int fail(int code, const std::string& msg) { g_err = msg; return code; }
+
+struct bam_target {
+    nvmt_t* t = nullptr;
+    void* bar = nullptr;
+    void* backing = nullptr;
+    size_t backing_bytes = 0;
+    nvmt_config_t cfg{};
+};
+struct bam_ctrl { Controller* c; };
+struct bam_page_cache { page_cache_t* pc; Controller* ctrl; };      /* ctrl: the first controller of the cache */
+struct bam_range { range_t<uint64_t>* r; };
+#define BAM_SUM_PARTIALS 4096
+struct bam_array { array_t<uint64_t>* a; BufferPtr partials; };
+struct bam_range32 { range_t<uint32_t>* r; };
+struct bam_array32 { array_t<uint32_t>* a; BufferPtr partials; };      /* partials: [BAM_SUM_PARTIALS] checksum shards, zero between launches */
+
+// ---------------------------------------------------------------------------
+// device helpers
+// ---------------------------------------------------------------------------
+namespace {
+
+__device__ __forceinline__ uint64_t mix64(uint64_t z)
+{
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+__device__ __forceinline__ uint64_t splitmix64(uint64_t seed, uint64_t i) { return mix64(seed + (i + 1) * 0x9E3779B97F4A7C15ull); }
+
+/* sum over the 64 lanes of a wave (all lanes active); result valid in every lane */
+__device__ __forceinline__ uint64_t wave_sum(uint64_t v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += bam::shfl(v, bam::lane() ^ o);
+    return v;
+}
+
+/*
+ * Add the wave's values into the launch's checksum.  A single word would take one atomic per wave of the
+ * whole grid, all serialised on one address (about 12 ns each: a million waves cost more than the reads they
+ * sum), so the sum is kept in BAM_SUM_PARTIALS shards picked by workgroup and folded by k_fold_partials.
+ */
+__device__ __forceinline__ void block_accumulate(unsigned long long* partials, uint64_t v)
+{
+    v = wave_sum(v);
+    if (bam::lane() == 0 && v) atomicAdd(&partials[(blockIdx.x * 0x9E3779B1u) >> 20], (unsigned long long)v);
+}
+
+/* a page that is not resident as far as one look at its state tells: what the read-ahead asks for (a page that is resident is
+ * left alone, which spares its state word two atomics per touch; if it goes before it is read, it is read on demand) */
+template <typename T>
+__device__ __forceinline__ bool page_absent(const bam::range_view<T>& view, const uint64_t page)
+{
+    return (bam::ld_relaxed(&view.pages[page].state) & VALID) == 0;
+}
+
+/*
+ * Read-ahead for kernels in which consecutive threads read consecutive elements (one element or two per thread, as in
+ * benchmarks/vectoradd, reduction and scan).  Left to themselves such kernels ask the store for one page per wave
+ * and trip, and the store path takes about a million such batches per second whatever their size: 1 GiB comes in
+ * at 5 GB/s.  Here the wave that reads the first element of a window of W pages (W = a 64th of the cache, at most
+ * 64) touches the W pages that lie up to 32 windows further on, one page per lane, taken and dropped again: they come
+ * in as one batch of W commands, before the waves that read them are started (workgroups start in order, and the
+ * device holds a few thousand waves, that is up to a thousand pages, at a time).  The first windows are touched by
+ * their own first waves.  `first` is the index of the wave's first element (wave-uniform), `wave_span` the elements
+ * from one wave's first to the next one's (more than 64 where the threads read with a stride).
+ */
+template <typename T>
+__device__ __forceinline__ void touch_ahead(array_d_t<T>* da, const uint64_t first, const uint64_t n_read, const uint64_t wave_span = BAM_WAVE_SIZE,
+                                            const uint32_t which = 0)
+{
+    if (da->n_ranges != 1) return;
+    const uint64_t n_elems = n_read < da->n_elems ? n_read : da->n_elems;         /* nothing is touched that the array does not hold */
+    const page_cache_d_t& cache = da->d_ranges[0].cache;
+    const uint64_t w_pages = cache.n_pages >> 6 > BAM_WAVE_SIZE ? BAM_WAVE_SIZE : cache.n_pages >> 6;
+    if (w_pages < 2) return;
+    const uint64_t epp = cache.page_size / sizeof(T), w_elems = w_pages * epp;
+    /* the wave that does it is the `which`-th of those that begin in the window (`wave_span` elements per wave): a kernel
+     * that walks several arrays gives each array's windows to a different wave, and their batches are in flight together */
+    if ((first % w_elems) / wave_span != which) return;
+    /* how far ahead: beyond what the waves in flight cover (a few thousand waves at one page per four to eight waves), within an
+     * eighth of the cache (a kernel may walk several arrays behind one cache at a time) */
+    uint64_t dist = (cache.n_pages / 8) / w_pages;
+    dist = (dist > 32 ? 32 : dist < 1 ? 1 : dist) * w_elems;
+    bam::range_view<T> view;
+    view.load(da->d_ranges);
+    auto touch = [](uint32_t) { return true; };
+    const uint64_t mine = first - first % w_elems + bam::lane() * epp;
+    if (first < dist) {
+        const uint64_t page = view.page_of(mine < n_elems ? mine : first);
+        const bool take = bam::lane() < w_pages && mine < n_elems && page_absent(view, page);
+        if (bam::ballot(take)) view.acquire_helped(page, take, false, touch, touch);
+    }
+    const uint64_t ahead = mine + dist;
+    if (first + dist < n_elems) {
+        const uint64_t page = view.page_of(ahead < n_elems ? ahead : first);
+        const bool take = bam::lane() < w_pages && ahead < n_elems && page_absent(view, page);
+        if (bam::ballot(take)) view.acquire_helped(page, take, false, touch, touch);
+    }
+    view.n_access = view.n_hit = 0;
+}
+
+inline uint32_t blocks_for(uint64_t n, uint32_t bs) { return (uint32_t)((n + bs - 1) / bs); }
+
+} // namespace
+#endif /* __BAM_CAPI_INTERNAL_H__ */

@@ -209,6 +209,8 @@ uint16_t do_rw(nvmt* t, Stats& st_, const nvm_cmd_t& c, bool write)
     if (c.dword[1] != 1) return ST_INVALID_FIELD;
     if (write && !t->cfg.backing) return ST_WRITE_RO;
     uint64_t done = 0;
+    static const bool no_payload = getenv("NVMT_EXPERIMENT_NO_PAYLOAD") != nullptr;
+    if (no_payload && !write) { st_.bump(st_.read_cmds); st_.bump(st_.bytes_read, bytes); return ST_OK; }
     alignas(64) uint64_t tmp[512];      /* sizeof(tmp) is the generation chunk */
     bool ok = for_each_prp(t, c, bytes, [&](uint64_t addr, uint64_t len) {
         uint8_t* p = (uint8_t*)addr;
@@ -279,28 +281,37 @@ void serve_sq(nvmt* t, IoThread* me, Sq& sq)
 {
     Cq& cq = t->cqs[sq.cqid];
     const uint32_t mask = sq.qs - 1;
-    uint32_t tail = ld<uint32_t>(sq.tail_db) & mask;
     Stats& st_ = me->stats;
-    if (tail != sq.last_tail) { st_.bump(st_.sq_doorbells); sq.last_tail = tail; }
-    while (((tail - sq.head) & mask) != 0) {
+    // A sealed queue is read by its seals: the entry at the head is looked at whether a doorbell has announced it or
+    // not (the line stays in this core's cache until the submitter writes it, so a look at an idle queue costs next to
+    // nothing), and entries are taken for as long as sequence number and checksum match.  Doorbells and entries are
+    // not ordered on their way here, and neither are two doorbells: the last doorbell of a burst may be an old one,
+    // and a queue read by its doorbell would then sit on entries nobody announces again.  The doorbell register is
+    // still read for the counters.  An unsealed queue is read by its doorbell, as the NVMe specification has it.
+    uint32_t tail = sq.sealed ? sq.last_tail : ld<uint32_t>(sq.tail_db) & mask;
+    if (!sq.sealed && tail != sq.last_tail) { st_.bump(st_.sq_doorbells); sq.last_tail = tail; }
+    for (;;) {
         nvm_cmd_t batch[64];
-        uint32_t n = (tail - sq.head) & mask;
-        if (n > 64) n = 64;
+        uint32_t n;
         if (sq.sealed) {
-            // take entries only while sequence number and checksum match: one that is stale, torn or still in
-            // flight (entry and doorbell are not ordered on the way here) is looked at again on a later pass
             uint32_t got = 0;
-            for (; got < n; got++) {
+            for (; got < 64; got++) {
                 batch[got] = sq.mem[(sq.head + got) & mask];
                 std::atomic_thread_fence(std::memory_order_acquire);
                 if (!nvm_cmd_seal_ok(&batch[got], sq.fetched + got)) break;
             }
-            if (got < n && !sq.retry_counted) {
-                st_.bump(st_.sqe_retries); sq.retry_counted = true;
-                if (getenv("NVMT_DEBUG_SEAL")) {
-                    const nvm_cmd_t& e = batch[got];
-                    fprintf(stderr, "[nvmt %p] sq %u slot %u: want ticket %u, entry dw0 %08x dw2 %08x dw3 %08x (seal %08x) slba %u head %u tail %u\n", (void*)t, sq.id,
-                            (sq.head + got) & mask, sq.fetched + got, e.dword[0], e.dword[2], e.dword[3], nvm_cmd_seal_value(&e, sq.fetched + got), e.dword[10], sq.head, tail);
+            if (got < 64) {
+                // an entry that a doorbell covers but that does not verify yet has been overtaken by its doorbell
+                tail = ld<uint32_t>(sq.tail_db) & mask;
+                if (tail != sq.last_tail) { st_.bump(st_.sq_doorbells); sq.last_tail = tail; }
+                const uint32_t announced = (tail - sq.head) & mask;
+                if (announced > got && announced <= sq.qs / 2 && !sq.retry_counted) {
+                    st_.bump(st_.sqe_retries); sq.retry_counted = true;
+                    if (getenv("NVMT_DEBUG_SEAL")) {
+                        const nvm_cmd_t& e = batch[got];
+                        fprintf(stderr, "[nvmt %p] sq %u slot %u: want ticket %u, entry dw0 %08x dw2 %08x dw3 %08x (seal %08x) slba %u head %u tail %u\n", (void*)t, sq.id,
+                                (sq.head + got) & mask, sq.fetched + got, e.dword[0], e.dword[2], e.dword[3], nvm_cmd_seal_value(&e, sq.fetched + got), e.dword[10], sq.head, tail);
+                    }
                 }
             }
             if (!got) return;
@@ -308,6 +319,9 @@ void serve_sq(nvmt* t, IoThread* me, Sq& sq)
             n = got;
             sq.fetched += n;
         } else {
+            n = (tail - sq.head) & mask;
+            if (!n) return;
+            if (n > 64) n = 64;
             for (uint32_t i = 0; i < n; i++) batch[i] = sq.mem[(sq.head + i) & mask];
         }
         sq.head = (sq.head + n) & mask;
@@ -657,5 +671,16 @@ void nvmt_reset_stats(nvmt_t* t)
 }
 
 void nvmt_fill_words(uint64_t seed, uint64_t first_word, uint64_t n, uint64_t* out) { gen_words(seed, first_word, n, out); }
+
+int nvmt_queue_state(nvmt_t* t, uint16_t qid, uint64_t* out8)
+{
+    if (!t || !out8 || qid == 0 || qid >= t->sqs.size()) return EINVAL;
+    const Sq& sq = t->sqs[qid];
+    if (!sq.valid) return ENOENT;
+    const Cq& cq = t->cqs[sq.cqid];
+    out8[0] = sq.head; out8[1] = sq.fetched; out8[2] = ld<uint32_t>(sq.tail_db); out8[3] = sq.sealed;
+    out8[4] = cq.tail; out8[5] = cq.head_seen; out8[6] = ld<uint32_t>(cq.head_db); out8[7] = cq.phase;
+    return 0;
+}
 
 } // extern "C"

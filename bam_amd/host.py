@@ -136,7 +136,7 @@ class PageCache:
         keys = ("batches", "commands", "t_cid", "t_submit", "t_wait", "t_copy", "t_find_slot", "find_slot_calls", "find_slot_lanes",
                 "t_sq_ticket", "t_sq_write", "t_sq_cover", "sq_cover_trips", "sq_sweeps", "sq_swept", "sq_doorbells",
                 "cq_wait_trips", "cq_drains", "cq_drained", "t_cq_drain", "cq_empty_looks", "t_cq_notice",
-                "n_ld_dev", "t_ld_dev", "n_sqe_store", "t_sqe_store", "t_doorbell", "n_ld_cqe", "t_ld_cqe")
+                "n_ld_dev", "t_ld_dev", "n_sqe_store", "t_sqe_store", "t_doorbell", "n_ld_cqe", "t_ld_cqe", "t_pull", "n_pull")
         return dict(zip(keys, list(out)))
 
     def block_io(self, n_reqs, req_bytes, lbas=None, write=False, queue_policy=1, block_size=64):

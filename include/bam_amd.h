@@ -53,6 +53,15 @@ int bam_ctrl_create(bam_ctrl_t** out, const char* path, uint32_t ns_id, uint32_t
 void bam_ctrl_destroy(bam_ctrl_t* c);
 /* out[6]: n_qps, queue depth, block size, namespace blocks, #SSDAccesses since last reset, error completions */
 int bam_ctrl_info(bam_ctrl_t* c, uint64_t* out, int reset);
+/* Where queue pair `qp` (0-based) stands, for diagnosis after a run that was given up; call with the device idle.
+ * out16[0..7]: queue depth, slot tickets handed out, SQ tail, SQ tail lock held, how far the controller has read the SQ
+ * (from completions), CQ head, CQ head lock held, error completions; [8..15] reserved.  slots (may be NULL): for each of
+ * the first n_slots slots three words: its free/lap counter, its written-for-lap mark, its command word (1 in flight,
+ * 3 completed, 7 completed with an error status). */
+int bam_ctrl_queue_state(bam_ctrl_t* c, uint32_t qp, uint64_t* out16, uint32_t* slots, uint32_t n_slots);
+/* the software target's side of I/O queue `qid` (1-based, as created): out8 = SQ head, commands fetched, SQ tail doorbell,
+ * sealed, CQ tail, CQ head as last seen, CQ head doorbell, CQ phase */
+int bam_target_queue_state(bam_target_t* t, uint32_t qid, uint64_t* out8);
 /* 1 if a device-side wait gave up (lost completion / spin limit); clear = reset the flag */
 int bam_ctrl_aborted(bam_ctrl_t* c, int clear);
 

@@ -5,21 +5,30 @@
  * reference (get_cid :35-52, put_cid :54-57, move_tail :59-80, move_head_cq
  * :82-123, sq_enqueue :167-330, cq_poll :378-422, cq_dequeue :424-535), and
  * the same wire behaviour towards the controller: ticketed SQ slots, one tail
- * doorbell per contiguous run of written entries, SQ slots recycled from the
- * SQHD field of completions, one CQ-head doorbell per run of consumed entries.
+ * doorbell per contiguous run of written entries, one CQ-head doorbell per run
+ * of consumed entries.
  *
  * The execution model is different.  A gfx950 wave runs its 64 lanes in lock
  * step, so a lane must never spin on something a masked-off sibling produces.
  * Every operation here is therefore done by the whole group of active lanes
- * that target the same queue:
- *   - one in_ticket fetch_add(n) per group reserves n consecutive SQ slots;
- *   - lanes write their own 64-byte entries and set tail_mark; the group's
- *     leader try-locks tail_lock and the group sweeps up to 64 marks per load;
- *   - completions are not searched for per thread.  Whichever group holds
- *     head_lock drains the CQ 64 entries per load and flags each completed
- *     command in the cid table (cid[c] = LOCKED|DONE); waiters poll their own
- *     word.  The drainer frees SQ slots from SQHD and rings the CQ doorbell
- *     once per sweep.
+ * that target the same queue.  And every step that has to wait for memory
+ * costs the wave a round trip of a microsecond or several (the payload that
+ * other waves of the compute unit pull from host memory comes back through
+ * the same in-order return path), so the protocol is laid out to need few of
+ * them, one after the other:
+ *   - one in_ticket fetch_add(n) per group reserves n consecutive SQ slots; a
+ *     command's id IS its slot, and the slot stays taken until the command's
+ *     owner has finished with the completion and the staged payload, so there
+ *     is no separate allocator of command ids (1 round trip, and 1 to see the
+ *     slot free);
+ *   - lanes write their own 64-byte entries and mark their slots with the
+ *     lap number; the lock of the tail holds the tail itself, so whoever takes
+ *     it (1 round trip) knows where to sweep from, reads up to 64 marks at a
+ *     time (1), rings one doorbell for the run and lets go without waiting;
+ *   - completions are not searched for per thread.  The lock of the CQ head
+ *     holds the head; whoever takes it reads 64 entries at a time and flags
+ *     each completed command in the cid table (cid[c] = LOCKED|DONE); waiters
+ *     poll their own word.  One CQ doorbell per drain.
  * All waits are bounded (bam_guard_t).
  */
 #ifndef __NVM_PARALLEL_QUEUE_H_
@@ -83,246 +92,74 @@ __device__ __forceinline__ uint32_t leading_run(uint64_t act, uint64_t ok)
     return miss ? popc(act & lanes_below(first_lane(miss))) : popc(act);
 }
 
-/* ---- command ids ---- */
+/* ---- lock words that carry the position they guard ---- */
 /*
- * Command ids are handed out to a group of lanes as one block of 64 (ids
- * 64*b .. 64*b+63): one atomic per wave instead of one per command, and a
- * wave never sits on a few ids while it waits for more, which would leave two
- * waves that share a queue each holding part of what the other needs.
- * Blocks are ticket locks: the n-th wave to ask gets block n mod n_blocks and
- * waits for that block's turn counter to reach n div n_blocks, so waves are
- * served in arrival order and none starves.  Returns the lane's id (block
- * base + rank of the lane in the group); the caller holds nothing else it
- * would have to give up while this waits.
+ * tail_lock of an SQ and head_lock of a CQ: bit 0 = held, bits 31:1 = the tail / head (free running, 31 bits).  Taking
+ * the lock with a fetch-or hands the taker the position in the same round trip, and letting go is one store of the new
+ * position.
  */
-__device__ __forceinline__ uint32_t get_cid_group(nvm_queue_t* sq)
+#define BAM_POS_MASK 0x7fffffffu
+__device__ __forceinline__ bool pos_before(uint32_t ticket, uint32_t pos31)          /* ticket < pos, both mod 2^31 */
 {
-    const uint64_t act = active_mask();
-    const uint32_t leader = first_lane(act);
-    const uint32_t n_blocks = (sq->cid_mask + 1u) >> 6;          /* power of two */
-    uint32_t base = 0;
-    if (lane() == leader) {
-        const uint32_t t = __hip_atomic_fetch_add(&sq->cid_ticket, 1u, __ATOMIC_RELAXED, BAM_AGENT);
-        const uint32_t b = t & (n_blocks - 1), shift = (uint32_t)__builtin_ctz(n_blocks);
-        const uint32_t turn_mask = 0xffffffffu >> shift;
-        spin_t sp;
-        /* polled with plain loads: an acquire per look would invalidate this compute unit's cache every time */
-        while (((ld_relaxed(&sq->pos_locks[b].val) - (t >> shift)) & turn_mask) != 0)
-            if (spin_giveup(sq, sp)) break;
-        fence_meta();
-        st_relaxed(&sq->head_mark[b].val, popc(act));       /* ids of this block still out */
-        base = b << 6;
-    }
-    base = bcast(base, leader);
-    const uint32_t id = base + rank_in(act);
-    st_relaxed(&sq->cid[id].val, (uint32_t)LOCKED);
-    return id;
+    const uint32_t d = (pos31 - ticket) & BAM_POS_MASK;
+    return d != 0 && d < 0x40000000u;
 }
+/* what a slot's mark reads once its entry for the lap of `idx` (free-running index, any width above 31 bits ignored) is written */
+__device__ __forceinline__ uint32_t lap_mark(uint32_t idx, uint32_t qs_log2) { return ((idx & BAM_POS_MASK) >> qs_log2) + 1u; }
 
-/*
- * Give command ids back.  The lanes that took a block together may return
- * their ids in one call or in several (the asynchronous entry points are
- * called thread by thread); the block's turn moves on when its last id is in.
- */
-__device__ __forceinline__ void put_cid_group(nvm_queue_t* sq, uint32_t id)
-{
-    st_relaxed(&sq->cid[id].val, (uint32_t)UNLOCKED);
-    fence_meta();                    /* whatever the lanes did with their ids and staging pages is over */
-    for_each_group((uint64_t)(id >> 6), [&](uint64_t b) {
-        const uint64_t grp = active_mask();
-        if (lane() == first_lane(grp)) {
-            const uint32_t k = popc(grp);
-            if (__hip_atomic_fetch_add(&sq->head_mark[b].val, 0u - k, __ATOMIC_RELAXED, BAM_AGENT) == k)
-                __hip_atomic_fetch_add(&sq->pos_locks[b].val, 1u, __ATOMIC_RELAXED, BAM_AGENT);   /* next turn */
-        }
-    });
-}
-
-__device__ __forceinline__ void cq_drain_group(nvm_queue_t* cq, nvm_queue_t* sq, uint64_t act);
+__device__ __forceinline__ void cq_drain_group(nvm_queue_t* cq, nvm_queue_t* sq, uint64_t act, uint32_t h);
 
 /*
  * Drain the completion queue if nobody else is doing so; true if this group
- * did.  The ring may live on the far side of the interconnect, and every
- * waiting wave comes through here, so an idle ring must cost next to nothing:
- * the holder of head_lock first reads the one entry at the head (a single
- * small read), and only when that entry is new does the group read a window
- * of 64; after an empty look a ring in host memory is left alone for
- * cq->idle_ticks (two microseconds; the time is kept in the otherwise unused
- * `tail` word of the CQ descriptor).  A ring in device memory has no such
- * pause: a look at it stays on the device.
+ * did.  Every waiting wave comes through here, so a look must cost next to
+ * nothing: one fetch-or for lock and head, one read of the entry at the head
+ * (by every lane: the window of 64 that a drain starts with).  A ring in host
+ * memory is left alone for cq->idle_ticks after an empty look (two
+ * microseconds; the time is kept in the otherwise unused `tail` word of the
+ * CQ descriptor): a look at it crosses the interconnect.  A ring in device
+ * memory has no such pause.
  */
 __device__ __forceinline__ bool try_drain_group(nvm_queue_t* cq, nvm_queue_t* sq)
 {
     const uint64_t act = active_mask();
     const uint32_t leader = first_lane(act);
-    uint32_t got = 0;
+    uint32_t got = 0, h = 0;
     if (lane() == leader) {
         /* the word holds the time of the next look (low 32 bits of the clock): wait only while that lies within
          * the next idle_ticks, so that a stale or never-written value can never hold anybody up */
         const uint32_t idle = cq->idle_ticks;
         const uint32_t ahead = idle ? ld_relaxed(&cq->tail) - (uint32_t)wall_clock64() : 0u;
-        if (ahead - 1u >= idle && ld_relaxed(&cq->head_lock) == UNLOCKED &&
-            __hip_atomic_exchange(&cq->head_lock, (uint32_t)LOCKED, __ATOMIC_RELAXED, BAM_AGENT) == UNLOCKED) {
-            fence_meta();
-            const uint32_t h = ld_relaxed(&cq->head);
-            [[maybe_unused]] const uint64_t po5 = BAM_PROF_NOW();
-            const uint32_t dw3 = ld_relaxed_sys(&((nvm_cpl_t*)cq->vaddr)[h & cq->qs_minus_1].dword[3]);
-            BAM_PROF_ADD(cq, 27, 1); BAM_PROF_ADD(cq, 28, BAM_PROF_NOW() - po5);
-            if (((dw3 >> 16) & 1u) == ((~(h >> cq->qs_log2)) & 1u)) got = 1;
-            else {
-                if (idle) st_relaxed(&cq->tail, (uint32_t)wall_clock64() + idle);      /* nothing new: leave the ring alone for a while */
-                st_publish(&cq->head_lock, (uint32_t)UNLOCKED);
-                BAM_PROF_ADD(cq, 20, 1);
-            }
+        if (ahead - 1u >= idle) {
+            const uint32_t old = __hip_atomic_fetch_or(&cq->head_lock, 1u, __ATOMIC_RELAXED, BAM_AGENT);
+            if ((old & 1u) == 0) { got = 1; h = old >> 1; }
         }
     }
     got = bcast(got, leader);
-    if (got) {
-        [[maybe_unused]] const uint64_t pd0 = BAM_PROF_NOW();
-        cq_drain_group(cq, sq, act);
-        if (lane() == leader) { st_publish(&cq->head_lock, (uint32_t)UNLOCKED); BAM_PROF_ADD(cq, 17, 1); BAM_PROF_ADD(cq, 19, BAM_PROF_NOW() - pd0); }
-    }
-    return got != 0;
+    if (!got) return false;
+    h = bcast(h, leader);
+    [[maybe_unused]] const uint64_t pd0 = BAM_PROF_NOW();
+    cq_drain_group(cq, sq, act, h);
+    if (lane() == leader) { BAM_PROF_ADD(cq, 17, 1); BAM_PROF_ADD(cq, 19, BAM_PROF_NOW() - pd0); }
+    return true;
 }
 
 /*
- * Submit one command per active lane to `sq` (wave-uniform).  Returns the
- * slot the lane's entry went to.  On return every entry is covered by a
- * doorbell write.
+ * Drain the completion queue from head `h`: the caller's group holds cq->head_lock and lets go of it here.  Flags
+ * every completed command in sq->cid[], notes how far the controller has read the SQ (SQHD of the newest completion;
+ * the tail sweep keeps the tail one entry short of it) and rings the CQ head doorbell once.
  */
-__device__ __forceinline__ uint32_t sq_enqueue_group(nvm_queue_t* sq, nvm_cmd_t* cmd)
-{
-    const uint64_t act = active_mask();
-    const uint32_t n = popc(act), rank = rank_in(act), leader = first_lane(act);
-    const uint32_t mask = sq->qs_minus_1;
-    uint32_t t0 = 0;
-    [[maybe_unused]] const uint64_t pq0 = BAM_PROF_NOW();
-    [[maybe_unused]] uint64_t pq2 = 0;
-    [[maybe_unused]] uint32_t p_trips = 0;
-    if (lane() == leader) t0 = __hip_atomic_fetch_add(&sq->in_ticket, n, __ATOMIC_RELAXED, BAM_AGENT);
-    t0 = bcast(t0, leader);
-    [[maybe_unused]] const uint64_t pq1 = BAM_PROF_NOW();
-    const uint32_t ticket = t0 + rank, pos = ticket & mask;
-    if (sq->sealed) nvm_cmd_seal(cmd, ticket);
-    bool written = false;
-    spin_t sp;
-    for (;;) {
-#ifdef BAM_PROFILE
-        const uint64_t po0 = BAM_PROF_NOW();
-        const uint32_t slot_word = ld_relaxed(&sq->tickets[pos].val);
-        const uint64_t po1 = BAM_PROF_NOW();
-        if (lane() == leader && !written) { BAM_PROF_ADD(sq, 22, 1); BAM_PROF_ADD(sq, 23, po1 - po0); }
-#else
-        const uint32_t slot_word = ld_relaxed(&sq->tickets[pos].val);
-#endif
-        if (!written && nvm_sq_slot_free(slot_word, ticket, sq->qs_log2)) {
-            fence_meta();
-            [[maybe_unused]] const uint64_t po2 = BAM_PROF_NOW();
-            /* written through to the ring, which may be host memory the L2 would otherwise hold on to */
-            uint64_t* dst = (uint64_t*)(((nvm_cmd_t*)sq->vaddr) + pos);
-            const uint64_t* src = (const uint64_t*)cmd->dword;
-#pragma unroll
-            for (int i = 0; i < 8; i++) __hip_atomic_store(dst + i, src[i], __ATOMIC_RELAXED, BAM_SYSTEM);
-            /*
-             * The entry must be in the ring before its mark can be swept into a doorbell.  A sealed queue leaves that
-             * to the controller (it takes an entry only once the seal verifies).  An unsealed one (a controller that
-             * follows the NVMe specification to the letter) has to know: the wait on the wave's own store counters
-             * says that the stores have been handed on, not that they have arrived, and the doorbell, written later by
-             * another wave, may travel another way.  Reading the entry back does say so: the reply to a read does not
-             * pass writes posted before it.
-             */
-#ifdef BAM_PROFILE
-            { const uint64_t po3 = BAM_PROF_NOW(); if (lane() == leader) { BAM_PROF_ADD(sq, 24, 1); BAM_PROF_ADD(sq, 25, po3 - po2); } }
-#endif
-            if (!sq->sealed) {
-                if (sq->flush == 1u) fence_release_sys();
-                else if (sq->flush == 2u) {
-                    fence_meta();
-                    const uint64_t back = __hip_atomic_load(dst + 7, __ATOMIC_RELAXED, BAM_SYSTEM);
-                    asm volatile("" :: "v"(back));
-                }
-            }
-            st_publish(&sq->tail_mark[pos].val, 1u);
-            written = true;
-        }
-        if (!pq2 && !ballot(!written)) pq2 = BAM_PROF_NOW();
-        p_trips++;
-        const uint32_t tl = ld_relaxed(&sq->tail);
-        const bool covered = written && (int32_t)(tl - ticket) > 0;
-        if (!ballot(!covered)) break;
-        bool progressed = false;
-        if (ballot(written && !covered)) {
-            /* try to become the tail mover for this queue */
-            uint32_t got = 0;
-            if (lane() == leader)
-                got = ld_relaxed(&sq->tail_lock) == UNLOCKED &&
-                      __hip_atomic_exchange(&sq->tail_lock, (uint32_t)LOCKED, __ATOMIC_RELAXED, BAM_AGENT) == UNLOCKED;
-            got = bcast(got, leader);
-            if (got) {
-                fence_meta();
-                const uint32_t cur = ld_relaxed(&sq->tail);
-                /* never let tail + 1 == head (mod qs): at most qs - 1 entries outstanding */
-                const uint32_t room = ld_relaxed(&sq->head) + sq->qs - 1u - cur;
-                uint32_t total = 0;
-                for (;;) {
-                    const uint32_t k = total + rank;
-                    const bool m = k < room && ld_relaxed(&sq->tail_mark[(cur + k) & mask].val) == 1u;
-                    const uint32_t run = leading_run(act, ballot(m));
-                    if (rank < run) st_relaxed(&sq->tail_mark[(cur + k) & mask].val, 0u);
-                    total += run;
-                    if (run < n) break;
-                }
-                fence_meta();                /* the marks read and cleared above: before the doorbell and the unlock */
-                if (lane() == leader) {
-                    if (total) {
-                        [[maybe_unused]] const uint64_t po4 = BAM_PROF_NOW();
-                        st_relaxed_sys(sq->db, (cur + total) & mask);     /* one doorbell for the whole run */
-                        BAM_PROF_ADD(sq, 26, BAM_PROF_NOW() - po4);
-                        st_relaxed(&sq->tail, cur + total);
-                        BAM_PROF_ADD(sq, 15, 1); BAM_PROF_ADD(sq, 14, total);
-                    }
-                    st_publish(&sq->tail_lock, (uint32_t)UNLOCKED);
-                    BAM_PROF_ADD(sq, 13, 1);
-                }
-                progressed = total != 0;
-            }
-        }
-        if (!progressed) {
-            /* a full SQ only empties when completions are consumed: do that here too, or a
-             * group larger than the queue would wait on itself */
-            try_drain_group((nvm_queue_t*)sq->pair, sq);
-            if (spin_giveup(sq, sp)) break;
-        }
-    }
-#ifdef BAM_PROFILE
-    if (lane() == leader) {
-        const uint64_t pq3 = BAM_PROF_NOW();
-        if (!pq2) pq2 = pq3;
-        BAM_PROF_ADD(sq, 9, pq1 - pq0); BAM_PROF_ADD(sq, 10, pq2 - pq1); BAM_PROF_ADD(sq, 11, pq3 - pq2); BAM_PROF_ADD(sq, 12, p_trips);
-    }
-#endif
-    return pos;
-}
-
-/*
- * Drain the completion queue: caller's group holds cq->head_lock.  Flags every
- * completed command in sq->cid[], frees the SQ slots the controller has
- * consumed (SQHD of the newest completion) and rings the CQ head doorbell once.
- */
-__device__ __forceinline__ void cq_drain_group(nvm_queue_t* cq, nvm_queue_t* sq, uint64_t act)
+__device__ __forceinline__ void cq_drain_group(nvm_queue_t* cq, nvm_queue_t* sq, uint64_t act, uint32_t h)
 {
     const uint32_t n = popc(act), rank = rank_in(act), leader = first_lane(act);
     const uint32_t mask = cq->qs_minus_1;
-    const uint32_t h = ld_relaxed(&cq->head);
     nvm_cpl_t* ring = (nvm_cpl_t*)cq->vaddr;
     uint32_t moved = 0, sqhd = 0;
     for (;;) {
-        const uint32_t idx = h + moved + rank, loc = idx & mask;
+        const uint32_t idx = (h + moved + rank) & BAM_POS_MASK, loc = idx & mask;
         const uint32_t phase = (~(idx >> cq->qs_log2)) & 1u;          /* first lap carries phase 1 */
         /* SQHD and the phase tag in one access: the controller may write an entry in pieces of eight bytes */
         const uint64_t dw23 = __hip_atomic_load((uint64_t*)&ring[loc].dword[2], __ATOMIC_RELAXED, BAM_SYSTEM);
         const uint32_t dw3 = (uint32_t)(dw23 >> 32);
-        fence_meta();
         const bool valid = ((dw3 >> 16) & 1u) == phase && moved + rank < mask;
         const uint32_t run = leading_run(act, ballot(valid));
         if (rank < run) {
@@ -338,20 +175,173 @@ __device__ __forceinline__ void cq_drain_group(nvm_queue_t* cq, nvm_queue_t* sq,
         moved += run;
         if (run < n) break;
     }
-    if (moved) {
-        const uint32_t smask = sq->qs_minus_1;
-        const uint32_t sh = ld_relaxed(&sq->head);
-        const uint32_t freed = (sqhd - sh) & smask;
-        fence_meta();
-        for (uint32_t i = rank; i < freed; i += n)
-            __hip_atomic_fetch_add(&sq->tickets[(sh + i) & smask].val, 2u, __ATOMIC_RELAXED, BAM_AGENT);
-        if (lane() == leader) {
-            if (freed) st_relaxed(&sq->head, sh + freed);
+    if (lane() == leader) {
+        if (moved) {
+            /* how far the controller has read the submission ring, free running: the newest SQHD is at most one lap ahead of the last */
+            const uint32_t sh = ld_relaxed(&sq->head);
+            st_relaxed(&sq->head, sh + ((sqhd - sh) & sq->qs_minus_1));
             st_relaxed_sys(cq->db, (h + moved) & mask);                /* one doorbell for the whole run */
             st_relaxed(&cq->head, h + moved);
+            st_relaxed(&cq->in_ticket, 0u);
+            /* The controller looks at this doorbell only when the ring is full as far as it knows, and then it must
+             * find the newest value: the store has been handed on before the next drainer can write another.  (Handed
+             * on is not arrived: see the empty look below.) */
+            fence_meta();
             BAM_PROF_ADD(cq, 18, moved);
+        } else {
+            if (cq->idle_ticks) st_relaxed(&cq->tail, (uint32_t)wall_clock64() + cq->idle_ticks);      /* nothing new: leave the ring alone for a while */
+            /* Two doorbell writes of two waves may still arrive in the wrong order, and the controller, finding the
+             * older value last, would wait with a full ring for a doorbell that nobody owes it.  Waves that keep
+             * finding the ring empty therefore write the head again now and then (the in_ticket word, unused on a CQ,
+             * counts the empty looks since the last drain). */
+            const uint32_t looks = ld_relaxed(&cq->in_ticket) + 1u;
+            st_relaxed(&cq->in_ticket, looks);
+            if ((looks & 63u) == 0) st_relaxed_sys(cq->db, h & mask);
+            BAM_PROF_ADD(cq, 20, 1);
+        }
+        /* the entries have been read (their values were used above): the next drainer may have the ring */
+        st_relaxed(&cq->head_lock, ((h + moved) & BAM_POS_MASK) << 1);
+    }
+}
+
+/* ---- submission ---- */
+/*
+ * Reserve one SQ slot per active lane on `sq` (wave-uniform) and wait until each is free.  Returns the lane's ticket;
+ * its slot, which is also its command id, is ticket & (qs - 1).  A slot is free again when the owner of the command
+ * that had it before has given it back (sq_release_group), so at most qs commands of a queue are out at a time and a
+ * command id never names two of them.
+ */
+__device__ __forceinline__ uint32_t sq_reserve_group(nvm_queue_t* sq)
+{
+    const uint64_t act = active_mask();
+    const uint32_t n = popc(act), rank = rank_in(act), leader = first_lane(act);
+    uint32_t t0 = 0;
+    [[maybe_unused]] const uint64_t pq0 = BAM_PROF_NOW();
+    if (lane() == leader) t0 = __hip_atomic_fetch_add(&sq->in_ticket, n, __ATOMIC_RELAXED, BAM_AGENT);
+    t0 = bcast(t0, leader);
+    [[maybe_unused]] const uint64_t pq1 = BAM_PROF_NOW();
+    const uint32_t ticket = t0 + rank, pos = ticket & sq->qs_minus_1;
+    spin_t sp;
+    for (;;) {
+        const bool is_free = nvm_sq_slot_free(ld_relaxed(&sq->tickets[pos].val), ticket, sq->qs_log2);
+        if (!ballot(!is_free)) break;
+        /* the slots come back when completions are consumed: do that here too, or a group larger than what is
+         * left of the queue would wait on itself */
+        try_drain_group((nvm_queue_t*)sq->pair, sq);
+        if (spin_giveup(sq, sp)) break;
+    }
+    st_relaxed(&sq->cid[pos].val, (uint32_t)LOCKED);
+    if (lane() == leader) { BAM_PROF_ADD(sq, 9, pq1 - pq0); BAM_PROF_ADD(sq, 10, BAM_PROF_NOW() - pq1); }
+    return ticket;
+}
+
+/* Give the slots (command ids) of the active lanes back: what the lanes did with their completions and staging pages is over. */
+__device__ __forceinline__ void sq_release_group(nvm_queue_t* sq, uint32_t pos)
+{
+    fence_meta();
+    __hip_atomic_fetch_add(&sq->tickets[pos].val, 2u, __ATOMIC_RELAXED, BAM_AGENT);
+}
+
+/*
+ * Write the entry of every active lane into its reserved slot of `sq` (wave-uniform) and see to it that a doorbell
+ * covers it.  `cmd` carries the slot as its command id.
+ */
+__device__ __forceinline__ void sq_submit_group(nvm_queue_t* sq, nvm_cmd_t* cmd, const uint32_t ticket)
+{
+    const uint64_t act = active_mask();
+    const uint32_t n = popc(act), rank = rank_in(act), leader = first_lane(act);
+    const uint32_t mask = sq->qs_minus_1, pos = ticket & mask;
+    const uint32_t t0 = bcast(ticket, leader);
+    [[maybe_unused]] const uint64_t pq2 = BAM_PROF_NOW();
+    if (sq->sealed) nvm_cmd_seal(cmd, ticket);
+    /* written through to the ring, which may be host memory the L2 would otherwise hold on to */
+    uint64_t* dst = (uint64_t*)(((nvm_cmd_t*)sq->vaddr) + pos);
+    const uint64_t* src = (const uint64_t*)cmd->dword;
+#pragma unroll
+    for (int i = 0; i < 8; i++) __hip_atomic_store(dst + i, src[i], __ATOMIC_RELAXED, BAM_SYSTEM);
+    /*
+     * The entry must be in the ring before a doorbell that covers it reaches the controller.  A sealed queue leaves
+     * that to the controller (it takes an entry only once the seal verifies, doorbell or no doorbell).  An unsealed
+     * one (a controller that follows the NVMe specification to the letter) has to know: a wait on the wave's own store
+     * counters says that the stores have been handed on, not that they have arrived, and the doorbell, written later by
+     * another wave, may travel another way.  Reading the entry back does say so: the reply to a read does not pass
+     * writes posted before it.
+     */
+    if (!sq->sealed) {
+        if (sq->flush == 1u) fence_release_sys();
+        else if (sq->flush == 2u) {
+            fence_meta();
+            const uint64_t back = __hip_atomic_load(dst + 7, __ATOMIC_RELAXED, BAM_SYSTEM);
+            asm volatile("" :: "v"(back));
+        }
+        fence_meta();
+    }
+    st_relaxed(&sq->tail_mark[pos].val, lap_mark(ticket, sq->qs_log2));
+    [[maybe_unused]] const uint64_t pq3 = BAM_PROF_NOW();
+    [[maybe_unused]] uint32_t p_trips = 0;
+    /* cover: sweep the marks from the tail on, or wait for whoever is doing that to get past this group's entries */
+    bool covered = false;
+    spin_t sp;
+    for (;;) {
+        p_trips++;
+        uint32_t got = 0, cur = 0;
+        if (lane() == leader) {
+            const uint32_t old = __hip_atomic_fetch_or(&sq->tail_lock, 1u, __ATOMIC_RELAXED, BAM_AGENT);
+            got = (old & 1u) == 0;
+            cur = old >> 1;
+        }
+        got = bcast(got, leader);
+        cur = bcast(cur, leader);
+        bool progressed = false;
+        if (got) {
+            /* never let tail + 1 == head (mod qs): at most qs - 1 entries between what the controller has read and the tail */
+            const uint32_t room = ((ld_relaxed(&sq->head) & BAM_POS_MASK) + sq->qs - 1u - cur) & BAM_POS_MASK;
+            uint32_t total = 0;
+            for (;;) {
+                const uint32_t k = total + rank, idx = (cur + k) & BAM_POS_MASK;
+                /* this group's own entries are written (above), whatever their marks read by now */
+                const bool own = ((idx - t0) & BAM_POS_MASK) < n;
+                const bool m = k < room && (own || ld_relaxed(&sq->tail_mark[idx & mask].val) == lap_mark(idx, sq->qs_log2));
+                const uint32_t run = leading_run(act, ballot(m));
+                total += run;
+                if (run < n) break;
+            }
+            const uint32_t new_tail = (cur + total) & BAM_POS_MASK;
+            if (lane() == leader) {
+                if (total) {
+                    st_relaxed_sys(sq->db, new_tail & mask);     /* one doorbell for the whole run */
+                    /* unsealed: the doorbell is there before the next one can leave */
+                    if (!sq->sealed && sq->flush) { fence_meta(); const uint32_t back = ld_relaxed_sys(sq->db); asm volatile("" :: "v"(back)); fence_meta(); }
+                    st_relaxed(&sq->tail, new_tail);
+                    BAM_PROF_ADD(sq, 15, 1); BAM_PROF_ADD(sq, 14, total);
+                }
+                st_relaxed(&sq->tail_lock, new_tail << 1);
+                BAM_PROF_ADD(sq, 13, 1);
+            }
+            covered = pos_before(ticket, new_tail);
+            progressed = total != 0;
+        } else
+            covered = pos_before(ticket, cur);
+        /* A sealed queue's controller takes entries by their seals, announced or not: the doorbell is a courtesy, rung
+         * by whoever finds the lock free, and nobody waits for it.  (Waiting would even be wrong: the controller may
+         * have read a whole lap of entries between two completions that report how far it has read, which looks like
+         * no progress at all, and the tail would stay one entry short of a head that never seems to move.) */
+        if (sq->sealed) break;
+        if (!ballot(!covered)) break;
+        if (!progressed) {
+            /* somebody else is sweeping, or the queue is full: watch the tail with plain loads until this group is
+             * covered or the lock is free again; a full SQ only empties when completions are consumed */
+            const uint32_t w = bcast(ld_relaxed(&sq->tail_lock), leader);
+            covered = pos_before(ticket, w >> 1);
+            if (!ballot(!covered)) break;
+            if (w & 1u) { if (spin_giveup(sq, sp)) break; }
+            else if (!got) continue;
+            else { try_drain_group((nvm_queue_t*)sq->pair, sq); if (spin_giveup(sq, sp)) break; }
         }
     }
+#ifdef BAM_PROFILE
+    if (lane() == leader) { BAM_PROF_ADD(sq, 11, BAM_PROF_NOW() - pq3); BAM_PROF_ADD(sq, 25, pq3 - pq2); BAM_PROF_ADD(sq, 24, 1); BAM_PROF_ADD(sq, 12, p_trips); }
+#endif
 }
 
 /*
@@ -372,7 +362,8 @@ __device__ __forceinline__ bool cq_wait_group(nvm_queue_t* cq, nvm_queue_t* sq, 
         if (spin_giveup(cq, sp)) break;
     }
     if (lane() == first_lane(active_mask())) BAM_PROF_ADD(cq, 16, p_trips);
-    /* what the controller wrote before posting the completion is visible from here on */
+    /* what the controller wrote before posting the completion is visible from here on: a staging page in host memory
+     * has had other tenants, and this compute unit's caches may remember them */
     fence_acquire_sys();
     return (w & (BAM_CID_DONE | BAM_CID_ERR)) == BAM_CID_DONE;
 }
@@ -381,25 +372,38 @@ __device__ __forceinline__ bool cq_wait_group(nvm_queue_t* cq, nvm_queue_t* sq, 
 
 /* ---- per-thread entry points with the reference's names ---- */
 
+/*
+ * A command id is the SQ slot its entry goes to: get_cid reserves the slot (the ticket is kept with it for sq_enqueue),
+ * put_cid gives it back.  To be called by the lanes of a wave as the reference's threads call them: get_cid, then
+ * sq_enqueue with that id in the entry, cq_poll, put_cid.
+ */
 inline __device__ uint16_t get_cid(nvm_queue_t* sq)
 {
     uint32_t id = 0;
-    bam::for_each_group((uint64_t)sq, [&](uint64_t q) { id = bam::get_cid_group((nvm_queue_t*)q); });
+    bam::for_each_group((uint64_t)sq, [&](uint64_t q) {
+        nvm_queue_t* s = (nvm_queue_t*)q;
+        const uint32_t ticket = bam::sq_reserve_group(s);
+        id = ticket & s->qs_minus_1;
+        bam::st_relaxed(&s->head_mark[id].val, ticket);
+    });
     return (uint16_t)id;
 }
 
-/* to be called by the same lanes that called get_cid together, all at once or in parts */
+/* to be called by the lanes that hold the ids, all at once or in parts */
 inline __device__ void put_cid(nvm_queue_t* sq, uint16_t id)
 {
-    bam::for_each_group((uint64_t)sq, [&](uint64_t q) { bam::put_cid_group((nvm_queue_t*)q, id); });
+    bam::for_each_group((uint64_t)sq, [&](uint64_t q) { bam::sq_release_group((nvm_queue_t*)q, id); });
 }
 
-/* returns the SQ slot used */
+/* the entry carries the id that get_cid handed out (nvm_cmd_header); returns the SQ slot used, which is that id */
 inline __device__ uint16_t sq_enqueue(nvm_queue_t* sq, nvm_cmd_t* cmd)
 {
-    uint32_t pos = 0;
-    bam::for_each_group((uint64_t)sq, [&](uint64_t q) { pos = bam::sq_enqueue_group((nvm_queue_t*)q, cmd); });
-    return (uint16_t)pos;
+    const uint32_t id = cmd->dword[0] >> 16;
+    bam::for_each_group((uint64_t)sq, [&](uint64_t q) {
+        nvm_queue_t* s = (nvm_queue_t*)q;
+        bam::sq_submit_group(s, cmd, bam::ld_relaxed(&s->head_mark[id & s->qs_minus_1].val));
+    });
+    return (uint16_t)id;
 }
 
 /*
@@ -412,7 +416,7 @@ inline __device__ uint16_t sq_enqueue(nvm_queue_t* sq, nvm_cmd_t* cmd)
 inline __device__ uint32_t cq_poll(nvm_queue_t* cq, uint16_t search_cid, uint32_t* loc_ = nullptr, uint32_t* cq_head = nullptr)
 {
     bam::for_each_group((uint64_t)cq, [&](uint64_t q) { bam::cq_wait_group((nvm_queue_t*)q, (nvm_queue_t*)((nvm_queue_t*)q)->pair, search_cid); });
-    uint32_t h = bam::ld_relaxed(&cq->head);
+    uint32_t h = bam::ld_relaxed(&cq->head_lock) >> 1;
     if (loc_) *loc_ = h;
     if (cq_head) *cq_head = h;
     return h & cq->qs_minus_1;

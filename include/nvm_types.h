@@ -71,20 +71,20 @@ typedef struct { uint32_t val; } padded_struct;
  */
 typedef struct
 {
-    uint32_t head_lock;  uint8_t pad0[60];  /* CQ: held by the wave draining completions */
-    uint32_t tail_lock;  uint8_t pad1[60];  /* SQ: held by the wave sweeping tail marks */
+    uint32_t head_lock;  uint8_t pad0[60];  /* CQ: bit 0 = held by the wave draining completions, bits 31:1 = head (free running) */
+    uint32_t tail_lock;  uint8_t pad1[60];  /* SQ: bit 0 = held by the wave sweeping tail marks, bits 31:1 = tail (free running) */
     uint32_t head;       uint8_t pad2[60];  /* free-running */
     uint32_t tail;       uint8_t pad3[60];  /* free-running */
     uint32_t in_ticket;  uint8_t pad4[60];  /* SQ: next slot ticket */
     uint32_t cid_ticket;                    /* SQ: next command-id probe */
     uint32_t n_errors;   uint8_t pad5[56];  /* CQ: completions seen with a non-zero status */
 
-    padded_struct*          tickets;        /* SQ [qs]: 2*lap = free for lap, odd = submitted */
-    padded_struct*          head_mark;      /* SQ [n_cids / 64]: command ids of the block still out (the reference marks consumed CQ entries here) */
-    padded_struct*          tail_mark;      /* SQ [qs]: 1 = written, waiting for the tail sweep */
-    padded_struct*          cid;            /* SQ [n_cids]: per command id, 0 idle, 1 in flight, 3 in flight + completed */
-    padded_struct*          pos_locks;      /* SQ [n_cids / 64]: command ids are handed out to a wave in blocks of 64; turn counter of each block */
-    uint32_t                cid_mask;       /* n_cids - 1 */
+    padded_struct*          tickets;        /* SQ [qs]: 2 * lap = free for the ticket of that lap (its owner adds 2 when done with the command) */
+    padded_struct*          head_mark;      /* SQ [qs]: the ticket a slot was reserved with by get_cid, for sq_enqueue (the reference marks consumed CQ entries here) */
+    padded_struct*          tail_mark;      /* SQ [qs]: lap + 1 of the entry last written to the slot, read by the tail sweep */
+    padded_struct*          cid;            /* SQ [qs]: per command id (= slot), 1 in flight, 3 in flight + completed, 7 completed with an error status */
+    padded_struct*          pos_locks;      /* unused (the reference's per-slot CQ locks) */
+    uint32_t                cid_mask;       /* qs - 1 */
     uint32_t                sealed;         /* SQ: entries carry a sequence number and checksum (nvm_cmd_seal) */
     uint32_t                flush;          /* SQ, unsealed: how a written entry is known to have reached the ring before its mark is set
                                                (0 nothing beyond the wave's own store counters, 1 system-scope release, 2 read the entry back) */

@@ -78,6 +78,10 @@ void     nvmt_reset_stats(nvmt_t* t);
 int      nvmt_publish(const char* path, nvmt_t* t);
 nvmt_t*  nvmt_lookup(const char* path);
 const nvmt_config_t* nvmt_config(nvmt_t* t);
+/* where the target stands on I/O queue pair `qid` (read without stopping the service threads: for diagnosis after a
+ * run that was given up).  out8: SQ head, commands fetched so far, SQ tail doorbell, sealed, CQ tail, CQ head as last
+ * seen, CQ head doorbell, CQ phase.  0, EINVAL or ENOENT (no such queue). */
+int      nvmt_queue_state(nvmt_t* t, uint16_t qid, uint64_t* out8);
 /* procedural content: fills out[0..n) with words first_word.. of a namespace with this seed */
 void     nvmt_fill_words(uint64_t seed, uint64_t first_word, uint64_t n, uint64_t* out);
 /*

@@ -88,8 +88,14 @@ typedef struct __attribute__((aligned(8))) { uint32_t state; uint32_t offset; } 
 typedef data_page_t* pages_t;
 __forceinline__ __device__ void bam_release_refs(data_page_t* dp, const uint32_t count, const bool wrote);
 
-/* one per cache slot */
-typedef struct { uint32_t page_take_lock; uint32_t pad; uint64_t page_translation; } cache_page_t;
+/*
+ * One per cache slot: which page the slot holds and who may change that, in one word, so that taking the slot's lock
+ * tells the taker in the same round trip what the slot holds.  Bits 63:62 are the reference's page_take_lock (FREE = 2,
+ * LOCKED = 1, UNLOCKED = 0; 3 = locked by the one who found it free), bits 61:0 its page_translation.
+ */
+typedef struct { uint64_t page_translation; } cache_page_t;
+#define BAM_TAKE_SHIFT 62
+#define BAM_TRANSLATION_MASK ((1ull << BAM_TAKE_SHIFT) - 1ull)
 
 /* statistics of one range, one shard per group of compute units */
 typedef struct { unsigned long long access_cnt, miss_cnt, hit_cnt, read_io_cnt, pad[4]; } bam_stat_shard_t;
@@ -200,15 +206,16 @@ __device__ __forceinline__ uint32_t* pull_begin(QueuePair* qp)
 {
     const uint32_t limit = qp->pull_limit;
     if (!limit) return nullptr;
+    /* two words per cluster: [0] turns taken, [1] turns finished; the n-th to ask goes ahead once n - finished < limit,
+     * so the waves are served in the order they asked and a turn that ends is taken up within one look of the next in line */
     uint32_t* word = qp->pull_tokens + xcc_id() * 16u;
     if (lane() == first_lane(active_mask())) {
+        const uint32_t turn = __hip_atomic_fetch_add(word, 1u, __ATOMIC_RELAXED, BAM_AGENT);
         spin_t sp;
-        for (;;) {
-            if (ld_relaxed(word) < limit) {
-                if (__hip_atomic_fetch_add(word, 1u, __ATOMIC_RELAXED, BAM_AGENT) < limit) break;
-                __hip_atomic_fetch_add(word, 0u - 1u, __ATOMIC_RELAXED, BAM_AGENT);
-            }
-            if (spin_giveup(&qp->cq, sp)) { __hip_atomic_fetch_add(word, 1u, __ATOMIC_RELAXED, BAM_AGENT); break; }
+        for (uint32_t looks = 1; (int32_t)(turn - ld_relaxed(word + 1)) >= (int32_t)limit; looks++) {
+            __builtin_amdgcn_s_sleep(4);
+            /* the abort flag and the clock once in a while (spin_giveup looks at them every 256th call) */
+            if ((looks & 255u) == 0) { sp.n = 255u; sp.slp = 1; if (spin_giveup(&qp->cq, sp)) break; }
         }
     }
     return word;
@@ -217,7 +224,21 @@ __device__ __forceinline__ void pull_end(uint32_t* word)
 {
     if (!word) return;
     fence_meta();                    /* the loads from host memory have come back */
-    if (lane() == first_lane(active_mask())) __hip_atomic_fetch_add(word, 0u - 1u, __ATOMIC_RELAXED, BAM_AGENT);
+    if (lane() == first_lane(active_mask())) __hip_atomic_fetch_add(word + 1, 1u, __ATOMIC_RELAXED, BAM_AGENT);
+}
+
+/*
+ * Run `body` for the active lanes in rounds of at most `max_n` lanes at a time (in rank order).  A group of lanes
+ * larger than half a queue is taken through the queue in such rounds, each a whole transfer: a round that held its
+ * slots while the next waited for slots would wait for itself.
+ */
+template <typename F>
+__device__ __forceinline__ void for_each_chunk(const uint32_t max_n, F&& body)
+{
+    const uint64_t act = active_mask();
+    const uint32_t n = popc(act), rank = rank_in(act), step = max_n ? max_n : 1u;
+    for (uint32_t base = 0; base < n; base += step)
+        if (rank >= base && rank - base < step) body();
 }
 
 /*
@@ -253,7 +274,9 @@ __device__ __forceinline__ uint32_t io_submit_group(page_cache_d_t* pc, QueuePai
 #ifdef BAM_PROFILE
     const uint64_t pt0 = wall_clock64();
 #endif
-    const uint32_t cid = get_cid_group(&qp->sq);
+    /* the command's id is the submission slot it goes to, taken until read_end / io_group / poll_async gives it back */
+    const uint32_t ticket = sq_reserve_group(&qp->sq);
+    const uint32_t cid = ticket & qp->sq.qs_minus_1;
 #ifdef BAM_PROFILE
     const uint64_t pt1 = wall_clock64();
 #endif
@@ -269,7 +292,7 @@ __device__ __forceinline__ uint32_t io_submit_group(page_cache_d_t* pc, QueuePai
      * batches of eight to the controller (12.3 against 11.4 M reads/s), raw block reads do best all staged (12.8
      * against 11.7 M).
      */
-    const bool direct = pc->prp1 && (bytes > qp->stage_stride || (opcode == NVM_IO_READ && bytes >= 2048 && ((cid >> 6) & 7u) < direct_share));
+    const bool direct = pc->prp1 && (bytes > qp->stage_stride || (opcode == NVM_IO_READ && bytes >= 2048 && ((ticket >> 6) & 7u) < direct_share));
     const bool staged = qp->stage && !direct;
     if (staged) {
         stage = qp->stage + (size_t)cid * qp->stage_stride;
@@ -289,7 +312,8 @@ __device__ __forceinline__ uint32_t io_submit_group(page_cache_d_t* pc, QueuePai
     nvm_cmd_header(&cmd, (uint16_t)cid, opcode, qp->nvmNamespace);
     nvm_cmd_data_ptr(&cmd, prp1, prp2);
     nvm_cmd_rw_blks(&cmd, lba, (uint16_t)n_blocks);
-    pos = sq_enqueue_group(&qp->sq, &cmd);
+    sq_submit_group(&qp->sq, &cmd, ticket);
+    pos = cid;
 #ifdef BAM_PROFILE
     if (pc->prof && rank == 0) {
         const uint64_t pt2 = wall_clock64();
@@ -322,7 +346,7 @@ __device__ __forceinline__ bool io_group(page_cache_d_t* pc, QueuePair* qp, uint
         copy_pages(pc->base_addr + pc_entry * pc->page_size, stage, stage && opcode == NVM_IO_READ && ok ? n_blocks << qp->block_size_log : 0u, act, popc(act), rank_in(act));
         pull_end(pull);
     }
-    put_cid_group(&qp->sq, cid);
+    sq_release_group(&qp->sq, cid);
 #ifdef BAM_PROFILE
     if (pc->prof && lane() == first_lane(act)) { atomicAdd(&pc->prof[4], pt3 - pt2); atomicAdd(&pc->prof[5], wall_clock64() - pt3); }
 #endif
@@ -334,7 +358,9 @@ __device__ __forceinline__ bool io_group(page_cache_d_t* pc, QueuePair* qp, uint
 inline __device__ void access_data(page_cache_d_t* pc, QueuePair* qp, const uint64_t starting_lba, const uint64_t n_blocks, const unsigned long long pc_entry, const uint8_t opcode)
 {
     bam::for_each_group((uint64_t)qp, (uint64_t)pc, [&](uint64_t q, uint64_t c) {
-        bam::io_group((page_cache_d_t*)c, (QueuePair*)q, starting_lba, (uint32_t)n_blocks, pc_entry, opcode, ((page_cache_d_t*)c)->direct_share_raw);
+        bam::for_each_chunk(((QueuePair*)q)->sq.qs >> 1, [&]() {
+            bam::io_group((page_cache_d_t*)c, (QueuePair*)q, starting_lba, (uint32_t)n_blocks, pc_entry, opcode, ((page_cache_d_t*)c)->direct_share_raw);
+        });
     });
 }
 
@@ -349,14 +375,18 @@ inline __device__ void read_begin(page_cache_d_t* pc, QueuePair* qp, const uint6
                                   uint32_t& cid, uint8_t*& stage, bool& held, bool& ok)
 {
     const uint64_t all = bam::active_mask();
-    const bool one_group = bam::ballot(qp == (QueuePair*)bam::first((uint64_t)qp) && pc == (page_cache_d_t*)bam::first((uint64_t)pc)) == all;
+    bool one_group = bam::ballot(qp == (QueuePair*)bam::first((uint64_t)qp) && pc == (page_cache_d_t*)bam::first((uint64_t)pc)) == all;
+    /* and one that the queue takes in one go: more commands than half its slots go through it in rounds */
+    if (one_group && bam::popc(all) > (((QueuePair*)bam::first((uint64_t)qp))->sq.qs >> 1)) one_group = false;
     held = one_group;
     stage = nullptr;
     cid = 0;
     ok = false;
     if (!one_group) {
         bam::for_each_group((uint64_t)qp, (uint64_t)pc, [&](uint64_t q, uint64_t c) {
-            ok = bam::io_group((page_cache_d_t*)c, (QueuePair*)q, starting_lba, (uint32_t)n_blocks, pc_entry, NVM_IO_READ, ((page_cache_d_t*)c)->direct_share);
+            bam::for_each_chunk(((QueuePair*)q)->sq.qs >> 1, [&]() {
+                ok = bam::io_group((page_cache_d_t*)c, (QueuePair*)q, starting_lba, (uint32_t)n_blocks, pc_entry, NVM_IO_READ, ((page_cache_d_t*)c)->direct_share);
+            });
         });
         return;
     }
@@ -375,7 +405,7 @@ inline __device__ void read_begin(page_cache_d_t* pc, QueuePair* qp, const uint6
 /* for the lanes of a read_begin that came back with `held`: one queue pair */
 inline __device__ void read_end(QueuePair* qp, const uint32_t cid)
 {
-    bam::put_cid_group(&((QueuePair*)bam::first((uint64_t)qp))->sq, cid);
+    bam::sq_release_group(&((QueuePair*)bam::first((uint64_t)qp))->sq, cid);
 }
 
 inline __device__ void read_data(page_cache_d_t* pc, QueuePair* qp, const uint64_t starting_lba, const uint64_t n_blocks, const unsigned long long pc_entry)
@@ -429,7 +459,7 @@ inline __device__ void poll_async(QueuePair* qp, uint16_t cid, uint16_t sq_pos)
             bam::copy_pages(dst, cur->stage + (size_t)cid * cur->stage_stride, dst ? len : 0, act, bam::popc(act), bam::rank_in(act));
             bam::pull_end(pull);
         }
-        bam::put_cid_group(&cur->sq, cid);
+        bam::sq_release_group(&cur->sq, cid);
     });
 }
 
@@ -462,53 +492,51 @@ uint32_t page_cache_d_t::find_slot(uint64_t address, uint64_t range_id, const ui
         const uint64_t need = ballot(looking);
         if (!need) break;
         if (looking) {
+            /* three round trips when the first slot will do: the hand, the slot's lock (which brings what the slot
+             * holds), the victim's state */
             const uint32_t ld = first_lane(need);
             uint32_t base = 0;
             if (lane() == ld) base = __hip_atomic_fetch_add(page_ticket, popc(need), __ATOMIC_RELAXED, BAM_AGENT);
             base = bcast(base, ld);
             const uint32_t p = (uint32_t)((base + rank_in(need)) % n_pages);
             cache_page_t* cp = &cache_pages[p];
-            uint32_t v = ld_relaxed(&cp->page_take_lock);
+            const uint64_t w = __hip_atomic_fetch_or(&cp->page_translation, (uint64_t)LOCKED << BAM_TAKE_SHIFT, __ATOMIC_RELAXED, BAM_AGENT);
+            const uint32_t v = (uint32_t)(w >> BAM_TAKE_SHIFT);
             if (v == FREE) {
-                if (__hip_atomic_compare_exchange_strong(&cp->page_take_lock, &v, (uint32_t)LOCKED, __ATOMIC_RELAXED, __ATOMIC_RELAXED, BAM_AGENT)) {
-                    st_relaxed(&cp->page_translation, global_address);
-                    st_publish(&cp->page_take_lock, (uint32_t)UNLOCKED);
-                    page = p; looking = false;
-                }
+                /* this lane holds it (the word reads FREE | LOCKED to everybody else until the store below) */
+                page = p; looking = false;
             } else if (v == UNLOCKED) {
-                if (__hip_atomic_compare_exchange_strong(&cp->page_take_lock, &v, (uint32_t)LOCKED, __ATOMIC_RELAXED, __ATOMIC_RELAXED, BAM_AGENT)) {
-                    fence_meta();
-                    const uint64_t prev = ld_relaxed(&cp->page_translation);
-                    const uint64_t prev_range = prev & n_ranges_mask, prev_page = prev >> n_ranges_bits;
-                    data_page_t* victim = &ranges[prev_range][prev_page];
-                    const uint32_t e = ld_relaxed(&victim->state);
-                    if ((e & CNT_MASK) == 0 && (e & BUSY) == 0) {
-                        const uint32_t o = __hip_atomic_fetch_or(&victim->state, BUSY, __ATOMIC_RELAXED, BAM_AGENT);
-                        if ((o & BUSY) == 0) {
-                            if ((o & CNT_MASK) == 0) {
-                                if (o & DIRTY) {
-                                    const data_dist_t dist = ranges_dists[prev_range];
-                                    const uint64_t index = get_backing_page_(ranges_page_starts[prev_range], prev_page, n_ctrls, dist);
-                                    uint64_t c = get_backing_ctrl_(prev_page, n_ctrls, dist);
-                                    const uint64_t c_end = c == ALL_CTRLS ? n_ctrls : c + 1;
-                                    for (c = c == ALL_CTRLS ? 0 : c; c < c_end; c++) {
-                                        Controller* ctl = d_ctrls[c];
-                                        write_data(this, ctl->d_qps + (queue_ % ctl->n_qps), index * n_blocks_per_page, n_blocks_per_page, p);
-                                    }
-                                }
-                                /* -> INVALID; references taken meanwhile stay counted and their owners reload */
-                                fence_meta();
-                                __hip_atomic_fetch_and(&victim->state, CNT_MASK, __ATOMIC_RELAXED, BAM_AGENT);
-                                st_relaxed(&cp->page_translation, global_address);
-                                page = p; looking = false;
-                            } else {
-                                __hip_atomic_fetch_and(&victim->state, DISABLE_BUSY_MASK, __ATOMIC_RELAXED, BAM_AGENT);
+                const uint64_t prev = w & BAM_TRANSLATION_MASK;
+                const uint64_t prev_range = prev & n_ranges_mask, prev_page = prev >> n_ranges_bits;
+                data_page_t* victim = &ranges[prev_range][prev_page];
+                /* BUSY first, questions later: a page that turns out to be in use has it taken off again (its users see a
+                 * page that is busy for a moment and look again) */
+                const uint32_t o = __hip_atomic_fetch_or(&victim->state, BUSY, __ATOMIC_RELAXED, BAM_AGENT);
+                if ((o & BUSY) == 0) {
+                    if ((o & CNT_MASK) == 0) {
+                        if (o & DIRTY) {
+                            const data_dist_t dist = ranges_dists[prev_range];
+                            const uint64_t index = get_backing_page_(ranges_page_starts[prev_range], prev_page, n_ctrls, dist);
+                            uint64_t c = get_backing_ctrl_(prev_page, n_ctrls, dist);
+                            const uint64_t c_end = c == ALL_CTRLS ? n_ctrls : c + 1;
+                            for (c = c == ALL_CTRLS ? 0 : c; c < c_end; c++) {
+                                Controller* ctl = d_ctrls[c];
+                                write_data(this, ctl->d_qps + (queue_ % ctl->n_qps), index * n_blocks_per_page, n_blocks_per_page, p);
                             }
+                            fence_meta();
                         }
+                        /* -> INVALID; references taken meanwhile stay counted and their owners reload */
+                        __hip_atomic_fetch_and(&victim->state, CNT_MASK, __ATOMIC_RELAXED, BAM_AGENT);
+                        page = p; looking = false;
+                    } else {
+                        __hip_atomic_fetch_and(&victim->state, DISABLE_BUSY_MASK, __ATOMIC_RELAXED, BAM_AGENT);
                     }
-                    st_publish(&cp->page_take_lock, (uint32_t)UNLOCKED);
                 }
+                /* taken: the new translation goes in with the lock coming off; not taken: the old one stays */
+                if (looking) st_relaxed(&cp->page_translation, prev);
             }
+            /* (v == LOCKED or FREE | LOCKED: somebody else has it, and the fetch-or changed nothing) */
+            if (page == p) st_relaxed(&cp->page_translation, global_address);
             if (looking && tries + 1 >= BAM_FIND_SLOT_TRIES) looking = false;
         }
     }
@@ -712,7 +740,11 @@ bool range_d_t<T>::slow_step(const size_t pg, const bool write, const uint32_t q
         /* all lanes that came in are here: the queue pair of any lane that has payload to move will do for the permission */
         QueuePair* pq = (QueuePair*)bam::bcast((uint64_t)qp, bam::first_lane(bam::ballot(load_me && io_ok && stage != nullptr)));
         uint32_t* pull = bam::pull_begin(pq);
+        [[maybe_unused]] const uint64_t pp0 = BAM_PROF_NOW();
         copy_pages_helped(cache.base_addr + (uint64_t)found * cache.page_size, stage, (uint32_t)cache.page_size, load_me && io_ok && stage != nullptr);
+#ifdef BAM_PROFILE
+        { const uint64_t pp1 = BAM_PROF_NOW(); if (cache.prof && bam::lane() == bam::first_lane(bam::active_mask())) { atomicAdd(&cache.prof[29], pp1 - pp0); atomicAdd(&cache.prof[30], (unsigned long long)bam::popc(bam::ballot(load_me && io_ok && stage != nullptr))); } }
+#endif
         bam::pull_end(pull);
     }
 #ifdef BAM_PROFILE
@@ -732,10 +764,10 @@ bool range_d_t<T>::slow_step(const size_t pg, const bool write, const uint32_t q
             bam::spin_t lk;
             bool locked = false;
             while (!locked) {
-                locked = __hip_atomic_exchange(&cp->page_take_lock, (uint32_t)LOCKED, __ATOMIC_RELAXED, BAM_AGENT) == UNLOCKED;
+                locked = (__hip_atomic_fetch_or(&cp->page_translation, (uint64_t)LOCKED << BAM_TAKE_SHIFT, __ATOMIC_RELAXED, BAM_AGENT) >> BAM_TAKE_SHIFT) == UNLOCKED;
                 if (!locked && cache.spin_giveup(lk)) break;
             }
-            if (locked) st_publish(&cp->page_take_lock, (uint32_t)FREE);
+            if (locked) st_relaxed(&cp->page_translation, (uint64_t)FREE << BAM_TAKE_SHIFT);
             fence_meta();
             __hip_atomic_fetch_and(&dp->state, DISABLE_BUSY_MASK, __ATOMIC_RELAXED, BAM_AGENT);
         } else {
@@ -1564,8 +1596,9 @@ static __global__ void __flush(page_cache_d_t* pc)
 {
     const uint64_t page = threadIdx.x + (uint64_t)blockIdx.x * blockDim.x;
     if (page >= pc->n_pages) return;
-    if (bam::ld_relaxed(&pc->cache_pages[page].page_take_lock) == FREE) return;
-    const uint64_t g = pc->cache_pages[page].page_translation;
+    const uint64_t w = bam::ld_relaxed(&pc->cache_pages[page].page_translation);
+    if ((w >> BAM_TAKE_SHIFT) & FREE) return;
+    const uint64_t g = w & BAM_TRANSLATION_MASK;
     const uint64_t range = g & pc->n_ranges_mask, addr = g >> pc->n_ranges_bits;
     data_page_t* dp = &pc->ranges[range][addr];
     const uint32_t s = bam::ld_relaxed(&dp->state);
@@ -1678,7 +1711,7 @@ struct page_cache_t {
         pdt.cache_pages = (cache_page_t*)cache_pages_buf.get();
         {
             std::vector<cache_page_t> tps(np);
-            for (size_t i = 0; i < np; i++) { tps[i].page_take_lock = FREE; tps[i].pad = 0; tps[i].page_translation = 0; }
+            for (size_t i = 0; i < np; i++) tps[i].page_translation = (uint64_t)FREE << BAM_TAKE_SHIFT;
             hip_err_chk(hipMemcpy(pdt.cache_pages, tps.data(), np * sizeof(cache_page_t), hipMemcpyHostToDevice));
         }
         page_ticket_buf = createBuffer(sizeof(uint32_t), hipDevice);

@@ -97,7 +97,7 @@ struct QueuePair
         cq.idle_ticks = cq_place == BAM_DMA_HOST ? BAM_CQ_IDLE_TICKS_DEFAULT : 0;
 
         /* device-side protocol state */
-        const uint32_t n_cids = qs < 64 ? 64 : qs;      /* handed out in blocks of 64, one block per wave */
+        const uint32_t n_cids = qs;                     /* a command's id is the submission slot it goes to */
         own->sq_tickets = createBuffer(qs * sizeof(padded_struct), hipDevice);
         own->sq_tail_mark = createBuffer(qs * sizeof(padded_struct), hipDevice);
         own->sq_cid = createBuffer(n_cids * sizeof(padded_struct), hipDevice);
@@ -105,10 +105,10 @@ struct QueuePair
         sq.tail_mark = (padded_struct*)own->sq_tail_mark.get();
         sq.cid = (padded_struct*)own->sq_cid.get();
         sq.cid_mask = n_cids - 1;
-        own->sq_cid_blocks = createBuffer((n_cids / 64) * sizeof(padded_struct), hipDevice);
-        sq.pos_locks = (padded_struct*)own->sq_cid_blocks.get();
-        own->sq_cid_left = createBuffer((n_cids / 64) * sizeof(padded_struct), hipDevice);
-        sq.head_mark = (padded_struct*)own->sq_cid_left.get();
+        own->sq_cid_blocks = createBuffer(sizeof(padded_struct), hipDevice);
+        sq.pos_locks = (padded_struct*)own->sq_cid_blocks.get();        /* unused */
+        own->sq_cid_left = createBuffer(qs * sizeof(padded_struct), hipDevice);
+        sq.head_mark = (padded_struct*)own->sq_cid_left.get();         /* per slot: the ticket get_cid reserved it with */
         cq.cid = sq.cid;
         cq.cid_mask = sq.cid_mask;
         sq.prof = cq.prof = prof;
