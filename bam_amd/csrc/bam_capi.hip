@@ -39,6 +39,13 @@ __global__ void k_array_read(array_d_t<uint64_t>* dr, uint64_t n_reqs, const uin
     block_accumulate(sum, v);
 }
 
+/* thread t hands out the element it read instead of adding it to a sum */
+__global__ void k_array_gather(array_d_t<uint64_t>* dr, uint64_t n_reqs, const uint64_t* assignment, uint64_t stride, uint64_t* out)
+{
+    const uint64_t tid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (tid < n_reqs) out[tid] = (*dr)[assignment ? assignment[tid] : tid * stride];
+}
+
 /*
  * The same read pattern through the other access routes of array_d_t:
  *   1  get_raw / release_raw            (the raw page handed out, lanes on one page share the references)
@@ -718,6 +725,18 @@ int bam_array_read(bam_array_t* a, uint64_t n_reqs, const uint64_t* d_assignment
     hipLaunchKernelGGL(k_array_read, dim3(blocks_for(n_reqs, block_size)), dim3(block_size), 0, (hipStream_t)stream,
                        a->a->d_array_ptr, n_reqs, d_assignment, stride, reqs_per_thread, (unsigned long long*)a->partials.get());
     hipLaunchKernelGGL(k_fold_partials, dim3(1), dim3(1024), 0, (hipStream_t)stream, (unsigned long long*)a->partials.get(), (unsigned long long*)d_sum);
+    hip_err_chk(hipGetLastError());
+    BAM_API_END
+}
+
+int bam_array_gather(bam_array_t* a, uint64_t n_reqs, const uint64_t* d_assignment, uint64_t stride, uint32_t block_size, uint64_t* d_out, void* stream)
+{
+    if (!a || !d_out) return fail(EINVAL, "bam_array_gather: null argument");
+    if (!block_size || block_size % BAM_WAVE_SIZE || block_size > 1024) return fail(EINVAL, "bam_array_gather: block size must be a multiple of 64, at most 1024");
+    if (!n_reqs) return 0;
+    BAM_API_BEGIN
+    hipLaunchKernelGGL(k_array_gather, dim3(blocks_for(n_reqs, block_size)), dim3(block_size), 0, (hipStream_t)stream,
+                       a->a->d_array_ptr, n_reqs, d_assignment, stride, d_out);
     hip_err_chk(hipGetLastError());
     BAM_API_END
 }

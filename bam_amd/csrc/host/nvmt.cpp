@@ -209,8 +209,6 @@ uint16_t do_rw(nvmt* t, Stats& st_, const nvm_cmd_t& c, bool write)
     if (c.dword[1] != 1) return ST_INVALID_FIELD;
     if (write && !t->cfg.backing) return ST_WRITE_RO;
     uint64_t done = 0;
-    static const bool no_payload = getenv("NVMT_EXPERIMENT_NO_PAYLOAD") != nullptr;
-    if (no_payload && !write) { st_.bump(st_.read_cmds); st_.bump(st_.bytes_read, bytes); return ST_OK; }
     alignas(64) uint64_t tmp[512];      /* sizeof(tmp) is the generation chunk */
     bool ok = for_each_prp(t, c, bytes, [&](uint64_t addr, uint64_t len) {
         uint8_t* p = (uint8_t*)addr;

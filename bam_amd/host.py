@@ -220,6 +220,12 @@ class Array:
         self.read_async(n_reqs, s, assignment, stride, reqs_per_thread, block_size)
         return int(s.item()) & MASK64
 
+    def gather(self, n_reqs, assignment=None, stride=1, block_size=64):
+        """The elements themselves: out[t] = element assignment[t] (or t * stride), an int64 tensor of bit patterns."""
+        out = torch.empty(n_reqs, dtype=torch.int64, device=f"cuda:{self.device}")
+        _chk(self.L.bam_array_gather(self.h, n_reqs, _ptr(assignment), stride, block_size, _ptr(out), _stream()), "bam_array_gather")
+        return out
+
     def read_via(self, api, n_reqs, assignment=None, span=1, block_size=64):
         """The read pattern through another access route of array_d_t (1 get_raw, 2 acquire_page_, 3 acquire_page,
         4 bam_ptr, 5 wave memcpy of up to `span` elements per request); sum of what was read."""

@@ -98,6 +98,9 @@ int bam_array_stats(bam_array_t* a, uint64_t* out, int reset);
  * (mod 2^64).  The reference discards the values; the checksum is what makes the result checkable. */
 int bam_array_read(bam_array_t* a, uint64_t n_reqs, const uint64_t* d_assignment, uint64_t stride, uint64_t reqs_per_thread,
                    uint32_t block_size, uint64_t* d_sum, void* stream);
+/* the same requests with the values handed out: d_out[t] = element d_assignment[t] (or t * stride); what a kernel of the
+ * reference's benchmark would hold in its register after array_d_t::operator[] (benchmarks/array/main.cu:57) */
+int bam_array_gather(bam_array_t* a, uint64_t n_reqs, const uint64_t* d_assignment, uint64_t stride, uint32_t block_size, uint64_t* d_out, void* stream);
 /* The read pattern of bam_array_read (one thread per request, element d_assignment[t] or t * span) through the other
  * access routes of array_d_t (include/page_cache.h:1240-1716, 414-485): api 1 get_raw/release_raw, 2 get_page_gid +
  * acquire_page_ + release_page, 3 acquire_page/release_page, 4 bam_ptr, 5 memcpy (one request per wave: up to `span`

@@ -230,6 +230,36 @@ __device__ __forceinline__ void ld_payload_stream16(const uint64_t* p, const uin
                  : "memory");
 }
 
+/*
+ * Sixteen bytes per lane at system scope, for moving payload between a staging page in host memory and a cache slot.
+ * The load is never served from a cache that remembers the staging page's last tenant, so nobody has to invalidate
+ * caches after a completion; the store goes through to memory, so the wave that moved a page in can publish it after
+ * a wait on its own store counter instead of a write-back of the whole L2.  Those two cache-wide operations, once per
+ * batch of commands, were what the miss path as a whole queued behind.  The compiler has no 16-byte access with a
+ * scope, hence the asm; what an asm load leaves in flight the compiler does not count, so the wait is spelt out and
+ * tied to the registers it is for.
+ */
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ u32x4_t ld16_sys(const void* p)
+{
+    u32x4_t v;
+    asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1" : "=v"(v) : "v"(p) : "memory");
+    return v;
+}
+__device__ __forceinline__ void wait_loads(u32x4_t& a, u32x4_t& b, u32x4_t& c, u32x4_t& d)
+{
+    asm volatile("s_waitcnt vmcnt(0)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d) :: "memory");
+}
+__device__ __forceinline__ void wait_loads(u32x4_t& a) { asm volatile("s_waitcnt vmcnt(0)" : "+v"(a) :: "memory"); }
+/* The two idle cycles after the store are part of it: a store of more than 8 bytes reads its data registers over the
+ * cycles that follow its issue, and a vector instruction that writes one of them in that window changes what is stored.
+ * The compiler keeps that distance for stores it emits itself, not for one inside an asm statement. */
+__device__ __forceinline__ void st16_sys(void* p, const u32x4_t v)
+{
+    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\ts_nop 1" :: "v"(p), "v"(v) : "memory");
+}
+__device__ __forceinline__ void wait_stores() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
 template <typename T> __device__ __forceinline__ T ld_payload(const T* p)
 {
     if constexpr (sizeof(T) == 8) { uint64_t v = __hip_atomic_load((const uint64_t*)p, __ATOMIC_RELAXED, BAM_AGENT); return *(T*)&v; }

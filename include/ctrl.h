@@ -178,7 +178,7 @@ private:
          * all its waves in order: while one wave waits for host memory, every other load of that unit waits with it.
          * With more pulls in flight than the interconnect needs to stay busy, each waits longer and so does everybody
          * else; the number of waves pulling at a time is therefore bounded (per cluster of compute units). */
-        pull_limit = 8;
+        pull_limit = 0;
         if (const char* e = getenv("BAM_PULL_LIMIT")) pull_limit = (uint32_t)atoi(e);
         own->pull_buff = createBuffer(8 * 64, deviceId);
         for (size_t i = 0; i < n_qps; i++) {

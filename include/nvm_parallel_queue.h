@@ -362,9 +362,10 @@ __device__ __forceinline__ bool cq_wait_group(nvm_queue_t* cq, nvm_queue_t* sq, 
         if (spin_giveup(cq, sp)) break;
     }
     if (lane() == first_lane(active_mask())) BAM_PROF_ADD(cq, 16, p_trips);
-    /* what the controller wrote before posting the completion is visible from here on: a staging page in host memory
-     * has had other tenants, and this compute unit's caches may remember them */
-    fence_acquire_sys();
+    /* What the controller wrote before posting the completion is in memory: staged payload in host memory, which
+     * copy_pages reads at system scope, or payload placed in a cache slot, which its readers load past the caches that
+     * could remember the slot's last tenant (bam::ld_payload).  No cache has to be invalidated for either. */
+    fence_meta();
     return (w & (BAM_CID_DONE | BAM_CID_ERR)) == BAM_CID_DONE;
 }
 

@@ -74,6 +74,10 @@ enum data_dist_t { REPLICATE = 0, STRIPE = 1 };
 #define BAM_SLOT_BITS 27u
 #define BAM_SLOT_MASK ((1u << BAM_SLOT_BITS) - 1u)
 
+/* batches smaller than this are never placed directly: the controller pushes a page into device memory in several
+ * microseconds, which a wave with a few commands waits for in full, while what it pulls itself is there in two */
+#define BAM_DIRECT_MIN_BATCH 24u
+
 #define BAM_TOKEN_SLOTS 4096u
 #define BAM_STAT_SHARDS 4096
 
@@ -185,17 +189,24 @@ __device__ __forceinline__ void copy_pages(uint8_t* dst, const uint8_t* src, uin
     const uint32_t movers = 1u << (31 - __builtin_clz(n));
     for (uint64_t m = act; m; m &= m - 1) {
         const uint32_t j = first_lane(m);
-        const uint4* s = (const uint4*)bcast((uint64_t)src, j);
-        uint4* d = (uint4*)bcast((uint64_t)dst, j);
+        const u32x4_t* s = (const u32x4_t*)bcast((uint64_t)src, j);
+        u32x4_t* d = (u32x4_t*)bcast((uint64_t)dst, j);
         const uint32_t nb = bcast(bytes, j) / 16;
         if (rank >= movers) continue;
+        /* system scope both ways (ld16_sys / st16_sys): nothing stale is read, and what is written is in memory when the
+         * wave's store counter says so */
         uint32_t i = rank;
         for (; i + 3 * movers < nb; i += 4 * movers) {
-            const uint4 x0 = s[i], x1 = s[i + movers], x2 = s[i + 2 * movers], x3 = s[i + 3 * movers];
-            d[i] = x0; d[i + movers] = x1; d[i + 2 * movers] = x2; d[i + 3 * movers] = x3;
+            u32x4_t x0 = ld16_sys(s + i), x1 = ld16_sys(s + i + movers), x2 = ld16_sys(s + i + 2 * movers), x3 = ld16_sys(s + i + 3 * movers);
+            wait_loads(x0, x1, x2, x3);
+            st16_sys(d + i, x0); st16_sys(d + i + movers, x1); st16_sys(d + i + 2 * movers, x2); st16_sys(d + i + 3 * movers, x3);
         }
-        for (; i < nb; i += movers) d[i] = s[i];
+        for (; i < nb; i += movers) { u32x4_t x = ld16_sys(s + i); wait_loads(x); st16_sys(d + i, x); }
     }
+    /* the compiler does not count stores issued from asm, and drops the counter wait of a later fence when it knows of
+     * nothing outstanding: wait here, so that what follows (publishing the page, releasing the staging slot) is ordered
+     * after the payload by the hardware and not by luck */
+    wait_stores();
 }
 /*
  * Permission to pull staged payload from host memory, taken by the wave (all active lanes call, one lane acts) before
@@ -292,7 +303,8 @@ __device__ __forceinline__ uint32_t io_submit_group(page_cache_d_t* pc, QueuePai
      * batches of eight to the controller (12.3 against 11.4 M reads/s), raw block reads do best all staged (12.8
      * against 11.7 M).
      */
-    const bool direct = pc->prp1 && (bytes > qp->stage_stride || (opcode == NVM_IO_READ && bytes >= 2048 && ((ticket >> 6) & 7u) < direct_share));
+    const bool direct = pc->prp1 && (bytes > qp->stage_stride ||
+                                     (opcode == NVM_IO_READ && bytes >= 2048 && n >= BAM_DIRECT_MIN_BATCH && ((ticket >> 6) & 7u) < direct_share));
     const bool staged = qp->stage && !direct;
     if (staged) {
         stage = qp->stage + (size_t)cid * qp->stage_stride;
@@ -300,7 +312,7 @@ __device__ __forceinline__ uint32_t io_submit_group(page_cache_d_t* pc, QueuePai
         if (bytes > qp->pageSize) prp2 = prp1 + qp->pageSize;         /* staging pages are contiguous: second controller page */
         if (opcode == NVM_IO_WRITE) {
             copy_pages(stage, pc->base_addr + pc_entry * pc->page_size, bytes, act, n, rank);
-            fence_release_sys();             /* plain stores to host memory: written back before the command goes out */
+            fence_meta();                    /* written through to host memory: there before the command goes out */
         }
     } else {
         prp1 = pc->prp1[pc_entry];
@@ -743,7 +755,10 @@ bool range_d_t<T>::slow_step(const size_t pg, const bool write, const uint32_t q
         [[maybe_unused]] const uint64_t pp0 = BAM_PROF_NOW();
         copy_pages_helped(cache.base_addr + (uint64_t)found * cache.page_size, stage, (uint32_t)cache.page_size, load_me && io_ok && stage != nullptr);
 #ifdef BAM_PROFILE
-        { const uint64_t pp1 = BAM_PROF_NOW(); if (cache.prof && bam::lane() == bam::first_lane(bam::active_mask())) { atomicAdd(&cache.prof[29], pp1 - pp0); atomicAdd(&cache.prof[30], (unsigned long long)bam::popc(bam::ballot(load_me && io_ok && stage != nullptr))); } }
+        {
+            const uint64_t pp1 = BAM_PROF_NOW(), pulled = bam::popc(bam::ballot(load_me && io_ok && stage != nullptr));
+            if (cache.prof && bam::lane() == bam::first_lane(bam::active_mask())) { atomicAdd(&cache.prof[29], pp1 - pp0); atomicAdd(&cache.prof[30], (unsigned long long)pulled); }
+        }
 #endif
         bam::pull_end(pull);
     }
@@ -776,12 +791,9 @@ bool range_d_t<T>::slow_step(const size_t pg, const bool write, const uint32_t q
             if (write) __hip_atomic_fetch_or(&dp->state, DIRTY, __ATOMIC_RELAXED, BAM_AGENT);
         }
     }
-    /* payload this wave (helpers included) moved in with plain stores has to be written back for the other
-     * compute units before the page shows as valid; payload the controller placed is in memory already */
-    if (bam::ballot(load_me && io_ok)) {
-        if (bam::ballot(load_me && io_ok && (stage != nullptr || !held))) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-        else fence_meta();
-    }
+    /* payload this wave (helpers included) moved in went through to memory (copy_pages): once the wave's store counter
+     * is down it is there for every compute unit; payload the controller placed is in memory already */
+    if (bam::ballot(load_me && io_ok)) fence_meta();
     if (load_me && io_ok) {
         /* BUSY -> 0 and VALID -> 1 in one step; publishes the payload and the offset */
         __hip_atomic_fetch_xor(&dp->state, DISABLE_BUSY_ENABLE_VALID, __ATOMIC_RELAXED, BAM_AGENT);
@@ -1723,7 +1735,7 @@ struct page_cache_t {
         if (const char* e = getenv("BAM_FAST_READS")) pdt.fast_reads = atoi(e) != 0;
         tokens_buf = createBuffer(BAM_TOKEN_SLOTS * 64, hipDevice);
         pdt.miss_tokens = (uint32_t*)tokens_buf.get();
-        pdt.miss_waves = 4;
+        pdt.miss_waves = 0;
         if (const char* e = getenv("BAM_MISS_WAVES")) pdt.miss_waves = (uint32_t)atoi(e);
         pdt.prof = ctrl.prof;
 

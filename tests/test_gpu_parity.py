@@ -143,6 +143,35 @@ def test_random_gather_with_eviction(bam, cache_pages, n_queues, depth, block):
         assert not r.c.aborted()
 
 
+@pytest.mark.parametrize("cache_pages,n_queues,depth,block", [(64, 4, 64, 64), (1024, 2, 16, 256), (4096, 16, 1024, 128)])
+def test_every_element_of_a_gather_and_of_an_update_under_eviction(bam, cache_pages, n_queues, depth, block):
+    """Element by element instead of a sum: 2^18 random reads through a cache that holds a fraction of the data, on queues so
+    shallow that a wave's misses go through them in rounds, and on deep ones.  Then the same requests as atomic adds of zero
+    (every page dirty, so every eviction is a write-back followed by a read into the same slot), the reads again, and adds
+    to distinct elements that must show up in a gather and, after a flush, in the store."""
+    n_elems, n = 1 << 22, 1 << 18
+    rng = np.random.default_rng(SEED)
+    with Rig(bam, n_elems * 8, backing=True, n_queues=n_queues, depth=depth) as r:
+        store = r.backing(n_elems)
+        store[:] = oracle.store(SEED, 0, n_elems)
+        model = store.copy()
+        a = r.array(n_elems, 4096, cache_pages)
+        idx = rng.integers(0, n_elems, n).astype(np.uint64)
+        d_idx, want = _dev(idx), model[idx.astype(np.int64)]
+        assert np.array_equal(_u64(a.gather(n, d_idx, block_size=block)), want)
+        assert np.array_equal(_u64(a.update(0, d_idx, _dev(np.zeros(n, dtype=np.uint64)), block_size=block)), want)
+        assert np.array_equal(_u64(a.gather(n, d_idx, block_size=block)), want)
+        didx = rng.permutation(n_elems)[:n].astype(np.uint64)
+        vals = rng.integers(1, 1 << 63, n).astype(np.uint64)
+        assert np.array_equal(_u64(a.update(0, _dev(didx), _dev(vals), block_size=block)), model[didx.astype(np.int64)])
+        model[didx.astype(np.int64)] += vals
+        assert np.array_equal(_u64(a.gather(n, _dev(didx), block_size=block)), model[didx.astype(np.int64)])
+        assert np.array_equal(_u64(a.gather(n, d_idx, block_size=block)), model[idx.astype(np.int64)])
+        r.objs[0][2].flush()
+        assert np.array_equal(r.backing(n_elems), model)
+        assert not r.c.aborted() and r.c.info()["error_completions"] == 0 and r.t.stats()["write_cmds"] > 0
+
+
 def test_ragged_and_empty_and_last_element(bam):
     n_elems = (1 << 16) + 37                 # last page partly used
     with Rig(bam, 1 << 20) as r:
