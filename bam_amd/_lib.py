@@ -48,6 +48,7 @@ SIGNATURES = {
     "bam_block_checksum": (c_int, [c_vp, c_u64, c_u32, c_vp, c_vp]),
     "bam_bfs": (c_int, [c_vp, c_vp, c_u64, c_u64, c_vp, c_u32, P(c_u32), c_vp]),
     "bam_cc": (c_int, [c_vp, c_vp, c_u64, c_vp, c_u32, P(c_u32), c_vp]),
+    "bam_array_set_graph": (c_int, [c_vp, c_vp, c_u64, c_vp]),
     "bam_array_gather": (c_int, [c_vp, c_u64, c_vp, c_u64, c_u32, c_vp, c_vp]),
     "bam_array_read_via": (c_int, [c_vp, c_int, c_u64, c_vp, c_u64, c_u32, c_vp, c_vp]),
     "bam_block_io_async": (c_int, [c_vp, c_vp, c_u64, c_u32, c_u32, c_vp, c_u32, c_vp]),
@@ -75,6 +76,8 @@ SIGNATURES = {
     "bam_gen_uniform": (c_int, [c_u64, c_u64, c_u64, c_u64, c_vp, c_vp, c_vp]),
     "bam_copy_kernel": (c_int, [c_vp, c_vp, c_u64, P(ctypes.c_float), c_vp]),
     "bam_read_kernel": (c_int, [c_vp, c_u64, P(ctypes.c_float), c_vp]),
+    "bam_atomic_pairs_kernel": (c_int, [c_vp, c_vp, c_u64, c_int, P(ctypes.c_float), c_vp]),
+    "bam_xcd_relay": (c_int, [c_vp, c_u64, c_u32, c_u32, c_u32, c_u32, c_u32, P(c_u64), c_vp]),
     "bam_gather_kernel": (c_int, [c_vp, c_vp, c_u64, P(ctypes.c_float), c_vp]),
     "bam_host_read_ceiling": (c_int, [c_u64, c_u32, P(ctypes.c_float)]),
     "bam_event_create": (c_int, [P(c_vp)]),

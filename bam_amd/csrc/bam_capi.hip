@@ -426,6 +426,67 @@ __global__ void k_gather8(const uint64_t* __restrict__ src, const uint64_t* __re
     const uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
     block_accumulate(partials, t < n ? src[idx[t]] : 0);
 }
+/* what a hit of the counted path costs the memory system: per request one 64-bit add that returns the old word and, once it
+ * is back, one add on the same word whose result nobody reads (take a reference, drop it), on words scattered by idx[] */
+template <int RETURNS>
+__global__ void k_atomic_pairs(unsigned long long* table, const uint64_t* __restrict__ idx, uint64_t n, unsigned long long* partials)
+{
+    const uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    unsigned long long v = 0;
+    if (t < n) {
+        unsigned long long* w = table + idx[t];
+        if (RETURNS) v = __hip_atomic_fetch_add(w, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        else __hip_atomic_fetch_add(w, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (v != ~0ull) __hip_atomic_fetch_add(w, ~0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    block_accumulate(partials, v);
+}
+
+/*
+ * Pages handed from one compute-unit cluster to the others.  The grid is one wave per workgroup, which the dispatcher
+ * deals out over the clusters in turn.  In round r the wave r % waves touches page r (a miss: the page is read into a
+ * slot that another page left a few rounds ago) and raises flag[r]; every other wave waits for the flag with a bounded
+ * spin, then reads elements of the page through array_d_t::operator[] and compares them with what the procedural store
+ * holds; the next round starts when all have reported.  out[0] elements that differed, out[1] waits given up,
+ * out[2] bit mask of the clusters that took part, out[3] reads checked.
+ */
+__global__ void k_xcd_relay(array_d_t<uint64_t>* dr, uint64_t seed, uint32_t n_pages, uint32_t rounds, uint32_t elems_per_page, uint32_t spin_limit,
+                            uint32_t* flag, uint32_t* done, unsigned long long* out)
+{
+    const uint32_t me = blockIdx.x, waves = gridDim.x, l = bam::lane();
+    if (l == 0) atomicOr(&out[2], 1ull << bam::xcc_id());
+    unsigned long long bad = 0, late = 0, checked = 0;
+    for (uint32_t r = 0; r < rounds; r++) {
+        const uint64_t first = (uint64_t)(r % n_pages) * elems_per_page;
+        if (me == r % waves) {
+            /* the wave before last round's readers are through: their reads of the slot's last tenant are over */
+            if (r) {
+                uint32_t spins = 0;
+                while (__hip_atomic_load(&done[r - 1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < waves - 1 && ++spins < spin_limit) __builtin_amdgcn_s_sleep(8);
+                late += spins >= spin_limit;
+            }
+            const uint64_t v = (*dr)[first + l];
+            bad += v != splitmix64(seed, first + l);
+            checked++;
+            bam::fence_meta();
+            if (l == 0) __hip_atomic_store(&flag[r], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        } else {
+            uint32_t spins = 0;
+            while (__hip_atomic_load(&flag[r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0 && ++spins < spin_limit) __builtin_amdgcn_s_sleep(8);
+            late += spins >= spin_limit;
+            for (uint32_t k = l; k < elems_per_page; k += 4 * BAM_WAVE_SIZE) {
+                const uint64_t v = (*dr)[first + k];
+                bad += v != splitmix64(seed, first + k);
+                checked++;
+            }
+            bam::fence_meta();
+            if (l == 0) __hip_atomic_fetch_add(&done[r], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+    atomicAdd(&out[0], bad); atomicAdd(&out[3], checked);
+    if (l == 0) atomicAdd(&out[1], late);
+}
+
 /* every wave pulls whole chunks of host-pinned memory into device memory, 16 bytes per lane per load */
 __global__ void k_host_pull(const uint4* __restrict__ host, uint4* __restrict__ dev, uint64_t n_chunks, uint32_t chunk16, uint64_t host_chunks)
 {
@@ -1138,6 +1199,39 @@ int bam_gather_kernel(const uint64_t* d_src, const uint64_t* d_idx, uint64_t n, 
     hip_err_chk(hipGetLastError());
     Event b(st);
     if (ms) *ms = (float)((b - a) / 1e3);
+    BAM_API_END
+}
+
+int bam_atomic_pairs_kernel(uint64_t* d_table, const uint64_t* d_idx, uint64_t n, int returns, float* ms, void* stream)
+{
+    if (!d_table || !d_idx || !n) return fail(EINVAL, "bam_atomic_pairs_kernel: bad argument");
+    BAM_API_BEGIN
+    hipStream_t st = (hipStream_t)stream;
+    BufferPtr partials = createBuffer(BAM_SUM_PARTIALS * sizeof(unsigned long long), 0);
+    Event a(st);
+    if (returns) hipLaunchKernelGGL(k_atomic_pairs<1>, dim3(blocks_for(n, 256)), dim3(256), 0, st, (unsigned long long*)d_table, d_idx, n, (unsigned long long*)partials.get());
+    else hipLaunchKernelGGL(k_atomic_pairs<0>, dim3(blocks_for(n, 256)), dim3(256), 0, st, (unsigned long long*)d_table, d_idx, n, (unsigned long long*)partials.get());
+    hip_err_chk(hipGetLastError());
+    Event b(st);
+    if (ms) *ms = (float)((b - a) / 1e3);
+    BAM_API_END
+}
+
+int bam_xcd_relay(bam_array_t* a, uint64_t seed, uint32_t page_bytes, uint32_t n_pages, uint32_t rounds, uint32_t n_waves, uint32_t spin_limit, uint64_t* out4, void* stream)
+{
+    if (!a || !out4 || page_bytes < 512 || !n_pages || !rounds || n_waves < 2 || n_waves > 256) return fail(EINVAL, "bam_xcd_relay: bad argument (2 to 256 waves)");
+    BAM_API_BEGIN
+    hipStream_t st = (hipStream_t)stream;
+    /* every wave must be running while the others wait for it: 256 workgroups of one wave fit the device many times over */
+    BufferPtr words = createBuffer((2ull * rounds) * sizeof(uint32_t) + 4 * sizeof(unsigned long long), 0);
+    hip_err_chk(hipMemsetAsync(words.get(), 0, (2ull * rounds) * sizeof(uint32_t) + 4 * sizeof(unsigned long long), st));
+    unsigned long long* out = (unsigned long long*)words.get();
+    uint32_t* flag = (uint32_t*)(out + 4);
+    const uint32_t per_page = page_bytes / (uint32_t)sizeof(uint64_t);
+    hipLaunchKernelGGL(k_xcd_relay, dim3(n_waves), dim3(BAM_WAVE_SIZE), 0, st, a->a->d_array_ptr, seed, n_pages, rounds, per_page, spin_limit ? spin_limit : 1u << 22, flag, flag + rounds, out);
+    hip_err_chk(hipGetLastError());
+    hip_err_chk(hipMemcpyAsync(out4, out, 4 * sizeof(uint64_t), hipMemcpyDeviceToHost, st));
+    hip_err_chk(hipStreamSynchronize(st));
     BAM_API_END
 }
 

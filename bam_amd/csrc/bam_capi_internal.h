@@ -4,6 +4,7 @@
 #define __BAM_CAPI_INTERNAL_H__
 #include "bam_amd.h"
 
+#include <memory>
 #include <hip/hip_runtime.h>
 #include <fcntl.h>
 #include <sys/mman.h>
@@ -50,7 +51,7 @@ struct bam_ctrl { Controller* c; };
 struct bam_page_cache { page_cache_t* pc; Controller* ctrl; };      /* ctrl: the first controller of the cache */
 struct bam_range { range_t<uint64_t>* r; };
 #define BAM_SUM_PARTIALS 4096
-struct bam_array { array_t<uint64_t>* a; BufferPtr partials; };
+struct bam_array { array_t<uint64_t>* a; BufferPtr partials; std::shared_ptr<void> graph; };      /* graph: what bam_array_set_graph prepared (bam_graph.hip) */
 struct bam_range32 { range_t<uint32_t>* r; };
 struct bam_array32 { array_t<uint32_t>* a; BufferPtr partials; };      /* partials: [BAM_SUM_PARTIALS] checksum shards, zero between launches */
 

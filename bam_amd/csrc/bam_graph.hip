@@ -621,36 +621,69 @@ __global__ void k_iota(unsigned long long* p, uint64_t n)
 extern "C" {
 
 namespace {
-/* the pieces of the long edge lists of a graph, listed once per call, and the counter that hands out the work of a sweep:
- * a list of d >= BAM_HEAVY_EDGES entries makes at most d / BAM_PIECE_EDGES + 1 <= 2 d / BAM_HEAVY_EDGES pieces */
-struct sweep_work {
-    BufferPtr buf, cnt;
-    heavy_piece_t* pieces;
-    unsigned long long* count;       /* [0] number of pieces, [1] next piece of work of the sweep */
+/* launch shape of the by-page graph kernels: pages per wave trip and number of waves, so that what the waves hold
+ * at any time stays under half of the cache */
+struct by_page_plan { uint64_t n_edges = 0, n_pages = 0; uint32_t epp = 0, ppw = 0, blocks = 0; BufferPtr first; };
+
+/* the end of a level: the device's `changed` word goes to the host through pinned memory, and it and the counter the next
+ * sweep takes its work from start the next level at zero.  One small launch instead of two copies and a fill. */
+__global__ void k_level_end(uint64_t* changed, unsigned long long* next_work, volatile uint64_t* host_flag)
+{
+    *host_flag = *changed;
+    *changed = 0;
+    *next_work = 0;
+}
+
+/*
+ * What the graph entry points need besides the graph, made once per graph (bam_array_set_graph) or, without that, once per
+ * call: the pieces of the long edge lists (a list of d >= BAM_HEAVY_EDGES entries makes at most d / BAM_PIECE_EDGES + 1 <=
+ * 2 d / BAM_HEAVY_EDGES pieces), the counter that hands out the work of a sweep, the `changed` word and its pinned copy,
+ * the first-vertex table of the by-page kernels, and the per-vertex buffers of the algorithms, which come when first asked for.
+ */
+struct graph_plan {
+    const uint64_t* offsets = nullptr;
+    uint64_t n_vertices = 0, n_edges = 0;
+    BufferPtr buf, words, host_words;
+    heavy_piece_t* pieces = nullptr;
+    unsigned long long* count = nullptr;     /* [0] number of pieces, [1] next piece of work of the sweep */
+    uint64_t* changed = nullptr;             /* device */
+    volatile uint64_t* host_flag = nullptr;  /* pinned host memory */
     uint64_t n_pieces = 0;
-    uint64_t group;                  /* vertices handed to a wave at a time */
-    uint64_t resident;               /* waves the device holds at a time */
-    sweep_work(uint64_t n_edges, uint64_t n_vertices, uint32_t coarse, const uint64_t* d_offsets, hipStream_t st)
+    uint64_t group = 512;                    /* vertices handed to a wave at a time */
+    uint64_t resident = 0;                   /* waves a sweep runs */
+    by_page_plan bp;
+    bool bp_built = false;
+    BufferPtr bytes_a, bytes_b, floats_a, floats_b, words_a;      /* per-vertex buffers: flags, PageRank's delta and residual, SSSP's new costs */
+
+    int build(bam_array_t* edges, const uint64_t* d_offsets, uint64_t nv, uint64_t other_cache_pages, hipStream_t st)
     {
+        offsets = d_offsets; n_vertices = nv; n_edges = edges->a->adt.n_elems;
         const uint64_t cap = 2 * (n_edges / BAM_HEAVY_EDGES) + 1;
         buf = createBuffer(cap * sizeof(heavy_piece_t), 0);
-        cnt = createBuffer(2 * sizeof(unsigned long long), 0);
+        words = createBuffer(64, 0);
+        host_words = createHostBuffer(64);
         pieces = (heavy_piece_t*)buf.get();
-        count = (unsigned long long*)cnt.get();
-        /* a group's lists are asked for as one batch of commands: a few hundred vertices make that batch large enough for the
-         * store path, and keep the one word all waves take their work from out of the way */
-        group = coarse > 512 ? coarse : 512;
+        count = (unsigned long long*)words.get();
+        changed = (uint64_t*)words.get() + 2;
+        host_flag = (volatile uint64_t*)host_words.get();
         int dev = 0, cus = 0;
         hip_err_chk(hipGetDevice(&dev));
         hip_err_chk(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
         resident = (uint64_t)cus * 16;
-        hip_err_chk(hipMemsetAsync(count, 0, 2 * sizeof(unsigned long long), st));
+        /* every lane of a running wave may hold a page of its own (its bam_ptr keeps the last one it read): more waves
+         * than the cache has pages for would wait for slots that only they can give back */
+        uint64_t cache_pages = edges->a->adt.n_ranges ? edges->a->h_ranges[0].cache.n_pages : 0;
+        if (other_cache_pages && other_cache_pages < cache_pages) cache_pages = other_cache_pages;
+        if (cache_pages && resident > cache_pages / BAM_WAVE_SIZE) resident = cache_pages / BAM_WAVE_SIZE;
+        if (resident < 2) resident = 2;
+        hip_err_chk(hipMemsetAsync(words.get(), 0, 64, st));
         hipLaunchKernelGGL(k_heavy_pieces, dim3(blocks_for(n_vertices, 256)), dim3(256), 0, st, d_offsets, n_vertices, pieces, count);
         hip_err_chk(hipGetLastError());
         unsigned long long n = 0;
         hip_err_chk(hipMemcpyAsync(&n, count, sizeof(n), hipMemcpyDeviceToHost, st));
         hip_err_chk(hipStreamSynchronize(st));
         n_pieces = n;
+        return 0;
     }
     /* workgroups of two waves for a sweep over `n_items` items in groups of `grp` */
     uint32_t blocks(uint64_t n_items, uint64_t grp) const
@@ -658,139 +691,23 @@ struct sweep_work {
         const uint64_t units = (n_pieces + BAM_PIECE_BUNDLE - 1) / BAM_PIECE_BUNDLE + (n_items + grp - 1) / grp;
         return (uint32_t)(((units < resident ? units : resident) + 1) / 2);
     }
-    void reset(hipStream_t st) { hip_err_chk(hipMemsetAsync(count + 1, 0, sizeof(unsigned long long), st)); }
+    unsigned long long* next_work() const { return count + 1; }
+    /* between sweeps `changed` and the work counter are zero; true if the sweep just queued on `st` changed anything */
+    bool level_end(hipStream_t st)
+    {
+        hipLaunchKernelGGL(k_level_end, dim3(1), dim3(1), 0, st, changed, count + 1, host_flag);
+        hip_err_chk(hipGetLastError());
+        hip_err_chk(hipStreamSynchronize(st));
+        return *host_flag != 0;
+    }
+    int by_page(bam_array_t* edges, hipStream_t st);
+    static void* sized(BufferPtr& b, uint64_t bytes) { if (!b) b = createBuffer(bytes ? bytes : 8, 0); return b.get(); }
 };
-} // namespace
 
-int bam_bfs(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t src, uint32_t* d_labels,
-            uint32_t coarse, uint32_t* iterations, void* stream)
+int graph_plan::by_page(bam_array_t* edges, hipStream_t st)
 {
-    if (!edges || !d_offsets || !d_labels) return fail(EINVAL, "bam_bfs: null argument");
-    if (src >= n_vertices || !coarse) return fail(EINVAL, "bam_bfs: source out of range or coarse = 0");
-    BAM_API_BEGIN
-    hipStream_t st = (hipStream_t)stream;
-    BufferPtr changed_buf = createBuffer(sizeof(uint64_t), 0);
-    uint64_t* changed_d = (uint64_t*)changed_buf.get();
-    const uint32_t zero = 0;
-    hip_err_chk(hipMemsetAsync(d_labels, 0xFF, n_vertices * sizeof(uint32_t), st));
-    hip_err_chk(hipMemcpyAsync(d_labels + src, &zero, sizeof(uint32_t), hipMemcpyHostToDevice, st));
-    const uint32_t threads = 128;
-    sweep_work work(edges->a->adt.n_elems, n_vertices, coarse, d_offsets, st);
-    uint32_t level = 0, iter = 0;
-    uint64_t changed_h;
-    do {
-        changed_h = 0;
-        hip_err_chk(hipMemcpyAsync(changed_d, &changed_h, sizeof(uint64_t), hipMemcpyHostToDevice, st));
-        work.reset(st);
-        hipLaunchKernelGGL(k_bfs_coalesce_coarse_ptr_pc, dim3(work.blocks(n_vertices, work.group)), dim3(threads), 0, st,
-                           edges->a->d_array_ptr, d_labels, level, n_vertices, d_offsets, changed_d, work.group, work.pieces, work.n_pieces, work.count + 1);
-        hip_err_chk(hipGetLastError());
-        iter++; level++;
-        hip_err_chk(hipMemcpyAsync(&changed_h, changed_d, sizeof(uint64_t), hipMemcpyDeviceToHost, st));
-        hip_err_chk(hipStreamSynchronize(st));
-    } while (changed_h);
-    if (iterations) *iterations = iter;
-    BAM_API_END
-}
-
-int bam_bfs_frontier(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t src, uint32_t* d_labels,
-                     uint32_t* iterations, void* stream)
-{
-    if (!edges || !d_offsets || !d_labels) return fail(EINVAL, "bam_bfs_frontier: null argument");
-    if (src >= n_vertices) return fail(EINVAL, "bam_bfs_frontier: source out of range");
-    if (n_vertices > 0xFFFFFFFFull) return fail(EINVAL, "bam_bfs_frontier: the queues hold 32-bit vertex numbers");
-    BAM_API_BEGIN
-    hipStream_t st = (hipStream_t)stream;
-    /* two queues of at most every vertex once (benchmarks/bfs/main.cu:1489-1492); the size of the next one is the reference's `changed` */
-    BufferPtr queue_a = createBuffer(n_vertices * sizeof(uint32_t), 0), queue_b = createBuffer(n_vertices * sizeof(uint32_t), 0);
-    BufferPtr size_buf = createBuffer(sizeof(unsigned long long), 0);
-    uint32_t* curr = (uint32_t*)queue_a.get();
-    uint32_t* next = (uint32_t*)queue_b.get();
-    unsigned long long* next_size = (unsigned long long*)size_buf.get();
-    const uint32_t zero = 0, src32 = (uint32_t)src;
-    hip_err_chk(hipMemsetAsync(d_labels, 0xFF, n_vertices * sizeof(uint32_t), st));
-    hip_err_chk(hipMemcpyAsync(d_labels + src, &zero, sizeof(uint32_t), hipMemcpyHostToDevice, st));
-    hip_err_chk(hipMemcpyAsync(curr, &src32, sizeof(uint32_t), hipMemcpyHostToDevice, st));
-    const uint32_t threads = 128;
-    uint64_t group = BAM_WAVE_SIZE;                 /* queue entries handed to a wave at a time: one per lane, more of a sorted queue */
-    bool sorted = true;                             /* the first queue holds the source alone */
-    sweep_work work(edges->a->adt.n_elems, n_vertices, 1, d_offsets, st);
-    uint32_t level = 0, iter = 0;
-    unsigned long long active = 1;
-    const char* e = getenv("BAM_FRONTIER_SORT");
-    const bool sort_queue = !e || atoi(e) != 0;
-    int vertex_bits = 1;
-    while (vertex_bits < 32 && (1ull << vertex_bits) < n_vertices) vertex_bits++;
-    size_t sort_bytes = 0;
-    if (sort_queue) hip_err_chk(hipcub::DeviceRadixSort::SortKeys(nullptr, sort_bytes, curr, next, (int)std::min<uint64_t>(n_vertices, 0x7FFFFFFFull), 0, vertex_bits, st));
-    BufferPtr sort_tmp = createBuffer(sort_bytes ? sort_bytes : 8, 0);
-    do {
-        hip_err_chk(hipMemsetAsync(next_size, 0, sizeof(unsigned long long), st));
-        work.reset(st);
-        hipLaunchKernelGGL(k_bfs_frontier_coalesce_ptr_pc, dim3(work.blocks(active, group)), dim3(threads), 0, st, edges->a->d_array_ptr, d_labels, level,
-                           d_offsets, curr, (uint64_t)active, next, next_size, group, work.pieces, work.n_pieces, work.count + 1, sorted);
-        hip_err_chk(hipGetLastError());
-        iter++; level++;
-        hip_err_chk(hipMemcpyAsync(&active, next_size, sizeof(unsigned long long), hipMemcpyDeviceToHost, st));
-        hip_err_chk(hipStreamSynchronize(st));
-        sorted = sort_queue && active <= 0x7FFFFFFFull;
-        group = sorted ? work.group : BAM_WAVE_SIZE;
-        if (sorted && active > 1) {
-            /* the queue comes out in the order of discovery; sorted by vertex, the level reads the edge array front to back
-             * (neighbouring lists share pages, a page is not evicted between two of its lists, and the pages under the
-             * lists of a group of entries can be asked for together as in the sweep over all vertices).  The sorted queue
-             * goes into the buffer the level just walked, so the two do not change places. */
-            size_t need = sort_bytes;
-            hip_err_chk(hipcub::DeviceRadixSort::SortKeys(sort_tmp.get(), need, next, curr, (int)active, 0, vertex_bits, st));
-        } else
-            std::swap(curr, next);
-    } while (active);
-    if (iterations) *iterations = iter;
-    BAM_API_END
-}
-
-int bam_cc(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t* d_labels,
-           uint32_t coarse, uint32_t* iterations, void* stream)
-{
-    if (!edges || !d_offsets || !d_labels) return fail(EINVAL, "bam_cc: null argument");
-    if (!coarse || !n_vertices) return fail(EINVAL, "bam_cc: empty graph or coarse = 0");
-    BAM_API_BEGIN
-    hipStream_t st = (hipStream_t)stream;
-    BufferPtr visit_a = createBuffer(n_vertices, 0), visit_b = createBuffer(n_vertices, 0), changed_buf = createBuffer(sizeof(uint64_t), 0);
-    bool* curr = (bool*)visit_a.get();
-    bool* next = (bool*)visit_b.get();
-    bool* changed_d = (bool*)changed_buf.get();
-    hipLaunchKernelGGL(k_iota, dim3(blocks_for(n_vertices, 256)), dim3(256), 0, st, (unsigned long long*)d_labels, n_vertices);
-    hip_err_chk(hipMemsetAsync(curr, 0x01, n_vertices, st));
-    hip_err_chk(hipMemsetAsync(next, 0x00, n_vertices, st));
-    const uint32_t threads = 128;
-    sweep_work work(edges->a->adt.n_elems, n_vertices, coarse, d_offsets, st);
-    uint32_t iter = 0;
-    bool changed_h;
-    do {
-        changed_h = false;
-        hip_err_chk(hipMemcpyAsync(changed_d, &changed_h, sizeof(bool), hipMemcpyHostToDevice, st));
-        work.reset(st);
-        hipLaunchKernelGGL(k_cc_coalesce_coarse_ptr_pc, dim3(work.blocks(n_vertices, work.group)), dim3(threads), 0, st, edges->a->d_array_ptr, curr, next,
-                           n_vertices, d_offsets, (unsigned long long*)d_labels, changed_d, work.group, work.pieces, work.n_pieces, work.count + 1, iter);
-        hip_err_chk(hipGetLastError());
-        hip_err_chk(hipMemsetAsync(curr, 0x00, n_vertices, st));
-        bool* t = curr; curr = next; next = t;
-        iter++;
-        hip_err_chk(hipMemcpyAsync(&changed_h, changed_d, sizeof(bool), hipMemcpyDeviceToHost, st));
-        hip_err_chk(hipStreamSynchronize(st));
-    } while (changed_h);
-    if (iterations) *iterations = iter;
-    BAM_API_END
-}
-
-namespace {
-/* launch shape of the by-page graph kernels: pages per wave trip and number of waves, so that what the waves hold
- * at any time stays under half of the cache */
-struct by_page_plan { uint64_t n_edges, n_pages; uint32_t epp, ppw, blocks; BufferPtr first; };
-
-int plan_by_page(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, hipStream_t st, by_page_plan& pl)
-{
+    if (bp_built) return 0;
+    by_page_plan& pl = bp;
     array_t<uint64_t>* a = edges->a;
     if (a->adt.n_ranges != 1) return fail(EINVAL, "by-page graph kernels take an array of one range");
     const range_d_t<uint64_t>& r = a->h_ranges[0];
@@ -814,12 +731,157 @@ int plan_by_page(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_verti
     pl.ppw = (uint32_t)ppw;
     pl.blocks = (uint32_t)waves;                               /* one wave per workgroup */
     pl.first = createBuffer((pl.n_pages + 1) * sizeof(uint64_t), dev);
-    hipLaunchKernelGGL(k_page_first_vertex, dim3(blocks_for(pl.n_pages + 1, 256)), dim3(256), 0, st, d_offsets, n_vertices, (uint64_t)pl.epp, pl.n_pages,
+    hipLaunchKernelGGL(k_page_first_vertex, dim3(blocks_for(pl.n_pages + 1, 256)), dim3(256), 0, st, offsets, n_vertices, (uint64_t)pl.epp, pl.n_pages,
                        (uint64_t*)pl.first.get());
     hip_err_chk(hipGetLastError());
+    bp_built = true;
     return 0;
 }
+
+/* the plan bam_array_set_graph made for this graph, or one made now in `local` that lives for the call */
+graph_plan* plan_for(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t other_cache_pages, hipStream_t st, std::unique_ptr<graph_plan>& local)
+{
+    graph_plan* p = (graph_plan*)edges->graph.get();
+    if (p && p->offsets == d_offsets && p->n_vertices == n_vertices && p->n_edges == edges->a->adt.n_elems && !other_cache_pages) return p;
+    local.reset(new graph_plan());
+    local->build(edges, d_offsets, n_vertices, other_cache_pages, st);
+    return local.get();
+}
 } // namespace
+
+int bam_array_set_graph(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, void* stream)
+{
+    if (!edges) return fail(EINVAL, "bam_array_set_graph: null argument");
+    if (!d_offsets) { edges->graph.reset(); return 0; }
+    if (!n_vertices) return fail(EINVAL, "bam_array_set_graph: empty graph");
+    BAM_API_BEGIN
+    hipStream_t st = (hipStream_t)stream;
+    std::shared_ptr<graph_plan> p(new graph_plan());
+    p->build(edges, d_offsets, n_vertices, 0, st);
+    if (edges->a->adt.n_ranges == 1) {
+        const range_d_t<uint64_t>& r = edges->a->h_ranges[0];
+        if (r.index_start == 0 && r.page_start_offset % r.cache.page_size == 0 && r.cache.n_pages >= 2) p->by_page(edges, st);
+    }
+    /* the per-vertex buffers the sweeps use, so that no later call has to allocate */
+    graph_plan::sized(p->bytes_a, n_vertices); graph_plan::sized(p->bytes_b, n_vertices);
+    graph_plan::sized(p->floats_a, n_vertices * sizeof(float)); graph_plan::sized(p->floats_b, n_vertices * sizeof(float));
+    hip_err_chk(hipStreamSynchronize(st));
+    edges->graph = p;
+    BAM_API_END
+}
+
+int bam_bfs(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t src, uint32_t* d_labels,
+            uint32_t coarse, uint32_t* iterations, void* stream)
+{
+    if (!edges || !d_offsets || !d_labels) return fail(EINVAL, "bam_bfs: null argument");
+    if (src >= n_vertices || !coarse) return fail(EINVAL, "bam_bfs: source out of range or coarse = 0");
+    BAM_API_BEGIN
+    hipStream_t st = (hipStream_t)stream;
+    std::unique_ptr<graph_plan> local;
+    graph_plan* pl = plan_for(edges, d_offsets, n_vertices, 0, st, local);
+    /* a group's lists are asked for as one batch of commands: a few hundred vertices make that batch large enough for the
+     * store path, and keep the one word all waves take their work from out of the way */
+    const uint64_t group = coarse > 512 ? coarse : 512;
+    hip_err_chk(hipMemsetAsync(d_labels, 0xFF, n_vertices * sizeof(uint32_t), st));
+    hip_err_chk(hipMemsetAsync(d_labels + src, 0, sizeof(uint32_t), st));
+    const uint32_t threads = 128;
+    uint32_t level = 0, iter = 0;
+    bool changed;
+    do {
+        hipLaunchKernelGGL(k_bfs_coalesce_coarse_ptr_pc, dim3(pl->blocks(n_vertices, group)), dim3(threads), 0, st,
+                           edges->a->d_array_ptr, d_labels, level, n_vertices, d_offsets, pl->changed, group, pl->pieces, pl->n_pieces, pl->next_work());
+        hip_err_chk(hipGetLastError());
+        iter++; level++;
+        changed = pl->level_end(st);
+    } while (changed);
+    if (iterations) *iterations = iter;
+    BAM_API_END
+}
+
+int bam_bfs_frontier(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t src, uint32_t* d_labels,
+                     uint32_t* iterations, void* stream)
+{
+    if (!edges || !d_offsets || !d_labels) return fail(EINVAL, "bam_bfs_frontier: null argument");
+    if (src >= n_vertices) return fail(EINVAL, "bam_bfs_frontier: source out of range");
+    if (n_vertices > 0xFFFFFFFFull) return fail(EINVAL, "bam_bfs_frontier: the queues hold 32-bit vertex numbers");
+    BAM_API_BEGIN
+    hipStream_t st = (hipStream_t)stream;
+    std::unique_ptr<graph_plan> local;
+    graph_plan* pl = plan_for(edges, d_offsets, n_vertices, 0, st, local);
+    /* two queues of at most every vertex once (benchmarks/bfs/main.cu:1489-1492); the size of the next one is the reference's `changed` */
+    BufferPtr queue_a = createBuffer(n_vertices * sizeof(uint32_t), 0), queue_b = createBuffer(n_vertices * sizeof(uint32_t), 0);
+    uint32_t* curr = (uint32_t*)queue_a.get();
+    uint32_t* next = (uint32_t*)queue_b.get();
+    unsigned long long* next_size = (unsigned long long*)pl->changed;
+    const uint32_t src32 = (uint32_t)src;
+    hip_err_chk(hipMemsetAsync(d_labels, 0xFF, n_vertices * sizeof(uint32_t), st));
+    hip_err_chk(hipMemsetAsync(d_labels + src, 0, sizeof(uint32_t), st));
+    hip_err_chk(hipMemcpyAsync(curr, &src32, sizeof(uint32_t), hipMemcpyHostToDevice, st));
+    const uint32_t threads = 128;
+    uint64_t group = BAM_WAVE_SIZE;                 /* queue entries handed to a wave at a time: one per lane, more of a sorted queue */
+    bool sorted = true;                             /* the first queue holds the source alone */
+    uint32_t level = 0, iter = 0;
+    unsigned long long active = 1;
+    const char* e = getenv("BAM_FRONTIER_SORT");
+    const bool sort_queue = !e || atoi(e) != 0;
+    int vertex_bits = 1;
+    while (vertex_bits < 32 && (1ull << vertex_bits) < n_vertices) vertex_bits++;
+    size_t sort_bytes = 0;
+    if (sort_queue) hip_err_chk(hipcub::DeviceRadixSort::SortKeys(nullptr, sort_bytes, curr, next, (int)std::min<uint64_t>(n_vertices, 0x7FFFFFFFull), 0, vertex_bits, st));
+    BufferPtr sort_tmp = createBuffer(sort_bytes ? sort_bytes : 8, 0);
+    do {
+        hipLaunchKernelGGL(k_bfs_frontier_coalesce_ptr_pc, dim3(pl->blocks(active, group)), dim3(threads), 0, st, edges->a->d_array_ptr, d_labels, level,
+                           d_offsets, curr, (uint64_t)active, next, next_size, group, pl->pieces, pl->n_pieces, pl->next_work(), sorted);
+        hip_err_chk(hipGetLastError());
+        iter++; level++;
+        pl->level_end(st);
+        active = *pl->host_flag;
+        sorted = sort_queue && active <= 0x7FFFFFFFull;
+        group = sorted ? pl->group : BAM_WAVE_SIZE;
+        if (sorted && active > 1) {
+            /* the queue comes out in the order of discovery; sorted by vertex, the level reads the edge array front to back
+             * (neighbouring lists share pages, a page is not evicted between two of its lists, and the pages under the
+             * lists of a group of entries can be asked for together as in the sweep over all vertices).  The sorted queue
+             * goes into the buffer the level just walked, so the two do not change places. */
+            size_t need = sort_bytes;
+            hip_err_chk(hipcub::DeviceRadixSort::SortKeys(sort_tmp.get(), need, next, curr, (int)active, 0, vertex_bits, st));
+        } else
+            std::swap(curr, next);
+    } while (active);
+    if (iterations) *iterations = iter;
+    BAM_API_END
+}
+
+int bam_cc(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t* d_labels,
+           uint32_t coarse, uint32_t* iterations, void* stream)
+{
+    if (!edges || !d_offsets || !d_labels) return fail(EINVAL, "bam_cc: null argument");
+    if (!coarse || !n_vertices) return fail(EINVAL, "bam_cc: empty graph or coarse = 0");
+    BAM_API_BEGIN
+    hipStream_t st = (hipStream_t)stream;
+    std::unique_ptr<graph_plan> local;
+    graph_plan* pl = plan_for(edges, d_offsets, n_vertices, 0, st, local);
+    const uint64_t group = coarse > 512 ? coarse : 512;
+    bool* curr = (bool*)graph_plan::sized(pl->bytes_a, n_vertices);
+    bool* next = (bool*)graph_plan::sized(pl->bytes_b, n_vertices);
+    hipLaunchKernelGGL(k_iota, dim3(blocks_for(n_vertices, 256)), dim3(256), 0, st, (unsigned long long*)d_labels, n_vertices);
+    hip_err_chk(hipMemsetAsync(curr, 0x01, n_vertices, st));
+    hip_err_chk(hipMemsetAsync(next, 0x00, n_vertices, st));
+    const uint32_t threads = 128;
+    uint32_t iter = 0;
+    bool changed;
+    do {
+        hipLaunchKernelGGL(k_cc_coalesce_coarse_ptr_pc, dim3(pl->blocks(n_vertices, group)), dim3(threads), 0, st, edges->a->d_array_ptr, curr, next,
+                           n_vertices, d_offsets, (unsigned long long*)d_labels, (bool*)pl->changed, group, pl->pieces, pl->n_pieces, pl->next_work(), iter);
+        hip_err_chk(hipGetLastError());
+        hip_err_chk(hipMemsetAsync(curr, 0x00, n_vertices, st));
+        bool* t = curr; curr = next; next = t;
+        iter++;
+        changed = pl->level_end(st);
+    } while (changed);
+    if (iterations) *iterations = iter;
+    BAM_API_END
+}
 
 int bam_bfs_by_page(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t src, uint32_t* d_labels,
                     uint32_t* iterations, void* stream)
@@ -828,26 +890,21 @@ int bam_bfs_by_page(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_ve
     if (src >= n_vertices) return fail(EINVAL, "bam_bfs_by_page: source out of range");
     BAM_API_BEGIN
     hipStream_t st = (hipStream_t)stream;
-    by_page_plan pl;
-    if (int rc = plan_by_page(edges, d_offsets, n_vertices, st, pl)) return rc;
-    BufferPtr changed_buf = createBuffer(sizeof(uint64_t), 0);
-    uint64_t* changed_d = (uint64_t*)changed_buf.get();
-    const uint32_t zero = 0;
+    std::unique_ptr<graph_plan> local;
+    graph_plan* pl = plan_for(edges, d_offsets, n_vertices, 0, st, local);
+    if (int rc = pl->by_page(edges, st)) return rc;
     hip_err_chk(hipMemsetAsync(d_labels, 0xFF, n_vertices * sizeof(uint32_t), st));
-    hip_err_chk(hipMemcpyAsync(d_labels + src, &zero, sizeof(uint32_t), hipMemcpyHostToDevice, st));
+    hip_err_chk(hipMemsetAsync(d_labels + src, 0, sizeof(uint32_t), st));
     uint32_t level = 0, iter = 0;
-    uint64_t changed_h;
+    bool changed;
     do {
-        changed_h = 0;
-        hip_err_chk(hipMemcpyAsync(changed_d, &changed_h, sizeof(uint64_t), hipMemcpyHostToDevice, st));
-        if (pl.n_pages)
-            hipLaunchKernelGGL(k_bfs_by_page, dim3(pl.blocks), dim3(BAM_WAVE_SIZE), 0, st, edges->a->d_array_ptr, d_labels, level, d_offsets,
-                               (const uint64_t*)pl.first.get(), pl.n_edges, pl.ppw, changed_d);
+        if (pl->bp.n_pages)
+            hipLaunchKernelGGL(k_bfs_by_page, dim3(pl->bp.blocks), dim3(BAM_WAVE_SIZE), 0, st, edges->a->d_array_ptr, d_labels, level, d_offsets,
+                               (const uint64_t*)pl->bp.first.get(), pl->bp.n_edges, pl->bp.ppw, pl->changed);
         hip_err_chk(hipGetLastError());
         iter++; level++;
-        hip_err_chk(hipMemcpyAsync(&changed_h, changed_d, sizeof(uint64_t), hipMemcpyDeviceToHost, st));
-        hip_err_chk(hipStreamSynchronize(st));
-    } while (changed_h);
+        changed = pl->level_end(st);
+    } while (changed);
     if (iterations) *iterations = iter;
     BAM_API_END
 }
@@ -858,30 +915,26 @@ int bam_cc_by_page(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_ver
     if (!n_vertices) return fail(EINVAL, "bam_cc_by_page: empty graph");
     BAM_API_BEGIN
     hipStream_t st = (hipStream_t)stream;
-    by_page_plan pl;
-    if (int rc = plan_by_page(edges, d_offsets, n_vertices, st, pl)) return rc;
-    BufferPtr visit_a = createBuffer(n_vertices, 0), visit_b = createBuffer(n_vertices, 0), changed_buf = createBuffer(sizeof(uint64_t), 0);
-    bool* curr = (bool*)visit_a.get();
-    bool* next = (bool*)visit_b.get();
-    bool* changed_d = (bool*)changed_buf.get();
+    std::unique_ptr<graph_plan> local;
+    graph_plan* pl = plan_for(edges, d_offsets, n_vertices, 0, st, local);
+    if (int rc = pl->by_page(edges, st)) return rc;
+    bool* curr = (bool*)graph_plan::sized(pl->bytes_a, n_vertices);
+    bool* next = (bool*)graph_plan::sized(pl->bytes_b, n_vertices);
     hipLaunchKernelGGL(k_iota, dim3(blocks_for(n_vertices, 256)), dim3(256), 0, st, (unsigned long long*)d_labels, n_vertices);
     hip_err_chk(hipMemsetAsync(curr, 0x01, n_vertices, st));
     hip_err_chk(hipMemsetAsync(next, 0x00, n_vertices, st));
     uint32_t iter = 0;
-    bool changed_h;
+    bool changed;
     do {
-        changed_h = false;
-        hip_err_chk(hipMemcpyAsync(changed_d, &changed_h, sizeof(bool), hipMemcpyHostToDevice, st));
-        if (pl.n_pages)
-            hipLaunchKernelGGL(k_cc_by_page, dim3(pl.blocks), dim3(BAM_WAVE_SIZE), 0, st, edges->a->d_array_ptr, curr, next, d_offsets,
-                               (const uint64_t*)pl.first.get(), pl.n_edges, pl.ppw, iter, (unsigned long long*)d_labels, changed_d);
+        if (pl->bp.n_pages)
+            hipLaunchKernelGGL(k_cc_by_page, dim3(pl->bp.blocks), dim3(BAM_WAVE_SIZE), 0, st, edges->a->d_array_ptr, curr, next, d_offsets,
+                               (const uint64_t*)pl->bp.first.get(), pl->bp.n_edges, pl->bp.ppw, iter, (unsigned long long*)d_labels, (bool*)pl->changed);
         hip_err_chk(hipGetLastError());
         hip_err_chk(hipMemsetAsync(curr, 0x00, n_vertices, st));
         bool* t = curr; curr = next; next = t;
         iter++;
-        hip_err_chk(hipMemcpyAsync(&changed_h, changed_d, sizeof(bool), hipMemcpyDeviceToHost, st));
-        hip_err_chk(hipStreamSynchronize(st));
-    } while (changed_h);
+        changed = pl->level_end(st);
+    } while (changed);
     if (iterations) *iterations = iter;
     BAM_API_END
 }
@@ -894,40 +947,31 @@ int bam_pagerank(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_verti
     if (!n_vertices) return 0;
     BAM_API_BEGIN
     hipStream_t st = (hipStream_t)stream;
-    BufferPtr delta = createBuffer(n_vertices * sizeof(float), 0), residual = createBuffer(n_vertices * sizeof(float), 0),
-              label = createBuffer(n_vertices, 0), changed_buf = createBuffer(sizeof(uint64_t), 0);
-    float* delta_d = (float*)delta.get();
-    float* residual_d = (float*)residual.get();
-    bool* label_d = (bool*)label.get();
-    bool* changed_d = (bool*)changed_buf.get();
-    by_page_plan pl{};
+    std::unique_ptr<graph_plan> local;
+    graph_plan* pl = plan_for(edges, d_offsets, n_vertices, 0, st, local);
     if (by_page)
-        if (int rc = plan_by_page(edges, d_offsets, n_vertices, st, pl)) return rc;
+        if (int rc = pl->by_page(edges, st)) return rc;
+    float* delta_d = (float*)graph_plan::sized(pl->floats_a, n_vertices * sizeof(float));
+    float* residual_d = (float*)graph_plan::sized(pl->floats_b, n_vertices * sizeof(float));
+    bool* label_d = (bool*)graph_plan::sized(pl->bytes_a, n_vertices);
     const uint32_t upd_blocks = blocks_for(n_vertices, 256);
-    sweep_work work(edges->a->adt.n_elems, n_vertices, 1, d_offsets, st);
     hipLaunchKernelGGL(k_pr_initialize, dim3(upd_blocks), dim3(256), 0, st, label_d, delta_d, residual_d, d_value, n_vertices, d_offsets, alpha);
     uint32_t iter = 0;
-    bool changed_h;
+    bool changed;
     do {
-        changed_h = false;
-        hip_err_chk(hipMemcpyAsync(changed_d, &changed_h, sizeof(bool), hipMemcpyHostToDevice, st));
         if (by_page) {
-            if (pl.n_pages)
-                hipLaunchKernelGGL(k_pr_by_page, dim3(pl.blocks), dim3(BAM_WAVE_SIZE), 0, st, edges->a->d_array_ptr, label_d, delta_d, residual_d, d_offsets,
-                                   (const uint64_t*)pl.first.get(), pl.n_edges, pl.ppw, iter);
-            hip_err_chk(hipMemsetAsync(label_d, 0, n_vertices, st));
-        } else {
-            work.reset(st);
-            hipLaunchKernelGGL(k_pr_coalesce_pc, dim3(work.blocks(n_vertices, work.group)), dim3(128), 0, st, edges->a->d_array_ptr, label_d, delta_d, residual_d,
-                               n_vertices, d_offsets, work.group, work.pieces, work.n_pieces, work.count + 1, iter);
-            hip_err_chk(hipMemsetAsync(label_d, 0, n_vertices, st));
-        }
+            if (pl->bp.n_pages)
+                hipLaunchKernelGGL(k_pr_by_page, dim3(pl->bp.blocks), dim3(BAM_WAVE_SIZE), 0, st, edges->a->d_array_ptr, label_d, delta_d, residual_d, d_offsets,
+                                   (const uint64_t*)pl->bp.first.get(), pl->bp.n_edges, pl->bp.ppw, iter);
+        } else
+            hipLaunchKernelGGL(k_pr_coalesce_pc, dim3(pl->blocks(n_vertices, pl->group)), dim3(128), 0, st, edges->a->d_array_ptr, label_d, delta_d, residual_d,
+                               n_vertices, d_offsets, pl->group, pl->pieces, pl->n_pieces, pl->next_work(), iter);
+        hip_err_chk(hipMemsetAsync(label_d, 0, n_vertices, st));
         iter++;
-        hipLaunchKernelGGL(k_pr_update, dim3(upd_blocks), dim3(256), 0, st, label_d, delta_d, residual_d, d_value, n_vertices, d_offsets, tolerance, alpha, changed_d);
+        hipLaunchKernelGGL(k_pr_update, dim3(upd_blocks), dim3(256), 0, st, label_d, delta_d, residual_d, d_value, n_vertices, d_offsets, tolerance, alpha, (bool*)pl->changed);
         hip_err_chk(hipGetLastError());
-        hip_err_chk(hipMemcpyAsync(&changed_h, changed_d, sizeof(bool), hipMemcpyDeviceToHost, st));
-        hip_err_chk(hipStreamSynchronize(st));
-    } while (changed_h && iter < max_iterations);
+        changed = pl->level_end(st);
+    } while (changed && iter < max_iterations);
     if (iterations) *iterations = iter;
     BAM_API_END
 }
@@ -938,10 +982,12 @@ namespace {
 void sssp_run(const bool FLOAT, bam_array_t* edges, bam_array32_t* weights, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t src, uint32_t* d_costs,
               uint32_t* iterations, hipStream_t st)
 {
-    BufferPtr new_cost = createBuffer(n_vertices * sizeof(uint32_t), 0), label = createBuffer(n_vertices, 0), changed_buf = createBuffer(sizeof(uint64_t), 0);
-    uint32_t* new_d = (uint32_t*)new_cost.get();
-    bool* label_d = (bool*)label.get();
-    bool* changed_d = (bool*)changed_buf.get();
+    /* a lane holds a page of the weights beside its page of the edges: the waves a sweep runs must fit the smaller cache too */
+    const uint64_t weight_pages = weights->a->adt.n_ranges ? weights->a->h_ranges[0].cache.n_pages : 0;
+    std::unique_ptr<graph_plan> local;
+    graph_plan* pl = plan_for(edges, d_offsets, n_vertices, weight_pages ? weight_pages : 1, st, local);
+    uint32_t* new_d = (uint32_t*)graph_plan::sized(pl->words_a, n_vertices * sizeof(uint32_t));
+    bool* label_d = (bool*)graph_plan::sized(pl->bytes_a, n_vertices);
     const uint32_t zero = 0;                    /* the pattern of 0.0f as well */
     const bool one = true;
     const float far = 1000000000.0f;
@@ -954,22 +1000,17 @@ void sssp_run(const bool FLOAT, bam_array_t* edges, bam_array32_t* weights, cons
     hip_err_chk(hipMemcpyAsync(d_costs + src, &zero, sizeof(uint32_t), hipMemcpyHostToDevice, st));
     hip_err_chk(hipMemcpyAsync(new_d + src, &zero, sizeof(uint32_t), hipMemcpyHostToDevice, st));
     const uint32_t threads = 128;
-    sweep_work work(edges->a->adt.n_elems, n_vertices, 1, d_offsets, st);
     uint32_t iter = 0;
-    bool changed_h;
+    bool changed;
     do {
-        changed_h = false;
-        hip_err_chk(hipMemcpyAsync(changed_d, &changed_h, sizeof(bool), hipMemcpyHostToDevice, st));
-        work.reset(st);
-        hipLaunchKernelGGL(FLOAT ? k_sssp_coalesce_pc<true> : k_sssp_coalesce_pc<false>, dim3(work.blocks(n_vertices, work.group)), dim3(threads), 0, st,
-                           edges->a->d_array_ptr, weights->a->d_array_ptr, label_d, new_d, n_vertices, d_offsets, work.group, work.pieces, work.n_pieces, work.count + 1, iter);
+        hipLaunchKernelGGL(FLOAT ? k_sssp_coalesce_pc<true> : k_sssp_coalesce_pc<false>, dim3(pl->blocks(n_vertices, pl->group)), dim3(threads), 0, st,
+                           edges->a->d_array_ptr, weights->a->d_array_ptr, label_d, new_d, n_vertices, d_offsets, pl->group, pl->pieces, pl->n_pieces, pl->next_work(), iter);
         hip_err_chk(hipMemsetAsync(label_d, 0, n_vertices, st));
-        hipLaunchKernelGGL(k_sssp_update, dim3(blocks_for(n_vertices, 256)), dim3(256), 0, st, label_d, d_costs, new_d, n_vertices, changed_d);
+        hipLaunchKernelGGL(k_sssp_update, dim3(blocks_for(n_vertices, 256)), dim3(256), 0, st, label_d, d_costs, new_d, n_vertices, (bool*)pl->changed);
         hip_err_chk(hipGetLastError());
         iter++;
-        hip_err_chk(hipMemcpyAsync(&changed_h, changed_d, sizeof(bool), hipMemcpyDeviceToHost, st));
-        hip_err_chk(hipStreamSynchronize(st));
-    } while (changed_h);
+        changed = pl->level_end(st);
+    } while (changed);
     if (iterations) *iterations = iter;
 }
 } // namespace

@@ -220,11 +220,23 @@ class Array:
         self.read_async(n_reqs, s, assignment, stride, reqs_per_thread, block_size)
         return int(s.item()) & MASK64
 
+    def set_graph(self, offsets=None):
+        """Prepare (or with None drop) what the graph entry points need for the CSR whose neighbour ids this array holds;
+        later calls with the same offsets tensor allocate nothing."""
+        _chk(self.L.bam_array_set_graph(self.h, _ptr(offsets), (offsets.numel() - 1) if offsets is not None else 0, _stream()), "bam_array_set_graph")
+        self._graph_offsets = offsets               # keeps the tensor alive while the plan names its address
+
     def gather(self, n_reqs, assignment=None, stride=1, block_size=64):
         """The elements themselves: out[t] = element assignment[t] (or t * stride), an int64 tensor of bit patterns."""
         out = torch.empty(n_reqs, dtype=torch.int64, device=f"cuda:{self.device}")
         _chk(self.L.bam_array_gather(self.h, n_reqs, _ptr(assignment), stride, block_size, _ptr(out), _stream()), "bam_array_gather")
         return out
+
+    def xcd_relay(self, seed, page_bytes, n_pages, rounds, n_waves=64, spin_limit=0):
+        """Pages loaded by a wave on one compute-unit cluster and read by waves on the others (bam_xcd_relay)."""
+        out = (c_u64 * 4)()
+        _chk(self.L.bam_xcd_relay(self.h, seed, page_bytes, n_pages, rounds, n_waves, spin_limit, out, _stream()), "bam_xcd_relay")
+        return dict(zip(("mismatches", "waits_given_up", "cluster_mask", "reads_checked"), list(out)))
 
     def read_via(self, api, n_reqs, assignment=None, span=1, block_size=64):
         """The read pattern through another access route of array_d_t (1 get_raw, 2 acquire_page_, 3 acquire_page,

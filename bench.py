@@ -168,6 +168,15 @@ def main():
     for _ in range(2):      # the same index pattern as a plain gather from a flat 1 GiB array, no cache protocol
         assert L.bam_gather_kernel(ctypes.c_void_p(probe.data_ptr()), ctypes.c_void_p(idx_hit.data_ptr()), ctypes.c_uint64(N_READS), ctypes.byref(ms_c), stream) == 0
     gather_hit["plain_gather_reads_per_s"] = N_READS / ms_c.value * 1e3
+    # what the counted hit path pays: a take-and-drop pair of atomics per read on words scattered like the page descriptors
+    table = torch.zeros(CACHE_PAGES, dtype=torch.int64, device=dev)
+    pages_hit = idx_hit // 512
+    for returns, key in ((1, "atomic_pairs_per_s"), (0, "atomic_pairs_unread_per_s")):
+        for _ in range(2):
+            assert L.bam_atomic_pairs_kernel(ctypes.c_void_p(table.data_ptr()), ctypes.c_void_p(pages_hit.data_ptr()), ctypes.c_uint64(N_READS), returns, ctypes.byref(ms_c), stream) == 0
+        gather_hit[key] = N_READS / ms_c.value * 1e3
+    assert int(table.abs().sum().item()) == 0
+    del table, pages_hit
     del probe
     arr.stats()
     del idx_hit
@@ -269,7 +278,16 @@ def main():
         del nb
         log("[bench] bfs graph: V=2^%d E=%d cache_pages=%d (%.1fs to build)" % (args.bfs_scale, n_e, cache_pages, time.time() - t0))
         nb_u = nb_h.view(np.uint64)
-        ref = cpu_bfs_s = cpu_bfs_edges = None
+        ag.set_graph(off)              # the per-graph preparation, outside the timed calls as in the reference's host code
+        # the serial oracle on every source: the first alone (timed: the CPU figure), the others side by side on the host's cores
+        from concurrent.futures import ThreadPoolExecutor
+        t1 = time.time()
+        refs = [oracle.bfs_levels(off_h, nb_u, int(srcs[0]))]
+        cpu_bfs_s = time.time() - t1
+        cpu_bfs_edges = O.bo_bfs_edges_scanned(len(off_h) - 1, off_h, refs[0][0])
+        with ThreadPoolExecutor(max(1, min(8, len(srcs) - 1))) as ex:
+            refs += list(ex.map(lambda x: oracle.bfs_levels(off_h, nb_u, int(x)), srcs[1:]))
+        log("[bench] bfs oracle: %d sources, %.1fs" % (len(refs), time.time() - t1))
         legs = {}
         # the edge-page kernel on every source; the reference-shaped kernel (a wave per vertex, bam_ptr per element) on the first two
         # (64 vertices per wave: consecutive vertices share pages, so the more vertices a wave has, the more distinct pages are asked for at a time)
@@ -285,13 +303,7 @@ def main():
                 L.bam_event_record(b, stream)
                 ms = elapsed_ms(a, b)
                 lv_h = lv.cpu().numpy().view(np.uint32)
-                if k == 0:                                              # full-size parity against the serial oracle (timed: the CPU figure)
-                    if ref is None:
-                        t1 = time.time()
-                        ref, rit = oracle.bfs_levels(off_h, nb_u, int(src))
-                        cpu_bfs_s = time.time() - t1
-                        cpu_bfs_edges = O.bo_bfs_edges_scanned(len(off_h) - 1, off_h, ref)
-                    levels_ok = levels_ok and np.array_equal(lv_h, ref) and it == rit
+                levels_ok = levels_ok and np.array_equal(lv_h, refs[k][0]) and it == refs[k][1]      # every source of every kernel, full size
                 tot_edges += O.bo_bfs_edges_scanned(len(off_h) - 1, off_h, lv_h)
                 tot_ms += ms
                 iters.append(it)
@@ -307,7 +319,7 @@ def main():
         bfs["cpu_serial_GTEPS"] = cpu_bfs_edges / cpu_bfs_s / 1e9
         log("[bench] bfs: %s" % bfs)
         ag.close(); rg.close(); pcg.close()
-        del off, nb_h, nb_u, off_h, lv, lv_h, ref
+        del off, nb_h, nb_u, off_h, lv, lv_h, refs
 
     # ------------------------------------------------------------------ CC on a uniform random graph (configuration 5)
     cc = None
@@ -326,6 +338,7 @@ def main():
         cache_pages = 1 << 21 if args.cc_logv == 26 else max(1 << 14, ns_bytes // PAGE // 2)        # 8 GiB at full size
         pcc, rc_, ac = make_array(ctrl, n_e, PAGE, cache_pages)
         log("[bench] cc graph: V=2^%d E=%d (%.1f GiB) cache_pages=%d (%.1fs to build)" % (args.cc_logv, n_e, n_e * 8 / 2**30, cache_pages, time.time() - t0))
+        ac.set_graph(off)
         a, b = event(), event()
         L.bam_event_record(a, stream)
         lb, it = ac.cc(off, by_page=True)

@@ -160,6 +160,16 @@ int bam_store_read_file(bam_ctrl_t* c, bam_page_cache_t* pc, const char* path, u
 /* sum of the 64-bit words of the first req_bytes of slots 0..n-1, one sum per slot */
 int bam_block_checksum(bam_page_cache_t* pc, uint64_t n_slots, uint32_t req_bytes, uint64_t* d_out, void* stream);
 
+/* ---- what the graph entry points prepare per graph (the host code around the reference's loops, benchmarks/bfs/main.cu:
+ * 1330-1560, allocates and fills its per-graph arrays once before the timed loop over sources) ----
+ * Lists the pieces of the long edge lists of the CSR (d_offsets[V+1], device memory), builds the first-vertex table of the
+ * by-page kernels when the array qualifies for them, and allocates the per-vertex flag and value buffers, the sweep counter
+ * and the word through which a level tells the host whether anything changed.  Calls of bam_bfs, bam_bfs_frontier, bam_cc,
+ * bam_bfs_by_page, bam_cc_by_page and bam_pagerank on `edges` with the same d_offsets and n_vertices then use it and
+ * allocate nothing themselves (bam_bfs_frontier still takes its queues); any other call prepares the same for itself and drops it
+ * at its end.  The offsets must not change while the plan is set.  d_offsets = NULL drops the plan; so does bam_array_destroy.
+ * The waves a sweep runs are limited to one per 64 pages of the cache, since every lane of a wave may hold a page. */
+int bam_array_set_graph(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, void* stream);
 /* ---- BFS (benchmarks/bfs/main.cu:658-689 kernel_coalesce_coarse_ptr_pc, host loop :1557-1566, 1577-1736) ----
  * Level-synchronous BFS from src: d_offsets[V+1] in device memory, neighbour ids read through the array,
  * d_labels[V] receives the level of every vertex (0xFFFFFFFF = unreachable).  *iterations = levels swept.
@@ -292,6 +302,17 @@ int bam_host_read_ceiling(uint64_t n_bytes, uint32_t chunk_bytes, float* ms);
  * read of n bytes, and a gather of n 8-byte words at d_idx[] from d_src; elapsed milliseconds */
 int bam_read_kernel(const void* d_src, uint64_t n_bytes, float* ms, void* stream);
 int bam_gather_kernel(const uint64_t* d_src, const uint64_t* d_idx, uint64_t n, float* ms, void* stream);
+/* the atomics of a hit that takes and drops a reference, without the cache around them: per request an add on the 8-byte
+ * word d_table[d_idx[t]] and, once it is back, the opposite add on the same word (the table ends as it began).
+ * returns != 0: the first add hands back the old word, as bam_try_hit needs it; 0: neither result is read. */
+int bam_atomic_pairs_kernel(uint64_t* d_table, const uint64_t* d_idx, uint64_t n, int returns, float* ms, void* stream);
+/* Pages handed between the compute-unit clusters of the device (each has an L2 of its own): n_waves workgroups of one wave,
+ * dealt out over the clusters by the dispatcher; in round r wave r % n_waves reads page r % n_pages (of page_bytes, the
+ * cache's page size) of a procedural store with seed `seed` into the cache (choose the cache smaller than n_pages, so every round re-uses a slot), the others wait
+ * for it (bounded by spin_limit looks, 0 = 2^22) and then compare elements of that page, read through operator[], with the
+ * store's words.  out4 (host): elements that differed, waits given up, bit mask of the clusters that ran waves, reads
+ * compared.  No counterpart in the reference, whose GPUs have one L2. */
+int bam_xcd_relay(bam_array_t* a, uint64_t seed, uint32_t page_bytes, uint32_t n_pages, uint32_t rounds, uint32_t n_waves, uint32_t spin_limit, uint64_t* out4, void* stream);
 /* time a callback-free region: record/elapsed on the stream the kernels above were launched on */
 int bam_event_create(void** ev);
 int bam_event_record(void* ev, void* stream);

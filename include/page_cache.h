@@ -124,6 +124,8 @@ struct page_cache_d_t {
     uint32_t* page_ticket;
     uint64_t* prp1;                  /* [n_pages] bus address of each slot (direct transfers) */
     uint32_t direct_share;           /* with staging available: of every 8 read batches of the cache's miss path, this many go direct all the same */
+    uint32_t direct_limit;           /* not 0: instead of that share, a read batch of the miss path goes direct while fewer than this many directly placed commands are in flight on the whole cache (*direct_gauge) */
+    uint32_t* direct_gauge;
     uint32_t direct_share_raw;       /* the same for reads through read_data / access_data (raw block I/O into slots the caller names) */
     uint64_t* prp2;                  /* [n_pages] second page or PRP list when page_size > controller page */
     uint64_t ctrl_page_size;
@@ -273,7 +275,7 @@ __device__ __forceinline__ void copy_pages_helped(uint8_t* dst, const uint8_t* s
  * itself) and `pos` the submission-queue slot its entry went to.
  */
 __device__ __forceinline__ uint32_t io_submit_group(page_cache_d_t* pc, QueuePair* qp, uint64_t lba, uint32_t n_blocks, uint64_t pc_entry, uint8_t opcode,
-                                                    uint8_t*& stage, uint32_t& pos, const uint32_t direct_share)
+                                                    uint8_t*& stage, uint32_t& pos, const uint32_t direct_share, uint32_t& gauged)
 {
     const uint64_t act = active_mask();
     const uint32_t n = popc(act), rank = rank_in(act);
@@ -285,8 +287,13 @@ __device__ __forceinline__ uint32_t io_submit_group(page_cache_d_t* pc, QueuePai
 #ifdef BAM_PROFILE
     const uint64_t pt0 = wall_clock64();
 #endif
+    /* placement by load: count this batch among the directly placed commands in flight, and see how many there were */
+    uint32_t gauge_before = 0;
+    gauged = gauged && direct_share && pc->direct_limit && pc->prp1 && qp->stage && opcode == NVM_IO_READ && bytes >= 2048 && bytes <= qp->stage_stride && n >= BAM_DIRECT_MIN_BATCH ? n : 0u;
+    if (gauged && lane() == first_lane(act)) gauge_before = __hip_atomic_fetch_add(pc->direct_gauge, n, __ATOMIC_RELAXED, BAM_AGENT);
     /* the command's id is the submission slot it goes to, taken until read_end / io_group / poll_async gives it back */
     const uint32_t ticket = sq_reserve_group(&qp->sq);
+    if (gauged) gauge_before = bcast(gauge_before, first_lane(act));
     const uint32_t cid = ticket & qp->sq.qs_minus_1;
 #ifdef BAM_PROFILE
     const uint64_t pt1 = wall_clock64();
@@ -303,8 +310,16 @@ __device__ __forceinline__ uint32_t io_submit_group(page_cache_d_t* pc, QueuePai
      * batches of eight to the controller (12.3 against 11.4 M reads/s), raw block reads do best all staged (12.8
      * against 11.7 M).
      */
-    const bool direct = pc->prp1 && (bytes > qp->stage_stride ||
-                                     (opcode == NVM_IO_READ && bytes >= 2048 && n >= BAM_DIRECT_MIN_BATCH && ((ticket >> 6) & 7u) < direct_share));
+    bool direct = pc->prp1 && (bytes > qp->stage_stride ||
+                               (opcode == NVM_IO_READ && bytes >= 2048 && n >= BAM_DIRECT_MIN_BATCH && ((ticket >> 6) & 7u) < direct_share));
+    if (gauged) {
+        /* the count was taken before the wait for the slots, so it cost no round trip of its own */
+        direct = gauge_before < pc->direct_limit;
+        if (!direct) {
+            if (lane() == first_lane(act)) __hip_atomic_fetch_sub(pc->direct_gauge, n, __ATOMIC_RELAXED, BAM_AGENT);
+            gauged = 0;
+        }
+    }
     const bool staged = qp->stage && !direct;
     if (staged) {
         stage = qp->stage + (size_t)cid * qp->stage_stride;
@@ -336,6 +351,12 @@ __device__ __forceinline__ uint32_t io_submit_group(page_cache_d_t* pc, QueuePai
     return cid;
 }
 
+/* the completions of a batch that io_submit_group counted as directly placed (`gauged` commands) are in */
+__device__ __forceinline__ void direct_done(page_cache_d_t* pc, const uint32_t gauged)
+{
+    if (gauged && lane() == first_lane(active_mask())) __hip_atomic_fetch_sub(pc->direct_gauge, gauged, __ATOMIC_RELAXED, BAM_AGENT);
+}
+
 /* the whole of one batch: submit, wait for all completions, move staged payload, recycle ids; true for the lanes whose
  * transfer happened (completed, without an error status) */
 __device__ __forceinline__ bool io_group(page_cache_d_t* pc, QueuePair* qp, uint64_t lba, uint32_t n_blocks, uint64_t pc_entry, uint8_t opcode,
@@ -344,11 +365,13 @@ __device__ __forceinline__ bool io_group(page_cache_d_t* pc, QueuePair* qp, uint
     const uint64_t act = active_mask();
     uint8_t* stage;
     uint32_t pos;
-    const uint32_t cid = io_submit_group(pc, qp, lba, n_blocks, pc_entry, opcode, stage, pos, direct_share);
+    uint32_t gauged = 1;
+    const uint32_t cid = io_submit_group(pc, qp, lba, n_blocks, pc_entry, opcode, stage, pos, direct_share, gauged);
 #ifdef BAM_PROFILE
     const uint64_t pt2 = wall_clock64();
 #endif
     const bool ok = cq_wait_group(&qp->cq, &qp->sq, cid);
+    direct_done(pc, gauged);
 #ifdef BAM_PROFILE
     const uint64_t pt3 = wall_clock64();
 #endif
@@ -405,11 +428,13 @@ inline __device__ void read_begin(page_cache_d_t* pc, QueuePair* qp, const uint6
     QueuePair* cur = (QueuePair*)bam::first((uint64_t)qp);
     page_cache_d_t* cpc = (page_cache_d_t*)bam::first((uint64_t)pc);
     uint32_t pos;
-    cid = bam::io_submit_group(cpc, cur, starting_lba, (uint32_t)n_blocks, pc_entry, NVM_IO_READ, stage, pos, cpc->direct_share);
+    uint32_t gauged = 1;
+    cid = bam::io_submit_group(cpc, cur, starting_lba, (uint32_t)n_blocks, pc_entry, NVM_IO_READ, stage, pos, cpc->direct_share, gauged);
 #ifdef BAM_PROFILE
     const uint64_t pt2 = wall_clock64();
 #endif
     ok = bam::cq_wait_group(&cur->cq, &cur->sq, cid);
+    bam::direct_done(cpc, gauged);
 #ifdef BAM_PROFILE
     if (cpc->prof && bam::lane() == bam::first_lane(all)) atomicAdd(&cpc->prof[4], wall_clock64() - pt2);
 #endif
@@ -444,7 +469,8 @@ inline __device__ void access_data_async(page_cache_d_t* pc, QueuePair* qp, cons
         page_cache_d_t* cpc = (page_cache_d_t*)c;
         uint8_t* stage;
         uint32_t pos;
-        const uint32_t id = bam::io_submit_group(cpc, cur, starting_lba, (uint32_t)n_blocks, pc_entry, opcode, stage, pos, cpc->direct_share_raw);
+        uint32_t gauged = 0;                 /* not counted: the completion is collected elsewhere, so this path keeps to the fixed share */
+        const uint32_t id = bam::io_submit_group(cpc, cur, starting_lba, (uint32_t)n_blocks, pc_entry, opcode, stage, pos, cpc->direct_share_raw, gauged);
         /* written for every command of a queue pair that has staging pages, staged or not: the id may have been used
          * by a staged read before, and poll_async must not find that command's destination */
         if (cur->stage) {
@@ -1645,6 +1671,7 @@ struct page_cache_t {
     BufferPtr ranges_page_starts_buf;
     BufferPtr ranges_dists_buf;
     BufferPtr page_ticket_buf;
+    BufferPtr direct_gauge_buf;
     BufferPtr ctrl_counter_buf;
     BufferPtr extra_reads_buf;
     BufferPtr tokens_buf;
@@ -1743,6 +1770,13 @@ struct page_cache_t {
         const uint64_t cache_size = ps * np;
         pdt.direct_share = 3;        /* measured best on the random-gather workload: 12.1M 4 KiB reads/s against 11.4M all staged, 10.4M all direct */
         if (const char* e = getenv("BAM_DIRECT_SHARE")) pdt.direct_share = (uint32_t)atoi(e);
+        /* 8192 measured best of 256 .. 65536: the random gather 12.9 M reads of 4 KiB per second (12.6 M with the fixed share of
+         * three in eight), the per-vertex traversal of a 2^24-vertex graph 4.1 thousand million edges per second (3.7) */
+        pdt.direct_limit = 8192;
+        if (const char* e = getenv("BAM_DIRECT_LIMIT")) pdt.direct_limit = (uint32_t)atoi(e);
+        direct_gauge_buf = createBuffer(64, hipDevice);
+        pdt.direct_gauge = (uint32_t*)direct_gauge_buf.get();
+        hip_err_chk(hipMemset(pdt.direct_gauge, 0, 64));
         pdt.direct_share_raw = 0;    /* raw 4 KiB block reads: 12.8 M/s all staged, 11.7 M with three of eight direct, 10.4 M all direct */
         if (const char* e = getenv("BAM_DIRECT_SHARE_RAW")) pdt.direct_share_raw = (uint32_t)atoi(e);
         if (!staged) pdt.direct_share = pdt.direct_share_raw = 0;

@@ -172,6 +172,23 @@ def test_every_element_of_a_gather_and_of_an_update_under_eviction(bam, cache_pa
         assert not r.c.aborted() and r.c.info()["error_completions"] == 0 and r.t.stats()["write_cmds"] > 0
 
 
+@pytest.mark.parametrize("stage_bytes,cache_pages", [(4096, 5), (0, 5), (4096, 16)])
+def test_pages_loaded_on_one_cluster_are_read_on_the_others(bam, stage_bytes, cache_pages):
+    """The device has eight clusters of compute units with an L2 each.  A page that a wave on one cluster brings into the
+    cache (pulled from a staging page, or placed by the controller when there is no staging) must be what waves on the
+    other clusters read a moment later, in a slot that held another page a few rounds before (their L2 may remember it).
+    bam_xcd_relay hands 600 pages round a ring of 64 waves through a cache of a few slots and compares every element read."""
+    n_pages = 600
+    with Rig(bam, 64 << 20, n_queues=4, depth=64, stage_bytes=stage_bytes) as r:
+        a = r.array(n_pages * 512, 4096, cache_pages)
+        res = a.xcd_relay(SEED, 4096, n_pages, rounds=n_pages, n_waves=64, spin_limit=1 << 18)
+        assert bin(res["cluster_mask"]).count("1") >= 2, "the waves ran on one cluster only: nothing was tested"
+        assert res["waits_given_up"] == 0
+        assert res["mismatches"] == 0 and res["reads_checked"] >= n_pages * 63 * 2
+        st = a.stats()
+        assert st["read_io_cnt"] >= n_pages and not r.c.aborted()
+
+
 def test_ragged_and_empty_and_last_element(bam):
     n_elems = (1 << 16) + 37                 # last page partly used
     with Rig(bam, 1 << 20) as r:
@@ -396,6 +413,34 @@ def test_block_reads_payload_checksums(bam, req, lba, order, raw_share, monkeypa
         pc.close()
 
 
+@pytest.mark.parametrize("req", [4096, 512])
+def test_block_reads_at_full_size_every_checksum(bam, req):
+    """The raw-read configuration at its full shape: 2^22 reads on 128 queue pairs of 1024 entries, every payload checked.
+    What a block must hold comes from the device generator of the store's words (pinned to the oracle by the generator
+    tests) through a running sum over the namespace: checksum(block) = S[w0 + words] - S[w0]; a sample is also checked
+    against the oracle's own checksum."""
+    import torch
+    from bam_amd import gen
+    n, ns, lba = 1 << 22, 2 << 30, 512
+    with Rig(bam, ns, lba=lba, n_queues=128, depth=1024, io_threads=12) as r:
+        pc = bam.PageCache(4096, n, 0, r.c)
+        lbas = gen.block_lbas(SEED, n, ns, req, lba)
+        pc.block_io(n, req, lbas)
+        cs = pc.block_checksums(n, req)
+        words = gen.words(SEED, 0, ns // 8)
+        run = torch.cumsum(words, 0)                       # wraps mod 2^64 like the checksum does
+        del words
+        w0 = lbas * (lba // 8)
+        want = run[w0 + (req // 8 - 1)] - torch.where(w0 > 0, run[torch.clamp(w0 - 1, min=0)], torch.zeros_like(w0))
+        assert bool(torch.equal(cs, want))
+        host_cs, host_lba = _u64(cs), _u64(lbas)
+        for k in np.random.default_rng(SEED).integers(0, n, 2048):
+            assert int(host_cs[k]) == oracle.lib().bo_block_checksum(SEED, int(host_lba[k]), lba, req)
+        ts = r.t.stats()
+        assert ts["read_cmds"] == n and ts["error_cpls"] == 0 and ts["bytes_read"] == n * req and not r.c.aborted()
+        pc.close()
+
+
 @pytest.mark.parametrize("depth,n_threads", [(1, 4096), (2, 2048), (4, 1024)])
 def test_block_reads_with_several_commands_in_flight_per_thread(bam, depth, n_threads):
     """access_data_async / poll_async: every payload arrives, ids come back (the launch can be repeated)"""
@@ -601,6 +646,50 @@ def test_bfs_levels_rmat_by_edge_page(bam, scale, cache_pages):
             assert np.array_equal(lv.cpu().numpy().view(np.uint32), ref) and it == rit
         st = a.stats()
         assert st["read_io_cnt"] > 0 and not r.c.aborted()
+
+
+@pytest.mark.parametrize("by_page", [False, True])
+def test_cc_labels_of_a_graph_with_millions_of_components(bam, by_page):
+    """2^24 vertices and 0.6 x 2^24 random pairs: below the threshold where a giant component takes over, so the answer is
+    millions of labels, not one.  Against the union-find oracle, through a cache that holds a quarter of the edge list."""
+    n_v = 1 << 24
+    off, nb = oracle.uniform_csr(SEED, n_v, int(0.6 * n_v))
+    r, a = _graph_rig(bam, nb, len(nb) // 512 // 4, n_queues=128, depth=1024, io_threads=12)
+    with r:
+        lb, it = a.cc(_dev(off), coarse=64, by_page=by_page)
+        ref, comps = oracle.cc_labels(off, nb)
+        got = _u64(lb)
+        assert np.array_equal(got, ref)
+        assert comps > 1 << 22 and len(np.unique(got)) == comps and it >= 2
+        assert a.stats()["read_io_cnt"] > 0 and not r.c.aborted()
+
+
+def test_graph_plan_gives_the_same_answers_and_is_dropped_when_the_graph_changes(bam):
+    """bam_array_set_graph prepares the per-graph tables once; every graph entry point must answer as it does without it, call
+    after call, and a call that names other offsets (here: a copy at another address) must not use the plan"""
+    off, nb = oracle.rmat_csr(SEED, 14)
+    r, a = _graph_rig(bam, nb, 300, n_queues=16, depth=256)
+    with r:
+        doff, doff2 = _dev(off), _dev(off.copy())
+        srcs = [int(x) for x in oracle.bfs_sources(SEED, off, 3)]
+        want_cc, comps = oracle.cc_labels(off, nb)
+        for planned in (False, True, True):
+            if planned:
+                a.set_graph(doff)
+            for use in (doff, doff2):
+                for src in srcs:
+                    ref, rit = oracle.bfs_levels(off, nb, src)
+                    for kw in ({"coarse": 64}, {"by_page": True}, {"frontier": True}):
+                        lv, it = a.bfs(use, src, **kw)
+                        assert np.array_equal(lv.cpu().numpy().view(np.uint32), ref) and it == rit, (planned, kw)
+                for kw in ({"coarse": 8}, {"by_page": True}):
+                    lb, it = a.cc(use, **kw)
+                    assert np.array_equal(_u64(lb), want_cc)
+        pr_plan, it_plan = a.pagerank(doff)
+        a.set_graph(None)
+        pr_none, it_none = a.pagerank(doff)
+        assert abs(it_plan - it_none) <= 3 and np.allclose(pr_plan.cpu().numpy(), pr_none.cpu().numpy(), rtol=2e-2)    # pushes land in any order: both within the tolerance of the fixed point
+        assert not r.c.aborted()
 
 
 @pytest.mark.parametrize("n_v,n_p,cache_pages", [(1 << 12, 3000, 256), (1 << 16, 1 << 18, 6), (1 << 14, 1 << 17, 4096)])
