@@ -39,6 +39,29 @@ __global__ void k_array_read(array_d_t<uint64_t>* dr, uint64_t n_reqs, const uin
     block_accumulate(sum, v);
 }
 
+/* the same sum for a launch of scattered requests, BAM_READS_PER_LANE of them per thread a quarter of the launch apart
+ * (request t + j * threads for j = 0 .. 3), read side by side (array_d_t::seq_read_n): what the lanes of a wave ask for
+ * together is as scattered as with one request per thread, and each lane keeps four requests in flight instead of one */
+#define BAM_READS_PER_LANE 4
+__global__ void k_array_read_n(array_d_t<uint64_t>* dr, uint64_t n_reqs, const uint64_t* __restrict__ assignment, uint64_t threads, unsigned long long* sum)
+{
+    const uint64_t tid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    size_t idx[BAM_READS_PER_LANE];
+    bool want[BAM_READS_PER_LANE];
+    uint64_t out[BAM_READS_PER_LANE];
+#pragma unroll
+    for (int j = 0; j < BAM_READS_PER_LANE; j++) {
+        const uint64_t t = tid + (uint64_t)j * threads;
+        want[j] = tid < threads && t < n_reqs;
+        idx[j] = want[j] ? assignment[t] : 0;
+    }
+    dr->seq_read_n(idx, want, out);
+    uint64_t v = 0;
+#pragma unroll
+    for (int j = 0; j < BAM_READS_PER_LANE; j++) v += want[j] ? out[j] : 0;
+    block_accumulate(sum, v);
+}
+
 /* thread t hands out the element it read instead of adding it to a sum */
 __global__ void k_array_gather(array_d_t<uint64_t>* dr, uint64_t n_reqs, const uint64_t* assignment, uint64_t stride, uint64_t* out)
 {
@@ -783,8 +806,14 @@ int bam_array_read(bam_array_t* a, uint64_t n_reqs, const uint64_t* d_assignment
     if (!block_size || block_size % BAM_WAVE_SIZE || block_size > 1024) return fail(EINVAL, "bam_array_read: block size must be a multiple of 64, at most 1024");
     if (!n_reqs) return 0;
     BAM_API_BEGIN
-    hipLaunchKernelGGL(k_array_read, dim3(blocks_for(n_reqs, block_size)), dim3(block_size), 0, (hipStream_t)stream,
-                       a->a->d_array_ptr, n_reqs, d_assignment, stride, reqs_per_thread, (unsigned long long*)a->partials.get());
+    /* a large launch of scattered requests, one read each: four requests per thread (results and counters are the same) */
+    if (d_assignment && reqs_per_thread == 1 && n_reqs >= (1ull << 16)) {
+        const uint64_t threads = (n_reqs + BAM_READS_PER_LANE - 1) / BAM_READS_PER_LANE;
+        hipLaunchKernelGGL(k_array_read_n, dim3(blocks_for(threads, block_size)), dim3(block_size), 0, (hipStream_t)stream,
+                           a->a->d_array_ptr, n_reqs, d_assignment, threads, (unsigned long long*)a->partials.get());
+    } else
+        hipLaunchKernelGGL(k_array_read, dim3(blocks_for(n_reqs, block_size)), dim3(block_size), 0, (hipStream_t)stream,
+                           a->a->d_array_ptr, n_reqs, d_assignment, stride, reqs_per_thread, (unsigned long long*)a->partials.get());
     hipLaunchKernelGGL(k_fold_partials, dim3(1), dim3(1024), 0, (hipStream_t)stream, (unsigned long long*)a->partials.get(), (unsigned long long*)d_sum);
     hip_err_chk(hipGetLastError());
     BAM_API_END

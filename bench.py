@@ -49,6 +49,24 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
+def splitmix_block_sums(torch, seed, first_word, n_words):
+    """sum over k < n_words of splitmix64(seed, first_word + k) (mod 2^64) for a tensor of first words, in int64 tensor
+    arithmetic: word i of the procedural store is mix64(seed + (i + 1) * 0x9E3779B97F4A7C15) with the published finalizer"""
+    def s64(x):
+        x &= (1 << 64) - 1
+        return x - (1 << 64) if x >> 63 else x
+    gamma, c1, c2 = s64(0x9E3779B97F4A7C15), s64(0xBF58476D1CE4E5B9), s64(0x94D049BB133111EB)
+    def lsr(z, k):
+        return (z >> k) & ((1 << (64 - k)) - 1)
+    acc = torch.zeros_like(first_word)
+    for k in range(n_words):
+        z = (first_word + (k + 1)) * gamma + s64(seed)
+        z = (z ^ lsr(z, 30)) * c1
+        z = (z ^ lsr(z, 27)) * c2
+        acc += z ^ lsr(z, 31)
+    return acc
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -65,6 +83,9 @@ def main():
     ap.add_argument("--cc-logv", type=int, default=26, help="log2 of the vertex count of the connected-components leg (0 = skip)")
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--skip-block", action="store_true")
+    ap.add_argument("--probe", action="store_true",
+                    help="the kernels the counter passes of the profiler look at, once each, and nothing else: the element gather at "
+                         "100 %% hits, the plain gather, the atomic pairs, the gather through the LDS translation table, the timed steps")
     ap.add_argument("--only-hit", action="store_true",
                     help="hit-path leg and a plain 1 GiB copy only (short; what the counter passes of the profiler are run on)")
     args = ap.parse_args()
@@ -178,6 +199,16 @@ def main():
     assert int(table.abs().sum().item()) == 0
     del table, pages_hit
     del probe
+    if args.probe:
+        # the same reads through bam_ptr_tlb over a translation table in LDS (what the LDS counters are for)
+        n_tlb = N_READS // 8
+        for _ in range(2):
+            a, b = event(), event()
+            L.bam_event_record(a, stream)
+            s_tlb = arr.read_via(6, n_tlb, idx_hit[:n_tlb], block_size=args.block)
+            L.bam_event_record(b, stream)
+        assert s_tlb == O.bo_gather_sum(SEED, SEED, 0, n_tlb, CACHE_PAGES * 512), "tlb gather checksum mismatch"
+        gather_hit["tlb_route_reads_per_s"] = n_tlb / elapsed_ms(a, b) * 1e3
     arr.stats()
     del idx_hit
     log("[bench] hit gather: %s" % gather_hit)
@@ -210,6 +241,10 @@ def main():
     log("[bench] cfg2: %.1f ms/step, %.2f M IOPS, %.1f M reads/s, hit rate %.3f, doorbells %d, sqe_retries %d (wall %.2fs)" %
         (ms_per_step, iops / 1e6, args.steps * N_READS / ms_total / 1e3, st["hit_cnt"] / st["access_cnt"], ts["sq_doorbells"], ts["sqe_retries"], t_wall))
     del idx, sums
+    if args.probe:
+        print(json.dumps({"probe": {"hit_gather": gather_hit, "cfg2_ms_per_step": ms_per_step, "cfg2_iops": iops, "cfg2_hit_rate": cfg2_hit_rate}}), flush=True)
+        arr.close(); rng.close(); pc.close(); ctrl.close(); target.close()
+        return
 
     # ------------------------------------------------------------------ what the store can do
     ms_c = ctypes.c_float(0)
@@ -248,10 +283,14 @@ def main():
             pcb.block_io(n_blk, req, lbas, block_size=64)
             L.bam_event_record(b, stream)
             ms = elapsed_ms(a, b)
-            cs = pcb.block_checksums(n_blk, req).cpu().numpy().view(np.uint64)
+            cs_d = pcb.block_checksums(n_blk, req)
+            # every payload: the sums of the store's words, restated with tensor arithmetic (SplitMix64 as published); and a
+            # sample against the oracle's C routine
+            good = bool(torch.equal(cs_d, splitmix_block_sums(torch, SEED, lbas * (512 // 8), req // 8)))
+            cs = cs_d.cpu().numpy().view(np.uint64)
             sample = np.random.default_rng(1).integers(0, n_blk, 4096)
             lb = lbas.cpu().numpy().view(np.uint64)
-            good = all(int(cs[k]) == O.bo_block_checksum(SEED, int(lb[k]), 512, req) for k in sample)
+            good = good and all(int(cs[k]) == O.bo_block_checksum(SEED, int(lb[k]), 512, req) for k in sample)
             assert good and not ctrl.aborted(), "raw block payload checksum mismatch"
             block["read_%dB" % req] = {"iops": n_blk / ms * 1e3, "GBps": n_blk * req / ms / 1e6, "ms": ms}
         block["frac_of_ceiling_4k"] = block["read_4096B"]["iops"] / ceiling
@@ -402,7 +441,13 @@ def main():
                    "seed": SEED, "block_size": args.block},
         "reads_per_s": args.steps * N_READS / ms_total * 1e3,
         "hit_rate": cfg2_hit_rate,
-        "roofline": roofline, "cpu_baseline": cpu, "store": store, "hit_gather": gather_hit, "block": block, "bfs": bfs, "cc": cc,
+        "roofline": roofline,
+        # the kernel that `value` times is bound by the store, not by HBM: its own entry, priced against what gets across the
+        # interconnect in 4 KiB pieces (measured in this run by bam_host_read_ceiling) or the target's service rate if lower
+        "roofline_miss_path": {"bound": "store", "kernel": "k_array_read (the timed steps)", "achieved": iops, "peak": ceiling, "unit": "IOPS",
+                               "frac": iops / ceiling, "peak_is": store["ceiling_is"], "bytes_per_unit": PAGE,
+                               "achieved_GBps": iops * PAGE / 1e9, "peak_GBps": ceiling * PAGE / 1e9},
+        "cpu_baseline": cpu, "store": store, "hit_gather": gather_hit, "block": block, "bfs": bfs, "cc": cc,
     }
     print(json.dumps(out), flush=True)
 

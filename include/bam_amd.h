@@ -95,7 +95,9 @@ int bam_array_stats(bam_array_t* a, uint64_t* out, int reset);
 /* ---- array benchmark kernels (benchmarks/array/main.cu:43-65) ----
  * One thread per request: thread t reads element d_assignment[t] (or t * stride when d_assignment is NULL)
  * reqs_per_thread times through array_d_t::operator[] and the launch adds every value read into *d_sum
- * (mod 2^64).  The reference discards the values; the checksum is what makes the result checkable. */
+ * (mod 2^64).  The reference discards the values; the checksum is what makes the result checkable.  A launch of 2^16 or
+ * more scattered requests read once each runs with a quarter of the threads, thread t taking requests t, t + n/4, t + 2n/4
+ * and t + 3n/4 side by side (array_d_t::seq_read_n): the same reads, sum and counters, four of them in flight per lane. */
 int bam_array_read(bam_array_t* a, uint64_t n_reqs, const uint64_t* d_assignment, uint64_t stride, uint64_t reqs_per_thread,
                    uint32_t block_size, uint64_t* d_sum, void* stream);
 /* the same requests with the values handed out: d_out[t] = element d_assignment[t] (or t * stride); what a kernel of the

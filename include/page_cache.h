@@ -956,11 +956,14 @@ struct range_view {
 
     /* WIDE: the lanes may hold more than one access each (a view that lived through many acquires) */
     template <bool WIDE = true>
-    __forceinline__ __device__ void flush_stats()
+    __forceinline__ __device__ void flush_stats() { flush_stats_bits<WIDE ? 32 : 1>(); }
+    /* every lane holds fewer than 2^BITS accesses */
+    template <int BITS>
+    __forceinline__ __device__ void flush_stats_bits()
     {
         if (!r) return;
-        stat_add<WIDE ? 32 : 1>(&shard->access_cnt, n_access);
-        stat_add<WIDE ? 32 : 1>(&shard->hit_cnt, n_hit);
+        stat_add<BITS>(&shard->access_cnt, n_access);
+        stat_add<BITS>(&shard->hit_cnt, n_hit);
         n_access = n_hit = 0;
     }
 
@@ -1182,6 +1185,52 @@ struct array_d_t {
         }
         v.template flush_stats<false>();
         return ret;
+    }
+
+    /*
+     * N reads per lane, the looks and loads of the unpinned route issued side by side: a read of a resident page is three
+     * dependent trips to memory (descriptor, element, descriptor again), and a lane that does them for one element at a
+     * time has one request in flight; N elements share the three waits.  out[j] for the j with want[j]; what is not
+     * resident goes the counted way one element after the other.  Same results and counters as N calls of seq_read.
+     */
+    template <int N>
+    __forceinline__ __device__ void seq_read_n(const size_t (&idx)[N], const bool (&want)[N], T (&out)[N]) const
+    {
+        static_assert(N >= 1 && N <= 7, "the counters are flushed with three ballots");
+        bool got[N];
+        bam::range_view<T> v;
+        const bool one = n_ranges == 1;
+        if (one) v.load(d_ranges);
+#pragma unroll
+        for (int j = 0; j < N; j++) { got[j] = false; out[j] = T(); }
+        if (one && v.r->cache.fast_reads) {
+            uint64_t s1[N], byte[N];
+            bool res[N];
+#pragma unroll
+            for (int j = 0; j < N; j++) {
+                res[j] = want[j] && d_ranges[0].index_start <= idx[j] && d_ranges[0].count > idx[j];
+                byte[j] = res[j] ? v.byte_of(idx[j]) : 0;
+                s1[j] = 0;
+                if (res[j]) s1[j] = __hip_atomic_load((const uint64_t*)(v.pages + (byte[j] >> v.page_size_log)), __ATOMIC_RELAXED, BAM_AGENT);
+            }
+#pragma unroll
+            for (int j = 0; j < N; j++) {
+                res[j] = res[j] && ((uint32_t)s1[j] >> (CNT_SHIFT + 1)) == V_NB;
+                if (res[j]) out[j] = bam::ld_payload((const T*)(v.base_addr + ((uint64_t)((uint32_t)(s1[j] >> 32) & BAM_SLOT_MASK) << v.page_size_log) + (byte[j] & (v.page_size - 1))));
+            }
+            bam::fence_meta();                           /* the elements are here before the second looks go out */
+#pragma unroll
+            for (int j = 0; j < N; j++) {
+                uint64_t s2 = ~s1[j];
+                if (res[j]) s2 = __hip_atomic_load((const uint64_t*)(v.pages + (byte[j] >> v.page_size_log)), __ATOMIC_RELAXED, BAM_AGENT);
+                got[j] = res[j] && ((s1[j] ^ s2) & 0xFFFFFFFFC0000000ull) == 0;
+                if (got[j]) v.account(true);
+            }
+            v.template flush_stats_bits<3>();
+        }
+#pragma unroll
+        for (int j = 0; j < N; j++)
+            if (want[j] && !got[j]) out[j] = seq_read(idx[j]);
     }
 
     __forceinline__ __device__ void seq_write(const size_t i, const T val) const
