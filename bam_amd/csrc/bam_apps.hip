@@ -5,9 +5,15 @@
 namespace {
 
 // ---- vectoradd (benchmarks/vectoradd/main.cu:102-117 kernel_baseline_ptr_pc): C[i] = A[i] + B[i], all three behind the cache ----
-__global__ __launch_bounds__(64) void k_vectoradd_ptr_pc(array_d_t<uint64_t>* da, array_d_t<uint64_t>* db, uint64_t n_elems, array_d_t<uint64_t>* dc)
+__global__ __launch_bounds__(64) void k_vectoradd_ptr_pc(array_d_t<uint64_t>* da, array_d_t<uint64_t>* db, uint64_t n_elems, array_d_t<uint64_t>* dc, const fetch_plan fp)
 {
-    const uint64_t tid = (uint64_t)blockDim.x * blockIdx.x + threadIdx.x;
+    if (fp.done && blockIdx.x < fp.blocks) {
+        array_d_t<uint64_t>* const arrays[3] = {da, db, dc};
+        fetch_role(arrays, n_elems, fp);
+        return;
+    }
+    const uint64_t bid = blockIdx.x - (fp.done ? fp.blocks : 0u);
+    const uint64_t tid = (uint64_t)blockDim.x * bid + threadIdx.x;
     bam_ptr<uint64_t> Aptr(da);
     bam_ptr<uint64_t> Bptr(db);
     bam_ptr<uint64_t> Cptr(dc);
@@ -20,13 +26,20 @@ __global__ __launch_bounds__(64) void k_vectoradd_ptr_pc(array_d_t<uint64_t>* da
         touch_ahead(dc, first, n_elems, BAM_WAVE_SIZE, 2);
     }
     if (tid < n_elems) Cptr[tid] = A[tid] + B[tid];
+    if (fp.done && threadIdx.x == 0) __hip_atomic_fetch_add(fp.done, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // ---- reduction (benchmarks/reduction/main.cu:166-195 kernel_reduce_baseline_ptr_pc): output[b] = sum of the 2 x blockDim elements of block b ----
-__global__ void k_reduce_ptr_pc(array_d_t<uint64_t>* da, unsigned long long* output, uint64_t len)
+__global__ void k_reduce_ptr_pc(array_d_t<uint64_t>* da, unsigned long long* output, uint64_t len, const fetch_plan fp)
 {
     __shared__ uint64_t wave_total[1024 / BAM_WAVE_SIZE];
-    const uint64_t tid = threadIdx.x, start = 2ull * blockDim.x * blockIdx.x;
+    if (fp.done && blockIdx.x < fp.blocks) {
+        array_d_t<uint64_t>* const arrays[1] = {da};
+        fetch_role(arrays, len, fp);
+        return;
+    }
+    const uint64_t bid = blockIdx.x - (fp.done ? fp.blocks : 0u);
+    const uint64_t tid = threadIdx.x, start = 2ull * blockDim.x * bid;
     uint64_t v = 0;
     {
         bam_ptr<uint64_t> in_ptr(da);
@@ -43,7 +56,8 @@ __global__ void k_reduce_ptr_pc(array_d_t<uint64_t>* da, unsigned long long* out
     __syncthreads();
     if (tid < BAM_WAVE_SIZE) {
         v = wave_sum(tid < blockDim.x / BAM_WAVE_SIZE ? wave_total[tid] : 0);
-        if (tid == 0) output[blockIdx.x] = v;
+        if (tid == 0) output[bid] = v;
+        if (fp.done && tid == 0) __hip_atomic_fetch_add(fp.done, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 }
 
@@ -66,12 +80,18 @@ __device__ __forceinline__ uint64_t wave_inclusive_sum(uint64_t v)
  * t + blockDim, so a wave reads consecutive elements through one page reference); the scan itself runs over wave
  * shuffles on pairs of neighbours rather than the two tree passes over shared memory.
  */
-__global__ void k_scan_ptr_pc(array_d_t<uint64_t>* da, unsigned long long* output, unsigned long long* intermediate, uint64_t len)
+__global__ void k_scan_ptr_pc(array_d_t<uint64_t>* da, unsigned long long* output, unsigned long long* intermediate, uint64_t len, const fetch_plan fp)
 {
     extern __shared__ uint64_t scan_mem[];                      /* 2 x blockDim elements, then one total per wave */
+    if (fp.done && blockIdx.x < fp.blocks) {
+        array_d_t<uint64_t>* const arrays[1] = {da};
+        fetch_role(arrays, len, fp);
+        return;
+    }
+    const uint32_t bid = blockIdx.x - (fp.done ? fp.blocks : 0u);
     const uint32_t B = blockDim.x, t = threadIdx.x;
     uint64_t* wave_total = scan_mem + 2 * B;
-    const uint64_t idx = 2ull * blockIdx.x * B + t;
+    const uint64_t idx = 2ull * bid * B + t;
     {
         bam_ptr<uint64_t> in_ptr(da);
         const bam_ptr<uint64_t>& ptr = in_ptr;
@@ -93,7 +113,8 @@ __global__ void k_scan_ptr_pc(array_d_t<uint64_t>* da, unsigned long long* outpu
     __syncthreads();
     if (idx < len) output[idx] = scan_mem[t];
     if (idx + B < len) output[idx + B] = scan_mem[t + B];
-    if (intermediate && t == B - 1) intermediate[blockIdx.x] = before + b;
+    if (intermediate && t == B - 1) intermediate[bid] = before + b;
+    if (fp.done && t == 0) __hip_atomic_fetch_add(fp.done, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 /* one block: v[i] = v[0] + ... + v[i] in place (the reference calls cub::DeviceScan::InclusiveSum here, scan/main.cu:416-418) */
@@ -129,6 +150,34 @@ __global__ void k_scan_finalsum(const unsigned long long* scanned_totals, unsign
 
 } // namespace
 
+namespace {
+/* fetch waves for a launch whose computing workgroups cover `elems_per_block` consecutive elements each: up to 256 waves
+ * (16384 pages on their way; measured on 1 GiB read from the store: 32 waves 18 GB/s, 64 waves 29, 256 waves 34-42, 512 waves
+ * 37-44, none 9-11), fewer where a quarter of the cache is less than that; BAM_FETCH_WAVES in the environment overrides the
+ * number (0: none); `done` is cleared on the stream */
+fetch_plan make_fetch_plan(bam_array_t* a, int n_arrays, uint32_t block_size, uint64_t elems_per_block, hipStream_t st)
+{
+    fetch_plan fp{nullptr, 0, 1u << 18, 0, elems_per_block};
+    if (a->a->adt.n_ranges != 1) return fp;
+    const page_cache_d_t& cache = a->a->h_ranges[0].cache;
+    const uint64_t w_pages = cache.n_pages >> 6 > BAM_WAVE_SIZE ? BAM_WAVE_SIZE : cache.n_pages >> 6;
+    if (w_pages < 2) return fp;
+    const uint64_t budget_pages = cache.n_pages / 4 / n_arrays;               /* what may lie fetched and unread, per array */
+    uint64_t waves = budget_pages / w_pages / 2;                              /* half of it on its way, half waiting to be read */
+    uint64_t most = 256;
+    if (const char* e = getenv("BAM_FETCH_WAVES")) most = (uint64_t)atoll(e);
+    if (waves > most) waves = most;
+    if (waves < 1) return fp;
+    const uint32_t waves_per_block = block_size / BAM_WAVE_SIZE;
+    fp.blocks = (uint32_t)((waves + waves_per_block - 1) / waves_per_block);
+    fp.lead_elems = budget_pages * (cache.page_size / sizeof(uint64_t));
+    if (!a->progress) a->progress = createBuffer(64, 0);
+    fp.done = (unsigned long long*)a->progress.get();
+    hip_err_chk(hipMemsetAsync(fp.done, 0, sizeof(unsigned long long), st));
+    return fp;
+}
+} // namespace
+
 extern "C" {
 
 int bam_vectoradd(bam_array_t* a, bam_array_t* b, bam_array_t* c, uint64_t n_elems, void* stream)
@@ -137,8 +186,9 @@ int bam_vectoradd(bam_array_t* a, bam_array_t* b, bam_array_t* c, uint64_t n_ele
     if (n_elems > a->a->adt.n_elems || n_elems > b->a->adt.n_elems || n_elems > c->a->adt.n_elems) return fail(EINVAL, "bam_vectoradd: more elements than the arrays hold");
     if (!n_elems) return 0;
     BAM_API_BEGIN
-    hipLaunchKernelGGL(k_vectoradd_ptr_pc, dim3(blocks_for(n_elems, 64)), dim3(64), 0, (hipStream_t)stream,
-                       a->a->d_array_ptr, b->a->d_array_ptr, n_elems, c->a->d_array_ptr);
+    const fetch_plan fp = make_fetch_plan(a, 3, 64, 64, (hipStream_t)stream);
+    hipLaunchKernelGGL(k_vectoradd_ptr_pc, dim3(blocks_for(n_elems, 64) + fp.blocks), dim3(64), 0, (hipStream_t)stream,
+                       a->a->d_array_ptr, b->a->d_array_ptr, n_elems, c->a->d_array_ptr, fp);
     hip_err_chk(hipGetLastError());
     BAM_API_END
 }
@@ -150,8 +200,9 @@ int bam_reduce(bam_array_t* a, uint64_t n_elems, uint32_t block_size, uint64_t* 
     if (n_elems > a->a->adt.n_elems) return fail(EINVAL, "bam_reduce: more elements than the array holds");
     if (!n_elems) return 0;
     BAM_API_BEGIN
-    hipLaunchKernelGGL(k_reduce_ptr_pc, dim3(blocks_for(n_elems, 2ull * block_size)), dim3(block_size), 0, (hipStream_t)stream,
-                       a->a->d_array_ptr, (unsigned long long*)d_partials, n_elems);
+    const fetch_plan fp = make_fetch_plan(a, 1, block_size, 2ull * block_size, (hipStream_t)stream);
+    hipLaunchKernelGGL(k_reduce_ptr_pc, dim3(blocks_for(n_elems, 2ull * block_size) + fp.blocks), dim3(block_size), 0, (hipStream_t)stream,
+                       a->a->d_array_ptr, (unsigned long long*)d_partials, n_elems, fp);
     hip_err_chk(hipGetLastError());
     BAM_API_END
 }
@@ -169,7 +220,8 @@ int bam_scan(bam_array_t* a, uint64_t n_elems, uint32_t block_size, uint64_t* d_
         BufferPtr totals = createBuffer(n_blocks * sizeof(uint64_t), 0);
         unsigned long long* out = (unsigned long long*)d_result + 1;
         const size_t lds = (2 * block_size + 1024 / BAM_WAVE_SIZE) * sizeof(uint64_t);
-        hipLaunchKernelGGL(k_scan_ptr_pc, dim3(n_blocks), dim3(block_size), lds, st, a->a->d_array_ptr, out, (unsigned long long*)totals.get(), n_elems);
+        const fetch_plan fp = make_fetch_plan(a, 1, block_size, 2ull * block_size, st);
+        hipLaunchKernelGGL(k_scan_ptr_pc, dim3(n_blocks + fp.blocks), dim3(block_size), lds, st, a->a->d_array_ptr, out, (unsigned long long*)totals.get(), n_elems, fp);
         hipLaunchKernelGGL(k_scan_block_totals, dim3(1), dim3(1024), 0, st, (unsigned long long*)totals.get(), n_blocks);
         hipLaunchKernelGGL(k_scan_finalsum, dim3(n_blocks), dim3(block_size), 0, st, (const unsigned long long*)totals.get(), out, n_elems);
         hip_err_chk(hipGetLastError());
@@ -233,7 +285,9 @@ int bam_scan_noalloc(bam_array_t* a, uint64_t n_elems, uint32_t block_size, uint
         /* totals[0 .. n_blocks) are written by the first kernel before the second reads them; what an earlier, longer call
          * left behind them is never read, so nothing has to be cleared */
         const size_t lds = (2 * block_size + 1024 / BAM_WAVE_SIZE) * sizeof(uint64_t);
-        hipLaunchKernelGGL(k_scan_ptr_pc, dim3((uint32_t)n_blocks), dim3(block_size), lds, st, a->a->d_array_ptr, out, totals, n_elems);
+        /* no fetch waves here: their counter would have to be allocated and cleared */
+        const fetch_plan none{nullptr, 0, 0, 0, 0};
+        hipLaunchKernelGGL(k_scan_ptr_pc, dim3((uint32_t)n_blocks), dim3(block_size), lds, st, a->a->d_array_ptr, out, totals, n_elems, none);
         hipLaunchKernelGGL(k_scan_block_totals, dim3(1), dim3(1024), 0, st, totals, n_blocks);
         hipLaunchKernelGGL(k_scan_finalsum, dim3((uint32_t)n_blocks), dim3(block_size), 0, st, (const unsigned long long*)totals, out, n_elems);
     }

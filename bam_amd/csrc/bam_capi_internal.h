@@ -51,7 +51,7 @@ struct bam_ctrl { Controller* c; };
 struct bam_page_cache { page_cache_t* pc; Controller* ctrl; };      /* ctrl: the first controller of the cache */
 struct bam_range { range_t<uint64_t>* r; };
 #define BAM_SUM_PARTIALS 4096
-struct bam_array { array_t<uint64_t>* a; BufferPtr partials; std::shared_ptr<void> graph; };      /* graph: what bam_array_set_graph prepared (bam_graph.hip) */
+struct bam_array { array_t<uint64_t>* a; BufferPtr partials, progress; std::shared_ptr<void> graph; };      /* progress: the word the computing workgroups of vectoradd, reduction and scan count themselves off in; graph: what bam_array_set_graph prepared (bam_graph.hip) */
 struct bam_range32 { range_t<uint32_t>* r; };
 struct bam_array32 { array_t<uint32_t>* a; BufferPtr partials; };      /* partials: [BAM_SUM_PARTIALS] checksum shards, zero between launches */
 
@@ -139,6 +139,56 @@ __device__ __forceinline__ void touch_ahead(array_d_t<T>* da, const uint64_t fir
         if (bam::ballot(take)) view.acquire_helped(page, take, false, touch, touch);
     }
     view.n_access = view.n_hit = 0;
+}
+
+/*
+ * Waves that only fetch.  The read-ahead above is done by waves that also compute, so what is on its way from the store is
+ * bounded by the windows the running waves happen to begin in (a few hundred pages).  A launch of these kernels therefore
+ * starts with a few workgroups whose waves do nothing else: wave k of them walks windows k, k + n_waves, ... of the
+ * arrays, takes the pages of a window that are not resident as one batch of commands per array (one page per lane), drops
+ * them again and goes on, so that n_waves batches are on their way at any time whatever the computing waves do.  They stay
+ * at most `lead_elems` elements ahead of the computing workgroups, which count themselves off in *done as they finish
+ * (elems_per_done elements each); a fetch wave that waits longer than the spin limit for that count to move gives up,
+ * and the computing waves read on demand as they would without it.  Nothing waits for a fetch wave.
+ */
+struct fetch_plan {
+    unsigned long long* done;       /* NULL: no fetch waves in this launch */
+    uint32_t blocks;                /* workgroups at the front of the grid that fetch */
+    uint32_t spin_limit;
+    uint64_t lead_elems, elems_per_done;
+};
+
+template <typename T, int N>
+__device__ __forceinline__ void fetch_role(array_d_t<T>* const (&arrays)[N], const uint64_t n_elems, const fetch_plan& fp)
+{
+    for (int a = 0; a < N; a++) if (arrays[a]->n_ranges != 1) return;
+    const page_cache_d_t& cache = arrays[0]->d_ranges[0].cache;
+    const uint64_t w_pages = cache.n_pages >> 6 > BAM_WAVE_SIZE ? BAM_WAVE_SIZE : cache.n_pages >> 6;
+    if (w_pages < 2) return;
+    const uint64_t epp = cache.page_size / sizeof(T), w_elems = w_pages * epp;
+    const uint64_t waves_per_block = blockDim.x / BAM_WAVE_SIZE;
+    const uint64_t wave = (uint64_t)blockIdx.x * waves_per_block + threadIdx.x / BAM_WAVE_SIZE, n_waves = (uint64_t)fp.blocks * waves_per_block;
+    const uint64_t n_windows = (n_elems + w_elems - 1) / w_elems;
+    auto touch = [](uint32_t) { return true; };
+    for (uint64_t w = wave; w < n_windows; w += n_waves) {
+        const uint64_t first = w * w_elems;
+        uint32_t spins = 0;
+        while (first > __hip_atomic_load(fp.done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * fp.elems_per_done + fp.lead_elems) {
+            if (++spins >= fp.spin_limit) return;
+            __builtin_amdgcn_s_sleep(64);
+        }
+        const uint64_t mine = first + bam::lane() * epp;
+#pragma unroll
+        for (int a = 0; a < N; a++) {
+            bam::range_view<T> view;
+            view.load(arrays[a]->d_ranges);
+            const uint64_t n_a = n_elems < arrays[a]->n_elems ? n_elems : arrays[a]->n_elems;
+            const uint64_t page = view.page_of(mine < n_a ? mine : 0);
+            const bool take = bam::lane() < w_pages && mine < n_a && page_absent(view, page);
+            if (bam::ballot(take)) view.acquire_helped(page, take, false, touch, touch);
+            view.n_access = view.n_hit = 0;
+        }
+    }
 }
 
 inline uint32_t blocks_for(uint64_t n, uint32_t bs) { return (uint32_t)((n + bs - 1) / bs); }
