@@ -170,7 +170,7 @@ private:
         hip_err_chk(hipMalloc((void**)&d_qps, sizeof(QueuePair) * n_qps));
         /* runtime policy of the queue pairs: where the completion rings live, whether submission entries are sealed, and
          * what an unsealed queue does to know its entries have arrived (see QueuePair and nvm_parallel_queue.h) */
-        cq_place = BAM_DMA_DEVICE; sq_seal = 1; sq_flush = 2;
+        cq_place = BAM_DMA_DEVICE; sq_seal = 0; sq_flush = 2;
         if (const char* e = getenv("BAM_CQ_PLACE")) cq_place = (e[0] == 'd' || e[0] == '1') ? BAM_DMA_DEVICE : BAM_DMA_HOST;
         if (const char* e = getenv("BAM_SQ_SEAL")) sq_seal = atoi(e) != 0;
         if (const char* e = getenv("BAM_SQ_FLUSH")) sq_flush = (uint32_t)atoi(e);

@@ -1045,27 +1045,27 @@ def test_completion_ring_placement(bam, place, order, depth, monkeypatch):
         pc.close()
 
 
-@pytest.mark.parametrize("flush", ["2", "1"])
-def test_unsealed_submission_entries(bam, flush, monkeypatch):
-    """submission queues as the NVMe specification has them, no seal in the entries (what a real controller needs): a
-    submitter makes sure its entry has arrived before the entry can be covered by a doorbell.  Checksum, no error
-    completions, no wait given up; the target's counters say what it saw."""
+@pytest.mark.parametrize("seal,flush", [("0", "2"), ("0", "1"), ("0", "0"), ("1", "2")])
+def test_submission_entries_sealed_and_unsealed(bam, seal, flush, monkeypatch):
+    """Submission queues as the NVMe specification has them (no seal in the entries, what a real controller needs; the
+    default), with each of the three ways a submitter has of making sure its entry arrives before a doorbell covers it
+    (2 read the entry back, 1 system-scope release, 0 the wave's store counter alone), and sealed (the target verifies a
+    ticket and a checksum in the entry and reads it again if they do not hold).  Checksum, no error completions, no wait
+    given up; the target's counters say what it saw."""
     from bam_amd import gen
-    monkeypatch.setenv("BAM_SQ_SEAL", "0")
+    monkeypatch.setenv("BAM_SQ_SEAL", seal)
     monkeypatch.setenv("BAM_SQ_FLUSH", flush)
     n_elems, n = 1 << 24, 1 << 20
     with Rig(bam, n_elems * 8, n_queues=32, depth=256, io_threads=8) as r:
         a = r.array(n_elems, 4096, 8192)
         for rep in range(3):
             idx = gen.gather_indices(SEED + rep, n, n_elems)
-            got = a.read(n, idx, block_size=256)
-            if flush == "2":
-                assert got == oracle.lib().bo_gather_sum(SEED, SEED + rep, 0, n, n_elems)
+            assert a.read(n, idx, block_size=256) == oracle.lib().bo_gather_sum(SEED, SEED + rep, 0, n, n_elems)
         ts = r.t.stats()
-        print("unsealed, flush %s: %d commands, %d doorbells, %d stale doorbells, %d entry retries" % (flush, ts["read_cmds"], ts["sq_doorbells"], ts["stale_doorbells"], ts["sqe_retries"]))
-        assert ts["sqe_retries"] == 0                                     # nothing is verified on an unsealed queue
-        if flush == "2":
-            assert not r.c.aborted() and r.c.info()["error_completions"] == 0 and ts["error_cpls"] == 0
+        print("seal %s, flush %s: %d commands, %d doorbells, %d stale doorbells, %d entry retries" % (seal, flush, ts["read_cmds"], ts["sq_doorbells"], ts["stale_doorbells"], ts["sqe_retries"]))
+        if seal == "0":
+            assert ts["sqe_retries"] == 0                                 # nothing is verified on an unsealed queue
+        assert not r.c.aborted() and r.c.info()["error_completions"] == 0 and ts["error_cpls"] == 0
 
 # ---------------------------------------------------------------- failure handling
 
