@@ -1075,7 +1075,7 @@ struct range_view {
                                 __builtin_amdgcn_s_sleep(127);
                                 __builtin_amdgcn_s_sleep(127);
                                 __builtin_amdgcn_s_sleep(127);
-                                /* no clock of its own: the waves inside time their waits, this one only watches for their verdict */
+                                /* no clock of its own: the waves inside time their waits, this one only watches for their outcome */
                                 if ((i & 15u) == 0 && cache->guard && ld_relaxed_sys(&cache->guard->abort)) break;
                             }
                         }
