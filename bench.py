@@ -444,7 +444,7 @@ def main():
         "roofline": roofline,
         # the kernel that `value` times is bound by the store, not by HBM: its own entry, priced against what gets across the
         # interconnect in 4 KiB pieces (measured in this run by bam_host_read_ceiling) or the target's service rate if lower
-        "roofline_miss_path": {"bound": "store", "kernel": "k_array_read (the timed steps)", "achieved": iops, "peak": ceiling, "unit": "IOPS",
+        "roofline_miss_path": {"bound": "store", "kernel": "k_array_read_n (the timed steps)", "achieved": iops, "peak": ceiling, "unit": "IOPS",
                                "frac": iops / ceiling, "peak_is": store["ceiling_is"], "bytes_per_unit": PAGE,
                                "achieved_GBps": iops * PAGE / 1e9, "peak_GBps": ceiling * PAGE / 1e9},
         "cpu_baseline": cpu, "store": store, "hit_gather": gather_hit, "block": block, "bfs": bfs, "cc": cc,
