@@ -151,8 +151,8 @@ __global__ void k_scan_finalsum(const unsigned long long* scanned_totals, unsign
 } // namespace
 
 namespace {
-/* fetch waves for a launch whose computing workgroups cover `elems_per_block` consecutive elements each: up to 256 waves
- * (16384 pages on their way; measured on 1 GiB read from the store: 32 waves 18 GB/s, 64 waves 29, 256 waves 34-42, 512 waves
+/* fetch waves for a launch whose computing workgroups cover `elems_per_block` consecutive elements each: up to 512 waves
+ * (32768 pages on their way; measured on 1 GiB read from the store: 32 waves 18 GB/s, 64 waves 29, 256 waves 34-42, 512 waves
  * 37-44, none 9-11), fewer where a quarter of the cache is less than that; BAM_FETCH_WAVES in the environment overrides the
  * number (0: none); `done` is cleared on the stream */
 fetch_plan make_fetch_plan(bam_array_t* a, int n_arrays, uint32_t block_size, uint64_t elems_per_block, hipStream_t st)
@@ -164,7 +164,7 @@ fetch_plan make_fetch_plan(bam_array_t* a, int n_arrays, uint32_t block_size, ui
     if (w_pages < 2) return fp;
     const uint64_t budget_pages = cache.n_pages / 4 / n_arrays;               /* what may lie fetched and unread, per array */
     uint64_t waves = budget_pages / w_pages / 2;                              /* half of it on its way, half waiting to be read */
-    uint64_t most = 256;
+    uint64_t most = 512;
     if (const char* e = getenv("BAM_FETCH_WAVES")) most = (uint64_t)atoll(e);
     if (waves > most) waves = most;
     if (waves < 1) return fp;

@@ -169,7 +169,8 @@ int bam_block_checksum(bam_page_cache_t* pc, uint64_t n_slots, uint32_t req_byte
  * and the word through which a level tells the host whether anything changed.  Calls of bam_bfs, bam_bfs_frontier, bam_cc,
  * bam_bfs_by_page, bam_cc_by_page and bam_pagerank on `edges` with the same d_offsets and n_vertices then use it and
  * allocate nothing themselves (bam_bfs_frontier still takes its queues); any other call prepares the same for itself and drops it
- * at its end.  The offsets must not change while the plan is set.  d_offsets = NULL drops the plan; so does bam_array_destroy.
+ * at its end.  The offsets must not change while the plan is set, and calls that use it must not overlap (they share its
+ * counters and buffers).  d_offsets = NULL drops the plan; so does bam_array_destroy.
  * The waves a sweep runs are limited to one per 64 pages of the cache, since every lane of a wave may hold a page. */
 int bam_array_set_graph(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, void* stream);
 /* ---- BFS (benchmarks/bfs/main.cu:658-689 kernel_coalesce_coarse_ptr_pc, host loop :1557-1566, 1577-1736) ----
