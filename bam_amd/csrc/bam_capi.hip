@@ -208,10 +208,45 @@ __device__ __attribute__((noinline)) void stream_touch(range_d_t<uint64_t>* r, c
 }
 
 // ---- cache / pattern benchmark (benchmarks/cache/main.cu:44-114): a wave streams whole pages ----
-template <int MODE>
-__device__ __forceinline__ void cache_stream_body(array_d_t<uint64_t>* dr, uint64_t n_waves, uint64_t n_pages_per_wave, const uint64_t* assignment, unsigned long long* sum)
+/* the fetch waves of the streaming modes for data that is not resident: the runs of the streaming waves laid end to end,
+ * 64 pages per batch (lane l of batch b looks after page (64 b + l) % n_pages_per_wave of streaming wave (64 b + l) /
+ * n_pages_per_wave), never further ahead of the waves that have finished than `lead_elems` pages */
+__device__ __forceinline__ void stream_fetch_role(array_d_t<uint64_t>* dr, const uint64_t n_waves, const uint64_t ppw, const uint64_t* assignment, const fetch_plan& fp)
 {
-    const uint64_t tid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (dr->n_ranges != 1) return;
+    bam::range_view<uint64_t> view;
+    view.load(dr->d_ranges);
+    const uint64_t epp = dr->d_ranges->n_elems_per_page;
+    const uint64_t fwave = ((uint64_t)blockIdx.x * blockDim.x + threadIdx.x) / BAM_WAVE_SIZE, n_fwaves = (uint64_t)fp.blocks * blockDim.x / BAM_WAVE_SIZE;
+    const uint64_t total = n_waves * ppw, n_batches = (total + BAM_WAVE_SIZE - 1) / BAM_WAVE_SIZE;
+    auto touch = [](uint32_t) { return true; };
+    for (uint64_t b = fwave; b < n_batches; b += n_fwaves) {
+        const uint64_t first_wave = b * BAM_WAVE_SIZE / ppw;
+        uint32_t spins = 0;
+        while (first_wave * ppw > __hip_atomic_load(fp.done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * ppw + fp.lead_elems) {
+            if (++spins >= fp.spin_limit) return;
+            __builtin_amdgcn_s_sleep(64);
+        }
+        const uint64_t at = b * BAM_WAVE_SIZE + bam::lane();
+        const uint64_t cw = at < total ? at / ppw : 0;
+        const uint64_t elem = ((assignment ? assignment[cw] : cw * ppw) + at % ppw) * epp;
+        const bool in = at < total && elem < dr->n_elems;
+        const uint64_t page = view.page_of(in ? elem : 0);
+        const bool take = in && page_absent(view, page);
+        if (bam::ballot(take)) view.acquire_helped(page, take, false, touch, touch);
+        view.n_access = view.n_hit = 0;
+    }
+}
+
+template <int MODE>
+__device__ __forceinline__ void cache_stream_body(array_d_t<uint64_t>* dr, uint64_t n_waves, uint64_t n_pages_per_wave, const uint64_t* assignment, unsigned long long* sum,
+                                                  const fetch_plan fp = fetch_plan{nullptr, 0, 0, 0, 0})
+{
+    if (MODE >= 3 && fp.done && blockIdx.x < fp.blocks) {
+        stream_fetch_role(dr, n_waves, n_pages_per_wave, assignment, fp);
+        return;
+    }
+    const uint64_t tid = (uint64_t)(blockIdx.x - (MODE >= 3 && fp.done ? fp.blocks : 0u)) * blockDim.x + threadIdx.x;
     const uint64_t wave = tid / BAM_WAVE_SIZE, lane = tid % BAM_WAVE_SIZE;
     uint64_t v = 0;
     if (wave < n_waves) {
@@ -289,6 +324,7 @@ __device__ __forceinline__ void cache_stream_body(array_d_t<uint64_t>* dr, uint6
                 }
             }
         }
+        if (MODE >= 3 && fp.done && lane == 0) __hip_atomic_fetch_add(fp.done, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     block_accumulate(sum, v);
 }
@@ -298,6 +334,13 @@ template <int MODE>
 __global__ __launch_bounds__(256) void k_cache_stream(array_d_t<uint64_t>* dr, uint64_t n_waves, uint64_t n_pages_per_wave, const uint64_t* assignment, unsigned long long* sum)
 {
     cache_stream_body<MODE>(dr, n_waves, n_pages_per_wave, assignment, sum);
+}
+/* modes 3 and 4 with fetch waves at the front of the grid */
+template <int MODE>
+__global__ __launch_bounds__(256) void k_cache_stream_fetched(array_d_t<uint64_t>* dr, uint64_t n_waves, uint64_t n_pages_per_wave, const uint64_t* assignment, unsigned long long* sum,
+                                                             const fetch_plan fp)
+{
+    cache_stream_body<MODE>(dr, n_waves, n_pages_per_wave, assignment, sum, fp);
 }
 __global__ __launch_bounds__(256) void k_cache_stream_pages(array_d_t<uint64_t>* dr, uint64_t n_waves, uint64_t n_pages_per_wave, const uint64_t* assignment, unsigned long long* sum)
 {
@@ -927,8 +970,14 @@ int bam_cache_stream(bam_array_t* a, uint64_t n_waves, uint64_t n_pages_per_wave
     unsigned long long* s = (unsigned long long*)a->partials.get();
     if (mode == 0) hipLaunchKernelGGL(k_cache_stream<0>, grid, block, 0, (hipStream_t)stream, d, n_waves, n_pages_per_wave, d_assignment, s);
     else if (mode == 1) hipLaunchKernelGGL(k_cache_stream<1>, grid, block, 0, (hipStream_t)stream, d, n_waves, n_pages_per_wave, d_assignment, s);
-    else if (mode == 3) hipLaunchKernelGGL(k_cache_stream<3>, grid, block, 0, (hipStream_t)stream, d, n_waves, n_pages_per_wave, d_assignment, s);
-    else if (mode == 4) hipLaunchKernelGGL(k_cache_stream<4>, grid, block, 0, (hipStream_t)stream, d, n_waves, n_pages_per_wave, d_assignment, s);
+    else if (mode >= 3) {
+        /* the lead is counted in pages here: one finished streaming wave stands for its n_pages_per_wave pages */
+        fetch_plan fp = make_fetch_plan(a, 1, bs, 1, (hipStream_t)stream);
+        fp.lead_elems /= a->a->h_ranges[0].cache.page_size / sizeof(uint64_t);
+        const dim3 grid_f(grid.x + fp.blocks);
+        if (mode == 3) hipLaunchKernelGGL(k_cache_stream_fetched<3>, grid_f, block, 0, (hipStream_t)stream, d, n_waves, n_pages_per_wave, d_assignment, s, fp);
+        else hipLaunchKernelGGL(k_cache_stream_fetched<4>, grid_f, block, 0, (hipStream_t)stream, d, n_waves, n_pages_per_wave, d_assignment, s, fp);
+    }
     else hipLaunchKernelGGL(k_cache_stream_pages, grid, block, 0, (hipStream_t)stream, d, n_waves, n_pages_per_wave, d_assignment, s);
     hipLaunchKernelGGL(k_fold_partials, dim3(1), dim3(1024), 0, (hipStream_t)stream, s, (unsigned long long*)d_sum);
     hip_err_chk(hipGetLastError());

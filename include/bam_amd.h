@@ -133,9 +133,11 @@ int bam_sqe_image(uint16_t cid, uint8_t opcode, uint32_t nsid, uint64_t prp1, ui
  * every element read once and summed into *d_sum.  mode 0: array_d_t::operator[] per element,
  * mode 1: bam_ptr per element (the reference's kernel, 64-wide), mode 2: one acquire per page and
  * streamed 8-byte loads (what the hit-path roofline is measured on); modes 3 and 4: modes 1 and 0 for data that is not
- * resident: the pages of a wave's run that are missing are touched ahead, up to 64 at a time, and reach the store as
- * one batch of commands (11 M instead of 1.5 M pages per second on a cold cache; on a resident one modes 1 and 0 are a
- * quarter faster, the kernels with the read-ahead run with fewer waves). */
+ * resident: a few workgroups at the front of the launch only fetch (they walk the runs of the streaming waves in order,
+ * 64 pages per batch of commands, at most a quarter of the cache ahead of the waves that have finished), and a streaming
+ * wave that gets ahead of them touches the missing pages of its run itself, up to 64 at a time (12 M instead of 2.5 M
+ * pages per second on a cold cache; on a resident one modes 1 and 0 are a quarter faster, the kernels with the read-ahead
+ * run with fewer waves). */
 int bam_cache_stream(bam_array_t* a, uint64_t n_waves, uint64_t n_pages_per_wave, const uint64_t* d_assignment, int mode,
                      uint64_t* d_sum, void* stream);
 
