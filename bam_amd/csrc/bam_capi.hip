@@ -311,7 +311,17 @@ __device__ __forceinline__ void cache_stream_body(array_d_t<uint64_t>* dr, uint6
                 if (MODE >= 3 && reach >= 2 && p % reach == 0) stream_touch(r0, start_page + p, n_pages_per_wave - p < reach ? n_pages_per_wave - p : reach);
                 const uint64_t start_idx = (start_page + p) * epp + lane;
                 if (MODE == 0 || MODE == 4) {
-                    for (uint64_t j = 0; j < epp; j += BAM_WAVE_SIZE) v += (*dr)[start_idx + j];
+                    /* operator[] per element, the eight elements a lane reads of a page side by side (array_d_t::seq_read_n) */
+                    for (uint64_t j = 0; j < epp; j += 8 * BAM_WAVE_SIZE) {
+                        size_t at[8];
+                        bool want[8];
+                        uint64_t x[8];
+#pragma unroll
+                        for (int u = 0; u < 8; u++) { at[u] = start_idx + j + u * BAM_WAVE_SIZE; want[u] = j + u * BAM_WAVE_SIZE + lane < epp; }
+                        dr->seq_read_n(at, want, x);
+#pragma unroll
+                        for (int u = 0; u < 8; u++) v += want[u] ? x[u] : 0;
+                    }
                 } else {
                     /* eight elements asked for before the first is used: the window test of an element needs nothing that
                      * an earlier load brings, so the loads of a page are in flight together */

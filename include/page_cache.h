@@ -1196,7 +1196,7 @@ struct array_d_t {
     template <int N>
     __forceinline__ __device__ void seq_read_n(const size_t (&idx)[N], const bool (&want)[N], T (&out)[N]) const
     {
-        static_assert(N >= 1 && N <= 7, "the counters are flushed with three ballots");
+        static_assert(N >= 1 && N <= 15, "the counters are flushed with three or four ballots");
         bool got[N];
         bam::range_view<T> v;
         const bool one = n_ranges == 1;
@@ -1226,7 +1226,7 @@ struct array_d_t {
                 got[j] = res[j] && ((s1[j] ^ s2) & 0xFFFFFFFFC0000000ull) == 0;
                 if (got[j]) v.account(true);
             }
-            v.template flush_stats_bits<3>();
+            v.template flush_stats_bits<(N < 8 ? 3 : 4)>();
         }
 #pragma unroll
         for (int j = 0; j < N; j++)
