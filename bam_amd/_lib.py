@@ -48,6 +48,8 @@ SIGNATURES = {
     "bam_block_checksum": (c_int, [c_vp, c_u64, c_u32, c_vp, c_vp]),
     "bam_bfs": (c_int, [c_vp, c_vp, c_u64, c_u64, c_vp, c_u32, P(c_u32), c_vp]),
     "bam_cc": (c_int, [c_vp, c_vp, c_u64, c_vp, c_u32, P(c_u32), c_vp]),
+    "bam_bfs_shaped": (c_int, [c_vp, c_vp, c_u64, c_u64, c_vp, c_int, c_u32, c_u32, P(c_u32), c_vp]),
+    "bam_cc_shaped": (c_int, [c_vp, c_vp, c_u64, c_vp, c_int, c_u32, c_u32, P(c_u32), c_vp]),
     "bam_array_set_graph": (c_int, [c_vp, c_vp, c_u64, c_vp]),
     "bam_array_gather": (c_int, [c_vp, c_u64, c_vp, c_u64, c_u32, c_vp, c_vp]),
     "bam_array_read_via": (c_int, [c_vp, c_int, c_u64, c_vp, c_u64, c_u32, c_vp, c_vp]),

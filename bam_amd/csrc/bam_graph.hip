@@ -380,6 +380,65 @@ __global__ __launch_bounds__(128) void k_bfs_coalesce_coarse_ptr_pc(array_d_t<ui
     if (any) *changed = 1;
 }
 
+// ---- the reference's other ways of sharing the vertices out (benchmarks/bfs/main.cu:733-760 hash, :810-850 hash + coarse,
+// :852-905 sixteen lanes per vertex, :961-1000 chunks; benchmarks/cc has the same set) ----
+/*
+ * The same relaxation as the kernels above, the vertices shared out as these variants of the reference do, with none of
+ * the machinery around the group walk (no touching ahead, no pieces of long lists): a unit of lanes walks a vertex's
+ * list through bam_ptr, and which vertex unit u takes is
+ *   SHAPE 0  unit = wave:       v = u / nep + (u % nep) * stride, nep = (V + stride) / stride          (hash)
+ *   SHAPE 1  unit = wave:       the `coarse` vertices c * coarse + j of c = u / nep + (u % nep) * stride,
+ *                               nep = (V + stride * coarse) / (stride * coarse)                          (hash, coarse)
+ *   SHAPE 2  unit = 16 lanes:   v as for SHAPE 0 (four vertices per wave side by side; the reference's page-cache
+ *                               version of this kernel has an empty loop body, its in-memory twin has the relaxation)
+ *   SHAPE 3  unit = wave:       the eight vertices 8 u .. 8 u + 7 one after the other                   (chunk)
+ * The units of a launch are walked by a bounded number of waves (`n_units` are shared out round robin), so that the
+ * pages the waves hold fit the cache.
+ */
+#define BAM_SHAPE_CHUNK 8
+template <int SHAPE, typename Active, typename Visit>
+__device__ __forceinline__ void walk_shaped(array_d_t<uint64_t>* da, const uint64_t* vertexList, const uint64_t n, const uint64_t coarse, const uint64_t stride,
+                                            const uint64_t n_units, Active active, Visit visit)
+{
+    const uint64_t tid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x, n_threads = (uint64_t)gridDim.x * blockDim.x;
+    bam_ptr<uint64_t> ptr(da);
+    const uint64_t width = SHAPE == 2 ? 16 : BAM_WAVE_SIZE;
+    const uint64_t l = tid % width;
+    auto walk = [&](const uint64_t v) {
+        const uint64_t start = vertexList[v], end = vertexList[v + 1];
+        for (uint64_t i = (start & 0xFFFFFFFFFFFFFFF0ull) + l; i < end; i += width)
+            if (i >= start) visit(v, ptr.read(i), i);
+    };
+    for (uint64_t u = tid / width; u < n_units; u += n_threads / width) {
+        if (SHAPE == 3) {
+            for (uint64_t v = u * BAM_SHAPE_CHUNK; v < (u + 1) * BAM_SHAPE_CHUNK && v < n; v++)
+                if (active(v)) walk(v);
+        } else if (SHAPE == 1) {
+            const uint64_t nep = (n + stride * coarse) / (stride * coarse);
+            const uint64_t c = u / nep + (u % nep) * stride;
+            for (uint64_t j = 0; j < coarse; j++) {
+                const uint64_t v = c * coarse + j;
+                if (v < n && active(v)) walk(v);
+            }
+        } else {
+            const uint64_t nep = (n + stride) / stride;
+            const uint64_t v = u / nep + (u % nep) * stride;
+            if (v < n && active(v)) walk(v);
+        }
+    }
+}
+
+template <int SHAPE>
+__global__ __launch_bounds__(128) void k_bfs_shaped(array_d_t<uint64_t>* da, uint32_t* label, const uint32_t level, const uint64_t vertex_count, const uint64_t* vertexList,
+                                                    uint64_t* changed, uint64_t coarse, uint64_t stride, uint64_t n_units)
+{
+    bool any = false;
+    walk_shaped<SHAPE>(da, vertexList, vertex_count, coarse, stride, n_units,
+                       [&](uint64_t v) { return label[v] == level; },
+                       [&](uint64_t, uint64_t next, uint64_t) { if (label[next] == MYINFINITY) { label[next] = level + 1; any = true; } });
+    if (any) *changed = 1;
+}
+
 // ---- BFS over a queue of the level's vertices (benchmarks/bfs/main.cu:409-451 kernel_frontier_coalesce_ptr_pc) ----
 /* a vertex found for the first time (the exchange on its label decides who found it) goes to the next level's queue;
  * the lanes of a wave that found one at the same step take their places in it with one atomic */
@@ -426,6 +485,15 @@ __global__ __launch_bounds__(128) void k_cc_coalesce_coarse_ptr_pc(array_d_t<uin
                                                                   const heavy_piece_t* heavy, uint64_t n_heavy, unsigned long long* next_work, uint32_t sweep)
 {
     walk_vertex_groups(da, vertexList, vertex_count, coarse, heavy, n_heavy, next_work, (sweep & 1u) != 0,
+                       [&](uint64_t v) { return curr_visit[v]; },
+                       [&](uint64_t v, uint64_t next, uint64_t) { cc_compute(v, comp, next, next_visit, changed); });
+}
+
+template <int SHAPE>
+__global__ __launch_bounds__(128) void k_cc_shaped(array_d_t<uint64_t>* da, bool* curr_visit, bool* next_visit, uint64_t vertex_count, const uint64_t* vertexList,
+                                                   unsigned long long* comp, bool* changed, uint64_t coarse, uint64_t stride, uint64_t n_units)
+{
+    walk_shaped<SHAPE>(da, vertexList, vertex_count, coarse, stride, n_units,
                        [&](uint64_t v) { return curr_visit[v]; },
                        [&](uint64_t v, uint64_t next, uint64_t) { cc_compute(v, comp, next, next_visit, changed); });
 }
@@ -804,6 +872,97 @@ int bam_bfs(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, 
                            edges->a->d_array_ptr, d_labels, level, n_vertices, d_offsets, pl->changed, group, pl->pieces, pl->n_pieces, pl->next_work());
         hip_err_chk(hipGetLastError());
         iter++; level++;
+        changed = pl->level_end(st);
+    } while (changed);
+    if (iterations) *iterations = iter;
+    BAM_API_END
+}
+
+namespace {
+/* units of a shaped launch and the waves that walk them (see walk_shaped): at most one wave per eight pages of the cache */
+struct shaped_launch { uint64_t n_units; uint32_t blocks; };
+shaped_launch shape_of(int shape, uint64_t n_vertices, uint64_t coarse, uint64_t stride, uint64_t cache_pages)
+{
+    shaped_launch sl{};
+    if (shape == 3) sl.n_units = (n_vertices + BAM_SHAPE_CHUNK - 1) / BAM_SHAPE_CHUNK;
+    else if (shape == 1) sl.n_units = ((n_vertices + stride * coarse) / (stride * coarse)) * stride;
+    else sl.n_units = ((n_vertices + stride) / stride) * stride;
+    const uint64_t per_wave = shape == 2 ? 4 : 1;
+    uint64_t waves = (sl.n_units + per_wave - 1) / per_wave;
+    int dev = 0, cus = 0;
+    hip_err_chk(hipGetDevice(&dev));
+    hip_err_chk(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    if (waves > (uint64_t)cus * 16) waves = (uint64_t)cus * 16;
+    if (cache_pages && waves > cache_pages / 8) waves = cache_pages / 8;
+    if (waves < 2) waves = 2;
+    sl.blocks = (uint32_t)((waves + 1) / 2);            /* workgroups of two waves */
+    return sl;
+}
+} // namespace
+
+int bam_bfs_shaped(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t src, uint32_t* d_labels,
+                   int shape, uint32_t coarse, uint32_t stride, uint32_t* iterations, void* stream)
+{
+    if (!edges || !d_offsets || !d_labels) return fail(EINVAL, "bam_bfs_shaped: null argument");
+    if (src >= n_vertices || shape < 0 || shape > 3 || !coarse || !stride) return fail(EINVAL, "bam_bfs_shaped: source out of range, shape not 0..3, or coarse / stride = 0");
+    BAM_API_BEGIN
+    hipStream_t st = (hipStream_t)stream;
+    std::unique_ptr<graph_plan> local;
+    graph_plan* pl = plan_for(edges, d_offsets, n_vertices, 0, st, local);
+    const shaped_launch sl = shape_of(shape, n_vertices, coarse, stride, edges->a->adt.n_ranges ? edges->a->h_ranges[0].cache.n_pages : 0);
+    hip_err_chk(hipMemsetAsync(d_labels, 0xFF, n_vertices * sizeof(uint32_t), st));
+    hip_err_chk(hipMemsetAsync(d_labels + src, 0, sizeof(uint32_t), st));
+    uint32_t level = 0, iter = 0;
+    bool changed;
+    do {
+        const dim3 grid(sl.blocks), block(128);
+        array_d_t<uint64_t>* d = edges->a->d_array_ptr;
+        switch (shape) {
+        case 0: hipLaunchKernelGGL(k_bfs_shaped<0>, grid, block, 0, st, d, d_labels, level, n_vertices, d_offsets, pl->changed, (uint64_t)coarse, (uint64_t)stride, sl.n_units); break;
+        case 1: hipLaunchKernelGGL(k_bfs_shaped<1>, grid, block, 0, st, d, d_labels, level, n_vertices, d_offsets, pl->changed, (uint64_t)coarse, (uint64_t)stride, sl.n_units); break;
+        case 2: hipLaunchKernelGGL(k_bfs_shaped<2>, grid, block, 0, st, d, d_labels, level, n_vertices, d_offsets, pl->changed, (uint64_t)coarse, (uint64_t)stride, sl.n_units); break;
+        default: hipLaunchKernelGGL(k_bfs_shaped<3>, grid, block, 0, st, d, d_labels, level, n_vertices, d_offsets, pl->changed, (uint64_t)coarse, (uint64_t)stride, sl.n_units); break;
+        }
+        hip_err_chk(hipGetLastError());
+        iter++; level++;
+        changed = pl->level_end(st);
+    } while (changed);
+    if (iterations) *iterations = iter;
+    BAM_API_END
+}
+
+int bam_cc_shaped(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t* d_labels,
+                  int shape, uint32_t coarse, uint32_t stride, uint32_t* iterations, void* stream)
+{
+    if (!edges || !d_offsets || !d_labels) return fail(EINVAL, "bam_cc_shaped: null argument");
+    if (!n_vertices || shape < 0 || shape > 3 || !coarse || !stride) return fail(EINVAL, "bam_cc_shaped: empty graph, shape not 0..3, or coarse / stride = 0");
+    BAM_API_BEGIN
+    hipStream_t st = (hipStream_t)stream;
+    std::unique_ptr<graph_plan> local;
+    graph_plan* pl = plan_for(edges, d_offsets, n_vertices, 0, st, local);
+    const shaped_launch sl = shape_of(shape, n_vertices, coarse, stride, edges->a->adt.n_ranges ? edges->a->h_ranges[0].cache.n_pages : 0);
+    bool* curr = (bool*)graph_plan::sized(pl->bytes_a, n_vertices);
+    bool* next = (bool*)graph_plan::sized(pl->bytes_b, n_vertices);
+    hipLaunchKernelGGL(k_iota, dim3(blocks_for(n_vertices, 256)), dim3(256), 0, st, (unsigned long long*)d_labels, n_vertices);
+    hip_err_chk(hipMemsetAsync(curr, 0x01, n_vertices, st));
+    hip_err_chk(hipMemsetAsync(next, 0x00, n_vertices, st));
+    uint32_t iter = 0;
+    bool changed;
+    do {
+        const dim3 grid(sl.blocks), block(128);
+        array_d_t<uint64_t>* d = edges->a->d_array_ptr;
+        unsigned long long* comp = (unsigned long long*)d_labels;
+        bool* ch = (bool*)pl->changed;
+        switch (shape) {
+        case 0: hipLaunchKernelGGL(k_cc_shaped<0>, grid, block, 0, st, d, curr, next, n_vertices, d_offsets, comp, ch, (uint64_t)coarse, (uint64_t)stride, sl.n_units); break;
+        case 1: hipLaunchKernelGGL(k_cc_shaped<1>, grid, block, 0, st, d, curr, next, n_vertices, d_offsets, comp, ch, (uint64_t)coarse, (uint64_t)stride, sl.n_units); break;
+        case 2: hipLaunchKernelGGL(k_cc_shaped<2>, grid, block, 0, st, d, curr, next, n_vertices, d_offsets, comp, ch, (uint64_t)coarse, (uint64_t)stride, sl.n_units); break;
+        default: hipLaunchKernelGGL(k_cc_shaped<3>, grid, block, 0, st, d, curr, next, n_vertices, d_offsets, comp, ch, (uint64_t)coarse, (uint64_t)stride, sl.n_units); break;
+        }
+        hip_err_chk(hipGetLastError());
+        hip_err_chk(hipMemsetAsync(curr, 0x00, n_vertices, st));
+        bool* t = curr; curr = next; next = t;
+        iter++;
         changed = pl->level_end(st);
     } while (changed);
     if (iterations) *iterations = iter;

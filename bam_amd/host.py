@@ -270,6 +270,22 @@ class Array:
             _chk(self.L.bam_bfs(self.h, _ptr(offsets), n_v, int(src), _ptr(labels), coarse, ctypes.byref(it), _stream()), "bam_bfs")
         return labels, it.value
 
+    def bfs_shaped(self, offsets, src, shape, coarse=1, stride=1):
+        """BFS with the vertices shared out as the reference's hash (0), hash + coarse (1), sixteen lanes per vertex (2) or
+        chunk (3) kernels do; levels and launch count."""
+        n_v = offsets.numel() - 1
+        labels = torch.empty(n_v, dtype=torch.int32, device=offsets.device)
+        it = c_u32(0)
+        _chk(self.L.bam_bfs_shaped(self.h, _ptr(offsets), n_v, int(src), _ptr(labels), shape, coarse, stride, ctypes.byref(it), _stream()), "bam_bfs_shaped")
+        return labels, it.value
+
+    def cc_shaped(self, offsets, shape, coarse=1, stride=1):
+        n_v = offsets.numel() - 1
+        labels = torch.empty(n_v, dtype=torch.int64, device=offsets.device)
+        it = c_u32(0)
+        _chk(self.L.bam_cc_shaped(self.h, _ptr(offsets), n_v, _ptr(labels), shape, coarse, stride, ctypes.byref(it), _stream()), "bam_cc_shaped")
+        return labels, it.value
+
     def cc(self, offsets, coarse=1, by_page=False):
         n_v = offsets.numel() - 1
         labels = torch.empty(n_v, dtype=torch.int64, device=offsets.device)

@@ -186,6 +186,19 @@ int bam_array_set_graph(bam_array_t* edges, const uint64_t* d_offsets, uint64_t 
  * for bam_cc, bam_sssp and bam_pagerank without by_page). */
 int bam_bfs(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t src, uint32_t* d_labels,
             uint32_t coarse, uint32_t* iterations, void* stream);
+/* ---- the reference's other launch shapes of BFS and CC (benchmarks/bfs/main.cu:733-760 kernel_coalesce_hash_ptr_pc,
+ * :810-850 kernel_coalesce_hash_coarse_ptr_pc, :852-905 kernel_coalesce_hash_half(_ptr_pc), :961-1000 kernel_coalesce_chunk_pc;
+ * benchmarks/cc/main.cu has the same set) ----
+ * The same levels and labels as bam_bfs / bam_cc, the vertices shared out as those variants do: shape 0 a wave per vertex,
+ * wave u taking vertex u / nep + (u % nep) * stride with nep = (V + stride) / stride; shape 1 the same over runs of `coarse`
+ * vertices; shape 2 sixteen lanes per vertex (four vertices per wave side by side), strided like shape 0; shape 3 a wave
+ * per chunk of eight consecutive vertices.  stride = 1 is the plain order.  These are the reference's kernels as they
+ * are, without read-ahead or splitting of long lists: for comparison and for programs that ask for them by name, not for
+ * speed (bam_bfs, bam_bfs_by_page). */
+int bam_bfs_shaped(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t src, uint32_t* d_labels,
+                   int shape, uint32_t coarse, uint32_t stride, uint32_t* iterations, void* stream);
+int bam_cc_shaped(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vertices, uint64_t* d_labels,
+                  int shape, uint32_t coarse, uint32_t stride, uint32_t* iterations, void* stream);
 /* ---- BFS over queues of vertices (benchmarks/bfs/main.cu:409-451 kernel_frontier_coalesce_ptr_pc, queues :1489-1492,
  * host loop :1561-1563, 1702-1711) ----
  * Instead of sweeping all labels, every level walks the queue of the vertices found by the level before and fills the

@@ -692,6 +692,28 @@ def test_graph_plan_gives_the_same_answers_and_is_dropped_when_the_graph_changes
         assert not r.c.aborted()
 
 
+@pytest.mark.parametrize("shape,coarse,stride", [(0, 1, 1), (0, 1, 7), (0, 1, 128), (1, 4, 3), (1, 16, 1), (2, 1, 1), (2, 1, 5), (3, 1, 1)])
+def test_bfs_and_cc_with_the_vertices_shared_out_as_the_reference_variants_do(bam, shape, coarse, stride):
+    """hash (0), hash + coarse (1), sixteen lanes per vertex (2) and chunk (3) assignment of vertices to waves: the same levels,
+    launch counts and labels as the oracle, whatever the stride"""
+    off, nb = oracle.rmat_csr(SEED, 13)
+    r, a = _graph_rig(bam, nb, 2048, n_queues=16, depth=256)
+    with r:
+        doff = _dev(off)
+        for src in oracle.bfs_sources(SEED, off, 2):
+            lv, it = a.bfs_shaped(doff, int(src), shape, coarse=coarse, stride=stride)
+            ref, rit = oracle.bfs_levels(off, nb, int(src))
+            assert np.array_equal(lv.cpu().numpy().view(np.uint32), ref) and it == rit
+        assert not r.c.aborted()
+    off, nb = oracle.uniform_csr(SEED, 1 << 13, 1 << 13)
+    r, a = _graph_rig(bam, nb, 2048, n_queues=16, depth=256)
+    with r:
+        lb, it = a.cc_shaped(_dev(off), shape, coarse=coarse, stride=stride)
+        ref, comps = oracle.cc_labels(off, nb)
+        assert np.array_equal(_u64(lb), ref) and len(np.unique(_u64(lb))) == comps
+        assert a.stats()["read_io_cnt"] > 0 and not r.c.aborted()
+
+
 @pytest.mark.parametrize("n_v,n_p,cache_pages", [(1 << 12, 3000, 256), (1 << 16, 1 << 18, 6), (1 << 14, 1 << 17, 4096)])
 def test_cc_labels_uniform_by_edge_page(bam, n_v, n_p, cache_pages):
     off, nb = oracle.uniform_csr(SEED, n_v, n_p)
