@@ -1,8 +1,8 @@
 #!/usr/bin/env python3
 """Benchmark of the GPU-side storage-access path on one MI355X.
 
-A step is one launch of the random-gather array benchmark: 2^26 element reads,
-one thread per read, at uniform-random indices into a 2^28-element u64 array
+A step is one launch of the random-gather array benchmark: 2^26 element reads
+(four per thread, side by side) at uniform-random indices into a 2^28-element u64 array
 (2 GiB store) behind a 1 GiB page cache with 4 KiB pages, the store being the
 software NVMe target.  The index tensors are generated and resident in HBM
 before the timed region.  `value` is 4 KiB read I/Os per second over the timed
@@ -436,7 +436,7 @@ def main():
         "value": iops, "unit": "IOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "u64", "data": "synthetic",
-        "config": {"workload": "random gather array bench: 2^28 u64 (2 GiB store), 4 KiB pages, 1 GiB page cache, 2^26 uniform-random reads per launch, one thread per read",
+        "config": {"workload": "random gather array bench: 2^28 u64 (2 GiB store), 4 KiB pages, 1 GiB page cache, 2^26 uniform-random reads per launch through bam_array_read (four reads per thread side by side)",
                    "store": "software NVMe target, procedural namespace, %d service threads, %d queue pairs x %d" % (args.io_threads, args.queues, args.depth),
                    "seed": SEED, "block_size": args.block},
         "reads_per_s": args.steps * N_READS / ms_total * 1e3,
