@@ -65,6 +65,15 @@ def test_argument_checks_without_a_gpu():
     assert L.bam_array_read(None, 1, None, 1, 1, 64, None, None) != 0
     assert b"null" in L.bam_last_error()
     assert L.bam_gen_mod(1, 0, 10, 0, 1, None, None) != 0
+    import errno
+    # the entry points added for element-wise results, graph plans, launch shapes and measurements refuse null handles too
+    assert L.bam_array_gather(None, 1, None, 1, 64, None, None) == errno.EINVAL and b"bam_array_gather" in L.bam_last_error()
+    assert L.bam_array_set_graph(None, None, 0, None) == errno.EINVAL
+    assert L.bam_bfs_shaped(None, None, 1, 0, None, 0, 1, 1, None, None) == errno.EINVAL
+    assert L.bam_cc_shaped(None, None, 1, None, 0, 1, 1, None, None) == errno.EINVAL
+    assert L.bam_atomic_pairs_kernel(None, None, 0, 1, None, None) == errno.EINVAL
+    assert L.bam_xcd_relay(None, 0, 4096, 1, 1, 64, 0, None, None) == errno.EINVAL
+    assert L.bam_scan_noalloc(None, 1, 64, None, None) == errno.EINVAL
     out = ctypes.c_void_p()
     assert L.bam_ctrl_create(ctypes.byref(out), b"/dev/not-published", 1, 0, 64, 1, 4096, 0) != 0
     assert b"no software NVMe target published" in L.bam_last_error() or b"HIP" in L.bam_last_error()
