@@ -247,12 +247,13 @@ __device__ __forceinline__ void cache_stream_body(array_d_t<uint64_t>* dr, uint6
         return;
     }
     const uint64_t tid = (uint64_t)(blockIdx.x - (MODE >= 3 && fp.done ? fp.blocks : 0u)) * blockDim.x + threadIdx.x;
-    const uint64_t wave = tid / BAM_WAVE_SIZE, lane = tid % BAM_WAVE_SIZE;
+    /* the same for all lanes of a wave, and said so: what follows from it (first page, loop counts) then lives in scalar registers */
+    const uint64_t wave = bam::first(tid / BAM_WAVE_SIZE), lane = tid % BAM_WAVE_SIZE;
     uint64_t v = 0;
     if (wave < n_waves) {
         range_d_t<uint64_t>* r0 = dr->d_ranges;
-        const uint64_t epp = r0->n_elems_per_page;
-        const uint64_t start_page = assignment ? assignment[wave] : wave * n_pages_per_wave;
+        const uint64_t epp = bam::first(r0->n_elems_per_page);
+        const uint64_t start_page = bam::first(assignment ? assignment[wave] : wave * n_pages_per_wave);
         if (MODE == 2) {
             /*
              * Descriptor read once.  Pages are taken sixteen at a time: lane l of the wave asks for page l of the
@@ -326,10 +327,22 @@ __device__ __forceinline__ void cache_stream_body(array_d_t<uint64_t>* dr, uint6
                     /* eight elements asked for before the first is used: the window test of an element needs nothing that
                      * an earlier load brings, so the loads of a page are in flight together */
                     for (uint64_t j = 0; j < epp; j += 8 * BAM_WAVE_SIZE) {
-                        uint64_t x[8];
+                        const uint64_t i0 = start_idx + j;
+                        const uint32_t n_here = (uint32_t)((epp - j + BAM_WAVE_SIZE - 1) / BAM_WAVE_SIZE < 8 ? (epp - j + BAM_WAVE_SIZE - 1) / BAM_WAVE_SIZE : 8);
+                        /* the first element opens the window (the one place where the page can change); when the others
+                         * lie in it, as they do unless a range ends inside the page, they are asked for side by side */
+                        uint64_t acc = (uint64_t)ptr[i0];
+                        if (ptr.covers(i0, i0 + (uint64_t)(n_here - 1) * BAM_WAVE_SIZE)) {
+                            uint64_t x[8];
+                            x[0] = 0;
 #pragma unroll
-                        for (int u = 0; u < 8; u++) x[u] = j + u * BAM_WAVE_SIZE < epp ? (uint64_t)ptr[start_idx + j + u * BAM_WAVE_SIZE] : 0;
-                        v += ((x[0] + x[1]) + (x[2] + x[3])) + ((x[4] + x[5]) + (x[6] + x[7]));
+                            for (int u = 1; u < 8; u++) x[u] = (uint32_t)u < n_here ? (uint64_t)ptr.peek(i0 + (uint64_t)u * BAM_WAVE_SIZE) : 0;
+                            acc += ((x[0] + x[1]) + (x[2] + x[3])) + ((x[4] + x[5]) + (x[6] + x[7]));
+                        } else {
+#pragma unroll 1
+                            for (uint32_t u = 1; u < n_here; u++) acc += (uint64_t)ptr[i0 + (uint64_t)u * BAM_WAVE_SIZE];
+                        }
+                        v += acc;
                     }
                 }
             }

@@ -1466,6 +1466,19 @@ struct bam_ptr {
 #endif
     }
 
+    /* whether elements a and b (a <= b), and so all between them, lie in the page this pointer holds now */
+    __forceinline__ __host__ __device__ bool covers(const size_t a, const size_t b) const { return a >= start && b < end; }
+    /* element i of the page held now, for callers that have asked covers() about it: no window test, so a lane's reads
+     * of one page go out side by side instead of one behind the test of the one before */
+    __forceinline__ __host__ __device__ T peek(const size_t i) const
+    {
+#if defined(__HIP_DEVICE_COMPILE__)
+        return bam::ld_payload(addr + (i - start));
+#else
+        return addr[i - start];
+#endif
+    }
+
     __forceinline__ __host__ __device__ void mark_dirty()
     {
 #if defined(__HIP_DEVICE_COMPILE__)
