@@ -353,8 +353,10 @@ __device__ __forceinline__ void cache_stream_body(array_d_t<uint64_t>* dr, uint6
 }
 
 /* one kernel per mode; the page-wise one has a name of its own because it is the one the hit-path roofline is quoted on */
+/* mode 1 is held to the registers of four waves per SIMD: it needs two more, which the compiler parks in scratch memory
+ * outside the loop over a page's elements */
 template <int MODE>
-__global__ __launch_bounds__(256) void k_cache_stream(array_d_t<uint64_t>* dr, uint64_t n_waves, uint64_t n_pages_per_wave, const uint64_t* assignment, unsigned long long* sum)
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MODE == 1 ? 4 : 1))) void k_cache_stream(array_d_t<uint64_t>* dr, uint64_t n_waves, uint64_t n_pages_per_wave, const uint64_t* assignment, unsigned long long* sum)
 {
     cache_stream_body<MODE>(dr, n_waves, n_pages_per_wave, assignment, sum);
 }

@@ -925,6 +925,17 @@ struct range_view {
     {
         flush_stats();
         r = r_;
+        fill();
+    }
+    /*
+     * The descriptor read (again).  Also called at the end of the miss path: what is read again there need not be
+     * kept in registers over the passes of that path, which is a call, and a value that lives across a call costs
+     * the caller a register the callee must not touch, of which there are few.  The path for resident pages, which
+     * has no call, then has the registers of a kernel with four waves per SIMD instead of three.
+     */
+    __forceinline__ __device__ void fill()
+    {
+        range_d_t<T>* const r_ = r;
         pages = r_->pages;
         base_addr = r_->cache.base_addr;
         shard = r_->shard();
@@ -1096,6 +1107,7 @@ struct range_view {
                 }
             }
             if (limit && admitted && me == leader) __hip_atomic_fetch_add(tokens, 0u - 1u, __ATOMIC_RELAXED, BAM_AGENT);
+            fill();
         }
     }
 
