@@ -310,7 +310,11 @@ __device__ __forceinline__ void cache_stream_body(array_d_t<uint64_t>* dr, uint6
             const uint32_t reach = MODE < 3 || dr->n_ranges != 1 ? 0 : (uint32_t)(r0->cache.n_pages >> 6 > BAM_WAVE_SIZE ? BAM_WAVE_SIZE : r0->cache.n_pages >> 6);
             for (uint64_t p = 0; p < n_pages_per_wave; p++) {
                 if (MODE >= 3 && reach >= 2 && p % reach == 0) stream_touch(r0, start_page + p, n_pages_per_wave - p < reach ? n_pages_per_wave - p : reach);
-                const uint64_t start_idx = (start_page + p) * epp + lane;
+                /* the lane number worked out afresh at every page (two instructions): held in a register across the
+                 * loop it is the value the compiler parks in scratch memory, and a reload with its wait costs more */
+                uint32_t lane_now;
+                asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lane_now));
+                const uint64_t start_idx = (start_page + p) * epp + lane_now;
                 if (MODE == 0 || MODE == 4) {
                     /* operator[] per element, the eight elements a lane reads of a page side by side (array_d_t::seq_read_n) */
                     for (uint64_t j = 0; j < epp; j += 8 * BAM_WAVE_SIZE) {

@@ -692,8 +692,16 @@ __device__ __forceinline__ void stat_add(unsigned long long* ctr, uint32_t v)
 {
     for_each_group((uint64_t)ctr, [&](uint64_t a0) {
         unsigned long long total = 0;
+        if constexpr (BITS > 8) {
+            /* any width: as many trips as the largest value of the group has bits (a view that lived through sixteen
+             * page changes makes five, not thirty-two) */
+            uint32_t rest = v;
+#pragma unroll 1
+            for (uint32_t b = 0; ballot(rest != 0); b++, rest >>= 1) total += (unsigned long long)popc(ballot(rest & 1u)) << b;
+        } else {
 #pragma unroll
-        for (uint32_t b = 0; b < BITS; b++) total += (unsigned long long)popc(ballot((v >> b) & 1u)) << b;
+            for (uint32_t b = 0; b < BITS; b++) total += (unsigned long long)popc(ballot((v >> b) & 1u)) << b;
+        }
         if (lane() == first_lane(active_mask()) && total)
             __hip_atomic_fetch_add((unsigned long long*)a0, total, __ATOMIC_RELAXED, BAM_AGENT);
     });
@@ -916,7 +924,6 @@ struct range_view {
     range_d_t<T>* r = nullptr;       /* full descriptor, for the miss path */
     data_page_t* pages;
     uint8_t* base_addr;
-    bam_stat_shard_t* shard;
     uint64_t index_start, index_end, pso;
     uint32_t page_size_log, page_size;
     uint32_t n_access = 0, n_hit = 0;   /* this lane's accesses since the last flush_stats() */
@@ -938,7 +945,6 @@ struct range_view {
         range_d_t<T>* const r_ = r;
         pages = r_->pages;
         base_addr = r_->cache.base_addr;
-        shard = r_->shard();
         index_start = r_->index_start;
         index_end = r_->count;
         pso = r_->page_start_offset;
@@ -973,6 +979,7 @@ struct range_view {
     __forceinline__ __device__ void flush_stats_bits()
     {
         if (!r) return;
+        bam_stat_shard_t* const shard = r->shard();      /* looked up here, once in a view's life, rather than carried along */
         stat_add<BITS>(&shard->access_cnt, n_access);
         stat_add<BITS>(&shard->hit_cnt, n_hit);
         n_access = n_hit = 0;
@@ -1009,10 +1016,11 @@ struct range_view {
         const uint32_t me = lane();
         /* helpers form a group of their own on a page number no range has; they take nothing */
         const uint64_t page = HELPERS && !take ? ~0ull : page_;
-        const uint64_t eq_mask = match_any(page, (uint64_t)r);
+        /* lanes with the same page of the same range have the same descriptor, and only they */
+        data_page_t* dp = pages + page;
+        const uint64_t eq_mask = match_any(HELPERS && !take ? 0ull : (uint64_t)dp);
         const uint32_t master = first_lane(eq_mask), count = popc(eq_mask);
         const bool dirty = (ballot(write) & eq_mask) != 0;
-        data_page_t* dp = pages + page;
         uint64_t sv = 0, pack = 0;
         uint32_t slot = 0;
         if (master == me && (!HELPERS || take)) { const bool h = bam_try_hit(dp, count, dirty, sv, slot); pack = (uint64_t)slot | ((uint64_t)h << 63); }
@@ -1114,7 +1122,7 @@ struct range_view {
     /* drop the reference each active lane holds on `page` (one atomic per group of lanes on the same page) */
     __forceinline__ __device__ void release(const uint64_t page, const bool wrote) const
     {
-        const uint64_t eq_mask = match_any(page, (uint64_t)r);
+        const uint64_t eq_mask = match_any((uint64_t)(pages + page));
         const bool any_wrote = (ballot(wrote) & eq_mask) != 0;
         if (first_lane(eq_mask) == lane()) bam_release_refs(pages + page, popc(eq_mask), any_wrote);
     }
