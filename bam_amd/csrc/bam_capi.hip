@@ -302,6 +302,8 @@ __device__ __forceinline__ void cache_stream_body(array_d_t<uint64_t>* dr, uint6
             view.flush_stats();
         } else {
             bam_ptr<uint64_t> ptr(dr);
+            bam::range_view<uint64_t> elem_view;            /* modes 0 and 4: the descriptor read once, the accesses counted here */
+            if ((MODE == 0 || MODE == 4) && dr->n_ranges == 1) elem_view.load(r0);
             /* a wave reads its pages one after the other: those of the next stretch that are not resident are touched
              * together, one page per lane, so that a cold run asks the store for a batch per stretch and not for a page
              * per trip (1.5 M pages/s otherwise); on a resident cache this costs one look at a state word per page */
@@ -323,7 +325,7 @@ __device__ __forceinline__ void cache_stream_body(array_d_t<uint64_t>* dr, uint6
                         uint64_t x[8];
 #pragma unroll
                         for (int u = 0; u < 8; u++) { at[u] = start_idx + j + u * BAM_WAVE_SIZE; want[u] = j + u * BAM_WAVE_SIZE + lane < epp; }
-                        dr->seq_read_n(at, want, x);
+                        dr->seq_read_n(at, want, x, elem_view);
 #pragma unroll
                         for (int u = 0; u < 8; u++) v += want[u] ? x[u] : 0;
                     }
@@ -350,6 +352,7 @@ __device__ __forceinline__ void cache_stream_body(array_d_t<uint64_t>* dr, uint6
                     }
                 }
             }
+            elem_view.flush_stats();
         }
         if (MODE >= 3 && fp.done && lane == 0) __hip_atomic_fetch_add(fp.done, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
@@ -357,10 +360,10 @@ __device__ __forceinline__ void cache_stream_body(array_d_t<uint64_t>* dr, uint6
 }
 
 /* one kernel per mode; the page-wise one has a name of its own because it is the one the hit-path roofline is quoted on */
-/* mode 1 is held to the registers of four waves per SIMD: it needs two more, which the compiler parks in scratch memory
- * outside the loop over a page's elements */
+/* mode 1 is held to the registers of four waves per SIMD (128; left alone the compiler takes 130): it fits, without a
+ * spill, since the lane number is worked out per page rather than kept; mode 0 to those of three (168; 171 left alone) */
 template <int MODE>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MODE == 1 ? 4 : 1))) void k_cache_stream(array_d_t<uint64_t>* dr, uint64_t n_waves, uint64_t n_pages_per_wave, const uint64_t* assignment, unsigned long long* sum)
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MODE == 1 ? 4 : MODE == 0 ? 3 : 1))) void k_cache_stream(array_d_t<uint64_t>* dr, uint64_t n_waves, uint64_t n_pages_per_wave, const uint64_t* assignment, unsigned long long* sum)
 {
     cache_stream_body<MODE>(dr, n_waves, n_pages_per_wave, assignment, sum);
 }

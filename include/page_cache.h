@@ -1216,22 +1216,37 @@ struct array_d_t {
     template <int N>
     __forceinline__ __device__ void seq_read_n(const size_t (&idx)[N], const bool (&want)[N], T (&out)[N]) const
     {
-        static_assert(N >= 1 && N <= 15, "the counters are flushed with three or four ballots");
-        bool got[N];
         bam::range_view<T> v;
-        const bool one = n_ranges == 1;
-        if (one) v.load(d_ranges);
+        if (n_ranges == 1) v.load(d_ranges);
+        seq_read_n(idx, want, out, v);
+        v.template flush_stats_bits<(N < 8 ? 3 : 4)>();
+    }
+    /*
+     * The same with the caller's view of the array's one range (`v.r` null: the array has several, and every read goes
+     * the counted way): a kernel that makes many such calls reads the range's descriptor once, and its lanes count their
+     * accesses in the view until the caller flushes it (range_view::flush_stats).
+     */
+    template <int N>
+    __forceinline__ __device__ void seq_read_n(const size_t (&idx)[N], const bool (&want)[N], T (&out)[N], bam::range_view<T>& v) const
+    {
+        static_assert(N >= 1 && N <= 15, "the counters of the plain form are flushed with three or four ballots");
+        bool got[N];
+        const bool one = v.r != nullptr;
 #pragma unroll
         for (int j = 0; j < N; j++) { got[j] = false; out[j] = T(); }
         if (one && v.r->cache.fast_reads) {
             uint64_t s1[N], byte[N];
-            bool res[N];
+            bool res[N], again[N];
+            /* an element on the page of the one before it (a lane that reads along an array) shares that one's two
+             * looks at the descriptor: what holds for the page holds for both */
 #pragma unroll
             for (int j = 0; j < N; j++) {
-                res[j] = want[j] && d_ranges[0].index_start <= idx[j] && d_ranges[0].count > idx[j];
+                res[j] = want[j] && v.index_start <= idx[j] && v.index_end > idx[j];
                 byte[j] = res[j] ? v.byte_of(idx[j]) : 0;
+                again[j] = j > 0 && res[j] && res[j - 1] && (byte[j] >> v.page_size_log) == (byte[j - 1] >> v.page_size_log);
                 s1[j] = 0;
-                if (res[j]) s1[j] = __hip_atomic_load((const uint64_t*)(v.pages + (byte[j] >> v.page_size_log)), __ATOMIC_RELAXED, BAM_AGENT);
+                if (again[j]) s1[j] = s1[j - 1];
+                else if (res[j]) s1[j] = __hip_atomic_load((const uint64_t*)(v.pages + (byte[j] >> v.page_size_log)), __ATOMIC_RELAXED, BAM_AGENT);
             }
 #pragma unroll
             for (int j = 0; j < N; j++) {
@@ -1239,14 +1254,15 @@ struct array_d_t {
                 if (res[j]) out[j] = bam::ld_payload((const T*)(v.base_addr + ((uint64_t)((uint32_t)(s1[j] >> 32) & BAM_SLOT_MASK) << v.page_size_log) + (byte[j] & (v.page_size - 1))));
             }
             bam::fence_meta();                           /* the elements are here before the second looks go out */
+            uint64_t s2[N];
 #pragma unroll
             for (int j = 0; j < N; j++) {
-                uint64_t s2 = ~s1[j];
-                if (res[j]) s2 = __hip_atomic_load((const uint64_t*)(v.pages + (byte[j] >> v.page_size_log)), __ATOMIC_RELAXED, BAM_AGENT);
-                got[j] = res[j] && ((s1[j] ^ s2) & 0xFFFFFFFFC0000000ull) == 0;
+                s2[j] = ~s1[j];
+                if (again[j]) s2[j] = s2[j - 1];
+                else if (res[j]) s2[j] = __hip_atomic_load((const uint64_t*)(v.pages + (byte[j] >> v.page_size_log)), __ATOMIC_RELAXED, BAM_AGENT);
+                got[j] = res[j] && ((s1[j] ^ s2[j]) & 0xFFFFFFFFC0000000ull) == 0;
                 if (got[j]) v.account(true);
             }
-            v.template flush_stats_bits<(N < 8 ? 3 : 4)>();
         }
 #pragma unroll
         for (int j = 0; j < N; j++)
