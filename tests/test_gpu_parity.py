@@ -350,6 +350,26 @@ def test_page_streaming_modes(bam, mode):
         assert not r.c.aborted()
 
 
+@pytest.mark.parametrize("mode", [0, 1, 3, 4])
+@pytest.mark.parametrize("page", [512, 4096, 16384])
+def test_element_streaming_over_other_page_sizes_and_a_ragged_last_page(bam, mode, page):
+    """The per-element streaming kernels where a lane reads one element of a page (512 B), eight (4 KiB) or thirty-two
+    (16 KiB), and over an array that ends inside its last page: the lanes past the end read nothing, and bam_ptr's
+    side-by-side reads (covers/peek) give way to operator[] per element on the page the array ends in."""
+    epp, n_pages = page // 8, 1024
+    n_elems = n_pages * epp - epp // 4
+    with Rig(bam, 64 << 20) as r:
+        a = r.array(n_elems, page, n_pages)
+        ref = oracle.lib().bo_store_sum(SEED, 0, 1, n_elems)
+        assert a.stream(n_pages // 4, 4, mode=mode) == ref          # cold
+        assert a.stats()["read_io_cnt"] == n_pages
+        assert a.stream(n_pages // 4, 4, mode=mode) == ref          # resident
+        assert a.stats()["read_io_cnt"] == 0 and not r.c.aborted()
+    with Rig(bam, 64 << 20) as r:
+        a = r.array(n_elems, page, 96)                              # a tenth of the data fits
+        assert a.stream(n_pages // 4, 4, mode=mode) == ref and not r.c.aborted()
+
+
 # ---------------------------------------------------------------- the other access routes of array_d_t
 
 @pytest.mark.parametrize("api", [1, 2, 3, 4, 6, 7])
