@@ -76,7 +76,9 @@ enum data_dist_t { REPLICATE = 0, STRIPE = 1 };
 
 /* batches smaller than this are never placed directly: the controller pushes a page into device memory in several
  * microseconds, which a wave with a few commands waits for in full, while what it pulls itself is there in two */
+#ifndef BAM_DIRECT_MIN_BATCH
 #define BAM_DIRECT_MIN_BATCH 24u
+#endif
 
 #define BAM_TOKEN_SLOTS 4096u
 #define BAM_STAT_SHARDS 4096
