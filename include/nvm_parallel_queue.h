@@ -256,9 +256,13 @@ __device__ __forceinline__ void sq_submit_group(nvm_queue_t* sq, nvm_cmd_t* cmd,
     if (sq->sealed) nvm_cmd_seal(cmd, ticket);
     /* written through to the ring, which may be host memory the L2 would otherwise hold on to */
     uint64_t* dst = (uint64_t*)(((nvm_cmd_t*)sq->vaddr) + pos);
-    const uint64_t* src = (const uint64_t*)cmd->dword;
+    /* four stores of sixteen bytes, not eight of eight: an entry in host memory leaves the GPU as one write per store,
+     * and the rate at which single-command batches go out doubled with half as many (2.5 to 5 M per second) */
+    {
+        const uint32_t* w = cmd->dword;
 #pragma unroll
-    for (int i = 0; i < 8; i++) __hip_atomic_store(dst + i, src[i], __ATOMIC_RELAXED, BAM_SYSTEM);
+        for (int i = 0; i < 4; i++) { u32x4_t v = {w[4 * i], w[4 * i + 1], w[4 * i + 2], w[4 * i + 3]}; st16_sys((uint8_t*)dst + 16 * i, v); }
+    }
     /*
      * The entry must be in the ring before a doorbell that covers it reaches the controller.  A sealed queue leaves
      * that to the controller (it takes an entry only once the seal verifies, doorbell or no doorbell).  An unsealed
