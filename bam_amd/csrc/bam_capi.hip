@@ -361,9 +361,9 @@ __device__ __forceinline__ void cache_stream_body(array_d_t<uint64_t>* dr, uint6
 
 /* one kernel per mode; the page-wise one has a name of its own because it is the one the hit-path roofline is quoted on */
 /* mode 1 is held to the registers of four waves per SIMD (128; left alone the compiler takes 130): it fits, without a
- * spill, since the lane number is worked out per page rather than kept; mode 0 to those of three (168; 171 left alone) */
+ * spill, since the lane number is worked out per page rather than kept */
 template <int MODE>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MODE == 1 ? 4 : MODE == 0 ? 3 : 1))) void k_cache_stream(array_d_t<uint64_t>* dr, uint64_t n_waves, uint64_t n_pages_per_wave, const uint64_t* assignment, unsigned long long* sum)
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MODE == 1 ? 4 : 1))) void k_cache_stream(array_d_t<uint64_t>* dr, uint64_t n_waves, uint64_t n_pages_per_wave, const uint64_t* assignment, unsigned long long* sum)
 {
     cache_stream_body<MODE>(dr, n_waves, n_pages_per_wave, assignment, sum);
 }
