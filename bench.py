@@ -42,7 +42,7 @@ STREAM_PAGES_PER_WAVE = 16      # one acquire batch of the page-wise streaming k
 # HBM bytes one launch of the page-wise streaming kernel moves over the 1 GiB cache, from the profiler's FETCH_SIZE and
 # WRITE_SIZE counters scaled by what they read for a plain 1 GiB copy (x2.0 and x1.0); figures and commands in
 # profiles/k_cache_stream_pages_hit_path_1GiB_cache.md.  Holds for this workload only.
-HIT_STREAM_TRAFFIC_BYTES = 1079601152
+HIT_STREAM_TRAFFIC_BYTES = 1079592960
 
 
 def log(*a):
