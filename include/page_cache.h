@@ -1256,20 +1256,24 @@ struct array_d_t {
                 if (res[j]) out[j] = bam::ld_payload((const T*)(v.base_addr + ((uint64_t)((uint32_t)(s1[j] >> 32) & BAM_SLOT_MASK) << v.page_size_log) + (byte[j] & (v.page_size - 1))));
             }
             bam::fence_meta();                           /* the elements are here before the second looks go out */
-            uint64_t s2[N];
+            uint64_t s2 = 0;                            /* the second look of the element before, for one that shares it */
 #pragma unroll
             for (int j = 0; j < N; j++) {
-                s2[j] = ~s1[j];
-                if (again[j]) s2[j] = s2[j - 1];
-                else if (res[j]) s2[j] = __hip_atomic_load((const uint64_t*)(v.pages + (byte[j] >> v.page_size_log)), __ATOMIC_RELAXED, BAM_AGENT);
-                got[j] = res[j] && ((s1[j] ^ s2[j]) & 0xFFFFFFFFC0000000ull) == 0;
+                if (!again[j]) {
+                    s2 = ~s1[j];
+                    if (res[j]) s2 = __hip_atomic_load((const uint64_t*)(v.pages + (byte[j] >> v.page_size_log)), __ATOMIC_RELAXED, BAM_AGENT);
+                }
+                got[j] = res[j] && ((s1[j] ^ s2) & 0xFFFFFFFFC0000000ull) == 0;
                 if (got[j]) v.account(true);
             }
         }
 #pragma unroll
         for (int j = 0; j < N; j++)
-            if (want[j] && !got[j]) out[j] = seq_read(idx[j]);
+            if (want[j] && !got[j]) out[j] = seq_read_call(idx[j]);
     }
+    /* seq_read as a call: the N places above where an element goes the counted way would otherwise each carry the whole
+     * of that path, and its registers with it */
+    __attribute__((noinline)) __device__ T seq_read_call(const size_t i) const { return seq_read(i); }
 
     __forceinline__ __device__ void seq_write(const size_t i, const T val) const
     {
