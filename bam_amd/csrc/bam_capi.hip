@@ -216,6 +216,7 @@ __device__ __forceinline__ void stream_fetch_role(array_d_t<uint64_t>* dr, const
     if (dr->n_ranges != 1) return;
     bam::range_view<uint64_t> view;
     view.load(dr->d_ranges);
+    view.read_ahead = true;
     const uint64_t epp = dr->d_ranges->n_elems_per_page;
     const uint64_t fwave = ((uint64_t)blockIdx.x * blockDim.x + threadIdx.x) / BAM_WAVE_SIZE, n_fwaves = (uint64_t)fp.blocks * blockDim.x / BAM_WAVE_SIZE;
     const uint64_t total = n_waves * ppw, n_batches = (total + BAM_WAVE_SIZE - 1) / BAM_WAVE_SIZE;

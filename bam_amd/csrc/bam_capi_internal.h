@@ -182,6 +182,7 @@ __device__ __forceinline__ void fetch_role(array_d_t<T>* const (&arrays)[N], con
         for (int a = 0; a < N; a++) {
             bam::range_view<T> view;
             view.load(arrays[a]->d_ranges);
+            view.read_ahead = true;
             const uint64_t n_a = n_elems < arrays[a]->n_elems ? n_elems : arrays[a]->n_elems;
             const uint64_t page = view.page_of(mine < n_a ? mine : 0);
             const bool take = bam::lane() < w_pages && mine < n_a && page_absent(view, page);

@@ -126,6 +126,7 @@ struct page_cache_d_t {
     uint32_t* page_ticket;
     uint64_t* prp1;                  /* [n_pages] bus address of each slot (direct transfers) */
     uint32_t direct_share;           /* with staging available: of every 8 read batches of the cache's miss path, this many go direct all the same */
+    uint32_t direct_limit_ahead;     /* the same bound for batches of waves that only fetch ahead of others (range_view::read_ahead): nobody copies for them */
     uint32_t direct_limit;           /* not 0: instead of that share, a read batch of the miss path goes direct while fewer than this many directly placed commands are in flight on the whole cache (*direct_gauge) */
     uint32_t* direct_gauge;
     uint32_t direct_share_raw;       /* the same for reads through read_data / access_data (raw block I/O into slots the caller names) */
@@ -291,6 +292,7 @@ __device__ __forceinline__ uint32_t io_submit_group(page_cache_d_t* pc, QueuePai
 #endif
     /* placement by load: count this batch among the directly placed commands in flight, and see how many there were */
     uint32_t gauge_before = 0;
+    const uint32_t gauged_kind = gauged;        /* 0: not counted (the caller has no end to report), 1: a batch somebody waits for, 2: read-ahead */
     gauged = gauged && direct_share && pc->direct_limit && pc->prp1 && qp->stage && opcode == NVM_IO_READ && bytes >= 2048 && bytes <= qp->stage_stride && n >= BAM_DIRECT_MIN_BATCH ? n : 0u;
     if (gauged && lane() == first_lane(act)) gauge_before = __hip_atomic_fetch_add(pc->direct_gauge, n, __ATOMIC_RELAXED, BAM_AGENT);
     /* the command's id is the submission slot it goes to, taken until read_end / io_group / poll_async gives it back */
@@ -316,7 +318,7 @@ __device__ __forceinline__ uint32_t io_submit_group(page_cache_d_t* pc, QueuePai
                                (opcode == NVM_IO_READ && bytes >= 2048 && n >= BAM_DIRECT_MIN_BATCH && ((ticket >> 6) & 7u) < direct_share));
     if (gauged) {
         /* the count was taken before the wait for the slots, so it cost no round trip of its own */
-        direct = gauge_before < pc->direct_limit;
+        direct = gauge_before < (gauged_kind == 2u ? pc->direct_limit_ahead : pc->direct_limit);
         if (!direct) {
             if (lane() == first_lane(act)) __hip_atomic_fetch_sub(pc->direct_gauge, n, __ATOMIC_RELAXED, BAM_AGENT);
             gauged = 0;
@@ -409,7 +411,7 @@ inline __device__ void access_data(page_cache_d_t* pc, QueuePair* qp, const uint
  * with several groups each one runs its whole transfer before the next starts, and `held` comes back false.
  */
 inline __device__ void read_begin(page_cache_d_t* pc, QueuePair* qp, const uint64_t starting_lba, const uint64_t n_blocks, const unsigned long long pc_entry,
-                                  uint32_t& cid, uint8_t*& stage, bool& held, bool& ok)
+                                  uint32_t& cid, uint8_t*& stage, bool& held, bool& ok, const bool ahead = false)
 {
     const uint64_t all = bam::active_mask();
     bool one_group = bam::ballot(qp == (QueuePair*)bam::first((uint64_t)qp) && pc == (page_cache_d_t*)bam::first((uint64_t)pc)) == all;
@@ -430,7 +432,7 @@ inline __device__ void read_begin(page_cache_d_t* pc, QueuePair* qp, const uint6
     QueuePair* cur = (QueuePair*)bam::first((uint64_t)qp);
     page_cache_d_t* cpc = (page_cache_d_t*)bam::first((uint64_t)pc);
     uint32_t pos;
-    uint32_t gauged = 1;
+    uint32_t gauged = ahead ? 2u : 1u;
     cid = bam::io_submit_group(cpc, cur, starting_lba, (uint32_t)n_blocks, pc_entry, NVM_IO_READ, stage, pos, cpc->direct_share, gauged);
 #ifdef BAM_PROFILE
     const uint64_t pt2 = wall_clock64();
@@ -623,7 +625,7 @@ struct range_d_t {
     /* spread by workgroup so that no counter word is shared by more than a few waves at a time */
     __forceinline__ __device__ bam_stat_shard_t* shard() const { return stats + (((blockIdx.x + blockIdx.y * gridDim.x) * 0x9E3779B1u) >> 20) % BAM_STAT_SHARDS; }
     __forceinline__ __device__ bool slow_step(const size_t pg, const bool write, const uint32_t queue, uint64_t& sv, uint32_t& slot, bool& was_hit, bool& progressed, const bool take_part = true,
-                                              const bool may_load = true, bool* wants_load = nullptr);
+                                              const bool may_load = true, bool* wants_load = nullptr, const bool ahead = false);
 };
 
 /*
@@ -729,7 +731,7 @@ __device__ __forceinline__ void stat_add(unsigned long long* ctr, uint32_t v)
 template <typename T>
 __forceinline__ __device__
 bool range_d_t<T>::slow_step(const size_t pg, const bool write, const uint32_t queue, uint64_t& sv, uint32_t& slot, bool& was_hit, bool& progressed, const bool take_part,
-                             const bool may_load, bool* wants_load)
+                             const bool may_load, bool* wants_load, const bool ahead)
 {
     using namespace bam;
     data_page_t* dp = &pages[pg];
@@ -777,7 +779,7 @@ bool range_d_t<T>::slow_step(const size_t pg, const bool write, const uint32_t q
             stat_add((unsigned long long*)&ctl->access_counter, 1);
             stat_add(&shard()->read_io_cnt, 1);
             qp = ctl->d_qps + (queue % ctl->n_qps);
-            read_begin(&cache, qp, get_backing_page(pg) * cache.n_blocks_per_page, cache.n_blocks_per_page, found, cid, stage, held, io_ok);
+            read_begin(&cache, qp, get_backing_page(pg) * cache.n_blocks_per_page, cache.n_blocks_per_page, found, cid, stage, held, io_ok, ahead);
         }
     }
     /* staged payload is moved by every lane that came in, whether it loaded a page itself or not */
@@ -855,12 +857,13 @@ struct bam_pass_t { uint64_t sv; uint32_t slot; uint32_t flags; };
 #define BAM_PASS_WRITE      16u     /* in: */
 #define BAM_PASS_TAKE_PART  32u
 #define BAM_PASS_MAY_LOAD   64u
+#define BAM_PASS_AHEAD      128u    /* the caller fetches for others (placement: page_cache_d_t::direct_limit_ahead) */
 template <typename T>
 __forceinline__ __device__ bam_pass_t bam_slow_pass_inline(range_d_t<T>* r, const uint64_t pg, const uint32_t queue, uint64_t sv, uint32_t slot, const uint32_t in)
 {
     bool hit = false, progressed = false, wants = false;
     const bool resolved = r->slow_step(pg, (in & BAM_PASS_WRITE) != 0, queue, sv, slot, hit, progressed, (in & BAM_PASS_TAKE_PART) != 0,
-                                       (in & BAM_PASS_MAY_LOAD) != 0, &wants);
+                                       (in & BAM_PASS_MAY_LOAD) != 0, &wants, (in & BAM_PASS_AHEAD) != 0);
     bam_pass_t out;
     out.sv = sv;
     out.slot = slot;
@@ -929,6 +932,7 @@ struct range_view {
     uint64_t index_start, index_end, pso;
     uint32_t page_size_log, page_size;
     uint32_t n_access = 0, n_hit = 0;   /* this lane's accesses since the last flush_stats() */
+    bool read_ahead = false;            /* set by waves that fetch for others: their batches may be placed directly up to the higher bound */
 
     __forceinline__ __device__ void load(range_d_t<T>* r_)
     {
@@ -1056,7 +1060,8 @@ struct range_view {
                 /* every lane of the miss branch goes in: the masters that still wait for their page take part, the rest help move payload */
                 const bool part = !done && master == me;
                 const bam_pass_t ps = bam_slow_pass<OUTLINE>(r, page, queue, sv, slot,
-                                                    (dirty ? BAM_PASS_WRITE : 0u) | (part ? BAM_PASS_TAKE_PART : 0u) | (admitted ? BAM_PASS_MAY_LOAD : 0u));
+                                                    (dirty ? BAM_PASS_WRITE : 0u) | (part ? BAM_PASS_TAKE_PART : 0u) | (admitted ? BAM_PASS_MAY_LOAD : 0u) |
+                                                    (read_ahead ? BAM_PASS_AHEAD : 0u));
                 const bool progressed = (ps.flags & BAM_PASS_PROGRESSED) != 0, wants = (ps.flags & BAM_PASS_WANTS) != 0;
                 if (part) {
                     sv = ps.sv;
@@ -1874,9 +1879,14 @@ struct page_cache_t {
         const uint64_t cache_size = ps * np;
         pdt.direct_share = 3;        /* measured best on the random-gather workload: 12.1M 4 KiB reads/s against 11.4M all staged, 10.4M all direct */
         if (const char* e = getenv("BAM_DIRECT_SHARE")) pdt.direct_share = (uint32_t)atoi(e);
-        /* 8192 measured best of 256 .. 65536: the random gather 12.9 M reads of 4 KiB per second (12.6 M with the fixed share of
-         * three in eight), the per-vertex traversal of a 2^24-vertex graph 4.1 thousand million edges per second (3.7) */
-        pdt.direct_limit = 8192;
+        /* 1024 measured: the random gather 13.2 M reads of 4 KiB per second (13.4 M at 64, 13.3 M all staged, 12.8 M at 8192,
+         * 11.9 M at 32768), connected components of 2^26 vertices 0.50 s (0.59 at 8192), the per-vertex traversal of a
+         * 2^24-vertex graph 4.5 thousand million edges per second (4.35 at 512 and at 8192) */
+        pdt.direct_limit = 1024;
+        /* waves that only fetch have nobody to copy staged pages for them: 8192, the cold streaming modes read every page
+         * once at 12.6 M pages per second (with 1024: a fifth of the pages twice) */
+        pdt.direct_limit_ahead = 8192;
+        if (const char* e = getenv("BAM_DIRECT_LIMIT_AHEAD")) pdt.direct_limit_ahead = (uint32_t)atoi(e);
         if (const char* e = getenv("BAM_DIRECT_LIMIT")) pdt.direct_limit = (uint32_t)atoi(e);
         direct_gauge_buf = createBuffer(64, hipDevice);
         pdt.direct_gauge = (uint32_t*)direct_gauge_buf.get();
