@@ -40,11 +40,13 @@ SIGNATURES = {
     "bam_array_destroy": (None, [c_vp]),
     "bam_array_stats": (c_int, [c_vp, P(c_u64), c_int]),
     "bam_array_read": (c_int, [c_vp, c_u64, c_vp, c_u64, c_u64, c_u32, c_vp, c_vp]),
+    "bam_array_read_shaped": (c_int, [c_vp, c_u64, c_vp, c_int, c_u32, c_u32, c_vp, c_vp]),
     "bam_array_write": (c_int, [c_vp, c_u64, c_vp, c_u64, c_vp, c_u32, c_vp]),
     "bam_array_update": (c_int, [c_vp, c_int, c_u64, c_vp, c_vp, c_vp, c_u32, c_vp]),
     "bam_sqe_image": (c_int, [ctypes.c_uint16, ctypes.c_uint8, c_u32, c_u64, c_u64, c_u64, ctypes.c_uint16, c_int, c_u32, P(c_u32), c_vp, c_vp]),
     "bam_cache_stream": (c_int, [c_vp, c_u64, c_u64, c_vp, c_int, c_vp, c_vp]),
     "bam_block_io": (c_int, [c_vp, c_vp, c_u64, c_u32, c_vp, c_int, c_int, c_u32, c_vp]),
+    "bam_warp_memcpy": (c_int, [c_vp, c_vp, c_u64, c_u64, c_vp]),
     "bam_block_checksum": (c_int, [c_vp, c_u64, c_u32, c_vp, c_vp]),
     "bam_bfs": (c_int, [c_vp, c_vp, c_u64, c_u64, c_vp, c_u32, P(c_u32), c_vp]),
     "bam_cc": (c_int, [c_vp, c_vp, c_u64, c_vp, c_u32, P(c_u32), c_vp]),

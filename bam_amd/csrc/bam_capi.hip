@@ -22,6 +22,54 @@ __global__ void k_fold_partials(unsigned long long* partials, unsigned long long
     if (bam::lane() == 0 && v) atomicAdd(sum, (unsigned long long)v);
 }
 
+/*
+ * The launch's checksum folded by the last workgroup of a kernel to finish, instead of by a launch of its own.  Called by
+ * all threads of every workgroup after their block_accumulate.  The partial sums are only ever touched with atomics at
+ * device scope, and a wave's additions have been performed when its memory counter says so (bam::fence_meta), so the
+ * workgroup that draws the last number finds them all.  The workgroups count themselves off in two steps (64 words, one per
+ * residue of the workgroup number, and one word for the residues that are complete): a single word would take one atomic
+ * per workgroup of the grid, all on one address.  finished[0 .. 64] are zero between launches.
+ */
+#define BAM_FINISHED_WORDS 65u
+__device__ __forceinline__ void fold_by_last_block(unsigned long long* partials, unsigned long long* sum, uint32_t* finished)
+{
+    __shared__ uint32_t last;
+    bam::fence_meta();
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t is_last = 0;
+        const uint32_t r = blockIdx.x & 63u, with_r = (gridDim.x - r + 63u) / 64u, residues = gridDim.x < 64u ? gridDim.x : 64u;
+        if (__hip_atomic_fetch_add(finished + 1 + r, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1 == with_r) {
+            __hip_atomic_store(finished + 1 + r, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            bam::fence_meta();
+            if (__hip_atomic_fetch_add(finished, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1 == residues) {
+                __hip_atomic_store(finished, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                is_last = 1;
+            }
+        }
+        last = is_last;
+    }
+    __syncthreads();
+    if (!last) return;
+    uint64_t v = 0;
+    for (uint32_t i = threadIdx.x; i < BAM_SUM_PARTIALS; i += blockDim.x) {
+        const unsigned long long x = __hip_atomic_load(partials + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (x) { v += x; __hip_atomic_store(partials + i, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+    }
+    v = wave_sum(v);
+    if (bam::lane() == 0 && v) atomicAdd(sum, (unsigned long long)v);
+}
+/* the word through which the first of two launches tells the second whether it left anything: the number of the call when it
+ * did (the host counts the calls per array), so that nobody has to clear it */
+#define BAM_LEFT_WORD 96u
+/* by a whole wave that left something; the word is written only while it does not say so yet (thousands of waves storing to
+ * one address take the device 12 ns a time, one after the other) */
+__device__ __forceinline__ void note_work_left(uint32_t* finished, const uint32_t call)
+{
+    if (bam::lane() == bam::first_lane(bam::active_mask()) && __hip_atomic_load(finished + BAM_LEFT_WORD, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != call)
+        __hip_atomic_store(finished + BAM_LEFT_WORD, call, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // ---- array benchmark (benchmarks/array/main.cu:43-65), with a checksum ----
 __global__ void k_array_read(array_d_t<uint64_t>* dr, uint64_t n_reqs, const uint64_t* assignment, uint64_t stride, uint64_t reqs_per_thread, unsigned long long* sum)
 {
@@ -43,7 +91,7 @@ __global__ void k_array_read(array_d_t<uint64_t>* dr, uint64_t n_reqs, const uin
  * (request t + j * threads for j = 0 .. 3), read side by side (array_d_t::seq_read_n): what the lanes of a wave ask for
  * together is as scattered as with one request per thread, and each lane keeps four requests in flight instead of one */
 #define BAM_READS_PER_LANE 4
-__global__ void k_array_read_n(array_d_t<uint64_t>* dr, uint64_t n_reqs, const uint64_t* __restrict__ assignment, uint64_t threads, unsigned long long* sum)
+__global__ void k_array_read_n_whole(array_d_t<uint64_t>* dr, uint64_t n_reqs, const uint64_t* __restrict__ assignment, uint64_t threads, unsigned long long* sum)
 {
     const uint64_t tid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
     size_t idx[BAM_READS_PER_LANE];
@@ -60,6 +108,104 @@ __global__ void k_array_read_n(array_d_t<uint64_t>* dr, uint64_t n_reqs, const u
 #pragma unroll
     for (int j = 0; j < BAM_READS_PER_LANE; j++) v += want[j] ? out[j] : 0;
     block_accumulate(sum, v);
+}
+
+/*
+ * A launch of scattered requests in two launches (arrays of one range).  The first, this kernel: thread t takes requests
+ * t, t + threads, ... (N at a time for `rounds` rounds, `threads` a multiple of 64) and reads those whose page is resident, without a reference
+ * (array_d_t::seq_read_n_resident); bit t of missed[] says whether request t is left for the second launch
+ * (k_array_read_deferred).  No call, no atomic but the checksum's and the counters', no stack: a kernel that can miss
+ * carries the registers of the miss path (four waves per SIMD) and its frame in scratch memory through every read.  The
+ * last workgroup folds the checksum of what was read; the second launch adds what it reads.
+ */
+#ifndef BAM_GATHER_MAX_WAVES
+#define BAM_GATHER_MAX_WAVES 8
+#endif
+template <int N>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, BAM_GATHER_MAX_WAVES))) void k_array_read_n(array_d_t<uint64_t>* dr, uint64_t n_reqs, const uint64_t* __restrict__ assignment, uint64_t threads, uint32_t rounds,
+                                                      unsigned long long* partials, uint64_t* missed, unsigned long long* sum, uint32_t* finished, uint32_t call)
+{
+    const uint64_t tid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    bam::range_view<uint64_t> view;
+    view.load(dr->d_ranges);
+    uint64_t v = 0, any_left = 0;
+    /* thread t takes requests t + k * threads, k = 0 .. N * rounds - 1, N at a time: what a wave, a workgroup and the launch
+     * do once (the range's descriptor, the counters, the checksum) is shared by more reads the more rounds there are */
+    for (uint32_t r = 0; r < rounds; r++) {
+        size_t idx[N];
+        bool want[N], got[N];
+        uint64_t out[N];
+#pragma unroll
+        for (int j = 0; j < N; j++) {
+            const uint64_t t = tid + (uint64_t)(r * N + j) * threads;
+            want[j] = tid < threads && t < n_reqs;
+            idx[j] = want[j] ? __builtin_nontemporal_load(assignment + t) : 0;      /* read once: not to be kept in the L2 the descriptors live in */
+        }
+        dr->template seq_read_n_resident<N, true>(idx, want, out, got, view);
+#pragma unroll
+        for (int j = 0; j < N; j++) {
+            v += got[j] ? out[j] : 0;
+            const uint64_t m = bam::ballot(want[j] && !got[j]);
+            if (bam::lane() == 0 && tid < threads) missed[(tid + (uint64_t)(r * N + j) * threads) / BAM_WAVE_SIZE] = m;
+            any_left |= m;
+        }
+    }
+    view.flush_stats();
+    if (any_left) note_work_left(finished, call);
+    block_accumulate(partials, v);
+    fold_by_last_block(partials, sum, finished);
+}
+
+/*
+ * The second launch: the requests the first one left, one per lane through array_d_t::operator[], which has the miss
+ * path.  A wave takes `words` words of missed[] at a time (1 to 16, a power of two: lane l looks after `words` bits),
+ * lines the requests noted there up in LDS and reads them 64 at a time: whatever the share of misses, the batches of
+ * commands that go to the store are whole waves' worth.  The last workgroup to finish adds the checksum of these reads
+ * to the first launch's.  When the first launch left nothing (it says so in a word of its own) this one ends at once.
+ */
+#define BAM_DEFER_MAX_WORDS 16u
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void k_array_read_deferred(array_d_t<uint64_t>* dr, uint64_t n_reqs, const uint64_t* __restrict__ assignment, const uint64_t* missed,
+                                                             uint64_t n_words, uint32_t words, unsigned long long* partials, unsigned long long* sum, uint32_t* finished, uint32_t call)
+{
+    __shared__ uint16_t ids[256 / BAM_WAVE_SIZE][BAM_DEFER_MAX_WORDS * BAM_WAVE_SIZE];
+    if (__hip_atomic_load(finished + BAM_LEFT_WORD, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != call) return;      /* nothing was left */
+    const uint32_t lane = bam::lane(), w_in_block = threadIdx.x / BAM_WAVE_SIZE;
+    const uint64_t gwave = ((uint64_t)blockIdx.x * blockDim.x + threadIdx.x) / BAM_WAVE_SIZE, n_gwaves = (uint64_t)gridDim.x * blockDim.x / BAM_WAVE_SIZE;
+    const uint64_t n_chunks = (n_words + words - 1) / words;
+    uint64_t v = 0;
+    bool any = false;
+    for (uint64_t c = gwave; c < n_chunks; c += n_gwaves) {
+        /* lane l: bits [l * words, (l + 1) * words) of the chunk's 64 * words */
+        const uint32_t bit0 = lane * words;
+        const uint64_t word = c * words + bit0 / 64;
+        const uint32_t seg = word < n_words ? (uint32_t)((missed[word] >> (bit0 % 64)) & ((1u << words) - 1u)) : 0u;
+        uint32_t incl = bam::popc((uint64_t)seg);
+        const uint32_t mine = incl;
+#pragma unroll
+        for (uint32_t o = 1; o < BAM_WAVE_SIZE; o <<= 1) {
+            const uint32_t u = bam::shfl(incl, lane >= o ? lane - o : lane);
+            if (lane >= o) incl += u;
+        }
+        const uint32_t total = bam::bcast(incl, BAM_WAVE_SIZE - 1);
+        if (!total) continue;
+        any = true;
+        uint32_t at = incl - mine;
+        for (uint32_t m = seg; m; m &= m - 1) ids[w_in_block][at++] = (uint16_t)(bit0 + (uint32_t)__builtin_ctz(m));
+        /* written and read by the lanes of one wave, which runs its LDS operations in order */
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        for (uint32_t b = 0; b < total; b += BAM_WAVE_SIZE) {
+            if (b + lane < total) {
+                const uint64_t t = c * words * BAM_WAVE_SIZE + ids[w_in_block][b + lane];
+                if (t < n_reqs) v += (*dr)[assignment[t]];
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    }
+    if (bam::ballot(any)) block_accumulate(partials, v);
+    fold_by_last_block(partials, sum, finished);
 }
 
 /* thread t hands out the element it read instead of adding it to a sum */
@@ -117,7 +263,7 @@ __global__ void k_array_read_via(array_d_t<uint64_t>* dr, uint64_t n_reqs, const
             if (q[0] != v || !(q - idx == p)) v = 0;
         } else if (API == 1) {
             returned_cache_page_t<uint64_t> pg = dr->get_raw(idx);
-            v = bam::ld_payload(pg.addr + pg.offset);
+            if (pg.addr) v = bam::ld_payload(pg.addr + pg.offset);      /* no address after a wait that was given up */
             dr->release_raw(idx);
         } else if (API == 2) {
             range_d_t<uint64_t>* r;
@@ -239,6 +385,75 @@ __device__ __forceinline__ void stream_fetch_role(array_d_t<uint64_t>* dr, const
     }
 }
 
+/*
+ * One page of a streaming wave, every element read once and added up: lane l reads elements l, l + 64, ... of the page
+ * whose first element is `first`.  ELEM: through array_d_t::operator[] per element (the eight elements a lane reads of a
+ * page side by side, array_d_t::seq_read_n); otherwise through bam_ptr per element.  DEFER: the page is read only if it is
+ * resident; true (for the whole wave) if it was not, and then nothing of it is counted, neither in `v` nor in the views.
+ */
+template <bool ELEM, bool DEFER, typename PTR>
+__device__ __forceinline__ bool stream_page(array_d_t<uint64_t>* dr, PTR& ptr, bam::range_view<uint64_t>& elem_view, const uint64_t first, const uint64_t epp,
+                                            const uint32_t lane, uint64_t& v)
+{
+    const uint64_t start_idx = first + lane;
+    uint64_t sum = 0;
+    bool miss = false;
+    [[maybe_unused]] uint32_t na = 0, nh = 0;
+    if constexpr (DEFER) { if (ELEM) { na = elem_view.n_access; nh = elem_view.n_hit; } else ptr.counted(na, nh); }
+    if constexpr (ELEM) {
+        for (uint64_t j = 0; j < epp; j += 8 * BAM_WAVE_SIZE) {
+            size_t at[8];
+            bool want[8];
+            uint64_t x[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) { at[u] = start_idx + j + u * BAM_WAVE_SIZE; want[u] = j + u * BAM_WAVE_SIZE + lane < epp; }
+            if constexpr (DEFER) {
+                bool got[8];
+                dr->seq_read_n_resident(at, want, x, got, elem_view);
+#pragma unroll
+                for (int u = 0; u < 8; u++) miss = miss || (want[u] && !got[u]);
+            } else
+                dr->seq_read_n(at, want, x, elem_view);
+#pragma unroll
+            for (int u = 0; u < 8; u++) sum += want[u] ? x[u] : 0;
+        }
+    } else {
+        /* The page changes in one place, update_page for the lane's first element of the stretch; when the lane's other
+         * elements lie in the window that opens, as they do unless a range ends inside the page, all eight are asked for
+         * side by side: the window test of an element needs nothing that an earlier load brings. */
+        for (uint64_t j = 0; j < epp; j += 8 * BAM_WAVE_SIZE) {
+            const uint64_t i0 = start_idx + j;
+            const uint32_t n_here = (uint32_t)((epp - j + BAM_WAVE_SIZE - 1) / BAM_WAVE_SIZE < 8 ? (epp - j + BAM_WAVE_SIZE - 1) / BAM_WAVE_SIZE : 8);
+            const uint64_t i_last = i0 + (uint64_t)(n_here - 1) * BAM_WAVE_SIZE;
+            if (!ptr.covers(i0, i_last)) ptr.update_page(i0);
+            if constexpr (DEFER) { if (bam::ballot(ptr.missed)) break; }
+            uint64_t acc = 0;
+            if (ptr.covers(i0, i_last)) {
+                uint64_t x[8];
+                if (n_here == 8) ptr.template peek_n<8>(i0, BAM_WAVE_SIZE, x);
+                else {
+#pragma unroll
+                    for (int u = 0; u < 8; u++) x[u] = (uint32_t)u < n_here ? (uint64_t)ptr.peek(i0 + (uint64_t)u * BAM_WAVE_SIZE) : 0;
+                }
+                acc = ((x[0] + x[1]) + (x[2] + x[3])) + ((x[4] + x[5]) + (x[6] + x[7]));
+            } else {
+#pragma unroll 1
+                for (uint32_t u = 0; u < n_here; u++) acc += (uint64_t)ptr[i0 + (uint64_t)u * BAM_WAVE_SIZE];
+            }
+            sum += acc;
+        }
+        if constexpr (DEFER) { miss = ptr.missed; ptr.missed = false; }
+    }
+    if constexpr (DEFER) {
+        if (bam::ballot(miss)) {
+            if (ELEM) { elem_view.n_access = na; elem_view.n_hit = nh; } else ptr.set_counted(na, nh);
+            return true;
+        }
+    }
+    v += sum;
+    return false;
+}
+
 template <int MODE>
 __device__ __forceinline__ void cache_stream_body(array_d_t<uint64_t>* dr, uint64_t n_waves, uint64_t n_pages_per_wave, const uint64_t* assignment, unsigned long long* sum,
                                                   const fetch_plan fp = fetch_plan{nullptr, 0, 0, 0, 0})
@@ -310,48 +525,14 @@ __device__ __forceinline__ void cache_stream_body(array_d_t<uint64_t>* dr, uint6
              * per trip (1.5 M pages/s otherwise); on a resident cache this costs one look at a state word per page */
             /* (modes 3 and 4: the helper needs more registers than the kernels themselves, which costs them a third of the
              * waves they run with on a resident cache, hence modes 0 and 1 without) */
-            const uint32_t reach = MODE < 3 || dr->n_ranges != 1 ? 0 : (uint32_t)(r0->cache.n_pages >> 6 > BAM_WAVE_SIZE ? BAM_WAVE_SIZE : r0->cache.n_pages >> 6);
+            const uint32_t reach = MODE < 3 || dr->n_ranges != 1 ? 1 : (uint32_t)(r0->cache.n_pages >> 6 > BAM_WAVE_SIZE ? BAM_WAVE_SIZE : r0->cache.n_pages >> 6);
             for (uint64_t p = 0; p < n_pages_per_wave; p++) {
                 if (MODE >= 3 && reach >= 2 && p % reach == 0) stream_touch(r0, start_page + p, n_pages_per_wave - p < reach ? n_pages_per_wave - p : reach);
                 /* the lane number worked out afresh at every page (two instructions): held in a register across the
                  * loop it is the value the compiler parks in scratch memory, and a reload with its wait costs more */
                 uint32_t lane_now;
                 asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lane_now));
-                const uint64_t start_idx = (start_page + p) * epp + lane_now;
-                if (MODE == 0 || MODE == 4) {
-                    /* operator[] per element, the eight elements a lane reads of a page side by side (array_d_t::seq_read_n) */
-                    for (uint64_t j = 0; j < epp; j += 8 * BAM_WAVE_SIZE) {
-                        size_t at[8];
-                        bool want[8];
-                        uint64_t x[8];
-#pragma unroll
-                        for (int u = 0; u < 8; u++) { at[u] = start_idx + j + u * BAM_WAVE_SIZE; want[u] = j + u * BAM_WAVE_SIZE + lane < epp; }
-                        dr->seq_read_n(at, want, x, elem_view);
-#pragma unroll
-                        for (int u = 0; u < 8; u++) v += want[u] ? x[u] : 0;
-                    }
-                } else {
-                    /* eight elements asked for before the first is used: the window test of an element needs nothing that
-                     * an earlier load brings, so the loads of a page are in flight together */
-                    for (uint64_t j = 0; j < epp; j += 8 * BAM_WAVE_SIZE) {
-                        const uint64_t i0 = start_idx + j;
-                        const uint32_t n_here = (uint32_t)((epp - j + BAM_WAVE_SIZE - 1) / BAM_WAVE_SIZE < 8 ? (epp - j + BAM_WAVE_SIZE - 1) / BAM_WAVE_SIZE : 8);
-                        /* the first element opens the window (the one place where the page can change); when the others
-                         * lie in it, as they do unless a range ends inside the page, they are asked for side by side */
-                        uint64_t acc = (uint64_t)ptr[i0];
-                        if (ptr.covers(i0, i0 + (uint64_t)(n_here - 1) * BAM_WAVE_SIZE)) {
-                            uint64_t x[8];
-                            x[0] = 0;
-#pragma unroll
-                            for (int u = 1; u < 8; u++) x[u] = (uint32_t)u < n_here ? (uint64_t)ptr.peek(i0 + (uint64_t)u * BAM_WAVE_SIZE) : 0;
-                            acc += ((x[0] + x[1]) + (x[2] + x[3])) + ((x[4] + x[5]) + (x[6] + x[7]));
-                        } else {
-#pragma unroll 1
-                            for (uint32_t u = 1; u < n_here; u++) acc += (uint64_t)ptr[i0 + (uint64_t)u * BAM_WAVE_SIZE];
-                        }
-                        v += acc;
-                    }
-                }
+                stream_page<MODE == 0 || MODE == 4, false>(dr, ptr, elem_view, (start_page + p) * epp, epp, lane_now, v);
             }
             elem_view.flush_stats();
         }
@@ -364,7 +545,7 @@ __device__ __forceinline__ void cache_stream_body(array_d_t<uint64_t>* dr, uint6
 /* mode 1 is held to the registers of four waves per SIMD (128; left alone the compiler takes 130): it fits, without a
  * spill, since the lane number is worked out per page rather than kept */
 template <int MODE>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MODE == 1 ? 4 : 1))) void k_cache_stream(array_d_t<uint64_t>* dr, uint64_t n_waves, uint64_t n_pages_per_wave, const uint64_t* assignment, unsigned long long* sum)
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MODE == 1 ? 4 : 1))) void k_cache_stream_whole(array_d_t<uint64_t>* dr, uint64_t n_waves, uint64_t n_pages_per_wave, const uint64_t* assignment, unsigned long long* sum)
 {
     cache_stream_body<MODE>(dr, n_waves, n_pages_per_wave, assignment, sum);
 }
@@ -378,6 +559,103 @@ __global__ __launch_bounds__(256) void k_cache_stream_fetched(array_d_t<uint64_t
 __global__ __launch_bounds__(256) void k_cache_stream_pages(array_d_t<uint64_t>* dr, uint64_t n_waves, uint64_t n_pages_per_wave, const uint64_t* assignment, unsigned long long* sum)
 {
     cache_stream_body<2>(dr, n_waves, n_pages_per_wave, assignment, sum);
+}
+
+/*
+ * Modes 0 and 1 in two launches (arrays of one range).  The first, this kernel, is the reference's kernel
+ * (benchmarks/cache/main.cu:44-114: a wave per run of pages, every element through bam_ptr or operator[]) with pointers
+ * that do not load: a page that is not resident is noted in deferred[wave * n_pages_per_wave + p] and left to the second
+ * launch (k_cache_stream_deferred), which has the miss path.  A kernel that can miss carries the registers and the stack of
+ * the miss path through every page visit (four waves per SIMD, a frame in scratch memory); this one has neither.
+ */
+#ifndef BAM_STREAM_MAX_WAVES
+#define BAM_STREAM_MAX_WAVES 8
+#endif
+template <int MODE>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, BAM_STREAM_MAX_WAVES))) void k_cache_stream(array_d_t<uint64_t>* dr, uint64_t n_waves, uint64_t n_pages_per_wave, const uint64_t* assignment, unsigned long long* partials,
+                                                      uint8_t* deferred, unsigned long long* sum, uint32_t* finished, uint32_t call)
+{
+    static_assert(MODE == 0 || MODE == 1, "the page-wise mode and the fetching modes are kernels of their own");
+    const uint64_t tid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const uint64_t wave = bam::first(tid / BAM_WAVE_SIZE);
+    const uint32_t lane = bam::lane();
+    uint64_t v = 0;
+    if (wave < n_waves) {
+        range_d_t<uint64_t>* r0 = dr->d_ranges;
+        const uint64_t epp = bam::first(r0->n_elems_per_page);
+        const uint64_t start_page = bam::first(assignment ? assignment[wave] : wave * n_pages_per_wave);
+        bam_ptr<uint64_t, true> ptr(dr);
+        bam::range_view<uint64_t> elem_view;
+        if (MODE == 0) elem_view.load(r0);
+        uint64_t later = 0;                 /* bit p % 64: page p is left to the second launch (the same in every lane) */
+        for (uint64_t p = 0; p < n_pages_per_wave; p++) {
+            if (stream_page<MODE == 0, true>(dr, ptr, elem_view, (start_page + p) * epp, epp, lane, v)) later |= 1ull << (p & 63u);
+            if ((p & 63u) == 63u || p + 1 == n_pages_per_wave) {
+                /* the notes of up to 64 pages with one store, a byte per lane */
+                const uint64_t first = p & ~63ull;
+                if (first + lane <= p) deferred[wave * n_pages_per_wave + first + lane] = (uint8_t)((later >> lane) & 1u);
+                if (later) note_work_left(finished, call);
+                later = 0;
+            }
+        }
+        elem_view.flush_stats();
+    }
+    block_accumulate(partials, v);
+    fold_by_last_block(partials, sum, finished);
+}
+
+/*
+ * The second launch: the pages the first one noted, read by waves that can load them.  A wave looks at 64 notes at a
+ * time; the pages it finds noted and not resident it asks for as one batch (one page per lane, taken and dropped again,
+ * as many at a time as a 64th of the cache allows), then it reads them one after the other as the one-launch kernel
+ * would.  On a resident cache the first launch noted nothing, says so, and this one ends at once.  The last workgroup
+ * to finish adds the checksum of what was read here to the first launch's.
+ */
+template <int MODE>
+__global__ __launch_bounds__(256) void k_cache_stream_deferred(array_d_t<uint64_t>* dr, uint64_t n_waves, uint64_t n_pages_per_wave, const uint64_t* assignment,
+                                                               unsigned long long* partials, const uint8_t* deferred, unsigned long long* sum, uint32_t* finished, uint32_t call)
+{
+    if (__hip_atomic_load(finished + BAM_LEFT_WORD, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != call) return;      /* nothing was noted */
+    const uint64_t gwave = ((uint64_t)blockIdx.x * blockDim.x + threadIdx.x) / BAM_WAVE_SIZE, n_gwaves = (uint64_t)gridDim.x * blockDim.x / BAM_WAVE_SIZE;
+    const uint64_t total = n_waves * n_pages_per_wave, n_chunks = (total + BAM_WAVE_SIZE - 1) / BAM_WAVE_SIZE;
+    uint64_t v = 0;
+    bool any = false;
+    for (uint64_t c = gwave; c < n_chunks; c += n_gwaves) {
+        const uint64_t q = c * BAM_WAVE_SIZE + bam::lane();
+        const bool noted = q < total && deferred[q] != 0;
+        const uint64_t m = bam::ballot(noted);
+        if (!m) continue;
+        any = true;
+        range_d_t<uint64_t>* r0 = dr->d_ranges;
+        const uint64_t epp = bam::first(r0->n_elems_per_page);
+        const uint64_t cw = noted ? q / n_pages_per_wave : 0;
+        const uint64_t page = noted ? (assignment ? assignment[cw] : cw * n_pages_per_wave) + q % n_pages_per_wave : 0;
+        {
+            bam::range_view<uint64_t> view;
+            view.load(r0);
+            const uint32_t reach = (uint32_t)(r0->cache.n_pages >> 6 > BAM_WAVE_SIZE ? BAM_WAVE_SIZE : r0->cache.n_pages >> 6);
+            auto touch = [](uint32_t) { return true; };
+            const bool in = noted && page * epp < dr->n_elems;
+            const uint64_t pg = view.page_of(in ? page * epp : 0);
+            const bool absent = in && page_absent(view, pg);
+            if (reach >= 2)
+                for (uint32_t b = 0; b < BAM_WAVE_SIZE; b += reach) {
+                    const bool take = absent && bam::lane() >= b && bam::lane() < b + reach;
+                    if (bam::ballot(take)) view.template acquire_helped<true>(pg, take, false, touch, touch);
+                }
+            view.n_access = view.n_hit = 0;
+        }
+        bam_ptr<uint64_t> ptr(dr);
+        bam::range_view<uint64_t> elem_view;
+        if (MODE == 0) elem_view.load(r0);
+        for (uint64_t mm = m; mm; mm &= mm - 1) {
+            const uint64_t first = bam::bcast(page, bam::first_lane(mm)) * epp;
+            stream_page<MODE == 0, false>(dr, ptr, elem_view, first, epp, bam::lane(), v);
+        }
+        elem_view.flush_stats();
+    }
+    if (bam::ballot(any)) block_accumulate(partials, v);
+    fold_by_last_block(partials, sum, finished);
 }
 
 // ---- raw block benchmark (benchmarks/block/main.cu:99-200) ----
@@ -401,6 +679,42 @@ __global__ void k_block_io(Controller** ctrls, page_cache_d_t* pc, uint32_t req_
         if (write) write_data(pc, qp, start_block, n_blocks, tid);
         else read_data(pc, qp, start_block, n_blocks, tid);
     }
+}
+
+/*
+ * One command per thread, put together by the thread itself from the per-thread queue operations, as the reference's
+ * read_data does it (include/page_cache.h:2009-2054: get_cid, the entry, sq_enqueue, cq_poll, cq_dequeue, put_cid), the
+ * controller addressing cache slot t directly.  Thread t uses queue pair t mod n_qps, so the lanes of a wave are on as many
+ * different queue pairs as there are; the calls take the lanes of one queue at a time.
+ */
+__global__ void k_block_io_per_thread(Controller** ctrls, page_cache_d_t* pc, uint32_t req_size, uint64_t n_reqs, const uint64_t* lbas, int write)
+{
+    const uint64_t tid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (tid >= n_reqs) return;
+    Controller* c = ctrls[0];
+    QueuePair* qp = c->d_qps + tid % c->n_qps;
+    const uint64_t start_block = lbas ? lbas[tid] : (tid * req_size) >> qp->block_size_log;
+    const uint64_t n_blocks = req_size >> qp->block_size_log;
+    if (write) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");      /* what the slot holds has reached memory before the controller fetches it */
+    nvm_cmd_t cmd;
+#pragma unroll
+    for (int i = 0; i < 16; i++) cmd.dword[i] = 0;
+    const uint16_t cid = get_cid(&qp->sq);
+    nvm_cmd_header(&cmd, cid, write ? NVM_IO_WRITE : NVM_IO_READ, qp->nvmNamespace);
+    nvm_cmd_data_ptr(&cmd, pc->prp1[tid], pc->prps ? pc->prp2[tid] : 0);
+    nvm_cmd_rw_blks(&cmd, start_block, (uint16_t)n_blocks);
+    const uint16_t sq_pos = sq_enqueue(&qp->sq, &cmd);
+    (void)sq_pos;
+    uint32_t head = 0, head_ = 0;
+    const uint32_t cq_pos = cq_poll(&qp->cq, cid, &head, &head_);
+    cq_dequeue(&qp->cq, (uint16_t)cq_pos, &qp->sq, head, head_);
+    put_cid(&qp->sq, cid);
+}
+
+/* one wave, the lanes named in `lanes` active: util.h's warp_memcpy of n words */
+__global__ void k_warp_memcpy(uint64_t* dst, const uint64_t* src, uint64_t n, uint64_t lanes)
+{
+    if ((lanes >> bam::lane()) & 1) warp_memcpy(dst, src, (size_t)n);
 }
 
 /*
@@ -875,21 +1189,83 @@ int bam_array_stats(bam_array_t* a, uint64_t* out, int reset)
     BAM_API_END
 }
 
+/* whether the entry points that have a two-launch form may use it on this array: one range, reads of resident pages
+ * without a reference switched on (the first launch reads that way) */
+static bool two_launches_ok(bam_array_t* a)
+{
+    return a->a->adt.n_ranges == 1 && a->a->h_ranges[0].cache.fast_reads != 0;
+}
+
+int bam_array_read_shaped(bam_array_t* a, uint64_t n_reqs, const uint64_t* d_assignment, int shape, uint32_t reads_per_lane, uint32_t block_size,
+                          uint64_t* d_sum, void* stream)
+{
+    if (!a || !d_sum || !d_assignment) return fail(EINVAL, "bam_array_read_shaped: null argument");
+    if (!block_size || block_size % BAM_WAVE_SIZE || block_size > 1024) return fail(EINVAL, "bam_array_read_shaped: block size must be a multiple of 64, at most 1024");
+    if (shape < BAM_READ_ONE_PER_THREAD || shape > BAM_READ_TWO_LAUNCHES) return fail(EINVAL, "bam_array_read_shaped: unknown shape");
+    if (shape == BAM_READ_TWO_LAUNCHES && reads_per_lane != 1 && reads_per_lane != 2 && reads_per_lane != 4 && reads_per_lane != 8)
+        return fail(EINVAL, "bam_array_read_shaped: 1, 2, 4 or 8 reads per lane");
+    if (shape == BAM_READ_TWO_LAUNCHES && !two_launches_ok(a)) return fail(EINVAL, "bam_array_read_shaped: two launches need an array of one range and BAM_FAST_READS on");
+    if (!n_reqs) return 0;
+    BAM_API_BEGIN
+    hipStream_t st = (hipStream_t)stream;
+    array_d_t<uint64_t>* d = a->a->d_array_ptr;
+    unsigned long long* part = (unsigned long long*)a->partials.get();
+    if (shape == BAM_READ_ONE_PER_THREAD) {
+        hipLaunchKernelGGL(k_array_read, dim3(blocks_for(n_reqs, block_size)), dim3(block_size), 0, st, d, n_reqs, d_assignment, (uint64_t)1, (uint64_t)1, part);
+        hipLaunchKernelGGL(k_fold_partials, dim3(1), dim3(1024), 0, st, part, (unsigned long long*)d_sum);
+    } else if (shape == BAM_READ_FOUR_PER_THREAD) {
+        const uint64_t threads = (n_reqs + BAM_READS_PER_LANE - 1) / BAM_READS_PER_LANE;
+        hipLaunchKernelGGL(k_array_read_n_whole, dim3(blocks_for(threads, block_size)), dim3(block_size), 0, st, d, n_reqs, d_assignment, threads, part);
+        hipLaunchKernelGGL(k_fold_partials, dim3(1), dim3(1024), 0, st, part, (unsigned long long*)d_sum);
+    } else {
+        const uint32_t N = reads_per_lane;
+        /* rounds of N reads per thread: as many as leave some eight thousand workgroups */
+        uint32_t rounds = 1;
+        while (rounds < 16 && n_reqs / ((uint64_t)N * rounds * 2 * 256) >= 8192) rounds *= 2;
+        const uint64_t per_thread = (uint64_t)N * rounds;
+        const uint64_t threads = ((n_reqs + per_thread - 1) / per_thread + BAM_WAVE_SIZE - 1) / BAM_WAVE_SIZE * BAM_WAVE_SIZE;
+        const uint64_t n_words = threads / BAM_WAVE_SIZE * per_thread;
+        uint64_t* missed = (uint64_t*)a->notes_for(n_words * sizeof(uint64_t));
+        const dim3 grid(blocks_for(threads, 256)), block(256);
+        unsigned long long* sum = (unsigned long long*)d_sum;
+        uint32_t* fin = (uint32_t*)a->finished.get();
+        const uint32_t call = a->next_call();
+        switch (N) {
+        case 1: hipLaunchKernelGGL(k_array_read_n<1>, grid, block, 0, st, d, n_reqs, d_assignment, threads, rounds, part, missed, sum, fin, call); break;
+        case 2: hipLaunchKernelGGL(k_array_read_n<2>, grid, block, 0, st, d, n_reqs, d_assignment, threads, rounds, part, missed, sum, fin, call); break;
+        case 4: hipLaunchKernelGGL(k_array_read_n<4>, grid, block, 0, st, d, n_reqs, d_assignment, threads, rounds, part, missed, sum, fin, call); break;
+        default: hipLaunchKernelGGL(k_array_read_n<8>, grid, block, 0, st, d, n_reqs, d_assignment, threads, rounds, part, missed, sum, fin, call); break;
+        }
+        /* the second launch: as many words per wave as leave some eight thousand waves' worth of chunks */
+        uint32_t words = 1;
+        while (words < BAM_DEFER_MAX_WORDS && n_words / (words * 2) >= 8192) words *= 2;
+        const uint64_t n_chunks = (n_words + words - 1) / words;
+        const uint64_t waves = n_chunks < 16384 ? n_chunks : 16384;
+        hipLaunchKernelGGL(k_array_read_deferred, dim3(blocks_for(waves * BAM_WAVE_SIZE, 256)), dim3(256), 0, st, d, n_reqs, d_assignment, missed, n_words, words,
+                           part, sum, fin, call);
+    }
+    hip_err_chk(hipGetLastError());
+    BAM_API_END
+}
+
 int bam_array_read(bam_array_t* a, uint64_t n_reqs, const uint64_t* d_assignment, uint64_t stride, uint64_t reqs_per_thread,
                    uint32_t block_size, uint64_t* d_sum, void* stream)
 {
     if (!a || !d_sum) return fail(EINVAL, "bam_array_read: null argument");
     if (!block_size || block_size % BAM_WAVE_SIZE || block_size > 1024) return fail(EINVAL, "bam_array_read: block size must be a multiple of 64, at most 1024");
     if (!n_reqs) return 0;
-    BAM_API_BEGIN
-    /* a large launch of scattered requests, one read each: four requests per thread (results and counters are the same) */
+    /* a large launch of scattered requests, one read each: in two launches where the array allows it, else four requests per
+     * thread (results and counters are the same) */
     if (d_assignment && reqs_per_thread == 1 && n_reqs >= (1ull << 16)) {
-        const uint64_t threads = (n_reqs + BAM_READS_PER_LANE - 1) / BAM_READS_PER_LANE;
-        hipLaunchKernelGGL(k_array_read_n, dim3(blocks_for(threads, block_size)), dim3(block_size), 0, (hipStream_t)stream,
-                           a->a->d_array_ptr, n_reqs, d_assignment, threads, (unsigned long long*)a->partials.get());
-    } else
-        hipLaunchKernelGGL(k_array_read, dim3(blocks_for(n_reqs, block_size)), dim3(block_size), 0, (hipStream_t)stream,
-                           a->a->d_array_ptr, n_reqs, d_assignment, stride, reqs_per_thread, (unsigned long long*)a->partials.get());
+        static const int shape_env = getenv("BAM_READ_SHAPE") ? atoi(getenv("BAM_READ_SHAPE")) : 0;
+        static const int lanes_env = getenv("BAM_READS_PER_LANE") ? atoi(getenv("BAM_READS_PER_LANE")) : BAM_READS_PER_LANE;
+        int shape = two_launches_ok(a) ? BAM_READ_TWO_LAUNCHES : BAM_READ_FOUR_PER_THREAD;
+        if (shape_env >= BAM_READ_ONE_PER_THREAD && shape_env <= BAM_READ_TWO_LAUNCHES && (shape_env != BAM_READ_TWO_LAUNCHES || two_launches_ok(a))) shape = shape_env;
+        return bam_array_read_shaped(a, n_reqs, d_assignment, shape, (uint32_t)lanes_env, block_size, d_sum, stream);
+    }
+    BAM_API_BEGIN
+    hipLaunchKernelGGL(k_array_read, dim3(blocks_for(n_reqs, block_size)), dim3(block_size), 0, (hipStream_t)stream,
+                       a->a->d_array_ptr, n_reqs, d_assignment, stride, reqs_per_thread, (unsigned long long*)a->partials.get());
     hipLaunchKernelGGL(k_fold_partials, dim3(1), dim3(1024), 0, (hipStream_t)stream, (unsigned long long*)a->partials.get(), (unsigned long long*)d_sum);
     hip_err_chk(hipGetLastError());
     BAM_API_END
@@ -994,15 +1370,31 @@ int bam_cache_stream(bam_array_t* a, uint64_t n_waves, uint64_t n_pages_per_wave
                      uint64_t* d_sum, void* stream)
 {
     if (!a || !d_sum) return fail(EINVAL, "bam_cache_stream: null argument");
-    if (mode < 0 || mode > 4) return fail(EINVAL, "bam_cache_stream: mode must be 0 to 4");
+    if (mode < 0 || mode > 6) return fail(EINVAL, "bam_cache_stream: mode must be 0 to 6");
     if (!n_waves || !n_pages_per_wave) return 0;
     BAM_API_BEGIN
     const uint32_t bs = 256;
     const dim3 grid(blocks_for(n_waves * BAM_WAVE_SIZE, bs)), block(bs);
     array_d_t<uint64_t>* d = a->a->d_array_ptr;
     unsigned long long* s = (unsigned long long*)a->partials.get();
-    if (mode == 0) hipLaunchKernelGGL(k_cache_stream<0>, grid, block, 0, (hipStream_t)stream, d, n_waves, n_pages_per_wave, d_assignment, s);
-    else if (mode == 1) hipLaunchKernelGGL(k_cache_stream<1>, grid, block, 0, (hipStream_t)stream, d, n_waves, n_pages_per_wave, d_assignment, s);
+    if (mode <= 1 && two_launches_ok(a)) {
+        /* the kernel that reads what is resident, then the one that reads what it noted (and folds the checksum) */
+        const uint64_t total = n_waves * n_pages_per_wave;
+        uint8_t* notes = (uint8_t*)a->notes_for(total);
+        unsigned long long* sum = (unsigned long long*)d_sum;
+        uint32_t* fin = (uint32_t*)a->finished.get();
+        const uint32_t call = a->next_call();
+        if (mode == 0) hipLaunchKernelGGL(k_cache_stream<0>, grid, block, 0, (hipStream_t)stream, d, n_waves, n_pages_per_wave, d_assignment, s, notes, sum, fin, call);
+        else hipLaunchKernelGGL(k_cache_stream<1>, grid, block, 0, (hipStream_t)stream, d, n_waves, n_pages_per_wave, d_assignment, s, notes, sum, fin, call);
+        const uint64_t n_chunks = (total + BAM_WAVE_SIZE - 1) / BAM_WAVE_SIZE;
+        const dim3 grid2(blocks_for((n_chunks < 1024 ? n_chunks : 1024) * BAM_WAVE_SIZE, bs));      /* a thousand waves with 64 pages each keep the store busy; when nothing was noted the fewer the better */
+        if (mode == 0) hipLaunchKernelGGL(k_cache_stream_deferred<0>, grid2, block, 0, (hipStream_t)stream, d, n_waves, n_pages_per_wave, d_assignment, s, notes, sum, fin, call);
+        else hipLaunchKernelGGL(k_cache_stream_deferred<1>, grid2, block, 0, (hipStream_t)stream, d, n_waves, n_pages_per_wave, d_assignment, s, notes, sum, fin, call);
+        hip_err_chk(hipGetLastError());
+        return 0;
+    }
+    if (mode == 0 || mode == 5) hipLaunchKernelGGL(k_cache_stream_whole<0>, grid, block, 0, (hipStream_t)stream, d, n_waves, n_pages_per_wave, d_assignment, s);
+    else if (mode == 1 || mode == 6) hipLaunchKernelGGL(k_cache_stream_whole<1>, grid, block, 0, (hipStream_t)stream, d, n_waves, n_pages_per_wave, d_assignment, s);
     else if (mode >= 3) {
         /* the lead is counted in pages here: one finished streaming wave stands for its n_pages_per_wave pages */
         fetch_plan fp = make_fetch_plan(a, 1, bs, 1, (hipStream_t)stream);
@@ -1024,10 +1416,25 @@ int bam_block_io(bam_ctrl_t* c, bam_page_cache_t* pc, uint64_t n_reqs, uint32_t 
     if (!block_size || block_size % BAM_WAVE_SIZE || block_size > 1024) return fail(EINVAL, "bam_block_io: block size must be a multiple of 64, at most 1024");
     if (n_reqs > pc->pc->pdt.n_pages) return fail(EINVAL, "bam_block_io: needs one cache page per request");
     if (!req_bytes || req_bytes % c->c->blk_size || req_bytes > pc->pc->pdt.page_size) return fail(EINVAL, "bam_block_io: request size must be a multiple of the block size and fit a page");
+    if (queue_policy < 0 || queue_policy > 2) return fail(EINVAL, "bam_block_io: queue policy must be 0, 1 or 2");
     if (!n_reqs) return 0;
     BAM_API_BEGIN
-    hipLaunchKernelGGL(k_block_io, dim3(blocks_for(n_reqs, block_size)), dim3(block_size), 0, (hipStream_t)stream,
-                       pc->pc->pdt.d_ctrls, pc->pc->d_pc_ptr, req_bytes, n_reqs, d_lbas, write, queue_policy);
+    if (queue_policy == 2) {
+        if (!pc->pc->pdt.prp1) return fail(EINVAL, "bam_block_io: the per-thread route addresses the cache slots directly, and this cache has no bus addresses for them");
+        hipLaunchKernelGGL(k_block_io_per_thread, dim3(blocks_for(n_reqs, block_size)), dim3(block_size), 0, (hipStream_t)stream,
+                           pc->pc->pdt.d_ctrls, pc->pc->d_pc_ptr, req_bytes, n_reqs, d_lbas, write);
+    } else
+        hipLaunchKernelGGL(k_block_io, dim3(blocks_for(n_reqs, block_size)), dim3(block_size), 0, (hipStream_t)stream,
+                           pc->pc->pdt.d_ctrls, pc->pc->d_pc_ptr, req_bytes, n_reqs, d_lbas, write, queue_policy);
+    hip_err_chk(hipGetLastError());
+    BAM_API_END
+}
+
+int bam_warp_memcpy(uint64_t* d_dst, const uint64_t* d_src, uint64_t n_words, uint64_t lanes, void* stream)
+{
+    if (!d_dst || !d_src || !lanes) return fail(EINVAL, "bam_warp_memcpy: null argument or no lane");
+    BAM_API_BEGIN
+    hipLaunchKernelGGL(k_warp_memcpy, dim3(1), dim3(BAM_WAVE_SIZE), 0, (hipStream_t)stream, d_dst, d_src, n_words, lanes);
     hip_err_chk(hipGetLastError());
     BAM_API_END
 }

@@ -51,7 +51,23 @@ struct bam_ctrl { Controller* c; };
 struct bam_page_cache { page_cache_t* pc; Controller* ctrl; };      /* ctrl: the first controller of the cache */
 struct bam_range { range_t<uint64_t>* r; };
 #define BAM_SUM_PARTIALS 4096
-struct bam_array { array_t<uint64_t>* a; BufferPtr partials, progress; std::shared_ptr<void> graph; };      /* progress: the word the computing workgroups of vectoradd, reduction and scan count themselves off in; graph: what bam_array_set_graph prepared (bam_graph.hip) */
+struct bam_array {
+    array_t<uint64_t>* a;
+    BufferPtr partials, progress;       /* progress: the word the computing workgroups of vectoradd, reduction and scan count themselves off in */
+    std::shared_ptr<void> graph;        /* what bam_array_set_graph prepared (bam_graph.hip) */
+    /* the entry points that read in two launches: what the first launch leaves for the second (grown on demand, kept),
+     * and the count of workgroups of the second that have finished (zero between launches) */
+    BufferPtr notes, finished;
+    size_t notes_bytes = 0;
+    uint32_t calls = 0;
+    void* notes_for(size_t bytes)
+    {
+        if (bytes > notes_bytes) { notes = createBuffer(bytes, 0); notes_bytes = bytes; }
+        if (!finished) finished = createBuffer(512, 0);      /* [0 .. 64] the count of workgroups done, [96] the call that left work for its second launch */
+        return notes.get();
+    }
+    uint32_t next_call() { if (++calls == 0) calls = 1; return calls; }      /* never 0: the word starts out as that */
+};
 struct bam_range32 { range_t<uint32_t>* r; };
 struct bam_array32 { array_t<uint32_t>* a; BufferPtr partials; };      /* partials: [BAM_SUM_PARTIALS] checksum shards, zero between launches */
 

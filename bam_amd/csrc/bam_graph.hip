@@ -2,9 +2,15 @@
 // PageRank and SSSP over CSR graphs whose neighbour ids (and weights) are read through the page cache.  Kernel shapes
 // follow the reference's benchmark kernels (cited per kernel); lane arithmetic is for 64-wide waves.
 #include "bam_capi_internal.h"
-#include <hipcub/hipcub.hpp>
 
 namespace {
+
+/* the per-vertex kernels (the group walk below) are held to the registers of this many waves per SIMD: left alone the
+ * compiler takes what a workgroup of two waves may have, all 512, and one wave per SIMD is what runs */
+#ifndef BAM_GRAPH_WAVES
+#define BAM_GRAPH_WAVES 2
+#endif
+#define BAM_GRAPH_KERNEL_WAVES __attribute__((amdgpu_waves_per_eu(BAM_GRAPH_WAVES)))
 
 // ---- BFS: wave per `coarse` vertices, edges through bam_ptr (benchmarks/bfs/main.cu:658-689) ----
 #define MYINFINITY 0xFFFFFFFFu
@@ -52,10 +58,10 @@ struct list_read_ahead {
         if (adopt) for (uint32_t i = 0; i < k; i++) m &= m - 1;
         const uint64_t adopted = bam::shfl(pl, adopt ? bam::first_lane(m) : 0u);
         const bool take_1 = take_f || adopt;
-        if (bam::ballot(take_1)) view.acquire_helped(take_f ? pf : adopted, take_1, false, touch, touch);
+        if (bam::ballot(take_1)) view.template acquire_helped<true>(take_f ? pf : adopted, take_1, false, touch, touch);
         /* last pages nobody had a lane for */
         const bool take_2 = take_l && bam::popc(need_l & bam::lanes_below(bam::lane())) >= bam::popc(idle);
-        if (bam::ballot(take_2)) view.acquire_helped(pl, take_2, false, touch, touch);
+        if (bam::ballot(take_2)) view.template acquire_helped<true>(pl, take_2, false, touch, touch);
         view.n_access = view.n_hit = 0;
     }
     /*
@@ -98,7 +104,7 @@ struct list_read_ahead {
 #pragma unroll
             for (uint32_t o = BAM_WAVE_SIZE / 2; o; o >>= 1) m |= bam::shfl(m, lane ^ o);
             const bool take = ((m >> lane) & 1) != 0 && page_absent(view, c + lane);
-            if (bam::ballot(take)) view.acquire_helped(c + lane, take, false, touch, touch);
+            if (bam::ballot(take)) view.template acquire_helped<true>(c + lane, take, false, touch, touch);
             seen |= m;
         }
         view.n_access = view.n_hit = 0;
@@ -123,7 +129,7 @@ struct list_read_ahead {
         auto touch = [](uint32_t) { return true; };
         const uint64_t page = want ? view.page_of(start) + (bam::lane() & 15u) : 0;
         const bool take = want && end > start && page <= view.page_of(end - 1) && page_absent(view, page);
-        if (bam::ballot(take)) view.acquire_helped(page, take, false, touch, touch);
+        if (bam::ballot(take)) view.template acquire_helped<true>(page, take, false, touch, touch);
         view.n_access = view.n_hit = 0;
         return true;
     }
@@ -136,7 +142,7 @@ struct list_read_ahead {
         const uint64_t p = pg + bam::lane();
         auto touch = [](uint32_t) { return true; };
         const bool take = bam::lane() < reach && p <= last_page && page_absent(view, p);
-        if (bam::ballot(take)) view.acquire_helped(p, take, false, touch, touch);
+        if (bam::ballot(take)) view.template acquire_helped<true>(p, take, false, touch, touch);
         asked_to = pg + reach;
         view.n_access = view.n_hit = 0;         /* not accesses of the kernel's own: kept out of the counters */
     }
@@ -369,7 +375,7 @@ __device__ __forceinline__ void walk_vertex_groups(array_d_t<uint64_t>* da, cons
                            [&](uint64_t i, uint64_t& v) { v = i; return active(i); }, active, visit, with);
 }
 
-__global__ __launch_bounds__(128) void k_bfs_coalesce_coarse_ptr_pc(array_d_t<uint64_t>* da, uint32_t* label, const uint32_t level, const uint64_t vertex_count,
+__global__ __launch_bounds__(128) BAM_GRAPH_KERNEL_WAVES void k_bfs_coalesce_coarse_ptr_pc(array_d_t<uint64_t>* da, uint32_t* label, const uint32_t level, const uint64_t vertex_count,
                                                                    const uint64_t* vertexList, uint64_t* changed, uint64_t coarse,
                                                                    const heavy_piece_t* heavy, uint64_t n_heavy, unsigned long long* next_work)
 {
@@ -454,7 +460,7 @@ __device__ __forceinline__ void bfs_frontier_visit(uint32_t* label, const uint32
     next_frontier[pos + bam::rank_in(mask)] = (uint32_t)next;
 }
 
-__global__ __launch_bounds__(128) void k_bfs_frontier_coalesce_ptr_pc(array_d_t<uint64_t>* da, uint32_t* label, const uint32_t level, const uint64_t* vertexList,
+__global__ __launch_bounds__(128) BAM_GRAPH_KERNEL_WAVES void k_bfs_frontier_coalesce_ptr_pc(array_d_t<uint64_t>* da, uint32_t* label, const uint32_t level, const uint64_t* vertexList,
                                                                      const uint32_t* curr_frontier, const uint64_t curr_size, uint32_t* next_frontier,
                                                                      unsigned long long* next_size, uint64_t group,
                                                                      const heavy_piece_t* heavy, uint64_t n_heavy, unsigned long long* next_work, bool sorted)
@@ -464,6 +470,59 @@ __global__ __launch_bounds__(128) void k_bfs_frontier_coalesce_ptr_pc(array_d_t<
                             [&](uint64_t v) { return label[v] == level; },
                             [&](uint64_t, uint64_t next, uint64_t) { bfs_frontier_visit(label, level, next_frontier, next_size, next); },
                             nullptr, sorted);
+}
+
+/*
+ * The queue of a level put in the order of its vertices.  A vertex enters a queue once, so the entries are distinct, and
+ * sorting distinct numbers below V is marking them in a map of V bits and reading the map front to back: four small
+ * kernels (mark; count the marks of every 4096 vertices, a wave each; running sums of those counts by one workgroup;
+ * write the vertices out, a wave per 4096 again, and clear the map), a few microseconds a level for 2^24 vertices,
+ * and no library.
+ */
+__global__ void k_queue_mark(const uint32_t* __restrict__ queue, const uint64_t n, unsigned long long* bits)
+{
+    const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) { const uint32_t v = queue[i]; atomicOr(&bits[v >> 6], 1ull << (v & 63u)); }
+}
+__global__ void k_bits_count(const unsigned long long* __restrict__ bits, const uint64_t n_words, uint32_t* totals)
+{
+    const uint64_t wave = ((uint64_t)blockIdx.x * blockDim.x + threadIdx.x) / BAM_WAVE_SIZE, at = wave * BAM_WAVE_SIZE + bam::lane();
+    const uint64_t c = wave_sum((uint64_t)bam::popc(at < n_words ? bits[at] : 0ull));
+    if (bam::lane() == 0 && wave * BAM_WAVE_SIZE < n_words) totals[wave] = (uint32_t)c;
+}
+/* totals[k] <- totals[0] + ... + totals[k - 1]; one workgroup of 1024 threads, a run of entries per thread */
+__global__ void k_totals_scan(uint32_t* totals, const uint64_t n)
+{
+    __shared__ uint32_t sums[1024];
+    const uint64_t per = (n + blockDim.x - 1) / blockDim.x, a = threadIdx.x * per, b = a + per < n ? a + per : n;
+    uint32_t mine = 0;
+    for (uint64_t k = a; k < b; k++) mine += totals[k];
+    sums[threadIdx.x] = mine;
+    __syncthreads();
+    for (uint32_t o = 1; o < blockDim.x; o <<= 1) {
+        const uint32_t add = threadIdx.x >= o ? sums[threadIdx.x - o] : 0;
+        __syncthreads();
+        sums[threadIdx.x] += add;
+        __syncthreads();
+    }
+    uint32_t run = sums[threadIdx.x] - mine;
+    for (uint64_t k = a; k < b; k++) { const uint32_t t = totals[k]; totals[k] = run; run += t; }
+}
+__global__ void k_bits_emit(unsigned long long* bits, const uint64_t n_words, const uint32_t* __restrict__ first_of_wave, uint32_t* out)
+{
+    const uint64_t wave = ((uint64_t)blockIdx.x * blockDim.x + threadIdx.x) / BAM_WAVE_SIZE, at = wave * BAM_WAVE_SIZE + bam::lane();
+    if (wave * BAM_WAVE_SIZE >= n_words) return;
+    unsigned long long w = at < n_words ? bits[at] : 0ull;
+    if (w) bits[at] = 0;
+    const uint32_t c = bam::popc(w);
+    uint32_t incl = c;
+#pragma unroll
+    for (uint32_t o = 1; o < BAM_WAVE_SIZE; o <<= 1) {
+        const uint32_t u = bam::shfl(incl, bam::lane() >= o ? bam::lane() - o : bam::lane());
+        if (bam::lane() >= o) incl += u;
+    }
+    uint32_t pos = first_of_wave[wave] + incl - c;
+    for (; w; w &= w - 1) out[pos++] = (uint32_t)(at * 64 + (uint64_t)__builtin_ctzll(w));
 }
 
 // ---- CC: min-label propagation (benchmarks/cc/main.cu:123-144, 595-617) ----
@@ -480,7 +539,7 @@ __device__ __forceinline__ void cc_compute(uint64_t cid, unsigned long long* com
     *changed = true;
 }
 
-__global__ __launch_bounds__(128) void k_cc_coalesce_coarse_ptr_pc(array_d_t<uint64_t>* da, bool* curr_visit, bool* next_visit, uint64_t vertex_count,
+__global__ __launch_bounds__(128) BAM_GRAPH_KERNEL_WAVES void k_cc_coalesce_coarse_ptr_pc(array_d_t<uint64_t>* da, bool* curr_visit, bool* next_visit, uint64_t vertex_count,
                                                                   const uint64_t* vertexList, unsigned long long* comp, bool* changed, uint64_t coarse,
                                                                   const heavy_piece_t* heavy, uint64_t n_heavy, unsigned long long* next_work, uint32_t sweep)
 {
@@ -622,7 +681,7 @@ __global__ void k_pr_initialize(bool* label, float* delta, float* residual, floa
 
 /* every neighbour of a flagged vertex receives the vertex's delta: the group walk of the per-vertex graph kernels; the flags
  * are cleared by the host loop after the sweep */
-__global__ __launch_bounds__(128) void k_pr_coalesce_pc(array_d_t<uint64_t>* da, const bool* label, const float* delta, float* residual,
+__global__ __launch_bounds__(128) BAM_GRAPH_KERNEL_WAVES void k_pr_coalesce_pc(array_d_t<uint64_t>* da, const bool* label, const float* delta, float* residual,
                                                         const uint64_t vertex_count, const uint64_t* vertexList, uint64_t group,
                                                         const heavy_piece_t* heavy, uint64_t n_heavy, unsigned long long* next_work, uint32_t sweep)
 {
@@ -667,7 +726,7 @@ __device__ __forceinline__ void sssp_relax(uint32_t* newCostList, const bam_ptr<
 }
 
 template <bool FLOAT>
-__global__ __launch_bounds__(128) void k_sssp_coalesce_pc(array_d_t<uint64_t>* de, array_d_t<uint32_t>* dw, const bool* label, uint32_t* newCostList,
+__global__ __launch_bounds__(128) BAM_GRAPH_KERNEL_WAVES void k_sssp_coalesce_pc(array_d_t<uint64_t>* de, array_d_t<uint32_t>* dw, const bool* label, uint32_t* newCostList,
                                                           const uint64_t vertex_count, const uint64_t* vertexList, uint64_t group,
                                                           const heavy_piece_t* heavy, uint64_t n_heavy, unsigned long long* next_work, uint32_t sweep)
 {
@@ -734,6 +793,7 @@ struct graph_plan {
     by_page_plan bp;
     bool bp_built = false;
     BufferPtr bytes_a, bytes_b, floats_a, floats_b, words_a;      /* per-vertex buffers: flags, PageRank's delta and residual, SSSP's new costs */
+    BufferPtr queue_a, queue_b, queue_bits, queue_totals;         /* bam_bfs_frontier: the two queues, the bit map that puts a queue in order and its counts per 4096 vertices */
 
     int build(bam_array_t* edges, const uint64_t* d_offsets, uint64_t nv, uint64_t other_cache_pages, hipStream_t st)
     {
@@ -845,6 +905,13 @@ int bam_array_set_graph(bam_array_t* edges, const uint64_t* d_offsets, uint64_t 
     /* the per-vertex buffers the sweeps use, so that no later call has to allocate */
     graph_plan::sized(p->bytes_a, n_vertices); graph_plan::sized(p->bytes_b, n_vertices);
     graph_plan::sized(p->floats_a, n_vertices * sizeof(float)); graph_plan::sized(p->floats_b, n_vertices * sizeof(float));
+    if (n_vertices <= 0xFFFFFFFFull) {
+        /* bam_bfs_frontier's queues and what puts them in order */
+        const uint64_t n_words = (n_vertices + 63) / 64;
+        graph_plan::sized(p->queue_a, n_vertices * sizeof(uint32_t)); graph_plan::sized(p->queue_b, n_vertices * sizeof(uint32_t));
+        graph_plan::sized(p->queue_bits, n_words * sizeof(unsigned long long));
+        graph_plan::sized(p->queue_totals, (n_words + BAM_WAVE_SIZE - 1) / BAM_WAVE_SIZE * sizeof(uint32_t));
+    }
     hip_err_chk(hipStreamSynchronize(st));
     edges->graph = p;
     BAM_API_END
@@ -979,10 +1046,13 @@ int bam_bfs_frontier(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_v
     hipStream_t st = (hipStream_t)stream;
     std::unique_ptr<graph_plan> local;
     graph_plan* pl = plan_for(edges, d_offsets, n_vertices, 0, st, local);
-    /* two queues of at most every vertex once (benchmarks/bfs/main.cu:1489-1492); the size of the next one is the reference's `changed` */
-    BufferPtr queue_a = createBuffer(n_vertices * sizeof(uint32_t), 0), queue_b = createBuffer(n_vertices * sizeof(uint32_t), 0);
-    uint32_t* curr = (uint32_t*)queue_a.get();
-    uint32_t* next = (uint32_t*)queue_b.get();
+    /* two queues of at most every vertex once (benchmarks/bfs/main.cu:1489-1492); the size of the next one is the reference's `changed`.
+     * They, and what puts a queue in order, belong to the plan: with bam_array_set_graph nothing is allocated here */
+    uint32_t* curr = (uint32_t*)graph_plan::sized(pl->queue_a, n_vertices * sizeof(uint32_t));
+    uint32_t* next = (uint32_t*)graph_plan::sized(pl->queue_b, n_vertices * sizeof(uint32_t));
+    const uint64_t n_words = (n_vertices + 63) / 64, n_bit_waves = (n_words + BAM_WAVE_SIZE - 1) / BAM_WAVE_SIZE;
+    unsigned long long* bits = (unsigned long long*)graph_plan::sized(pl->queue_bits, n_words * sizeof(unsigned long long));      /* zero between levels */
+    uint32_t* totals = (uint32_t*)graph_plan::sized(pl->queue_totals, n_bit_waves * sizeof(uint32_t));
     unsigned long long* next_size = (unsigned long long*)pl->changed;
     const uint32_t src32 = (uint32_t)src;
     hip_err_chk(hipMemsetAsync(d_labels, 0xFF, n_vertices * sizeof(uint32_t), st));
@@ -995,11 +1065,6 @@ int bam_bfs_frontier(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_v
     unsigned long long active = 1;
     const char* e = getenv("BAM_FRONTIER_SORT");
     const bool sort_queue = !e || atoi(e) != 0;
-    int vertex_bits = 1;
-    while (vertex_bits < 32 && (1ull << vertex_bits) < n_vertices) vertex_bits++;
-    size_t sort_bytes = 0;
-    if (sort_queue) hip_err_chk(hipcub::DeviceRadixSort::SortKeys(nullptr, sort_bytes, curr, next, (int)std::min<uint64_t>(n_vertices, 0x7FFFFFFFull), 0, vertex_bits, st));
-    BufferPtr sort_tmp = createBuffer(sort_bytes ? sort_bytes : 8, 0);
     do {
         hipLaunchKernelGGL(k_bfs_frontier_coalesce_ptr_pc, dim3(pl->blocks(active, group)), dim3(threads), 0, st, edges->a->d_array_ptr, d_labels, level,
                            d_offsets, curr, (uint64_t)active, next, next_size, group, pl->pieces, pl->n_pieces, pl->next_work(), sorted);
@@ -1007,15 +1072,18 @@ int bam_bfs_frontier(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_v
         iter++; level++;
         pl->level_end(st);
         active = *pl->host_flag;
-        sorted = sort_queue && active <= 0x7FFFFFFFull;
+        sorted = sort_queue;
         group = sorted ? pl->group : BAM_WAVE_SIZE;
         if (sorted && active > 1) {
-            /* the queue comes out in the order of discovery; sorted by vertex, the level reads the edge array front to back
-             * (neighbouring lists share pages, a page is not evicted between two of its lists, and the pages under the
-             * lists of a group of entries can be asked for together as in the sweep over all vertices).  The sorted queue
-             * goes into the buffer the level just walked, so the two do not change places. */
-            size_t need = sort_bytes;
-            hip_err_chk(hipcub::DeviceRadixSort::SortKeys(sort_tmp.get(), need, next, curr, (int)active, 0, vertex_bits, st));
+            /* the queue comes out in the order of discovery; in the order of the vertices the level reads the edge array
+             * front to back (neighbouring lists share pages, a page is not evicted between two of its lists, and the pages
+             * under the lists of a group of entries can be asked for together as in the sweep over all vertices).  The
+             * ordered queue goes into the buffer the level just walked, so the two do not change places. */
+            hipLaunchKernelGGL(k_queue_mark, dim3(blocks_for(active, 256)), dim3(256), 0, st, next, (uint64_t)active, bits);
+            hipLaunchKernelGGL(k_bits_count, dim3(blocks_for(n_bit_waves * BAM_WAVE_SIZE, 256)), dim3(256), 0, st, bits, n_words, totals);
+            hipLaunchKernelGGL(k_totals_scan, dim3(1), dim3(1024), 0, st, totals, n_bit_waves);
+            hipLaunchKernelGGL(k_bits_emit, dim3(blocks_for(n_bit_waves * BAM_WAVE_SIZE, 256)), dim3(256), 0, st, bits, n_words, totals, curr);
+            hip_err_chk(hipGetLastError());
         } else
             std::swap(curr, next);
     } while (active);

@@ -23,6 +23,7 @@
 #include <thread>
 #include <fcntl.h>
 #include <sys/mman.h>
+#include <sys/stat.h>
 #include <unistd.h>
 
 namespace {
@@ -112,6 +113,11 @@ int nvm_ctrl_init(nvm_ctrl_t** ctrl, int fd)
     if (!ctrl) return EINVAL;
     *ctrl = nullptr;
     if (fcntl(fd, F_GETFL) == -1) return errno;
+    /* a regular file shorter than the window maps all the same, and the first register read behind its end would be a
+     * bus error instead of an error code */
+    struct stat sb;
+    if (fstat(fd, &sb) == -1) return errno;
+    if (S_ISREG(sb.st_mode) && (uint64_t)sb.st_size < NVM_CTRL_MEM_MINSIZE) return ENODEV;
     void* mm = mmap(nullptr, NVM_CTRL_MEM_MINSIZE, PROT_READ | PROT_WRITE, MAP_SHARED, fd, 0);
     if (mm == MAP_FAILED) return errno ? errno : ENODEV;
     int err = nvm_raw_ctrl_init(ctrl, mm, NVM_CTRL_MEM_MINSIZE);

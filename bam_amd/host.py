@@ -220,6 +220,19 @@ class Array:
         self.read_async(n_reqs, s, assignment, stride, reqs_per_thread, block_size)
         return int(s.item()) & MASK64
 
+    ONE_PER_THREAD, FOUR_PER_THREAD, TWO_LAUNCHES = 1, 2, 3
+
+    def read_shaped_async(self, n_reqs, d_sum, assignment, shape, reads_per_lane=4, block_size=64):
+        _chk(self.L.bam_array_read_shaped(self.h, n_reqs, _ptr(assignment), shape, reads_per_lane, block_size, _ptr(d_sum), _stream()),
+             "bam_array_read_shaped")
+
+    def read_shaped(self, n_reqs, assignment, shape, reads_per_lane=4, block_size=64):
+        """The scattered reads of read() with the launch shape named: ONE_PER_THREAD (the reference's kernel as it is),
+        FOUR_PER_THREAD, or TWO_LAUNCHES with 1, 2, 4 or 8 reads per lane in the first."""
+        s = self._sum_buf()
+        self.read_shaped_async(n_reqs, s, assignment, shape, reads_per_lane, block_size)
+        return int(s.item()) & MASK64
+
     def set_graph(self, offsets=None):
         """Prepare (or with None drop) what the graph entry points need for the CSR whose neighbour ids this array holds;
         later calls with the same offsets tensor allocate nothing."""

@@ -100,6 +100,21 @@ int bam_array_stats(bam_array_t* a, uint64_t* out, int reset);
  * and t + 3n/4 side by side (array_d_t::seq_read_n): the same reads, sum and counters, four of them in flight per lane. */
 int bam_array_read(bam_array_t* a, uint64_t n_reqs, const uint64_t* d_assignment, uint64_t stride, uint64_t reqs_per_thread,
                    uint32_t block_size, uint64_t* d_sum, void* stream);
+/* The same scattered requests (thread t reads element d_assignment[t] once; sum into *d_sum) with the launch shape named,
+ * whatever the size of the launch; sums and counters of accesses do not depend on the shape.
+ *   BAM_READ_ONE_PER_THREAD   the reference's kernel as it is: one thread per request, one launch (benchmarks/array/main.cu:43-65)
+ *   BAM_READ_FOUR_PER_THREAD  a quarter of the threads, four requests per thread side by side, one launch
+ *   BAM_READ_TWO_LAUNCHES     a first launch reads what is resident, reads_per_lane (1, 2, 4, 8) requests per thread, with a
+ *                             kernel that cannot miss (no call, no stack, a fraction of the registers) and notes the rest;
+ *                             a second launch reads the rest, one request per lane and 64 per wave whatever the share of
+ *                             misses was.  Arrays of one range only (EINVAL otherwise).
+ * bam_array_read picks BAM_READ_TWO_LAUNCHES with four reads per lane for launches of 2^16 requests and more where the array
+ * allows it (BAM_READ_FOUR_PER_THREAD where not) and BAM_READ_ONE_PER_THREAD below that. */
+#define BAM_READ_ONE_PER_THREAD  1
+#define BAM_READ_FOUR_PER_THREAD 2
+#define BAM_READ_TWO_LAUNCHES    3
+int bam_array_read_shaped(bam_array_t* a, uint64_t n_reqs, const uint64_t* d_assignment, int shape, uint32_t reads_per_lane, uint32_t block_size,
+                          uint64_t* d_sum, void* stream);
 /* the same requests with the values handed out: d_out[t] = element d_assignment[t] (or t * stride); what a kernel of the
  * reference's benchmark would hold in its register after array_d_t::operator[] (benchmarks/array/main.cu:57) */
 int bam_array_gather(bam_array_t* a, uint64_t n_reqs, const uint64_t* d_assignment, uint64_t stride, uint32_t block_size, uint64_t* d_out, void* stream);
@@ -132,19 +147,28 @@ int bam_sqe_image(uint16_t cid, uint8_t opcode, uint32_t nsid, uint64_t prp1, ui
  * One wave per run of n_pages_per_wave whole pages starting at page d_assignment[w] (or w * n_pages_per_wave),
  * every element read once and summed into *d_sum.  mode 0: array_d_t::operator[] per element,
  * mode 1: bam_ptr per element (the reference's kernel, 64-wide), mode 2: one acquire per page and
- * streamed 8-byte loads (what the hit-path roofline is measured on); modes 3 and 4: modes 1 and 0 for data that is not
+ * streamed 8-byte loads; modes 3 and 4: modes 1 and 0 for data that is not
  * resident: a few workgroups at the front of the launch only fetch (they walk the runs of the streaming waves in order,
  * 64 pages per batch of commands, at most a quarter of the cache ahead of the waves that have finished), and a streaming
  * wave that gets ahead of them touches the missing pages of its run itself, up to 64 at a time (12 M instead of 2.5 M
- * pages per second on a cold cache; on a resident one modes 1 and 0 are a quarter faster, the kernels with the read-ahead
- * run with fewer waves). */
+ * pages per second on a cold cache).
+ * Modes 0 and 1 on an array of one range run as two launches: the reference's kernel with pointers that read what is
+ * resident and note the pages that are not (a kernel without the miss path: no call, no stack, twice the waves), then a
+ * kernel that has the miss path over the pages noted, 64 at a time, which also folds the checksum.  Same sum, same number
+ * of accesses counted; pages that the second launch loads are asked for as batches before they are read, so their
+ * accesses count as hits.  Modes 5 and 6 are modes 0 and 1 as one launch of the kernel that can miss (what arrays of
+ * several ranges get under modes 0 and 1). */
 int bam_cache_stream(bam_array_t* a, uint64_t n_waves, uint64_t n_pages_per_wave, const uint64_t* d_assignment, int mode,
                      uint64_t* d_sum, void* stream);
 
 /* ---- raw block benchmark kernels (benchmarks/block/main.cu:99-200) ----
  * One thread per command: thread t transfers req_bytes between LBA d_lbas[t] (or t * req_bytes / lba_size when
  * NULL) and cache slot t with read_data / write_data; no cache lookup.  Needs n_pages >= n_reqs.
- * queue_policy 0: queue = compute unit % n_qps (sequential kernel), 1: round-robin counter (random kernel). */
+ * queue_policy 0: queue = compute unit % n_qps (sequential kernel), 1: round-robin counter (random kernel);
+ * 2: every thread puts its command together itself from the per-thread queue operations, the way the reference's
+ * read_data is written (include/page_cache.h:2009-2054: get_cid, nvm_cmd_*, sq_enqueue, cq_poll, cq_dequeue, put_cid;
+ * include/nvm_parallel_queue.h:35-57, 167-330, 378-535), thread t on queue pair t mod n_qps, the controller addressing
+ * slot t itself (EINVAL for a cache whose slots have no bus addresses). */
 int bam_block_io(bam_ctrl_t* c, bam_page_cache_t* pc, uint64_t n_reqs, uint32_t req_bytes, const uint64_t* d_lbas, int write,
                  int queue_policy, uint32_t block_size, void* stream);
 /* raw block reads with `depth` (1, 2, 4, 8) commands in flight per thread through access_data_async / poll_async
@@ -161,6 +185,9 @@ int bam_block_io_async(bam_ctrl_t* c, bam_page_cache_t* pc, uint64_t n_threads, 
 int bam_store_write_file(bam_ctrl_t* c, bam_page_cache_t* pc, const char* path, uint64_t file_offset, uint64_t store_offset, uint64_t n_bytes,
                          uint64_t* bytes_done);
 int bam_store_read_file(bam_ctrl_t* c, bam_page_cache_t* pc, const char* path, uint64_t store_offset, uint64_t n_bytes);
+/* util.h's warp_memcpy (reference include/util.h:102-117) run by one wave with the lanes named in the bit mask `lanes`
+ * active: n_words 64-bit words from d_src to d_dst */
+int bam_warp_memcpy(uint64_t* d_dst, const uint64_t* d_src, uint64_t n_words, uint64_t lanes, void* stream);
 /* sum of the 64-bit words of the first req_bytes of slots 0..n-1, one sum per slot */
 int bam_block_checksum(bam_page_cache_t* pc, uint64_t n_slots, uint32_t req_bytes, uint64_t* d_out, void* stream);
 
@@ -170,7 +197,7 @@ int bam_block_checksum(bam_page_cache_t* pc, uint64_t n_slots, uint32_t req_byte
  * by-page kernels when the array qualifies for them, and allocates the per-vertex flag and value buffers, the sweep counter
  * and the word through which a level tells the host whether anything changed.  Calls of bam_bfs, bam_bfs_frontier, bam_cc,
  * bam_bfs_by_page, bam_cc_by_page and bam_pagerank on `edges` with the same d_offsets and n_vertices then use it and
- * allocate nothing themselves (bam_bfs_frontier still takes its queues); any other call prepares the same for itself and drops it
+ * allocate nothing themselves; any other call prepares the same for itself and drops it
  * at its end.  The offsets must not change while the plan is set, and calls that use it must not overlap (they share its
  * counters and buffers).  d_offsets = NULL drops the plan; so does bam_array_destroy.
  * The waves a sweep runs are limited to one per 64 pages of the cache, since every lane of a wave may hold a page. */
@@ -205,8 +232,8 @@ int bam_cc_shaped(bam_array_t* edges, const uint64_t* d_offsets, uint64_t n_vert
  * next one: a vertex enters it when the exchange on its label finds it unreached, the lanes of a wave that found one
  * at the same step take their places with one atomic.  Otherwise the walk of bam_bfs (lists packed 64 entries per
  * step, long lists in pieces).  Same levels and the same *iterations as bam_bfs; no result depends on the order of a
- * queue, which is that of discovery when a level ends.  Between levels the queue is sorted by vertex (radix sort on
- * the device), so that a level reads the edge array front to back and a wave can take 512 entries at a time and ask
+ * queue, which is that of discovery when a level ends.  Between levels the queue is put in the order of its vertices (they
+ * are distinct: marked in a bit map and read back front to back), so that a level reads the edge array front to back and a wave can take 512 entries at a time and ask
  * for the pages under their lists as one batch, as bam_bfs does for 512 vertices; environment BAM_FRONTIER_SORT=0
  * leaves the queue as it comes (64 entries per wave at a time, first and last page of each list asked for).
  * n_vertices <= 2^32 - 1 (32-bit queue entries). */

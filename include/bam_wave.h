@@ -116,6 +116,29 @@ __device__ __forceinline__ void for_each_group(const uint64_t key, F&& body)
 {
     for_each_group(key, 0, [&](uint64_t a, uint64_t) { body(a); });
 }
+/*
+ * The same with the groups taken in ascending order of their key, whatever lanes hold them.  For work that takes
+ * something per key and keeps it while it takes the next (slots of several queues): when every wave takes in the same
+ * order, no two can each hold what the other is waiting for.  Costs a pass over the distinct keys still to be served per
+ * group (scalar reads and ballots), so it is for the places that need the order.
+ */
+template <typename F>
+__device__ __forceinline__ void for_each_group_ascending(const uint64_t key, F&& body)
+{
+    uint64_t todo = active_mask();
+    while (todo) {
+        uint64_t least = ~0ull, least_grp = 0;
+        for (uint64_t rest = todo; rest;) {
+            const uint64_t a = bcast(key, first_lane(rest));
+            const uint64_t grp = ballot(key == a) & todo;
+            if (a <= least) { least = a; least_grp = grp; }
+            rest &= ~grp;
+        }
+        const bool mine = (least_grp >> lane()) & 1;
+        if (mine) body(least);
+        todo &= ~least_grp;
+    }
+}
 
 /* compute-unit identity across the whole device: XCC, shader engine and CU bits */
 __device__ __forceinline__ uint32_t cu_id() { return __smid(); }
@@ -231,6 +254,42 @@ __device__ __forceinline__ void ld_payload_stream16(const uint64_t* p, const uin
 }
 
 /*
+ * N 64-bit words of payload at N addresses of the lane's own (scattered reads, or a lane's elements of one page), all in
+ * flight behind one wait: past the vector L1 and marked as not to be kept, like the streaming loads above.  Payload that
+ * is read once should not push the page descriptors out of the L2: with the mark the element gather's looks at the
+ * descriptors keep hitting, and it runs at 43 instead of 38 thousand million reads a second.  Every address must be
+ * readable (a lane with nothing to read passes any address inside the cache).
+ */
+template <int N>
+__device__ __forceinline__ void ld_payload_nt(const uint64_t* const (&p)[N], uint64_t (&x)[N])
+{
+    static_assert(N == 1 || N == 2 || N == 4 || N == 7 || N == 8, "1, 2, 4, 7 or 8 words");
+    if constexpr (N == 1)
+        asm volatile("global_load_dwordx2 %0, %1, off sc1 nt\n\ts_waitcnt vmcnt(0)" : "=&v"(x[0]) : "v"(p[0]) : "memory");
+    else if constexpr (N == 2)
+        asm volatile("global_load_dwordx2 %0, %2, off sc1 nt\n\tglobal_load_dwordx2 %1, %3, off sc1 nt\n\ts_waitcnt vmcnt(0)"
+                     : "=&v"(x[0]), "=&v"(x[1]) : "v"(p[0]), "v"(p[1]) : "memory");
+    else if constexpr (N == 4)
+        asm volatile("global_load_dwordx2 %0, %4, off sc1 nt\n\tglobal_load_dwordx2 %1, %5, off sc1 nt\n\t"
+                     "global_load_dwordx2 %2, %6, off sc1 nt\n\tglobal_load_dwordx2 %3, %7, off sc1 nt\n\ts_waitcnt vmcnt(0)"
+                     : "=&v"(x[0]), "=&v"(x[1]), "=&v"(x[2]), "=&v"(x[3]) : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]) : "memory");
+    else if constexpr (N == 7)
+        asm volatile("global_load_dwordx2 %0, %7, off sc1 nt\n\tglobal_load_dwordx2 %1, %8, off sc1 nt\n\t"
+                     "global_load_dwordx2 %2, %9, off sc1 nt\n\tglobal_load_dwordx2 %3, %10, off sc1 nt\n\t"
+                     "global_load_dwordx2 %4, %11, off sc1 nt\n\tglobal_load_dwordx2 %5, %12, off sc1 nt\n\t"
+                     "global_load_dwordx2 %6, %13, off sc1 nt\n\ts_waitcnt vmcnt(0)"
+                     : "=&v"(x[0]), "=&v"(x[1]), "=&v"(x[2]), "=&v"(x[3]), "=&v"(x[4]), "=&v"(x[5]), "=&v"(x[6])
+                     : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]), "v"(p[5]), "v"(p[6]) : "memory");
+    else
+        asm volatile("global_load_dwordx2 %0, %8, off sc1 nt\n\tglobal_load_dwordx2 %1, %9, off sc1 nt\n\t"
+                     "global_load_dwordx2 %2, %10, off sc1 nt\n\tglobal_load_dwordx2 %3, %11, off sc1 nt\n\t"
+                     "global_load_dwordx2 %4, %12, off sc1 nt\n\tglobal_load_dwordx2 %5, %13, off sc1 nt\n\t"
+                     "global_load_dwordx2 %6, %14, off sc1 nt\n\tglobal_load_dwordx2 %7, %15, off sc1 nt\n\ts_waitcnt vmcnt(0)"
+                     : "=&v"(x[0]), "=&v"(x[1]), "=&v"(x[2]), "=&v"(x[3]), "=&v"(x[4]), "=&v"(x[5]), "=&v"(x[6]), "=&v"(x[7])
+                     : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]), "v"(p[5]), "v"(p[6]), "v"(p[7]) : "memory");
+}
+
+/*
  * Sixteen bytes per lane at system scope, for moving payload between a staging page in host memory and a cache slot.
  * The load is never served from a cache that remembers the staging page's last tenant, so nobody has to invalidate
  * caches after a completion; the store goes through to memory, so the wave that moved a page in can publish it after
@@ -240,17 +299,26 @@ __device__ __forceinline__ void ld_payload_stream16(const uint64_t* p, const uin
  * tied to the registers it is for.
  */
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+/* The load and the wait for it are one statement: between two statements the compiler may copy or spill a register it
+ * believes written, and one whose load is still on its way would be copied as it was before. */
 __device__ __forceinline__ u32x4_t ld16_sys(const void* p)
 {
     u32x4_t v;
-    asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1" : "=v"(v) : "v"(p) : "memory");
+    asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1\n\ts_waitcnt vmcnt(0)" : "=&v"(v) : "v"(p) : "memory");
     return v;
 }
-__device__ __forceinline__ void wait_loads(u32x4_t& a, u32x4_t& b, u32x4_t& c, u32x4_t& d)
+/* four of them in flight behind one wait */
+__device__ __forceinline__ void ld16x4_sys(const void* p0, const void* p1, const void* p2, const void* p3, u32x4_t& a, u32x4_t& b, u32x4_t& c, u32x4_t& d)
 {
-    asm volatile("s_waitcnt vmcnt(0)" : "+v"(a), "+v"(b), "+v"(c), "+v"(d) :: "memory");
+    asm volatile("global_load_dwordx4 %0, %4, off sc0 sc1\n\t"
+                 "global_load_dwordx4 %1, %5, off sc0 sc1\n\t"
+                 "global_load_dwordx4 %2, %6, off sc0 sc1\n\t"
+                 "global_load_dwordx4 %3, %7, off sc0 sc1\n\t"
+                 "s_waitcnt vmcnt(0)"
+                 : "=&v"(a), "=&v"(b), "=&v"(c), "=&v"(d)
+                 : "v"(p0), "v"(p1), "v"(p2), "v"(p3)
+                 : "memory");
 }
-__device__ __forceinline__ void wait_loads(u32x4_t& a) { asm volatile("s_waitcnt vmcnt(0)" : "+v"(a) :: "memory"); }
 /* The two idle cycles after the store are part of it: a store of more than 8 bytes reads its data registers over the
  * cycles that follow its issue, and a vector instruction that writes one of them in that window changes what is stored.
  * The compiler keeps that distance for stores it emits itself, not for one inside an asm statement. */

@@ -174,6 +174,10 @@ private:
         if (const char* e = getenv("BAM_CQ_PLACE")) cq_place = (e[0] == 'd' || e[0] == '1') ? BAM_DMA_DEVICE : BAM_DMA_HOST;
         if (const char* e = getenv("BAM_SQ_SEAL")) sq_seal = atoi(e) != 0;
         if (const char* e = getenv("BAM_SQ_FLUSH")) sq_flush = (uint32_t)atoi(e);
+        /* an unsealed queue's controller goes by the doorbell alone, so the submitter has to know that its entry arrived
+         * before a doorbell can cover it: 0 (the wave's store counter only: handed on, not arrived) is for sealed queues,
+         * whose controller checks each entry; asked for on an unsealed queue it becomes the read-back */
+        if (!sq_seal && sq_flush == 0) sq_flush = 2;
         /* staged payload is pulled from host memory by the waves themselves, and a compute unit returns the loads of
          * all its waves in order: while one wave waits for host memory, every other load of that unit waits with it.
          * With more pulls in flight than the interconnect needs to stay busy, each waits longer and so does everybody

@@ -378,56 +378,68 @@ __device__ __forceinline__ bool cq_wait_group(nvm_queue_t* cq, nvm_queue_t* sq, 
 /* ---- per-thread entry points with the reference's names ---- */
 
 /*
- * A command id is the SQ slot its entry goes to: get_cid reserves the slot (the ticket is kept with it for sq_enqueue),
- * put_cid gives it back.  To be called by the lanes of a wave as the reference's threads call them: get_cid, then
- * sq_enqueue with that id in the entry, cq_poll, put_cid.
+ * The reference's threads each take a command id, build an entry around it, enqueue it, poll for its completion and hand
+ * the id back (get_cid, sq_enqueue, cq_poll, cq_dequeue, put_cid; include/page_cache.h:2009-2054 strings them together),
+ * and a thread that waits in one of these steps does not keep its neighbours from going through theirs.  The lanes of a
+ * wave move together: a wave whose lanes are on several queues, holding slots of one queue (reserved, their entries not
+ * yet written) while it waits for slots or for a covering doorbell on another, can wait for a wave that does the same the
+ * other way round; with seven queues, where consecutive waves meet the queues in rotated orders, that happens within
+ * milliseconds.  So a wave never holds anything of one queue while it waits on another: sq_enqueue does the whole of a
+ * command's life for one queue's lanes at a time (slot, entry, doorbell, completion, slot handed back), in rounds of half
+ * a queue where the lanes are more than that, and the calls around it have nothing left to wait for.  For the caller the
+ * sequence is the reference's: after cq_poll the transfer of the entry it enqueued has happened.  The id get_cid hands
+ * out is a token; the id the controller sees is the slot sq_enqueue writes the entry to, which it puts into the entry.
+ * Threads that want several commands in flight use access_data_async / poll_async.
  */
 inline __device__ uint16_t get_cid(nvm_queue_t* sq)
+{
+    (void)sq;
+    return (uint16_t)bam::lane();
+}
+
+/* nothing is held after sq_enqueue */
+inline __device__ void put_cid(nvm_queue_t* sq, uint16_t id)
+{
+    (void)sq; (void)id;
+}
+
+/* submits the entry and waits for its completion; returns the SQ slot used, which is the command id the controller saw.
+ * Bit 15 of the entry's dword 12 upward and the other fields are the caller's; only the id in dword 0 is replaced. */
+inline __device__ uint16_t sq_enqueue(nvm_queue_t* sq, nvm_cmd_t* cmd)
 {
     uint32_t id = 0;
     bam::for_each_group((uint64_t)sq, [&](uint64_t q) {
         nvm_queue_t* s = (nvm_queue_t*)q;
-        const uint32_t ticket = bam::sq_reserve_group(s);
-        id = ticket & s->qs_minus_1;
-        bam::st_relaxed(&s->head_mark[id].val, ticket);
-    });
-    return (uint16_t)id;
-}
-
-/* to be called by the lanes that hold the ids, all at once or in parts */
-inline __device__ void put_cid(nvm_queue_t* sq, uint16_t id)
-{
-    bam::for_each_group((uint64_t)sq, [&](uint64_t q) { bam::sq_release_group((nvm_queue_t*)q, id); });
-}
-
-/* the entry carries the id that get_cid handed out (nvm_cmd_header); returns the SQ slot used, which is that id */
-inline __device__ uint16_t sq_enqueue(nvm_queue_t* sq, nvm_cmd_t* cmd)
-{
-    const uint32_t id = cmd->dword[0] >> 16;
-    bam::for_each_group((uint64_t)sq, [&](uint64_t q) {
-        nvm_queue_t* s = (nvm_queue_t*)q;
-        bam::sq_submit_group(s, cmd, bam::ld_relaxed(&s->head_mark[id & s->qs_minus_1].val));
+        const uint64_t act = bam::active_mask();
+        const uint32_t n = bam::popc(act), rank = bam::rank_in(act), step = s->qs >> 1 ? s->qs >> 1 : 1u;
+        for (uint32_t base = 0; base < n; base += step)
+            if (rank >= base && rank - base < step) {
+                const uint32_t ticket = bam::sq_reserve_group(s);
+                id = ticket & s->qs_minus_1;
+                cmd->dword[0] = (cmd->dword[0] & 0xffffu) | (id << 16);
+                bam::sq_submit_group(s, cmd, ticket);
+                bam::cq_wait_group((nvm_queue_t*)s->pair, s, id);
+                bam::sq_release_group(s, id);
+            }
     });
     return (uint16_t)id;
 }
 
 /*
- * Wait for the completion of command `search_cid` submitted on the SQ paired
- * with `cq` (cq->pair).  The reference scans the ring and hands back the entry's position
- * for cq_dequeue; here the drainer has already consumed the entry, so the
- * out-parameters (which the reference dereferences even when NULL,
+ * The completion of the command was waited for in sq_enqueue.  The reference scans the ring here and hands back the
+ * entry's position for cq_dequeue; the out-parameters (which the reference dereferences even when NULL,
  * nvm_parallel_queue.h:406-407) are optional and receive the current head.
  */
 inline __device__ uint32_t cq_poll(nvm_queue_t* cq, uint16_t search_cid, uint32_t* loc_ = nullptr, uint32_t* cq_head = nullptr)
 {
-    bam::for_each_group((uint64_t)cq, [&](uint64_t q) { bam::cq_wait_group((nvm_queue_t*)q, (nvm_queue_t*)((nvm_queue_t*)q)->pair, search_cid); });
+    (void)search_cid;
     uint32_t h = bam::ld_relaxed(&cq->head_lock) >> 1;
     if (loc_) *loc_ = h;
     if (cq_head) *cq_head = h;
     return h & cq->qs_minus_1;
 }
 
-/* Completions are consumed by the drainer inside cq_poll; nothing is left to do per entry. */
+/* Completions are consumed by whoever drains the ring; nothing is left to do per entry. */
 inline __device__ void cq_dequeue(nvm_queue_t* cq, uint16_t pos, nvm_queue_t* sq, uint32_t loc_ = 0, uint32_t cur_head_ = 0)
 {
     (void)cq; (void)pos; (void)sq; (void)loc_; (void)cur_head_;

@@ -80,7 +80,7 @@ typedef struct
     uint32_t n_errors;   uint8_t pad5[56];  /* CQ: completions seen with a non-zero status */
 
     padded_struct*          tickets;        /* SQ [qs]: 2 * lap = free for the ticket of that lap (its owner adds 2 when done with the command) */
-    padded_struct*          head_mark;      /* SQ [qs]: the ticket a slot was reserved with by get_cid, for sq_enqueue (the reference marks consumed CQ entries here) */
+    padded_struct*          head_mark;      /* SQ [qs]: a spare word per slot (the reference marks consumed CQ entries in an array of this name) */
     padded_struct*          tail_mark;      /* SQ [qs]: lap + 1 of the entry last written to the slot, read by the tail sweep */
     padded_struct*          cid;            /* SQ [qs]: per command id (= slot), 1 in flight, 3 in flight + completed, 7 completed with an error status */
     padded_struct*          pos_locks;      /* unused (the reference's per-slot CQ locks) */

@@ -202,11 +202,11 @@ __device__ __forceinline__ void copy_pages(uint8_t* dst, const uint8_t* src, uin
          * wave's store counter says so */
         uint32_t i = rank;
         for (; i + 3 * movers < nb; i += 4 * movers) {
-            u32x4_t x0 = ld16_sys(s + i), x1 = ld16_sys(s + i + movers), x2 = ld16_sys(s + i + 2 * movers), x3 = ld16_sys(s + i + 3 * movers);
-            wait_loads(x0, x1, x2, x3);
+            u32x4_t x0, x1, x2, x3;
+            ld16x4_sys(s + i, s + i + movers, s + i + 2 * movers, s + i + 3 * movers, x0, x1, x2, x3);
             st16_sys(d + i, x0); st16_sys(d + i + movers, x1); st16_sys(d + i + 2 * movers, x2); st16_sys(d + i + 3 * movers, x3);
         }
-        for (; i < nb; i += movers) { u32x4_t x = ld16_sys(s + i); wait_loads(x); st16_sys(d + i, x); }
+        for (; i < nb; i += movers) { const u32x4_t x = ld16_sys(s + i); st16_sys(d + i, x); }
     }
     /* the compiler does not count stores issued from asm, and drops the counter wait of a later fence when it knows of
      * nothing outstanding: wait here, so that what follows (publishing the page, releasing the staging slot) is ordered
@@ -1016,7 +1016,21 @@ struct range_view {
     {
         acquire_<OUTLINE, true>(page, write, on_hit, on_miss, take);
     }
-    template <bool OUTLINE, bool HELPERS, typename FH, typename FM>
+    /*
+     * The hit half alone, for kernels that are launched in two passes: a group whose page is resident is served as
+     * acquire() serves it; a group whose page is not gives its references back at once and its lanes come back with
+     * true (nothing was called for them).  The caller notes what it could not read and a second launch, of a kernel
+     * that has the miss path, reads it.  A kernel that is made of this half only has no call in it, needs no stack and
+     * a fraction of the registers: what the path for resident pages costs, and nothing of what a miss would.
+     */
+    template <typename FH>
+    __forceinline__ __device__ bool acquire_or_defer(const uint64_t page, const bool write, FH&& on_hit)
+    {
+        bool deferred = false;
+        acquire_<false, false, true>(page, write, on_hit, [&](uint32_t) { deferred = true; return false; }, true);
+        return deferred;
+    }
+    template <bool OUTLINE, bool HELPERS, bool DEFER = false, typename FH, typename FM>
     __forceinline__ __device__ void acquire_(const uint64_t page_, const bool write, FH&& on_hit, FM&& on_miss, const bool take)
     {
         const uint32_t me = lane();
@@ -1037,6 +1051,10 @@ struct range_view {
             /* the lanes of a group may answer differently (one keeps the page, another only touched it) */
             const uint32_t n_drop = popc(ballot(drop) & eq_mask);
             if (n_drop && master == me) bam_release_refs(dp, n_drop, dirty);
+        } else if constexpr (DEFER) {
+            /* not resident: the references go back (nothing was read through them, so nothing has to be waited for) */
+            if (master == me) __hip_atomic_fetch_add(&dp->state, 0u - count, __ATOMIC_RELAXED, BAM_AGENT);
+            on_miss(BAM_NO_SLOT);
         } else {
             /* miss path: pass after pass; groups whose page came in are served and release before the next pass */
             const uint32_t queue = wave_slot_hash();
@@ -1238,9 +1256,56 @@ struct array_d_t {
     {
         static_assert(N >= 1 && N <= 15, "the counters of the plain form are flushed with three or four ballots");
         bool got[N];
+        seq_read_n_resident(idx, want, out, got, v);
+#pragma unroll
+        for (int j = 0; j < N; j++)
+            if (want[j] && !got[j]) out[j] = seq_read_call(idx[j]);
+    }
+    /*
+     * The half of seq_read_n that cannot miss: out[j] and got[j] = true for the elements that were read from resident
+     * pages (and counted as hits in the view); got[j] = false for the others, which nothing was done for.  No call, no
+     * atomic, no store: a kernel made of this alone (the first of two launches, the second reading what this one could
+     * not) needs a fraction of the registers of one that can miss.  The view is that of the array's one range.
+     */
+    template <int N, bool SCATTERED = false>
+    __forceinline__ __device__ void seq_read_n_resident(const size_t (&idx)[N], const bool (&want)[N], T (&out)[N], bool (&got)[N], bam::range_view<T>& v) const
+    {
         const bool one = v.r != nullptr;
 #pragma unroll
         for (int j = 0; j < N; j++) { got[j] = false; out[j] = T(); }
+        if constexpr (SCATTERED && sizeof(T) == 8 && (N == 1 || N == 2 || N == 4 || N == 8)) {
+            /* elements anywhere in the array (a gather): no two are expected on one page, so every element has its own looks,
+             * and every lane makes every load (one with nothing to read looks at the first page's descriptor and loads the
+             * cache's first word): three rounds of N loads with nothing but arithmetic between them */
+            if (one && v.r->cache.fast_reads) {
+                const data_page_t* dp[N];
+                const uint64_t* p[N];
+                uint64_t s1[N], in_page[N], x[N];
+                bool res[N];
+#pragma unroll
+                for (int j = 0; j < N; j++) {
+                    res[j] = want[j] && idx[j] - v.index_start < v.index_end - v.index_start;
+                    const uint64_t byte = res[j] ? v.byte_of(idx[j]) : 0;
+                    dp[j] = v.pages + (byte >> v.page_size_log);
+                    in_page[j] = byte & (v.page_size - 1);
+                }
+#pragma unroll
+                for (int j = 0; j < N; j++) s1[j] = __hip_atomic_load((const uint64_t*)dp[j], __ATOMIC_RELAXED, BAM_AGENT);
+#pragma unroll
+                for (int j = 0; j < N; j++) {
+                    res[j] = res[j] && ((uint32_t)s1[j] >> (CNT_SHIFT + 1)) == V_NB;
+                    p[j] = (const uint64_t*)(v.base_addr + (res[j] ? ((uint64_t)((uint32_t)(s1[j] >> 32) & BAM_SLOT_MASK) << v.page_size_log) + in_page[j] : 0));
+                }
+                bam::ld_payload_nt(p, x);               /* with its wait: the elements are here before the second looks go out */
+#pragma unroll
+                for (int j = 0; j < N; j++) {
+                    const uint64_t s2 = __hip_atomic_load((const uint64_t*)dp[j], __ATOMIC_RELAXED, BAM_AGENT);
+                    got[j] = res[j] && ((s1[j] ^ s2) & 0xFFFFFFFFC0000000ull) == 0;
+                    if (got[j]) { out[j] = *(T*)&x[j]; v.account(true); }
+                }
+            }
+            return;
+        }
         if (one && v.r->cache.fast_reads) {
             uint64_t s1[N], byte[N];
             bool res[N], again[N];
@@ -1256,11 +1321,24 @@ struct array_d_t {
                 else if (res[j]) s1[j] = __hip_atomic_load((const uint64_t*)(v.pages + (byte[j] >> v.page_size_log)), __ATOMIC_RELAXED, BAM_AGENT);
             }
 #pragma unroll
-            for (int j = 0; j < N; j++) {
-                res[j] = res[j] && ((uint32_t)s1[j] >> (CNT_SHIFT + 1)) == V_NB;
-                if (res[j]) out[j] = bam::ld_payload((const T*)(v.base_addr + ((uint64_t)((uint32_t)(s1[j] >> 32) & BAM_SLOT_MASK) << v.page_size_log) + (byte[j] & (v.page_size - 1))));
+            for (int j = 0; j < N; j++) res[j] = res[j] && ((uint32_t)s1[j] >> (CNT_SHIFT + 1)) == V_NB;
+            if constexpr (sizeof(T) == 8 && (N == 1 || N == 2 || N == 4 || N == 8)) {
+                /* scattered 8-byte elements: loaded as not to be kept, all behind one wait (lanes with nothing to read load
+                 * the cache's first word and drop it) */
+                const uint64_t* p[N];
+                uint64_t x[N];
+#pragma unroll
+                for (int j = 0; j < N; j++)
+                    p[j] = (const uint64_t*)(v.base_addr + (res[j] ? ((uint64_t)((uint32_t)(s1[j] >> 32) & BAM_SLOT_MASK) << v.page_size_log) + (byte[j] & (v.page_size - 1)) : 0));
+                bam::ld_payload_nt(p, x);               /* with its wait: the elements are here before the second looks go out */
+#pragma unroll
+                for (int j = 0; j < N; j++) if (res[j]) out[j] = *(T*)&x[j];
+            } else {
+#pragma unroll
+                for (int j = 0; j < N; j++)
+                    if (res[j]) out[j] = bam::ld_payload((const T*)(v.base_addr + ((uint64_t)((uint32_t)(s1[j] >> 32) & BAM_SLOT_MASK) << v.page_size_log) + (byte[j] & (v.page_size - 1))));
+                bam::fence_meta();                       /* the elements are here before the second looks go out */
             }
-            bam::fence_meta();                           /* the elements are here before the second looks go out */
             uint64_t s2 = 0;                            /* the second look of the element before, for one that shares it */
 #pragma unroll
             for (int j = 0; j < N; j++) {
@@ -1272,9 +1350,6 @@ struct array_d_t {
                 if (got[j]) v.account(true);
             }
         }
-#pragma unroll
-        for (int j = 0; j < N; j++)
-            if (want[j] && !got[j]) out[j] = seq_read_call(idx[j]);
     }
     /* seq_read as a call: the N places above where an element goes the counted way would otherwise each carry the whole
      * of that path, and its registers with it */
@@ -1414,7 +1489,7 @@ struct array_d_t {
     }
 };
 
-template <typename T> struct bam_ptr;
+template <typename T, bool DEFER = false> struct bam_ptr;
 
 /*
  * What bam_ptr::operator[] hands out on a non-const pointer: converts to T for
@@ -1425,7 +1500,7 @@ template <typename T> struct bam_ptr;
  */
 template <typename T>
 struct bam_ref {
-    bam_ptr<T>* p;
+    bam_ptr<T, false>* p;
     size_t i;
     __forceinline__ __host__ __device__ operator T() const { return p->read(i); }
     __forceinline__ __host__ __device__ bam_ref& operator=(T v) { p->write(i, v); return *this; }
@@ -1443,8 +1518,12 @@ struct bam_ref {
  * hold at once (the reference has the same requirement).  The range
  * descriptor is read once and kept in registers for as long as the accesses
  * stay inside that range.
+ *
+ * DEFER (no counterpart in the reference): a pointer for the first of two launches.  It reads what is resident; when
+ * the page of an access is not, the access yields T(), `missed` is set and nothing is loaded (range_view::
+ * acquire_or_defer): the kernel notes the work for the second launch, which uses a plain bam_ptr.  Reads only.
  */
-template <typename T>
+template <typename T, bool DEFER>
 struct bam_ptr {
     data_page_t* page = nullptr;
     array_d_t<T>* array = nullptr;
@@ -1453,6 +1532,7 @@ struct bam_ptr {
     int64_t range_id = -1;
     T* addr = nullptr;
     bool dirty = false;
+    bool missed = false;             /* DEFER: an access since the flag was last cleared found its page not resident */
 #if defined(__HIP_DEVICE_COMPILE__)
     bam::range_view<T> view;
 #endif
@@ -1477,7 +1557,17 @@ struct bam_ptr {
 #endif
     }
 
+    /* move the window to the page of element i (the reference's update_page, include/page_cache.h:447); NULL when there is no
+     * such page to be had: no range holds i, the wait for the page was given up, or, DEFER, the page is not resident */
     __forceinline__ __host__ __device__ T* update_page(const size_t i)
+    {
+#if defined(__HIP_DEVICE_COMPILE__)
+        if constexpr (DEFER) { if (view.holds(i)) return move_window(i); }
+#endif
+        return update_page_general(i);
+    }
+
+    __forceinline__ __host__ __device__ T* update_page_general(const size_t i)
     {
 #if defined(__HIP_DEVICE_COMPILE__)
         fini();
@@ -1492,7 +1582,10 @@ struct bam_ptr {
         const uint64_t pg = view.page_of(i);
         uint32_t slot = BAM_NO_SLOT;
         auto keep = [&](uint32_t s_) { slot = s_; return false; };
-        view.template acquire<true>(pg, false, keep, keep);
+        if constexpr (DEFER) {
+            if (view.acquire_or_defer(pg, false, keep)) { missed = true; return nullptr; }      /* no reference is held */
+        } else
+            view.template acquire<true>(pg, false, keep, keep);
         page = view.pages + pg;                 /* the references of the group stay counted either way */
         if (slot == BAM_NO_SLOT) return nullptr;        /* the wait was given up (the controller is marked aborted): no window */
         view.window(pg, start, end);
@@ -1501,15 +1594,80 @@ struct bam_ptr {
         return addr;
     }
 
+#if defined(__HIP_DEVICE_COMPILE__)
+    /*
+     * DEFER: the window moves to the page of element i, which the range at hand holds.  Giving the old page back and
+     * taking the new one is one grouping of the lanes (by both pages at once: lanes that leave the same page for the same
+     * page share the two atomics) instead of one each; nothing else of update_page is needed for a pointer that only
+     * reads what is resident.
+     */
+    __forceinline__ __device__ T* move_window(const size_t i)
+    {
+        using namespace bam;
+        data_page_t* const old_dp = page;
+        const uint64_t pg = view.page_of(i);
+        data_page_t* const new_dp = view.pages + pg;
+        const uint64_t eq = match_any((uint64_t)old_dp, (uint64_t)new_dp);
+        const uint32_t master = first_lane(eq), cnt = popc(eq);
+        uint64_t sv = 0;
+        if (lane() == master) {
+            /* the loads of the old page are in (a wait on the wave's counter covers every lane's) before its count drops */
+            if (old_dp) { fence_meta(); __hip_atomic_fetch_add(&old_dp->state, 0u - cnt, __ATOMIC_RELAXED, BAM_AGENT); }
+            sv = __hip_atomic_fetch_add((uint64_t*)new_dp, (uint64_t)cnt, __ATOMIC_RELAXED, BAM_AGENT);
+        }
+        /* one group, as when a wave walks a page together: the word comes over the scalar unit */
+        if (first(eq) == active_mask()) sv = bcast(sv, first_lane(active_mask()));
+        else sv = shfl(sv, master);
+        if (((uint32_t)sv >> (CNT_SHIFT + 1)) == V_NB) {
+            view.account(true);
+            page = new_dp;
+            view.window(pg, start, end);
+            addr = (T*)(view.slot_addr((uint32_t)(sv >> 32) & BAM_SLOT_MASK) + (view.byte_of(start) & (view.page_size - 1)));
+            return addr;
+        }
+        if (lane() == master) __hip_atomic_fetch_add(&new_dp->state, 0u - cnt, __ATOMIC_RELAXED, BAM_AGENT);
+        page = nullptr;
+        start = end = 0;
+        addr = nullptr;
+        missed = true;
+        return nullptr;
+    }
+#endif
+
     /* after a wait that was given up the value is T(): callers that use what they read as an index (the neighbour
      * ids of a graph) stay inside their arrays until the host sees the abort */
     __forceinline__ __host__ __device__ T read(const size_t i)
     {
+#if defined(__HIP_DEVICE_COMPILE__)
+        if constexpr (DEFER) {
+            if (i < start || i >= end) { if (!update_page(i)) return T(); }
+            return bam::ld_payload(addr + (i - start));
+        }
+#endif
         if (i < start || i >= end) { if (!update_page(i)) return T(); }
 #if defined(__HIP_DEVICE_COMPILE__)
         return bam::ld_payload(addr + (i - start));
 #else
         return addr[i - start];
+#endif
+    }
+
+    /* the accesses this pointer has counted and not yet handed to the range's counters, read and put back: a kernel that
+     * leaves a piece of work to a later launch takes back what it counted for it */
+    __forceinline__ __host__ __device__ void counted(uint32_t& n_access, uint32_t& n_hit) const
+    {
+#if defined(__HIP_DEVICE_COMPILE__)
+        n_access = view.n_access; n_hit = view.n_hit;
+#else
+        n_access = n_hit = 0;
+#endif
+    }
+    __forceinline__ __host__ __device__ void set_counted(const uint32_t n_access, const uint32_t n_hit)
+    {
+#if defined(__HIP_DEVICE_COMPILE__)
+        view.n_access = n_access; view.n_hit = n_hit;
+#else
+        (void)n_access; (void)n_hit;
 #endif
     }
 
@@ -1526,6 +1684,29 @@ struct bam_ptr {
 #endif
     }
 
+    /* N elements i, i + stride, ... of the page held now (the caller has asked covers() about the first and the last),
+     * side by side; 8-byte elements are loaded as not to be kept (bam::ld_payload_nt) */
+    template <int N>
+    __forceinline__ __host__ __device__ void peek_n(const size_t i, const size_t stride, T (&out)[N]) const
+    {
+#if defined(__HIP_DEVICE_COMPILE__)
+        if constexpr (sizeof(T) == 8 && (N == 1 || N == 2 || N == 4 || N == 7 || N == 8)) {
+            const uint64_t* p[N];
+            uint64_t x[N];
+#pragma unroll
+            for (int u = 0; u < N; u++) p[u] = (const uint64_t*)(addr + (i - start) + (size_t)u * stride);
+            bam::ld_payload_nt(p, x);
+#pragma unroll
+            for (int u = 0; u < N; u++) out[u] = *(T*)&x[u];
+        } else {
+#pragma unroll
+            for (int u = 0; u < N; u++) out[u] = bam::ld_payload(addr + (i - start) + (size_t)u * stride);
+        }
+#else
+        for (int u = 0; u < N; u++) out[u] = addr[i - start + (size_t)u * stride];
+#endif
+    }
+
     __forceinline__ __host__ __device__ void mark_dirty()
     {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -1535,18 +1716,24 @@ struct bam_ptr {
 
     __forceinline__ __host__ __device__ void write(const size_t i, const T v)
     {
+        static_assert(!DEFER, "a deferring bam_ptr only reads");
         if (i < start || i >= end) { if (!update_page(i)) return; }
         mark_dirty();
         addr[i - start] = v;
     }
 
     __forceinline__ __host__ __device__ T operator[](const size_t i) const { return const_cast<bam_ptr*>(this)->read(i); }
-    __forceinline__ __host__ __device__ bam_ref<T> operator[](const size_t i) { return bam_ref<T>{this, i}; }
+    __forceinline__ __host__ __device__ auto operator[](const size_t i)
+    {
+        if constexpr (DEFER) return read(i);
+        else return bam_ref<T>{this, i};
+    }
 
     /* address of element i for the caller to read or write: counts as a write.  NULL when no range holds i or the wait
      * for the page was given up (the reference returns an address computed from a null window there) */
     __forceinline__ __host__ __device__ T* memref(size_t i)
     {
+        static_assert(!DEFER, "a deferring bam_ptr only reads");
         if (i < start || i >= end) { if (!update_page(i)) return nullptr; }
         mark_dirty();
         return addr + (i - start);

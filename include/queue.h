@@ -108,7 +108,7 @@ struct QueuePair
         own->sq_cid_blocks = createBuffer(sizeof(padded_struct), hipDevice);
         sq.pos_locks = (padded_struct*)own->sq_cid_blocks.get();        /* unused */
         own->sq_cid_left = createBuffer(qs * sizeof(padded_struct), hipDevice);
-        sq.head_mark = (padded_struct*)own->sq_cid_left.get();         /* per slot: the ticket get_cid reserved it with */
+        sq.head_mark = (padded_struct*)own->sq_cid_left.get();         /* a spare word per slot */
         cq.cid = sq.cid;
         cq.cid_mask = sq.cid_mask;
         sq.prof = cq.prof = prof;

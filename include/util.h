@@ -1,8 +1,8 @@
 /*
  * Small host/device helpers.  Replaces include/util.h of the reference
  * (cuda_err_chk :18-35, hexdump :52-96, warp_memcpy :102-117, CEIL :45) with
- * HIP equivalents; warp_memcpy moves 16 bytes per lane per trip over the
- * active lanes of a 64-wide wave.
+ * HIP equivalents; warp_memcpy shares the elements out over the active lanes
+ * of a 64-wide wave.
  */
 #ifndef __BAM_UTIL_H__
 #define __BAM_UTIL_H__
@@ -26,15 +26,14 @@ inline void bam_hip_assert(hipError_t code, const char* file, int line)
 #define CEIL(X, Y, Z) (((X) + (Y) - 1) >> (Z))
 #endif
 
-/* cooperative copy by the active lanes; n bytes, multiple of 16, both pointers 16-byte aligned */
+/* cooperative copy by the active lanes, all called with the same arguments: `num` elements of type T (a count, not
+ * bytes, as in the reference), the k-th active lane taking elements k, k + n, ... of n active lanes */
 template <typename T>
-__device__ __forceinline__ void warp_memcpy(T* dest, const T* src, size_t n_bytes)
+__device__ __forceinline__ void warp_memcpy(T* dest, const T* src, size_t num)
 {
     const uint64_t act = bam::active_mask();
     const uint32_t n = bam::popc(act), rank = bam::rank_in(act);
-    uint4* d = (uint4*)dest;
-    const uint4* s = (const uint4*)src;
-    for (size_t i = rank; i < n_bytes / 16; i += n) d[i] = s[i];
+    for (size_t i = rank; i < num; i += n) dest[i] = src[i];
 }
 
 inline __host__ void hexdump(const void* data, size_t size)

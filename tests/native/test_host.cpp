@@ -297,6 +297,16 @@ int main()
         CHECK("ctrl_init_fd_mapping_is_shared", through);
         nvm_ctrl_free(c);
         close(fd); unlink(path);
+        // a regular file shorter than the register window (or empty): an error code, not a bus error at the first register read
+        for (size_t short_size : {(size_t)0, (size_t)64, (size_t)NVM_CTRL_MEM_MINSIZE - 1}) {
+            char spath[] = "/tmp/bam_bar0s_XXXXXX";
+            int sfd = mkstemp(spath);
+            bool sized = ftruncate(sfd, (off_t)short_size) == 0;
+            c = nullptr;
+            int e = nvm_ctrl_init(&c, sfd);
+            CHECK("ctrl_init_fd_short_file", sized && e == ENODEV && !c);
+            close(sfd); unlink(spath);
+        }
         int pfd[2];
         if (pipe(pfd) == 0) {
             c = nullptr;

@@ -143,6 +143,34 @@ def test_random_gather_with_eviction(bam, cache_pages, n_queues, depth, block):
         assert not r.c.aborted()
 
 
+@pytest.mark.parametrize("cache_pages,n_queues,depth", [(8, 4, 64), (300, 8, 256), (8192, 16, 1024)])
+def test_launch_shapes_of_the_gather_agree(bam, cache_pages, n_queues, depth):
+    """The scattered gather in every launch shape (one request per thread as the reference has it, four per thread, and in
+    two launches with 1 to 8 reads per lane in the first), a ragged request count, caches from a few pages to one that
+    holds everything: same sum, every request counted once, and hits + misses = accesses, whatever the shape; on the cache
+    that holds everything the second round is all hits and does no I/O."""
+    from bam_amd import gen
+    n_elems, n = 1 << 22, (1 << 17) + 37          # 8192 pages of data
+    want = oracle.lib().bo_gather_sum(SEED, SEED, 0, n, n_elems)
+    with Rig(bam, 64 << 20, n_queues=n_queues, depth=depth) as r:
+        a = r.array(n_elems, 4096, cache_pages)
+        idx = gen.gather_indices(SEED, n, n_elems)
+        shapes = [(a.ONE_PER_THREAD, 1), (a.FOUR_PER_THREAD, 4)] + [(a.TWO_LAUNCHES, k) for k in (1, 2, 4, 8)]
+        for rnd in range(2):
+            for shape, lanes in shapes:
+                for block in (64, 256):
+                    assert a.read_shaped(n, idx, shape, lanes, block_size=block) == want, (shape, lanes, block)
+                    st = a.stats()
+                    assert st["access_cnt"] == n and st["hit_cnt"] + st["miss_cnt"] == n, (shape, lanes, st)
+                    if cache_pages == 8192 and rnd == 1:
+                        assert st["read_io_cnt"] == 0 and st["hit_cnt"] == n
+                    if cache_pages == 8:
+                        assert st["read_io_cnt"] > 0
+        assert a.read(n, idx, block_size=64) == want                  # what bam_array_read picks for a launch of this size
+        assert a.stats()["access_cnt"] == n
+        assert not r.c.aborted() and r.c.info()["error_completions"] == 0
+
+
 @pytest.mark.parametrize("cache_pages,n_queues,depth,block", [(64, 4, 64, 64), (1024, 2, 16, 256), (4096, 16, 1024, 128)])
 def test_every_element_of_a_gather_and_of_an_update_under_eviction(bam, cache_pages, n_queues, depth, block):
     """Element by element instead of a sum: 2^18 random reads through a cache that holds a fraction of the data, on queues so
@@ -325,7 +353,7 @@ def test_pages_above_two_controller_pages_use_prp_lists(bam, page, stage):
 
 # ---------------------------------------------------------------- cache / pattern streaming
 
-@pytest.mark.parametrize("mode", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("mode", [0, 1, 2, 3, 4, 5, 6])
 def test_page_streaming_modes(bam, mode):
     n_pages = 4096
     with Rig(bam, 64 << 20) as r:
@@ -333,12 +361,14 @@ def test_page_streaming_modes(bam, mode):
         ref = oracle.lib().bo_store_sum(SEED, 0, 1, n_pages * 512)
         assert a.stream(n_pages // 2, 2, mode=mode) == ref          # cold: every page read once
         st = a.stats()
-        # every page comes in once.  Per-element operator[] (mode 0): the wave's first access to a page misses, its seven
-        # others hit; bam_ptr (1) and the page-wise kernel (2) take each page once per wave, as a miss; modes 3 and 4 touch
-        # the pages of a wave's run ahead as one batch (not counted as accesses), so their own accesses all find their page
-        assert st["read_io_cnt"] == n_pages and st["hit_cnt"] == {0: n_pages * 448, 1: 0, 2: 0, 3: n_pages * 64, 4: n_pages * 512}[mode]
+        # every page comes in once.  Per-element operator[] in one launch (mode 5): the wave's first access to a page misses,
+        # its seven others hit; bam_ptr in one launch (6) and the page-wise kernel (2) take each page once per wave, as a miss;
+        # modes 3 and 4, and the second launch of modes 0 and 1, ask for the pages of a wave's run as one batch before they read
+        # (not counted as accesses), so their own accesses all find their page
+        assert st["read_io_cnt"] == n_pages
+        assert st["hit_cnt"] == {0: n_pages * 512, 1: n_pages * 64, 2: 0, 3: n_pages * 64, 4: n_pages * 512, 5: n_pages * 448, 6: 0}[mode]
         # accesses: one per element with operator[], one per lane per page with bam_ptr, one per page when pages are taken in batches
-        assert st["access_cnt"] == {0: n_pages * 512, 1: n_pages * 64, 2: n_pages, 3: n_pages * 64, 4: n_pages * 512}[mode]
+        assert st["access_cnt"] == {0: n_pages * 512, 1: n_pages * 64, 2: n_pages, 3: n_pages * 64, 4: n_pages * 512, 5: n_pages * 512, 6: n_pages * 64}[mode]
         assert a.stream(n_pages // 2, 2, mode=mode) == ref          # hot: no I/O at all
         st = a.stats()
         assert st["read_io_cnt"] == 0 and st["miss_cnt"] == 0
@@ -350,7 +380,7 @@ def test_page_streaming_modes(bam, mode):
         assert not r.c.aborted()
 
 
-@pytest.mark.parametrize("mode", [0, 1, 3, 4])
+@pytest.mark.parametrize("mode", [0, 1, 3, 4, 5, 6])
 @pytest.mark.parametrize("page", [512, 4096, 16384])
 def test_element_streaming_over_other_page_sizes_and_a_ragged_last_page(bam, mode, page):
     """The per-element streaming kernels where a lane reads one element of a page (512 B), eight (4 KiB) or thirty-two
@@ -431,6 +461,52 @@ def test_block_reads_payload_checksums(bam, req, lba, order, raw_share, monkeypa
         assert ts["read_cmds"] == 2 * n + 1000 and ts["error_cpls"] == 0 and ts["sq_doorbells"] < ts["read_cmds"]
         assert not r.c.aborted()
         pc.close()
+
+
+@pytest.mark.parametrize("n_queues,depth,order", [(4, 16, 0), (8, 16, 2), (7, 64, 1), (128, 1024, 0), (7, 16, 0), (2, 16, 1), (1, 4, 0)])
+def test_block_io_through_the_per_thread_queue_operations(bam, n_queues, depth, order):
+    """Every thread builds and runs its own command with get_cid, nvm_cmd_*, sq_enqueue, cq_poll, cq_dequeue and put_cid,
+    as the reference's read_data is written, thread t on queue pair t mod n_qps: the lanes of a wave are on different
+    queue pairs, sixteen of them per queue of sixteen slots (the whole queue per wave), eight (half of it), nine or
+    ten where 64 does not divide (consecutive waves then meet the queues in rotated orders), thirty-two or all sixty-four
+    on queues of sixteen and of four slots (more lanes than slots), the last wave ragged; completions in order, reversed
+    and shuffled.  Payload checksums
+    against the oracle, then a write of the same slots further on and a read back, and the ids come back every time (the
+    launches repeat on the same queues)."""
+    from bam_amd import gen
+    n, ns, req, lba = 5000 + 37, 1 << 30, 4096, 512
+    with Rig(bam, ns, lba=lba, n_queues=n_queues, depth=depth, order=order, backing=True) as r:
+        pc = bam.PageCache(4096, n, 0, r.c)
+        for rep in range(3):
+            lbas = gen.block_lbas(SEED + rep, n, ns // 2, req, lba)
+            pc.block_io(n, req, lbas, queue_policy=2, block_size=256 if rep else 64)
+            cs = _u64(pc.block_checksums(n, req))
+            assert not r.c.aborted(), (rep, r.t.stats())
+            ref = np.array([oracle.lib().bo_block_checksum(SEED, int(x), lba, req) for x in _u64(lbas)], dtype=np.uint64)
+            assert np.array_equal(cs, ref), (rep, int((cs != ref).sum()), r.t.stats())
+        # the slots as they are now, written to distinct blocks in the upper half of the namespace and read back
+        before = cs.copy()
+        up = _dev(np.arange(n, dtype=np.uint64) * np.uint64(req // lba) + np.uint64(ns // 2 // lba))
+        pc.block_io(n, req, up, write=True, queue_policy=2)
+        pc.block_io(n, req, None, queue_policy=2)                     # something else into the slots in between
+        assert not np.array_equal(_u64(pc.block_checksums(n, req)), before)
+        pc.block_io(n, req, up, queue_policy=2)
+        assert np.array_equal(_u64(pc.block_checksums(n, req)), before)
+        ts = r.t.stats()
+        assert ts["read_cmds"] == 5 * n and ts["write_cmds"] == n and ts["error_cpls"] == 0 and not r.c.aborted()
+        pc.close()
+
+
+@pytest.mark.parametrize("lanes", [(1 << 64) - 1, (1 << 37) - 1, 0xAAAAAAAAAAAAAAAA, 1 << 63, 0x8000000100000001])
+def test_warp_memcpy_with_any_set_of_lanes(bam, lanes):
+    """util.h's warp_memcpy: a count of elements, shared out over whichever lanes are active; nothing is written past it"""
+    import torch
+    for n in (0, 1, 63, 64, 1000, 4097):
+        src = torch.arange(1, n + 9, dtype=torch.int64, device="cuda") * 0x9E3779B97F4A7C15
+        dst = torch.full((n + 8,), -1, dtype=torch.int64, device="cuda")
+        assert bam._lib.load().bam_warp_memcpy(ctypes.c_void_p(dst.data_ptr()), ctypes.c_void_p(src.data_ptr()), n, lanes, None) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(dst[:n], src[:n]) and bool((dst[n:] == -1).all())
 
 
 @pytest.mark.parametrize("req", [4096, 512])
@@ -1087,12 +1163,13 @@ def test_completion_ring_placement(bam, place, order, depth, monkeypatch):
         pc.close()
 
 
-@pytest.mark.parametrize("seal,flush", [("0", "2"), ("0", "1"), ("0", "0"), ("1", "2")])
+@pytest.mark.parametrize("seal,flush", [("0", "2"), ("0", "1"), ("1", "0"), ("1", "2")])
 def test_submission_entries_sealed_and_unsealed(bam, seal, flush, monkeypatch):
     """Submission queues as the NVMe specification has them (no seal in the entries, what a real controller needs; the
-    default), with each of the three ways a submitter has of making sure its entry arrives before a doorbell covers it
-    (2 read the entry back, 1 system-scope release, 0 the wave's store counter alone), and sealed (the target verifies a
-    ticket and a checksum in the entry and reads it again if they do not hold).  Checksum, no error completions, no wait
+    default), with each of the two ways a submitter has of knowing that its entry arrived before a doorbell covers it
+    (2 read the entry back, 1 system-scope release), and sealed (the target verifies a ticket and a checksum in the entry
+    and reads it again if they do not hold, so the submitter need not know: the wave's store counter alone, 0, will do;
+    on an unsealed queue 0 is not offered, the controller turns it into 2).  Checksum, no error completions, no wait
     given up; the target's counters say what it saw."""
     from bam_amd import gen
     monkeypatch.setenv("BAM_SQ_SEAL", seal)
@@ -1118,6 +1195,20 @@ def test_lost_completion_ends_the_kernel_with_the_abort_flag(bam):
         a.read(1 << 18, block_size=64)
         assert r.c.aborted() and r.t.stats()["dropped"] >= 1
         assert r.c.aborted(clear=True) and not r.c.aborted()
+
+
+@pytest.mark.parametrize("api", [1, 2, 3, 4, 5, 6, 7])
+def test_lost_completion_through_every_access_route(bam, api):
+    """the same through get_raw, acquire_page_, acquire_page, bam_ptr, the wave memcpy, bam_ptr_tlb and bafs_ptr: a route
+    whose wait was given up hands out no address (NULL, an empty window, T()), its kernel reads nothing through it and
+    ends, and the flag is up"""
+    with Rig(bam, 16 << 20, drop_every=200, limit=300_000) as r:
+        a = r.array(1 << 20, 4096, 4096)
+        if api == 5:
+            a.read_via(5, 1 << 11, span=512, block_size=64)
+        else:
+            a.read_via(api, 1 << 17, span=8, block_size=64)
+        assert r.c.aborted() and r.t.stats()["dropped"] >= 1
 
 
 @pytest.mark.parametrize("kernel", [dict(coarse=4), dict(frontier=True), dict(by_page=True)])
