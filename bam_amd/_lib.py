@@ -82,6 +82,7 @@ SIGNATURES = {
     "bam_read_kernel": (c_int, [c_vp, c_u64, P(ctypes.c_float), c_vp]),
     "bam_atomic_pairs_kernel": (c_int, [c_vp, c_vp, c_u64, c_int, P(ctypes.c_float), c_vp]),
     "bam_xcd_relay": (c_int, [c_vp, c_u64, c_u32, c_u32, c_u32, c_u32, c_u32, P(c_u64), c_vp]),
+    "bam_hit_path_parts": (c_int, [c_vp, c_int, c_int, c_u64, c_u64, c_vp, c_vp]),
     "bam_gather_kernel": (c_int, [c_vp, c_vp, c_u64, P(ctypes.c_float), c_vp]),
     "bam_host_read_ceiling": (c_int, [c_u64, c_u32, P(ctypes.c_float)]),
     "bam_event_create": (c_int, [P(c_vp)]),

@@ -118,11 +118,11 @@ __global__ void k_array_read_n_whole(array_d_t<uint64_t>* dr, uint64_t n_reqs, c
  * carries the registers of the miss path (four waves per SIMD) and its frame in scratch memory through every read.  The
  * last workgroup folds the checksum of what was read; the second launch adds what it reads.
  */
-#ifndef BAM_GATHER_MAX_WAVES
-#define BAM_GATHER_MAX_WAVES 8
+#ifndef BAM_GATHER_MIN_WAVES
+#define BAM_GATHER_MIN_WAVES 1
 #endif
 template <int N>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, BAM_GATHER_MAX_WAVES))) void k_array_read_n(array_d_t<uint64_t>* dr, uint64_t n_reqs, const uint64_t* __restrict__ assignment, uint64_t threads, uint32_t rounds,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BAM_GATHER_MIN_WAVES))) void k_array_read_n(array_d_t<uint64_t>* dr, uint64_t n_reqs, const uint64_t* __restrict__ assignment, uint64_t threads, uint32_t rounds,
                                                       unsigned long long* partials, uint64_t* missed, unsigned long long* sum, uint32_t* finished, uint32_t call)
 {
     const uint64_t tid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -131,6 +131,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, BAM_GATH
     uint64_t v = 0, any_left = 0;
     /* thread t takes requests t + k * threads, k = 0 .. N * rounds - 1, N at a time: what a wave, a workgroup and the launch
      * do once (the range's descriptor, the counters, the checksum) is shared by more reads the more rounds there are */
+    /* the indices of a round are asked for a round ahead: a read is four trips to memory one after the other (index,
+     * descriptor, element, descriptor again), and this takes the first out of the chain (44 against 41 thousand million reads
+     * a second with eight reads per lane).  Every lane loads (one without a request the first index): N loads side by side,
+     * no branch around any.  Read once: not to be kept in the L2 the descriptors live in */
+    size_t ahead[N];
+#pragma unroll
+    for (int j = 0; j < N; j++) {
+        const uint64_t t = tid + (uint64_t)j * threads;
+        ahead[j] = __builtin_nontemporal_load(assignment + (tid < threads && t < n_reqs ? t : 0));
+    }
     for (uint32_t r = 0; r < rounds; r++) {
         size_t idx[N];
         bool want[N], got[N];
@@ -139,16 +149,27 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, BAM_GATH
         for (int j = 0; j < N; j++) {
             const uint64_t t = tid + (uint64_t)(r * N + j) * threads;
             want[j] = tid < threads && t < n_reqs;
-            idx[j] = want[j] ? __builtin_nontemporal_load(assignment + t) : 0;      /* read once: not to be kept in the L2 the descriptors live in */
+            idx[j] = ahead[j];
+        }
+        if (r + 1 < rounds) {
+#pragma unroll
+            for (int j = 0; j < N; j++) {
+                const uint64_t t = tid + (uint64_t)((r + 1) * N + j) * threads;
+                ahead[j] = __builtin_nontemporal_load(assignment + (tid < threads && t < n_reqs ? t : 0));
+            }
         }
         dr->template seq_read_n_resident<N, true>(idx, want, out, got, view);
+        /* the N words of notes of the round with one store: lane j writes the j-th */
+        uint64_t mine = 0;
 #pragma unroll
         for (int j = 0; j < N; j++) {
             v += got[j] ? out[j] : 0;
-            const uint64_t m = bam::ballot(want[j] && !got[j]);
-            if (bam::lane() == 0 && tid < threads) missed[(tid + (uint64_t)(r * N + j) * threads) / BAM_WAVE_SIZE] = m;
+            const uint64_t m = bam::ballot(want[j] & !got[j]);
+            if (bam::lane() == (uint32_t)j) mine = m;
             any_left |= m;
         }
+        if (bam::lane() < (uint32_t)N && tid - bam::lane() < threads)
+            missed[(tid - bam::lane() + (uint64_t)(r * N + bam::lane()) * threads) / BAM_WAVE_SIZE] = mine;
     }
     view.flush_stats();
     if (any_left) note_work_left(finished, call);
@@ -833,6 +854,60 @@ __global__ __launch_bounds__(256) void k_read_stream(const uint64_t* __restrict_
     for (i += lane; i < mine; i += BAM_WAVE_SIZE) a += p[i];
     block_accumulate(partials, a);
 }
+/*
+ * The hit path of the streaming kernels taken apart, for measurement: a wave reads a run of resident pages of the cache,
+ * 4 KiB each, and what it does around the payload loads is chosen.  REFS 0: the page's descriptor is read for the slot and
+ * no reference is taken (only safe while nothing is evicted: a measurement, not an access route); 1: a reference per page,
+ * taken before the page is read and dropped after (what bam_ptr does); 2: the references of sixteen pages taken with one
+ * vector atomic and dropped with one (what the page-wise kernel does).  NT: the payload loads marked as not to be kept.
+ * The differences between the six and the plain reader (k_read_stream) are what each part of the protocol costs.
+ */
+template <int REFS, bool NT>
+__global__ __launch_bounds__(256) void k_hit_path_parts(array_d_t<uint64_t>* dr, uint64_t n_waves, uint64_t ppw, unsigned long long* partials)
+{
+    const uint64_t tid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const uint64_t wave = bam::first(tid / BAM_WAVE_SIZE);
+    const uint32_t lane = bam::lane();
+    uint64_t v = 0;
+    if (wave < n_waves) {
+        bam::range_view<uint64_t> view;
+        view.load(dr->d_ranges);
+        const uint64_t start_page = wave * ppw;
+        auto read_page = [&](const uint32_t slot) {
+            const uint64_t* base = (const uint64_t*)view.slot_addr(slot) + lane;
+            uint64_t x[8];
+            if (NT) bam::ld_payload_stream8(base, x);
+            else {
+#pragma unroll
+                for (int j = 0; j < 8; j++) x[j] = bam::ld_payload(base + j * BAM_WAVE_SIZE);
+            }
+            v += ((x[0] + x[1]) + (x[2] + x[3])) + ((x[4] + x[5]) + (x[6] + x[7]));
+        };
+        if (REFS == 2) {
+            for (uint64_t p0 = 0; p0 < ppw; p0 += 16) {
+                const uint32_t nb = (uint32_t)(ppw - p0 < 16 ? ppw - p0 : 16);
+                data_page_t* dp = view.pages + start_page + p0 + (lane < nb ? lane : 0);
+                uint64_t sv = 0;
+                if (lane < nb) sv = __hip_atomic_fetch_add((uint64_t*)dp, 1ull, __ATOMIC_RELAXED, BAM_AGENT);
+                const uint32_t slot = (uint32_t)(sv >> 32) & BAM_SLOT_MASK;
+                for (uint32_t k = 0; k < nb; k++) read_page(bam::bcast(slot, k));
+                bam::fence_meta();
+                if (lane < nb) __hip_atomic_fetch_add(&dp->state, 0u - 1u, __ATOMIC_RELAXED, BAM_AGENT);
+            }
+        } else {
+            for (uint64_t p = 0; p < ppw; p++) {
+                data_page_t* dp = view.pages + start_page + p;
+                uint64_t sv = 0;
+                if (REFS == 0) sv = __hip_atomic_load((uint64_t*)dp, __ATOMIC_RELAXED, BAM_AGENT);
+                else if (lane == 0) sv = __hip_atomic_fetch_add((uint64_t*)dp, (uint64_t)BAM_WAVE_SIZE, __ATOMIC_RELAXED, BAM_AGENT);
+                sv = bam::bcast(sv, 0);
+                read_page((uint32_t)(sv >> 32) & BAM_SLOT_MASK);
+                if (REFS == 1) { bam::fence_meta(); if (lane == 0) __hip_atomic_fetch_add(&dp->state, 0u - (uint32_t)BAM_WAVE_SIZE, __ATOMIC_RELAXED, BAM_AGENT); }
+            }
+        }
+    }
+    block_accumulate(partials, v);
+}
 /* plain random gather of 8-byte words from device memory: the ceiling of that access pattern without any cache protocol */
 __global__ void k_gather8(const uint64_t* __restrict__ src, const uint64_t* __restrict__ idx, uint64_t n, unsigned long long* partials)
 {
@@ -1219,9 +1294,10 @@ int bam_array_read_shaped(bam_array_t* a, uint64_t n_reqs, const uint64_t* d_ass
         hipLaunchKernelGGL(k_fold_partials, dim3(1), dim3(1024), 0, st, part, (unsigned long long*)d_sum);
     } else {
         const uint32_t N = reads_per_lane;
-        /* rounds of N reads per thread: as many as leave some eight thousand workgroups */
+        /* rounds of N reads per thread: as many as leave sixteen thousand workgroups, several times what the device holds at a time
+         * (a launch of about as many workgroups as the device holds ends with most of the device idle) */
         uint32_t rounds = 1;
-        while (rounds < 16 && n_reqs / ((uint64_t)N * rounds * 2 * 256) >= 8192) rounds *= 2;
+        while (rounds < 32 && n_reqs / ((uint64_t)N * rounds * 2 * 256) >= 16384) rounds *= 2;
         const uint64_t per_thread = (uint64_t)N * rounds;
         const uint64_t threads = ((n_reqs + per_thread - 1) / per_thread + BAM_WAVE_SIZE - 1) / BAM_WAVE_SIZE * BAM_WAVE_SIZE;
         const uint64_t n_words = threads / BAM_WAVE_SIZE * per_thread;
@@ -1258,7 +1334,9 @@ int bam_array_read(bam_array_t* a, uint64_t n_reqs, const uint64_t* d_assignment
      * thread (results and counters are the same) */
     if (d_assignment && reqs_per_thread == 1 && n_reqs >= (1ull << 16)) {
         static const int shape_env = getenv("BAM_READ_SHAPE") ? atoi(getenv("BAM_READ_SHAPE")) : 0;
-        static const int lanes_env = getenv("BAM_READS_PER_LANE") ? atoi(getenv("BAM_READS_PER_LANE")) : BAM_READS_PER_LANE;
+        /* eight reads per lane in the first launch: 44 thousand million reads a second on resident data against 39 with four
+         * (what bounds the kernel is how many requests a compute unit's L1 keeps in flight, and for how long each) */
+        static const int lanes_env = getenv("BAM_READS_PER_LANE") ? atoi(getenv("BAM_READS_PER_LANE")) : 8;
         int shape = two_launches_ok(a) ? BAM_READ_TWO_LAUNCHES : BAM_READ_FOUR_PER_THREAD;
         if (shape_env >= BAM_READ_ONE_PER_THREAD && shape_env <= BAM_READ_TWO_LAUNCHES && (shape_env != BAM_READ_TWO_LAUNCHES || two_launches_ok(a))) shape = shape_env;
         return bam_array_read_shaped(a, n_reqs, d_assignment, shape, (uint32_t)lanes_env, block_size, d_sum, stream);
@@ -1703,6 +1781,30 @@ int bam_read_kernel(const void* d_src, uint64_t n_bytes, float* ms, void* stream
     hip_err_chk(hipGetLastError());
     Event b(st);
     if (ms) *ms = (float)((b - a) / 1e3);
+    BAM_API_END
+}
+
+int bam_hit_path_parts(bam_array_t* a, int refs, int not_kept, uint64_t n_waves, uint64_t n_pages_per_wave, uint64_t* d_sum, void* stream)
+{
+    if (!a || !d_sum || refs < 0 || refs > 2) return fail(EINVAL, "bam_hit_path_parts: bad argument");
+    if (a->a->adt.n_ranges != 1 || a->a->h_ranges[0].cache.page_size != 4096) return fail(EINVAL, "bam_hit_path_parts: one range of 4 KiB pages");
+    if (n_waves * n_pages_per_wave > a->a->h_ranges[0].page_count) return fail(EINVAL, "bam_hit_path_parts: more pages than the range has");
+    if (!n_waves || !n_pages_per_wave) return 0;
+    BAM_API_BEGIN
+    hipStream_t st = (hipStream_t)stream;
+    array_d_t<uint64_t>* d = a->a->d_array_ptr;
+    unsigned long long* s = (unsigned long long*)a->partials.get();
+    const dim3 grid(blocks_for(n_waves * BAM_WAVE_SIZE, 256)), block(256);
+    switch (refs * 2 + (not_kept ? 1 : 0)) {
+    case 0: hipLaunchKernelGGL((k_hit_path_parts<0, false>), grid, block, 0, st, d, n_waves, n_pages_per_wave, s); break;
+    case 1: hipLaunchKernelGGL((k_hit_path_parts<0, true>), grid, block, 0, st, d, n_waves, n_pages_per_wave, s); break;
+    case 2: hipLaunchKernelGGL((k_hit_path_parts<1, false>), grid, block, 0, st, d, n_waves, n_pages_per_wave, s); break;
+    case 3: hipLaunchKernelGGL((k_hit_path_parts<1, true>), grid, block, 0, st, d, n_waves, n_pages_per_wave, s); break;
+    case 4: hipLaunchKernelGGL((k_hit_path_parts<2, false>), grid, block, 0, st, d, n_waves, n_pages_per_wave, s); break;
+    default: hipLaunchKernelGGL((k_hit_path_parts<2, true>), grid, block, 0, st, d, n_waves, n_pages_per_wave, s); break;
+    }
+    hipLaunchKernelGGL(k_fold_partials, dim3(1), dim3(1024), 0, st, s, (unsigned long long*)d_sum);
+    hip_err_chk(hipGetLastError());
     BAM_API_END
 }
 

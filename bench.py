@@ -229,6 +229,23 @@ def main():
     roofline["plain_read_kernel_GBps"] = (1 << 30) / best / 1e6
     log("[bench] hit path: %s" % hit)
     if args.only_hit:
+        # the hit path taken apart: what taking references (none / per page / sixteen at a time) and keeping the payload in the L2
+        # or not cost, against the plain reader above
+        parts = {}
+        for refs, rname in ((0, "no_reference"), (1, "reference_per_page"), (2, "references_16_at_a_time")):
+            for nt, nname in ((0, "kept"), (1, "not_kept")):
+                args_ = (arr.h, refs, nt, ctypes.c_uint64(CACHE_PAGES // STREAM_PAGES_PER_WAVE), ctypes.c_uint64(STREAM_PAGES_PER_WAVE), ctypes.c_void_p(s_hit.data_ptr()), stream)
+                s_hit.zero_()
+                assert L.bam_hit_path_parts(*args_) == 0
+                torch.cuda.synchronize()
+                assert int(s_hit.item()) & (2**64 - 1) == O.bo_store_sum(SEED, 0, 1, CACHE_PAGES * 512), "hit-path parts checksum mismatch"
+                a, b = event(), event()
+                L.bam_event_record(a, stream)
+                for _ in range(hit_reps):
+                    L.bam_hit_path_parts(*args_)
+                L.bam_event_record(b, stream)
+                parts["%s_%s_GBps" % (rname, nname)] = CACHE_PAGES * PAGE / (elapsed_ms(a, b) / hit_reps) / 1e6
+        roofline["hit_path_parts"] = parts
         # a plain device copy of known size in the same process: the scale of the profiler's traffic counters
         src = torch.empty(1 << 27, dtype=torch.int64, device=dev).fill_(1)
         dst = torch.empty_like(src)
@@ -252,7 +269,7 @@ def main():
     ms = elapsed_ms(a, b)
     assert int(s_hit.item()) & (2**64 - 1) == O.bo_gather_sum(SEED, SEED, 0, N_READS, CACHE_PAGES * 512), "hit gather checksum mismatch"
     gather_hit = {"reads_per_s": N_READS / ms * 1e3, "GBps_of_u64": N_READS * 8 / ms / 1e6, "ms": ms,
-                  "kernel": "k_array_read_n<4> (what bam_array_read launches for a launch of this size), with the launch that follows it for "
+                  "kernel": "k_array_read_n<8> (what bam_array_read launches for a launch of this size: eight reads per lane), with the launch that follows it for "
                             "requests whose page is not resident (none here) inside the timed region"}
     for shape, key in ((arr.ONE_PER_THREAD, "one_read_per_thread_reads_per_s"), (arr.FOUR_PER_THREAD, "four_per_thread_one_launch_reads_per_s")):
         arr.read_shaped_async(N_READS, s_hit.zero_(), idx_hit, shape, 4, block_size=args.block)
@@ -323,7 +340,7 @@ def main():
     # the same steps as bam_array_read runs a launch of this size by default: what is resident is read by a kernel that cannot
     # miss, the rest 64 requests to a wave by one that can; the first launch leaves the second only requests whose page it did
     # not find, and the pages those bring in are the ones the rest of the step asks for
-    two = run_steps(arr.TWO_LAUNCHES, 4)
+    two = run_steps(arr.TWO_LAUNCHES, 8)
     log("[bench] cfg2, two launches: %s" % two)
     del idx, sums
     if args.probe:

@@ -108,7 +108,7 @@ int bam_array_read(bam_array_t* a, uint64_t n_reqs, const uint64_t* d_assignment
  *                             kernel that cannot miss (no call, no stack, a fraction of the registers) and notes the rest;
  *                             a second launch reads the rest, one request per lane and 64 per wave whatever the share of
  *                             misses was.  Arrays of one range only (EINVAL otherwise).
- * bam_array_read picks BAM_READ_TWO_LAUNCHES with four reads per lane for launches of 2^16 requests and more where the array
+ * bam_array_read picks BAM_READ_TWO_LAUNCHES with eight reads per lane for launches of 2^16 requests and more where the array
  * allows it (BAM_READ_FOUR_PER_THREAD where not) and BAM_READ_ONE_PER_THREAD below that. */
 #define BAM_READ_ONE_PER_THREAD  1
 #define BAM_READ_FOUR_PER_THREAD 2
@@ -347,6 +347,13 @@ int bam_host_read_ceiling(uint64_t n_bytes, uint32_t chunk_bytes, float* ms);
  * read of n bytes, and a gather of n 8-byte words at d_idx[] from d_src; elapsed milliseconds */
 int bam_read_kernel(const void* d_src, uint64_t n_bytes, float* ms, void* stream);
 int bam_gather_kernel(const uint64_t* d_src, const uint64_t* d_idx, uint64_t n, float* ms, void* stream);
+/* The hit path of the streaming kernels taken apart (measurement only): n_waves waves read runs of n_pages_per_wave pages of
+ * the array's one range, which must all be resident and must stay so (nothing may evict meanwhile), and add every word into
+ * *d_sum.  refs 0: the descriptor is read for the slot, no reference taken; 1: a reference per page, taken before and dropped
+ * after, as bam_ptr does; 2: the references of sixteen pages per vector atomic, as the page-wise kernel does.  not_kept:
+ * payload loads marked as not to be kept in the L2.  Against bam_read_kernel (no protocol at all) the six say what each part
+ * costs.  4 KiB pages. */
+int bam_hit_path_parts(bam_array_t* a, int refs, int not_kept, uint64_t n_waves, uint64_t n_pages_per_wave, uint64_t* d_sum, void* stream);
 /* the atomics of a hit that takes and drops a reference, without the cache around them: per request an add on the 8-byte
  * word d_table[d_idx[t]] and, once it is back, the opposite add on the same word (the table ends as it began).
  * returns != 0: the first add hands back the old word, as bam_try_hit needs it; 0: neither result is read. */

@@ -1280,28 +1280,39 @@ struct array_d_t {
             if (one && v.r->cache.fast_reads) {
                 const data_page_t* dp[N];
                 const uint64_t* p[N];
-                uint64_t s1[N], in_page[N], x[N];
+                uint64_t s1[N], x[N];
+                uint32_t in_page[N];
                 bool res[N];
 #pragma unroll
                 for (int j = 0; j < N; j++) {
                     res[j] = want[j] && idx[j] - v.index_start < v.index_end - v.index_start;
                     const uint64_t byte = res[j] ? v.byte_of(idx[j]) : 0;
                     dp[j] = v.pages + (byte >> v.page_size_log);
-                    in_page[j] = byte & (v.page_size - 1);
+                    in_page[j] = (uint32_t)byte & (v.page_size - 1);
                 }
 #pragma unroll
                 for (int j = 0; j < N; j++) s1[j] = __hip_atomic_load((const uint64_t*)dp[j], __ATOMIC_RELAXED, BAM_AGENT);
 #pragma unroll
+                for (int j = 0; j < N; j++) asm volatile("" : "+v"(s1[j]));
+#pragma unroll
                 for (int j = 0; j < N; j++) {
-                    res[j] = res[j] && ((uint32_t)s1[j] >> (CNT_SHIFT + 1)) == V_NB;
+                    res[j] = res[j] & (((uint32_t)s1[j] >> (CNT_SHIFT + 1)) == V_NB);
                     p[j] = (const uint64_t*)(v.base_addr + (res[j] ? ((uint64_t)((uint32_t)(s1[j] >> 32) & BAM_SLOT_MASK) << v.page_size_log) + in_page[j] : 0));
                 }
                 bam::ld_payload_nt(p, x);               /* with its wait: the elements are here before the second looks go out */
+                uint64_t s2[N];
+#pragma unroll
+                for (int j = 0; j < N; j++) s2[j] = __hip_atomic_load((const uint64_t*)dp[j], __ATOMIC_RELAXED, BAM_AGENT);
+                /* all N looks are out before the first is used (left to itself the compiler moves each look into the branch
+                 * that uses it, one wait per look) */
+#pragma unroll
+                for (int j = 0; j < N; j++) asm volatile("" : "+v"(s2[j]));
 #pragma unroll
                 for (int j = 0; j < N; j++) {
-                    const uint64_t s2 = __hip_atomic_load((const uint64_t*)dp[j], __ATOMIC_RELAXED, BAM_AGENT);
-                    got[j] = res[j] && ((s1[j] ^ s2) & 0xFFFFFFFFC0000000ull) == 0;
-                    if (got[j]) { out[j] = *(T*)&x[j]; v.account(true); }
+                    got[j] = res[j] & (((s1[j] ^ s2[j]) & 0xFFFFFFFFC0000000ull) == 0);
+                    out[j] = got[j] ? *(T*)&x[j] : T();
+                    v.n_access += got[j] ? 1u : 0u;
+                    v.n_hit += got[j] ? 1u : 0u;
                 }
             }
             return;
