@@ -48,8 +48,8 @@ STREAM_PAGES_PER_WAVE = 16      # pages per wave of the streaming kernels (one a
 # counters scaled by what they read for a plain 1 GiB copy; figures, commands and date in the files named.  They hold for
 # this workload and the tree state the profile was taken on, which is why the source is printed beside them.
 HIT_TRAFFIC = {
-    "bam_ptr": {"bytes": None, "source": None},
-    "page_wise": {"bytes": 1079592960, "source": "profiles/k_cache_stream_pages_hit_path_1GiB_cache.md"},
+    "bam_ptr": {"bytes": 1092679680, "source": "profiles/k_cache_stream_hit_path_1GiB_cache.md"},
+    "page_wise": {"bytes": 1079590912, "source": "profiles/k_cache_stream_hit_path_1GiB_cache.md"},
 }
 
 
@@ -110,6 +110,7 @@ def main():
     ap.add_argument("--probe-batches", type=str, default="",
                     help="comma-separated K: 65536 waves whose 64 lanes read K distinct pages of a cold 4 GiB cache, one launch per K, "
                          "batches per second and I/Os per second (with BAM_AMD_LIB naming the build with the phase timers, those too); nothing else")
+    ap.add_argument("--pages-per-wave", type=int, default=STREAM_PAGES_PER_WAVE, help="pages a wave of the streaming kernels reads (a power of two up to 16)")
     ap.add_argument("--only-hit", action="store_true",
                     help="hit-path leg and a plain 1 GiB copy only (short; what the counter passes of the profiler are run on)")
     args = ap.parse_args()
@@ -150,6 +151,7 @@ def main():
         rows = []
         for K in [int(x) for x in args.probe_batches.split(",")]:
             pc, rng, arr = make_array(ctrl, n_el, PAGE, 1 << 20)
+            waves = min(1 << 16, n_el // 512 // K)          # every wave its own K pages of the store
             tid = torch.arange(waves * 64, dtype=torch.int64, device=dev)
             idx_k = ((tid // 64) * K + (tid % 64) % K) * 512 + (tid % 64)
             s_k = torch.zeros(1, dtype=torch.int64, device=dev)
@@ -160,7 +162,8 @@ def main():
             L.bam_event_record(b, stream)
             ms = elapsed_ms(a, b)
             st, pr = arr.stats(), pc.profile()
-            row = {"K": K, "ms": ms, "read_ios": st["read_io_cnt"], "M_batches_per_s": waves / ms / 1e3, "MIOPS": st["read_io_cnt"] / ms / 1e3}
+            assert st["read_io_cnt"] == waves * K
+            row = {"K": K, "waves": waves, "ms": ms, "read_ios": st["read_io_cnt"], "M_batches_per_s": waves / ms / 1e3, "MIOPS": st["read_io_cnt"] / ms / 1e3}
             if pr["batches"]:
                 nb_ = pr["batches"]
                 row["per_batch_us"] = {k: pr[k] / nb_ / 100 for k in ("t_cid", "t_submit", "t_wait", "t_copy")}
@@ -185,7 +188,9 @@ def main():
     log("[bench] set-up %.1fs: %s %s" % (time.time() - t0, ctrl.info(), pc.info()))
 
     # ------------------------------------------------------------------ hit path (roofline): stream the resident cache
-    arr.stream(CACHE_PAGES // STREAM_PAGES_PER_WAVE, STREAM_PAGES_PER_WAVE, mode=2)             # cold pass fills the cache with pages 0 .. CACHE_PAGES-1
+    ppw = args.pages_per_wave
+    assert ppw in (1, 2, 4, 8, 16)
+    arr.stream(CACHE_PAGES // ppw, ppw, mode=2)             # cold pass fills the cache with pages 0 .. CACHE_PAGES-1
     arr.stats()
     ref_stream = O.bo_store_sum(SEED, 0, 1, 1 << 24)
     hit_reps = 20
@@ -196,14 +201,14 @@ def main():
     kinds = ((1, "bam_ptr"), (2, "page_wise"), (6, "bam_ptr_one_launch"), (0, "element_operator"))
     for mode, name in kinds:
         assert arr.stream((1 << 24) // 512 // 4, 4, mode=mode) == ref_stream, "hit-path checksum mismatch (%s)" % name
-        arr.stream_async(CACHE_PAGES // STREAM_PAGES_PER_WAVE, STREAM_PAGES_PER_WAVE, s_hit, mode=mode)
+        arr.stream_async(CACHE_PAGES // ppw, ppw, s_hit, mode=mode)
     torch.cuda.synchronize()
     hit = {}
     for mode, name in kinds:
         a, b = event(), event()
         L.bam_event_record(a, stream)
         for _ in range(hit_reps):
-            arr.stream_async(CACHE_PAGES // STREAM_PAGES_PER_WAVE, STREAM_PAGES_PER_WAVE, s_hit, mode=mode)
+            arr.stream_async(CACHE_PAGES // ppw, ppw, s_hit, mode=mode)
         L.bam_event_record(b, stream)
         ms = elapsed_ms(a, b) / hit_reps
         hit[name] = {"ms_per_launch": ms, "GBps": CACHE_PAGES * PAGE / ms / 1e6}
@@ -213,7 +218,7 @@ def main():
                                           "with the launch that follows it for pages that are not resident (none here) inside the timed region",
                 "achieved": hit["bam_ptr"]["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": hit["bam_ptr"]["GBps"] / HBM_PEAK_GBS, "traffic": HIT_TRAFFIC["bam_ptr"]["bytes"], "traffic_source": HIT_TRAFFIC["bam_ptr"]["source"],
-                "bytes_per_launch": CACHE_PAGES * PAGE, "ms_per_launch": hit["bam_ptr"]["ms_per_launch"], "pages_per_wave": STREAM_PAGES_PER_WAVE,
+                "bytes_per_launch": CACHE_PAGES * PAGE, "ms_per_launch": hit["bam_ptr"]["ms_per_launch"], "pages_per_wave": ppw,
                 "page_wise_kernel": {"kernel": "k_cache_stream_pages (one acquire per 16 pages, streamed loads; no counterpart in the reference)",
                                      "achieved": hit["page_wise"]["GBps"], "frac": hit["page_wise"]["GBps"] / HBM_PEAK_GBS,
                                      "ms_per_launch": hit["page_wise"]["ms_per_launch"],
@@ -234,7 +239,7 @@ def main():
         parts = {}
         for refs, rname in ((0, "no_reference"), (1, "reference_per_page"), (2, "references_16_at_a_time")):
             for nt, nname in ((0, "kept"), (1, "not_kept")):
-                args_ = (arr.h, refs, nt, ctypes.c_uint64(CACHE_PAGES // STREAM_PAGES_PER_WAVE), ctypes.c_uint64(STREAM_PAGES_PER_WAVE), ctypes.c_void_p(s_hit.data_ptr()), stream)
+                args_ = (arr.h, refs, nt, ctypes.c_uint64(CACHE_PAGES // ppw), ctypes.c_uint64(ppw), ctypes.c_void_p(s_hit.data_ptr()), stream)
                 s_hit.zero_()
                 assert L.bam_hit_path_parts(*args_) == 0
                 torch.cuda.synchronize()
