@@ -200,6 +200,29 @@ def test_every_element_of_a_gather_and_of_an_update_under_eviction(bam, cache_pa
         assert not r.c.aborted() and r.c.info()["error_completions"] == 0 and r.t.stats()["write_cmds"] > 0
 
 
+@pytest.mark.parametrize("fast", ["1", "0"])
+def test_reads_with_and_without_a_reference_give_the_same_elements(bam, fast, monkeypatch):
+    """BAM_FAST_READS=0 takes out the read of a resident page that holds no reference (two looks at the page's descriptor
+    around the load instead): every read then counts itself in and out, as in the reference.  The elements of a gather
+    under eviction (a cache of 256 pages under 2^18 random reads, so every slot changes hands a thousand times while other
+    waves read), the sum of the same launch as bam_array_read shapes it and the number of accesses are the same either way."""
+    monkeypatch.setenv("BAM_FAST_READS", fast)
+    n_elems, n = 1 << 22, 1 << 18
+    rng = np.random.default_rng(SEED + 1)
+    with Rig(bam, n_elems * 8, backing=True, n_queues=4, depth=64) as r:
+        store = r.backing(n_elems)
+        store[:] = oracle.store(SEED, 0, n_elems)
+        a = r.array(n_elems, 4096, 256)
+        idx = rng.integers(0, n_elems, n).astype(np.uint64)
+        d_idx, want = _dev(idx), store[idx.astype(np.int64)]
+        for _ in range(2):
+            assert np.array_equal(_u64(a.gather(n, d_idx, block_size=64)), want)
+        a.stats()
+        assert a.read(n, d_idx, block_size=256) == int(np.sum(want, dtype=np.uint64))
+        assert a.stats()["access_cnt"] == n
+        assert not r.c.aborted() and r.c.info()["error_completions"] == 0
+
+
 @pytest.mark.parametrize("stage_bytes,cache_pages", [(4096, 5), (0, 5), (4096, 16)])
 def test_pages_loaded_on_one_cluster_are_read_on_the_others(bam, stage_bytes, cache_pages):
     """The device has eight clusters of compute units with an L2 each.  A page that a wave on one cluster brings into the

@@ -13,7 +13,7 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 REF = "/root/reference"
 
-# (namespace, file under the reference tree, [(first line, last line), ...]) - the kernels VERDICT-style citations name:
+# (namespace, file under the reference tree, [(first line, last line), ...]) - the kernels of the five benchmarks:
 # array: sequential_access_kernel / random_access_kernel; block: sequential_access_kernel; cache: random_access_warp /
 # sequential_access_warp; bfs: kernel_coalesce_coarse_ptr_pc; cc: cc_compute + kernel_coalesce_coarse_ptr_pc
 KERNELS = [
