@@ -627,6 +627,11 @@ def main():
         "cpu_baseline": cpu, "store": store, "hit_gather": gather_hit, "block": block, "bfs": bfs, "cc": cc,
     }
     print(json.dumps(out), flush=True)
+    # nothing of this process outlives the line above: every target, controller and CPU-path handle has been closed (their
+    # service threads joined), the thread pool of the serial BFS oracle was a context manager
+    import threading
+    log("[bench] done; python threads alive: %d, native threads of the process: %d"
+        % (threading.active_count(), len(os.listdir("/proc/self/task"))))
 
 
 if __name__ == "__main__":
