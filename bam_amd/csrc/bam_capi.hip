@@ -118,11 +118,8 @@ __global__ void k_array_read_n_whole(array_d_t<uint64_t>* dr, uint64_t n_reqs, c
  * carries the registers of the miss path (four waves per SIMD) and its frame in scratch memory through every read.  The
  * last workgroup folds the checksum of what was read; the second launch adds what it reads.
  */
-#ifndef BAM_GATHER_MIN_WAVES
-#define BAM_GATHER_MIN_WAVES 1
-#endif
 template <int N>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BAM_GATHER_MIN_WAVES))) void k_array_read_n(array_d_t<uint64_t>* dr, uint64_t n_reqs, const uint64_t* __restrict__ assignment, uint64_t threads, uint32_t rounds,
+__global__ __launch_bounds__(256) void k_array_read_n(array_d_t<uint64_t>* dr, uint64_t n_reqs, const uint64_t* __restrict__ assignment, uint64_t threads, uint32_t rounds,
                                                       unsigned long long* partials, uint64_t* missed, unsigned long long* sum, uint32_t* finished, uint32_t call)
 {
     const uint64_t tid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -589,11 +586,8 @@ __global__ __launch_bounds__(256) void k_cache_stream_pages(array_d_t<uint64_t>*
  * launch (k_cache_stream_deferred), which has the miss path.  A kernel that can miss carries the registers and the stack of
  * the miss path through every page visit (four waves per SIMD, a frame in scratch memory); this one has neither.
  */
-#ifndef BAM_STREAM_MAX_WAVES
-#define BAM_STREAM_MAX_WAVES 8
-#endif
 template <int MODE>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, BAM_STREAM_MAX_WAVES))) void k_cache_stream(array_d_t<uint64_t>* dr, uint64_t n_waves, uint64_t n_pages_per_wave, const uint64_t* assignment, unsigned long long* partials,
+__global__ __launch_bounds__(256) void k_cache_stream(array_d_t<uint64_t>* dr, uint64_t n_waves, uint64_t n_pages_per_wave, const uint64_t* assignment, unsigned long long* partials,
                                                       uint8_t* deferred, unsigned long long* sum, uint32_t* finished, uint32_t call)
 {
     static_assert(MODE == 0 || MODE == 1, "the page-wise mode and the fetching modes are kernels of their own");

@@ -116,30 +116,6 @@ __device__ __forceinline__ void for_each_group(const uint64_t key, F&& body)
 {
     for_each_group(key, 0, [&](uint64_t a, uint64_t) { body(a); });
 }
-/*
- * The same with the groups taken in ascending order of their key, whatever lanes hold them.  For work that takes
- * something per key and keeps it while it takes the next (slots of several queues): when every wave takes in the same
- * order, no two can each hold what the other is waiting for.  Costs a pass over the distinct keys still to be served per
- * group (scalar reads and ballots), so it is for the places that need the order.
- */
-template <typename F>
-__device__ __forceinline__ void for_each_group_ascending(const uint64_t key, F&& body)
-{
-    uint64_t todo = active_mask();
-    while (todo) {
-        uint64_t least = ~0ull, least_grp = 0;
-        for (uint64_t rest = todo; rest;) {
-            const uint64_t a = bcast(key, first_lane(rest));
-            const uint64_t grp = ballot(key == a) & todo;
-            if (a <= least) { least = a; least_grp = grp; }
-            rest &= ~grp;
-        }
-        const bool mine = (least_grp >> lane()) & 1;
-        if (mine) body(least);
-        todo &= ~least_grp;
-    }
-}
-
 /* compute-unit identity across the whole device: XCC, shader engine and CU bits */
 __device__ __forceinline__ uint32_t cu_id() { return __smid(); }
 
