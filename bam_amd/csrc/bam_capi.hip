@@ -460,7 +460,8 @@ __device__ __forceinline__ bool stream_page(array_d_t<uint64_t>* dr, PTR& ptr, b
             }
             sum += acc;
         }
-        if constexpr (DEFER) { miss = ptr.missed; ptr.missed = false; }
+        /* a pointer that holds no reference: what it read of the page counts if the page is still what it was */
+        if constexpr (DEFER) { ptr.still(); miss = ptr.missed; ptr.missed = false; }
     }
     if constexpr (DEFER) {
         if (bam::ballot(miss)) {

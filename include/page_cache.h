@@ -1016,21 +1016,7 @@ struct range_view {
     {
         acquire_<OUTLINE, true>(page, write, on_hit, on_miss, take);
     }
-    /*
-     * The hit half alone, for kernels that are launched in two passes: a group whose page is resident is served as
-     * acquire() serves it; a group whose page is not gives its references back at once and its lanes come back with
-     * true (nothing was called for them).  The caller notes what it could not read and a second launch, of a kernel
-     * that has the miss path, reads it.  A kernel that is made of this half only has no call in it, needs no stack and
-     * a fraction of the registers: what the path for resident pages costs, and nothing of what a miss would.
-     */
-    template <typename FH>
-    __forceinline__ __device__ bool acquire_or_defer(const uint64_t page, const bool write, FH&& on_hit)
-    {
-        bool deferred = false;
-        acquire_<false, false, true>(page, write, on_hit, [&](uint32_t) { deferred = true; return false; }, true);
-        return deferred;
-    }
-    template <bool OUTLINE, bool HELPERS, bool DEFER = false, typename FH, typename FM>
+    template <bool OUTLINE, bool HELPERS, typename FH, typename FM>
     __forceinline__ __device__ void acquire_(const uint64_t page_, const bool write, FH&& on_hit, FM&& on_miss, const bool take)
     {
         const uint32_t me = lane();
@@ -1051,10 +1037,6 @@ struct range_view {
             /* the lanes of a group may answer differently (one keeps the page, another only touched it) */
             const uint32_t n_drop = popc(ballot(drop) & eq_mask);
             if (n_drop && master == me) bam_release_refs(dp, n_drop, dirty);
-        } else if constexpr (DEFER) {
-            /* not resident: the references go back (nothing was read through them, so nothing has to be waited for) */
-            if (master == me) __hip_atomic_fetch_add(&dp->state, 0u - count, __ATOMIC_RELAXED, BAM_AGENT);
-            on_miss(BAM_NO_SLOT);
         } else {
             /* miss path: pass after pass; groups whose page came in are served and release before the next pass */
             const uint32_t queue = wave_slot_hash();
@@ -1531,8 +1513,12 @@ struct bam_ref {
  * stay inside that range.
  *
  * DEFER (no counterpart in the reference): a pointer for the first of two launches.  It reads what is resident; when
- * the page of an access is not, the access yields T(), `missed` is set and nothing is loaded (range_view::
- * acquire_or_defer): the kernel notes the work for the second launch, which uses a plain bam_ptr.  Reads only.
+ * the page of an access is not, the access yields T(), `missed` is set and nothing is loaded: the kernel notes the work
+ * for the second launch, which uses a plain bam_ptr.  Reads only, and it holds no reference: the window is opened on a
+ * look at the page's descriptor (valid, not busy: slot and load count noted), and what was read through it counts only
+ * once still() has looked again and found the same, as for every read of a resident page that takes no reference
+ * (bam_read_unpinned).  A reference is two read-modify-writes of the descriptor per page, and those are performed at
+ * the memory, not in a cache: taking them out is worth a fifth of the rate of a wave that streams through pages.
  */
 template <typename T, bool DEFER>
 struct bam_ptr {
@@ -1543,7 +1529,10 @@ struct bam_ptr {
     int64_t range_id = -1;
     T* addr = nullptr;
     bool dirty = false;
-    bool missed = false;             /* DEFER: an access since the flag was last cleared found its page not resident */
+    bool missed = false;             /* DEFER: an access since the flag was last cleared found its page not resident (any more) */
+    uint64_t seen = 0;               /* DEFER: the descriptor as it was when the window was opened */
+    data_page_t* ahead = nullptr;    /* DEFER: the descriptor after the window's, looked at when the window was opened, */
+    uint64_t ahead_sv = 0;           /* and what was seen there: a walk along an array finds its next look already made */
 #if defined(__HIP_DEVICE_COMPILE__)
     bam::range_view<T> view;
 #endif
@@ -1561,10 +1550,8 @@ struct bam_ptr {
     __forceinline__ __host__ __device__ void fini(void)
     {
 #if defined(__HIP_DEVICE_COMPILE__)
-        if (page) {
-            view.release((uint64_t)(page - view.pages), dirty);
-            page = nullptr;
-        }
+        if constexpr (!DEFER) { if (page) view.release((uint64_t)(page - view.pages), dirty); }
+        page = nullptr;
 #endif
     }
 
@@ -1573,7 +1560,15 @@ struct bam_ptr {
     __forceinline__ __host__ __device__ T* update_page(const size_t i)
     {
 #if defined(__HIP_DEVICE_COMPILE__)
-        if constexpr (DEFER) { if (view.holds(i)) return move_window(i); }
+        if constexpr (DEFER) {
+            if (!view.holds(i)) {
+                page = nullptr; start = end = 0; addr = nullptr;
+                range_id = array->find_range(i);
+                if (range_id == -1) { view.r = nullptr; return nullptr; }
+                view.load(array->d_ranges + range_id);
+            }
+            return move_window(i);
+        }
 #endif
         return update_page_general(i);
     }
@@ -1593,10 +1588,7 @@ struct bam_ptr {
         const uint64_t pg = view.page_of(i);
         uint32_t slot = BAM_NO_SLOT;
         auto keep = [&](uint32_t s_) { slot = s_; return false; };
-        if constexpr (DEFER) {
-            if (view.acquire_or_defer(pg, false, keep)) { missed = true; return nullptr; }      /* no reference is held */
-        } else
-            view.template acquire<true>(pg, false, keep, keep);
+        view.template acquire<true>(pg, false, keep, keep);
         page = view.pages + pg;                 /* the references of the group stay counted either way */
         if (slot == BAM_NO_SLOT) return nullptr;        /* the wait was given up (the controller is marked aborted): no window */
         view.window(pg, start, end);
@@ -1607,36 +1599,41 @@ struct bam_ptr {
 
 #if defined(__HIP_DEVICE_COMPILE__)
     /*
-     * DEFER: the window moves to the page of element i, which the range at hand holds.  Giving the old page back and
-     * taking the new one is one grouping of the lanes (by both pages at once: lanes that leave the same page for the same
-     * page share the two atomics) instead of one each; nothing else of update_page is needed for a pointer that only
-     * reads what is resident.
+     * DEFER: the window moves to the page of element i, which the range at hand holds: one look at the page's descriptor.
+     * Where the lanes of the wave all go to the same page (a wave that walks pages together) the window and the address
+     * of its first element are worked out once per wave, over the scalar unit, instead of once per lane.
      */
     __forceinline__ __device__ T* move_window(const size_t i)
     {
         using namespace bam;
-        data_page_t* const old_dp = page;
         const uint64_t pg = view.page_of(i);
-        data_page_t* const new_dp = view.pages + pg;
-        const uint64_t eq = match_any((uint64_t)old_dp, (uint64_t)new_dp);
-        const uint32_t master = first_lane(eq), cnt = popc(eq);
-        uint64_t sv = 0;
-        if (lane() == master) {
-            /* the loads of the old page are in (a wait on the wave's counter covers every lane's) before its count drops */
-            if (old_dp) { fence_meta(); __hip_atomic_fetch_add(&old_dp->state, 0u - cnt, __ATOMIC_RELAXED, BAM_AGENT); }
-            sv = __hip_atomic_fetch_add((uint64_t*)new_dp, (uint64_t)cnt, __ATOMIC_RELAXED, BAM_AGENT);
-        }
-        /* one group, as when a wave walks a page together: the word comes over the scalar unit */
-        if (first(eq) == active_mask()) sv = bcast(sv, first_lane(active_mask()));
-        else sv = shfl(sv, master);
+        const uint64_t upg = first(pg);
+        const bool together = ballot(pg != upg) == 0;
+        data_page_t* const dp = view.pages + (together ? upg : pg);
+        uint64_t sv = ahead_sv;
+        if (ahead != dp) sv = __hip_atomic_load((const uint64_t*)dp, __ATOMIC_RELAXED, BAM_AGENT);
+        ahead = nullptr;
         if (((uint32_t)sv >> (CNT_SHIFT + 1)) == V_NB) {
             view.account(true);
-            page = new_dp;
-            view.window(pg, start, end);
-            addr = (T*)(view.slot_addr((uint32_t)(sv >> 32) & BAM_SLOT_MASK) + (view.byte_of(start) & (view.page_size - 1)));
+            page = dp;
+            seen = sv;
+            if (together) {
+                size_t s_, e_;
+                view.window(upg, s_, e_);
+                start = s_; end = e_;
+                addr = (T*)(view.slot_addr((uint32_t)(sv >> 32) & BAM_SLOT_MASK) + (view.byte_of(s_) & (view.page_size - 1)));
+            } else {
+                view.window(pg, start, end);
+                addr = (T*)(view.slot_addr((uint32_t)(sv >> 32) & BAM_SLOT_MASK) + (view.byte_of(start) & (view.page_size - 1)));
+            }
+            /* the look at the next page goes out now, beside this page's reads, and is not used before the next move: a
+             * page then costs a walking wave its reads and the look that confirms them, not a third trip between them */
+            if (end < view.index_end) {
+                ahead = dp + 1;
+                ahead_sv = __hip_atomic_load((const uint64_t*)(dp + 1), __ATOMIC_RELAXED, BAM_AGENT);
+            }
             return addr;
         }
-        if (lane() == master) __hip_atomic_fetch_add(&new_dp->state, 0u - cnt, __ATOMIC_RELAXED, BAM_AGENT);
         page = nullptr;
         start = end = 0;
         addr = nullptr;
@@ -1644,6 +1641,27 @@ struct bam_ptr {
         return nullptr;
     }
 #endif
+
+    /*
+     * DEFER: whether what was read through the window since it was opened stands: the page is still valid, not busy, in
+     * the same slot and loaded the same number of times (the reads have come back: callers ask after using them).  If
+     * not, `missed` is set and the window is closed, as if the page had not been resident in the first place.
+     */
+    __forceinline__ __host__ __device__ bool still()
+    {
+#if defined(__HIP_DEVICE_COMPILE__)
+        if (!page) return true;
+        const uint64_t now = __hip_atomic_load((const uint64_t*)page, __ATOMIC_RELAXED, BAM_AGENT);
+        if (((seen ^ now) & 0xFFFFFFFFC0000000ull) == 0) return true;
+        page = nullptr;
+        start = end = 0;
+        addr = nullptr;
+        missed = true;
+        return false;
+#else
+        return true;
+#endif
+    }
 
     /* after a wait that was given up the value is T(): callers that use what they read as an index (the neighbour
      * ids of a graph) stay inside their arrays until the host sees the abort */
@@ -1701,6 +1719,15 @@ struct bam_ptr {
     __forceinline__ __host__ __device__ void peek_n(const size_t i, const size_t stride, T (&out)[N]) const
     {
 #if defined(__HIP_DEVICE_COMPILE__)
+        if constexpr (sizeof(T) == 8 && N == 8) {
+            if (stride == BAM_WAVE_SIZE) {              /* a wave's share of a page side by side: one address, eight offsets */
+                uint64_t x[8];
+                bam::ld_payload_stream8((const uint64_t*)(addr + (i - start)), x);
+#pragma unroll
+                for (int u = 0; u < N; u++) out[u] = *(T*)&x[u];
+                return;
+            }
+        }
         if constexpr (sizeof(T) == 8 && (N == 1 || N == 2 || N == 4 || N == 7 || N == 8)) {
             const uint64_t* p[N];
             uint64_t x[N];

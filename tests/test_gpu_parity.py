@@ -403,6 +403,46 @@ def test_page_streaming_modes(bam, mode):
         assert not r.c.aborted()
 
 
+def test_streaming_what_is_resident_while_another_stream_evicts(bam):
+    """Two arrays behind one cache, each driven from a stream of its own.  One is streamed element by element (modes 0 and
+    1: first a launch that reads what is resident without holding it, every page confirmed by a second look at its
+    descriptor, then a launch for the rest) while random reads of the other, four times the cache, take its pages away
+    under it: a page that goes between the two looks must be left to the second launch, and a page that goes and comes
+    back must not be read half old, half new.  Every sum of both arrays is exact, launch after launch."""
+    import torch
+    page, nx_pages, ny_pages, cache_pages, n = 4096, 2048, 8192, 1024, 1 << 17
+    nx, ny = nx_pages * 512, ny_pages * 512
+    with Rig(bam, (nx + ny) * 8, n_queues=16, depth=256) as r:
+        pc = bam.PageCache(page, cache_pages, 0, r.c)
+        rx = bam.Range(0, nx, 0, nx_pages, 0, page, pc, 0)
+        ry = bam.Range(0, ny, nx_pages, ny_pages, 0, page, pc, 0)
+        ax, ay = bam.Array(nx, 0, [rx], 0), bam.Array(ny, nx_pages * page, [ry], 0)
+        want_x = oracle.lib().bo_store_sum(SEED, 0, 1, nx)
+        words_y = oracle.store(SEED, nx, ny)
+        rng = np.random.default_rng(SEED + 5)
+        reps = 8
+        idx = [rng.integers(0, ny, n).astype(np.uint64) for _ in range(reps)]
+        d_idx = [_dev(i) for i in idx]
+        sums_x = [torch.zeros(1, dtype=torch.int64, device="cuda:0") for _ in range(reps)]
+        sums_y = [torch.zeros(1, dtype=torch.int64, device="cuda:0") for _ in range(reps)]
+        sx, sy = torch.cuda.Stream(), torch.cuda.Stream()
+        torch.cuda.synchronize()
+        for k in range(reps):
+            with torch.cuda.stream(sx):
+                ax.stream_async(nx_pages // 16, 16, sums_x[k], mode=k % 2)
+            with torch.cuda.stream(sy):
+                ay.read_async(n, sums_y[k], d_idx[k], block_size=256)
+        torch.cuda.synchronize()
+        for k in range(reps):
+            assert int(sums_x[k].item()) & (2**64 - 1) == want_x, "streamed array, launch %d" % k
+            assert int(sums_y[k].item()) & (2**64 - 1) == int(np.sum(words_y[idx[k].astype(np.int64)], dtype=np.uint64)), "gathered array, launch %d" % k
+        # one access per element through operator[] (mode 0), one per lane and page through bam_ptr (mode 1): a page that was
+        # given up on in the first launch is counted in the second and nowhere else
+        assert ax.stats()["access_cnt"] == reps // 2 * (nx + nx_pages * 64) and ay.stats()["access_cnt"] == reps * n
+        assert r.t.stats()["read_cmds"] > reps * nx_pages // 2 and not r.c.aborted() and r.c.info()["error_completions"] == 0
+        ax.close(); ay.close(); rx.close(); ry.close(); pc.close()
+
+
 @pytest.mark.parametrize("mode", [0, 1, 3, 4, 5, 6])
 @pytest.mark.parametrize("page", [512, 4096, 16384])
 def test_element_streaming_over_other_page_sizes_and_a_ragged_last_page(bam, mode, page):
