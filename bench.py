@@ -48,7 +48,7 @@ STREAM_PAGES_PER_WAVE = 16      # pages per wave of the streaming kernels (one a
 # counters scaled by what they read for a plain 1 GiB copy; figures, commands and date in the files named.  They hold for
 # this workload and the tree state the profile was taken on, which is why the source is printed beside them.
 HIT_TRAFFIC = {
-    "bam_ptr": {"bytes": 1092679680, "source": "profiles/k_cache_stream_hit_path_1GiB_cache.md"},
+    "bam_ptr": {"bytes": 1078487040, "source": "profiles/k_cache_stream_hit_path_1GiB_cache.md"},
     "page_wise": {"bytes": 1079590912, "source": "profiles/k_cache_stream_hit_path_1GiB_cache.md"},
 }
 

@@ -153,8 +153,10 @@ int bam_sqe_image(uint16_t cid, uint8_t opcode, uint32_t nsid, uint64_t prp1, ui
  * wave that gets ahead of them touches the missing pages of its run itself, up to 64 at a time (12 M instead of 2.5 M
  * pages per second on a cold cache).
  * Modes 0 and 1 on an array of one range run as two launches: the reference's kernel with pointers that read what is
- * resident and note the pages that are not (a kernel without the miss path: no call, no stack, twice the waves), then a
- * kernel that has the miss path over the pages noted, 64 at a time, which also folds the checksum.  Same sum, same number
+ * resident and note the pages that are not (a kernel without the miss path: no call, no stack, twice the waves; it holds
+ * no reference on a page, it looks at the page's descriptor before and after reading it, and a page whose two looks
+ * differ is noted like one that was not there), then a kernel that has the miss path over the pages noted, 64 at a time,
+ * which also folds the checksum.  Same sum, same number
  * of accesses counted; pages that the second launch loads are asked for as batches before they are read, so their
  * accesses count as hits.  Modes 5 and 6 are modes 0 and 1 as one launch of the kernel that can miss (what arrays of
  * several ranges get under modes 0 and 1). */

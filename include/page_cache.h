@@ -1545,7 +1545,14 @@ struct bam_ptr {
         view.flush_stats();
 #endif
     }
-    __forceinline__ __host__ __device__ void init(array_d_t<T>* a) { array = a; }
+    __forceinline__ __host__ __device__ void init(array_d_t<T>* a)
+    {
+        array = a;
+#if defined(__HIP_DEVICE_COMPILE__)
+        /* a deferring pointer is for arrays of one range: its descriptor is read here, once */
+        if constexpr (DEFER) { range_id = 0; view.load(a->d_ranges); }
+#endif
+    }
 
     __forceinline__ __host__ __device__ void fini(void)
     {
@@ -1561,12 +1568,7 @@ struct bam_ptr {
     {
 #if defined(__HIP_DEVICE_COMPILE__)
         if constexpr (DEFER) {
-            if (!view.holds(i)) {
-                page = nullptr; start = end = 0; addr = nullptr;
-                range_id = array->find_range(i);
-                if (range_id == -1) { view.r = nullptr; return nullptr; }
-                view.load(array->d_ranges + range_id);
-            }
+            if (!view.holds(i)) { page = nullptr; start = end = 0; addr = nullptr; return nullptr; }       /* past the array's one range */
             return move_window(i);
         }
 #endif
