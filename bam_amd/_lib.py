@@ -32,6 +32,7 @@ SIGNATURES = {
     "bam_page_cache_create_multi": (c_int, [P(c_vp), c_u64, c_u64, c_u32, P(c_vp), c_u32, c_u64]),
     "bam_page_cache_destroy": (None, [c_vp]),
     "bam_page_cache_info": (c_int, [c_vp, P(c_u64)]),
+    "bam_page_cache_export_dmabuf": (c_int, [c_vp, P(c_int), P(c_u64)]),
     "bam_page_cache_flush": (c_int, [c_vp]),
     "bam_page_cache_profile": (c_int, [c_vp, P(c_u64), c_int]),
     "bam_range_create": (c_int, [P(c_vp), c_u64, c_u64, c_u64, c_u64, c_u64, c_u64, c_vp, c_u32, c_int]),

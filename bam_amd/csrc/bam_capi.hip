@@ -1178,6 +1178,23 @@ int bam_page_cache_info(bam_page_cache_t* pc, uint64_t* out)
     return 0;
 }
 
+int bam_page_cache_export_dmabuf(bam_page_cache_t* pc, int* fd, uint64_t* bytes)
+{
+    if (!pc || !fd || !bytes) return fail(EINVAL, "bam_page_cache_export_dmabuf: null argument");
+    *fd = -1;
+    /* whole host pages: the allocation behind the slots is at least that large (allocations are made in larger pieces) */
+    const uint64_t want = (pc->pc->pdt.n_pages * pc->pc->pdt.page_size + 4095ull) & ~4095ull;
+    int out = -1;
+    const hipError_t e = hipMemGetHandleForAddressRange(&out, (hipDeviceptr_t)pc->pc->pdt.base_addr, want, hipMemRangeHandleTypeDmaBufFd, 0);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(ENOTSUP, std::string("bam_page_cache_export_dmabuf: ") + hipGetErrorString(e));
+    }
+    *fd = out;
+    *bytes = want;
+    return 0;
+}
+
 int bam_page_cache_profile(bam_page_cache_t* pc, uint64_t* out32, int reset)
 {
     if (!pc || !out32) return fail(EINVAL, "bam_page_cache_profile: null argument");

@@ -8,6 +8,7 @@ buffers are torch tensors on the handle's device; 64-bit unsigned data travels
 as int64 tensors (same bits).
 """
 import ctypes
+import errno
 import os
 
 import torch
@@ -128,6 +129,15 @@ class PageCache:
 
     def flush(self):
         _chk(self.L.bam_page_cache_flush(self.h), "bam_page_cache_flush")
+
+    def export_dmabuf(self):
+        """(fd, bytes) of a dma-buf descriptor over the cache's slots, or None where device memory cannot be exported."""
+        fd, n = ctypes.c_int(-1), c_u64(0)
+        rc = self.L.bam_page_cache_export_dmabuf(self.h, ctypes.byref(fd), ctypes.byref(n))
+        if rc == errno.ENOTSUP:
+            return None
+        _chk(rc, "bam_page_cache_export_dmabuf")
+        return fd.value, n.value
 
     def profile(self, reset=True):
         """Miss-path phase timers (only a library built with -DBAM_PROFILE fills them)."""

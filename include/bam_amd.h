@@ -75,6 +75,13 @@ int bam_page_cache_create_multi(bam_page_cache_t** out, uint64_t page_size, uint
 void bam_page_cache_destroy(bam_page_cache_t* pc);
 /* out[5]: n_pages, page_size, wave_batch, staged(0/1), of every 8 read batches how many bypass the staging pages */
 int bam_page_cache_info(bam_page_cache_t* pc, uint64_t* out);
+/* The cache's payload memory as a dma-buf descriptor (reference: module/map.c:307-399, where the kernel module pins the
+ * GPU pages of the cache with nvidia_p2p_get_pages and hands the controller their bus addresses).  This is the GPU side
+ * of the same step for a real NVMe device here: the descriptor names the device memory [base, base + *bytes) of the
+ * cache's slots, and whoever drives the device (a kernel driver, VFIO / iommufd) imports it, maps it for the device's
+ * DMA and supplies the bus addresses to nvm_dma_map_device.  The caller owns *fd and closes it.  ENOTSUP where the
+ * runtime or the machine cannot export device memory. */
+int bam_page_cache_export_dmabuf(bam_page_cache_t* pc, int* fd, uint64_t* bytes);
 int bam_page_cache_flush(bam_page_cache_t* pc);
 /* phase timers of the miss path (100 MHz ticks, summed over the batches of the cache's first controller), non-zero only in
  * a library built with -DBAM_PROFILE (make prof); out32[0..8]: I/O batches, commands, ticks waiting for command ids,

@@ -374,6 +374,29 @@ def test_pages_above_two_controller_pages_use_prp_lists(bam, page, stage):
         assert np.array_equal(r.backing(1 << 15), vals) and not r.c.aborted()
 
 
+def test_cache_slots_exported_as_a_dma_buf(bam):
+    """The GPU side of putting a real NVMe device behind the cache: the slots' device memory as a dma-buf descriptor that
+    a driver can import and map for the device's DMA.  Where the runtime exports it, the descriptor is a real one, as
+    large as the slots; where it cannot, the call says so (ENOTSUP) and nothing else changes."""
+    import os
+    import stat
+    with Rig(bam, 64 << 20) as r:
+        a = r.array(1 << 20, 4096, 256)
+        pc = r.objs[0][2]
+        got = pc.export_dmabuf()
+        if got is None:
+            pytest.skip("this runtime does not export device memory")
+        fd, n = got
+        try:
+            assert fd >= 0 and n == 256 * 4096
+            st = os.fstat(fd)
+            assert not stat.S_ISREG(st.st_mode) and not stat.S_ISDIR(st.st_mode)
+            assert st.st_size in (0, n) or st.st_size >= n
+        finally:
+            os.close(fd)
+        assert a.read(1 << 16, stride=16) == oracle.lib().bo_store_sum(SEED, 0, 16, 1 << 16)      # the cache works as before
+
+
 # ---------------------------------------------------------------- cache / pattern streaming
 
 @pytest.mark.parametrize("mode", [0, 1, 2, 3, 4, 5, 6])
