@@ -48,6 +48,7 @@ SIGNATURES = {
     "bam_cache_stream": (c_int, [c_vp, c_u64, c_u64, c_vp, c_int, c_vp, c_vp]),
     "bam_block_io": (c_int, [c_vp, c_vp, c_u64, c_u32, c_vp, c_int, c_int, c_u32, c_vp]),
     "bam_warp_memcpy": (c_int, [c_vp, c_vp, c_u64, c_u64, c_vp]),
+    "bam_unheld_window_cases": (c_int, [c_vp, c_u64, P(c_u32)]),
     "bam_block_checksum": (c_int, [c_vp, c_u64, c_u32, c_vp, c_vp]),
     "bam_bfs": (c_int, [c_vp, c_vp, c_u64, c_u64, c_vp, c_u32, P(c_u32), c_vp]),
     "bam_cc": (c_int, [c_vp, c_vp, c_u64, c_vp, c_u32, P(c_u32), c_vp]),

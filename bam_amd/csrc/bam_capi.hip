@@ -734,6 +734,41 @@ __global__ void k_warp_memcpy(uint64_t* dst, const uint64_t* src, uint64_t n, ui
 }
 
 /*
+ * The second look of a pointer that holds no reference, case by case: one wave opens a window on a resident page through
+ * bam_ptr<T, true>, the page's descriptor is changed under it in one way (by the same wave: nobody else uses the cache
+ * meanwhile), still() is asked, and the descriptor is put back.  out[c] = 1 if still() found the window standing.
+ * Cases: 0 nothing changed, 1 other readers' references (the count in the state word), 2 the dirty bit, 3 busy, 4 not
+ * valid, 5 another slot, 6 the same slot loaded once more.  Only the first three may stand.
+ */
+__global__ void k_unheld_window_cases(array_d_t<uint64_t>* dr, uint64_t page, uint32_t* out)
+{
+    uint64_t* const word = (uint64_t*)(dr->d_ranges[0].pages + page);
+    const uint64_t epp = dr->d_ranges[0].n_elems_per_page;
+    for (uint32_t c = 0; c < 7; c++) {
+        bam_ptr<uint64_t, true> ptr(dr);
+        const uint64_t x = ptr[page * epp + bam::lane()];
+        const bool opened = !ptr.missed;
+        const uint64_t was = __hip_atomic_load(word, __ATOMIC_RELAXED, BAM_AGENT);
+        uint64_t now = was;
+        switch (c) {
+        case 1: now = was + 5; break;
+        case 2: now = was | (uint64_t)DIRTY; break;
+        case 3: now = was | (uint64_t)BUSY; break;
+        case 4: now = was & ~(uint64_t)VALID; break;
+        case 5: now = was ^ (1ull << 32); break;
+        case 6: now = was + (1ull << (32 + BAM_SLOT_BITS)); break;
+        default: break;
+        }
+        if (bam::lane() == 0) { __hip_atomic_store(word, now, __ATOMIC_RELAXED, BAM_AGENT); bam::fence_meta(); }
+        const bool stands = ptr.still();
+        if (bam::lane() == 0) { __hip_atomic_store(word, was, __ATOMIC_RELAXED, BAM_AGENT); bam::fence_meta(); }
+        const uint64_t all = bam::ballot(stands), none = bam::ballot(!stands);
+        /* every lane says the same; a window that fell must have set `missed`, one that stands must not */
+        if (bam::lane() == 0) out[c] = (opened && none == 0 && !ptr.missed ? 1u : 0u) | (opened && all == 0 && ptr.missed ? 2u : 0u) | (x == 0 && !opened ? 4u : 0u);
+    }
+}
+
+/*
  * Raw block reads with several commands in flight per thread (benchmarks/iodepth-block/main.cu:97-140): thread t
  * submits its `depth` commands with access_data_async (command k of thread t reads LBA lbas[t * depth + k] into slot
  * t * depth + k), then collects them with poll_async.  Wave w uses queue pair w mod n_qps.
@@ -1526,6 +1561,20 @@ int bam_warp_memcpy(uint64_t* d_dst, const uint64_t* d_src, uint64_t n_words, ui
     BAM_API_BEGIN
     hipLaunchKernelGGL(k_warp_memcpy, dim3(1), dim3(BAM_WAVE_SIZE), 0, (hipStream_t)stream, d_dst, d_src, n_words, lanes);
     hip_err_chk(hipGetLastError());
+    BAM_API_END
+}
+
+int bam_unheld_window_cases(bam_array_t* a, uint64_t page, uint32_t* host_out7)
+{
+    if (!a || !host_out7) return fail(EINVAL, "bam_unheld_window_cases: null argument");
+    if (a->a->adt.n_ranges != 1 || page >= a->a->h_ranges[0].page_count) return fail(EINVAL, "bam_unheld_window_cases: an array of one range and a page of it");
+    BAM_API_BEGIN
+    BufferPtr out = createBuffer(7 * sizeof(uint32_t), 0);
+    hip_err_chk(hipMemset(out.get(), 0, 7 * sizeof(uint32_t)));
+    hipLaunchKernelGGL(k_unheld_window_cases, dim3(1), dim3(BAM_WAVE_SIZE), 0, 0, a->a->d_array_ptr, page, (uint32_t*)out.get());
+    hip_err_chk(hipGetLastError());
+    hip_err_chk(hipDeviceSynchronize());
+    hip_err_chk(hipMemcpy(host_out7, out.get(), 7 * sizeof(uint32_t), hipMemcpyDeviceToHost));
     BAM_API_END
 }
 

@@ -271,6 +271,12 @@ class Array:
     def write(self, n_reqs, values, assignment=None, stride=1, block_size=64):
         _chk(self.L.bam_array_write(self.h, n_reqs, _ptr(assignment), stride, _ptr(values), block_size, _stream()), "bam_array_write")
 
+    def unheld_window_cases(self, page):
+        """bam_unheld_window_cases: what the second look of the pointer that holds no reference says, case by case."""
+        out = (c_u32 * 7)()
+        _chk(self.L.bam_unheld_window_cases(self.h, page, out), "bam_unheld_window_cases")
+        return list(out)
+
     def stream_async(self, n_waves, n_pages_per_wave, d_sum, assignment=None, mode=2):
         _chk(self.L.bam_cache_stream(self.h, n_waves, n_pages_per_wave, _ptr(assignment), mode, _ptr(d_sum), _stream()), "bam_cache_stream")
 

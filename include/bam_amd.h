@@ -197,6 +197,12 @@ int bam_store_read_file(bam_ctrl_t* c, bam_page_cache_t* pc, const char* path, u
 /* util.h's warp_memcpy (reference include/util.h:102-117) run by one wave with the lanes named in the bit mask `lanes`
  * active: n_words 64-bit words from d_src to d_dst */
 int bam_warp_memcpy(uint64_t* d_dst, const uint64_t* d_src, uint64_t n_words, uint64_t lanes, void* stream);
+/* The second look of bam_ptr<T, true> (the pointer of the first streaming launch, which holds no reference) case by case
+ * on a resident page of an array of one range, with nothing else using the cache: host_out7[c] is 1 if the window stood
+ * and 2 if it fell after the page's descriptor was changed under it in way c: 0 not at all, 1 other readers' references,
+ * 2 the dirty bit, 3 busy, 4 not valid, 5 another slot, 6 the same slot loaded once more (4 if the page was not resident
+ * to begin with).  A test helper; no counterpart in the reference. */
+int bam_unheld_window_cases(bam_array_t* a, uint64_t page, uint32_t* host_out7);
 /* sum of the 64-bit words of the first req_bytes of slots 0..n-1, one sum per slot */
 int bam_block_checksum(bam_page_cache_t* pc, uint64_t n_slots, uint32_t req_bytes, uint64_t* d_out, void* stream);
 

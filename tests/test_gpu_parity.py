@@ -426,6 +426,21 @@ def test_page_streaming_modes(bam, mode):
         assert not r.c.aborted()
 
 
+def test_second_look_of_the_pointer_that_holds_no_reference(bam):
+    """bam_ptr<T, true> opens its window on a look at the page's descriptor and what was read counts once still() finds the
+    descriptor as it was.  Changed under the window, one way at a time: other readers' references and the dirty bit do
+    not matter; busy, not valid, another slot, or the same slot after one more load of the page, and the window falls
+    (a mask with a bit too few in it would let one of them through)."""
+    with Rig(bam, 8 << 20) as r:
+        a = r.array(1 << 18, 4096, 64)
+        assert a.read(1 << 15, stride=1) == oracle.lib().bo_store_sum(SEED, 0, 1, 1 << 15)      # pages 0..63 are resident now
+        assert a.unheld_window_cases(5) == [1, 1, 1, 2, 2, 2, 2]
+        assert a.unheld_window_cases(63) == [1, 1, 1, 2, 2, 2, 2]
+        assert a.unheld_window_cases(200) == [4] * 7                                              # never loaded: no window at all
+        assert a.read(1 << 15, stride=1) == oracle.lib().bo_store_sum(SEED, 0, 1, 1 << 15) and a.stats()["read_io_cnt"] == 64
+        assert not r.c.aborted()
+
+
 def test_streaming_what_is_resident_while_another_stream_evicts(bam):
     """Two arrays behind one cache, each driven from a stream of its own.  One is streamed element by element (modes 0 and
     1: first a launch that reads what is resident without holding it, every page confirmed by a second look at its
