@@ -288,6 +288,13 @@ def main():
         assert L.bam_gather_kernel(ctypes.c_void_p(probe.data_ptr()), ctypes.c_void_p(idx_hit.data_ptr()), ctypes.c_uint64(N_READS), ctypes.byref(ms_c), stream) == 0
     gather_hit["plain_gather_reads_per_s"] = N_READS / ms_c.value * 1e3
     gather_hit["frac_of_plain_gather"] = gather_hit["reads_per_s"] / gather_hit["plain_gather_reads_per_s"]
+    # a random 8-byte read costs a 128-byte line from HBM whatever the load's cache policy (FETCH_SIZE: 136 bytes per read with
+    # the 8-byte index, profiles/k_array_read_counters_hits_and_random_gather.md), so the roofline of any gather is
+    # 8 TB/s / 128 B = 62.5 G reads/s, and in bytes moved the gather through the cache runs at this fraction of the HBM peak
+    gather_hit["hbm_bytes_per_read"] = 136
+    gather_hit["hbm_GBps_by_traffic"] = gather_hit["reads_per_s"] * 136 / 1e9
+    gather_hit["frac_of_hbm_peak_by_traffic"] = gather_hit["hbm_GBps_by_traffic"] / HBM_PEAK_GBS
+    gather_hit["plain_gather_frac_of_hbm_peak_by_traffic"] = gather_hit["plain_gather_reads_per_s"] * 136 / 1e9 / HBM_PEAK_GBS
     # what the counted hit path pays: a take-and-drop pair of atomics per read on words scattered like the page descriptors
     table = torch.zeros(CACHE_PAGES, dtype=torch.int64, device=dev)
     pages_hit = idx_hit // 512
